@@ -1,0 +1,554 @@
+"""CPU restatement of one PBG training step (test infrastructure only).
+
+Every function cites the reference lines it follows.  The tensor ops are
+issued in the reference's order so that fp32 rounding stays comparable, and
+uniform-negative indices are INPUTS (the reference draws them with
+torch.randint inside the model, model.py:70-75), so that the oracle and the
+GPU path can be fed identical negatives.
+"""
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+OPERATOR_NAMES = ("none", "diagonal", "translation", "linear", "complex_diagonal")
+COMPARATOR_NAMES = ("dot", "cos", "l2")
+LOSS_NAMES = ("ranking", "logistic", "softmax")
+
+
+@dataclass
+class StepConfig:
+    """The fields of the reference's ConfigSchema that parameterise the step
+    (config.py:115-347): operator / comparator / loss_fn / margin /
+    num_batch_negs / num_uniform_negs / disable_*_negs / dynamic_relations /
+    lr / relation_lr, plus per-relation weights (RelationSchema.weight)."""
+
+    dim: int
+    operator: str = "none"
+    comparator: str = "dot"
+    loss: str = "ranking"
+    margin: float = 0.1
+    num_batch_negs: int = 50
+    num_uniform_negs: int = 50
+    disable_lhs_negs: bool = False
+    disable_rhs_negs: bool = False
+    dynamic: bool = False
+    num_relations: int = 1
+    lr: float = 0.1
+    relation_lr: Optional[float] = None
+    relation_weights: Sequence[float] = field(default_factory=lambda: [1.0])
+
+    def chunking(self, num_pos: int) -> Tuple[int, int, str]:
+        """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
+        if self.num_batch_negs == 0:
+            chunk = min(self.num_uniform_negs, num_pos)
+            mode = "uniform"
+        else:
+            chunk = min(self.num_batch_negs, num_pos)
+            mode = "batch_uniform"
+        if num_pos == 0 or chunk == 0:
+            return chunk, 0, mode
+        return chunk, (num_pos - 1) // chunk + 1, mode
+
+
+# --------------------------------------------------------------------------
+# operators (operators.py:49-157 static, :197-338 dynamic)
+# --------------------------------------------------------------------------
+
+def init_operator_params(name: str, dim: int, num_ops: int) -> Dict[str, torch.Tensor]:
+    """Initial parameters with a leading [num_ops] axis (operators.py:62,76,
+    90,137-138 and :215,234,255-257,315-316).  Standard mode keeps one
+    operator object per relation; stacking them changes nothing because a
+    relation with a zero gradient is left untouched by Adagrad."""
+    if name == "none":
+        return {}
+    if name == "diagonal":
+        return {"diagonal": torch.ones(num_ops, dim)}
+    if name == "translation":
+        return {"translation": torch.zeros(num_ops, dim)}
+    if name == "linear":
+        return {"linear_transformation": torch.eye(dim).repeat(num_ops, 1, 1)}
+    if name == "complex_diagonal":
+        if dim % 2 != 0:
+            raise ValueError(
+                "Need even dimension as 1st half is real and 2nd half is imaginary coordinates"
+            )
+        return {"real": torch.ones(num_ops, dim // 2), "imag": torch.zeros(num_ops, dim // 2)}
+    raise NotImplementedError(f"Unknown operator {name}")
+
+
+def apply_operator(
+    name: str,
+    embs: torch.Tensor,
+    params: Dict[str, torch.Tensor],
+    rel,
+) -> torch.Tensor:
+    """y = op_rel(x) on the last axis.  ``rel`` is an int (one operator for
+    every row: operators.py:53-157) or a LongTensor shaped like
+    embs.shape[:-1] (one operator per row: operators.py:200-338)."""
+    dim = embs.shape[-1]
+    if name == "none":
+        return embs
+    pick = (lambda p: p[rel])
+    if name == "diagonal":
+        return pick(params["diagonal"]) * embs
+    if name == "translation":
+        return embs + pick(params["translation"])
+    if name == "linear":
+        mat = pick(params["linear_transformation"])
+        return torch.matmul(mat, embs.unsqueeze(-1)).squeeze(-1)
+    if name == "complex_diagonal":
+        half = dim // 2
+        real_a, imag_a = embs[..., :half], embs[..., half:]
+        real_b, imag_b = pick(params["real"]), pick(params["imag"])
+        prod = torch.empty_like(embs)
+        prod[..., :half] = real_a * real_b - imag_a * imag_b
+        prod[..., half:] = real_a * imag_b + imag_a * real_b
+        return prod
+    raise NotImplementedError(f"Unknown operator {name}")
+
+
+# --------------------------------------------------------------------------
+# comparators (model.py:159-278)
+# --------------------------------------------------------------------------
+
+def comparator_prepare(name: str, embs: torch.Tensor) -> torch.Tensor:
+    """model.py:161-162 (dot), :187-192 (cos), :251-252 (l2)."""
+    if name == "cos":
+        norm = embs.norm(2, dim=-1)
+        return embs * norm.reciprocal().unsqueeze(-1)
+    if name in ("dot", "l2"):
+        return embs
+    raise NotImplementedError(f"Unknown comparator {name}")
+
+
+def _f32(x: torch.Tensor) -> torch.Tensor:
+    """The reference's ``.float()`` casts (model.py:177,268,827-829); float64
+    inputs are let through so that tests can take finite differences."""
+    return x if x.dtype == torch.float64 else x.float()
+
+
+def _all_pairs_l2(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """model.py:215-246: ||a||^2 - 2ab + ||b||^2 through baddbmm, clamped at
+    1e-30, square-rooted."""
+    a_squared = a.norm(dim=-1).pow(2)
+    b_squared = b.norm(dim=-1).pow(2)
+    res = torch.baddbmm(b_squared.unsqueeze(-2), a, b.transpose(-2, -1), alpha=-2).add_(
+        a_squared.unsqueeze(-1)
+    )
+    return res.clamp_min_(1e-30).sqrt_()
+
+
+def comparator_scores(
+    name: str,
+    lhs_pos: torch.Tensor,
+    rhs_pos: torch.Tensor,
+    lhs_neg: torch.Tensor,
+    rhs_neg: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(pos[C,P], lhs_neg_scores[C,P,Ln] = rhs_pos x lhs_neg,
+    rhs_neg_scores[C,P,Rn] = lhs_pos x rhs_neg); model.py:164-182, 194-212,
+    254-278.  Note the cross pairing of the negative scores."""
+    if lhs_pos.dim() != 3 or rhs_pos.shape != lhs_pos.shape:
+        raise TypeError("Shape doesn't match")
+    c, p, d = lhs_pos.shape
+    if lhs_neg.dim() != 3 or lhs_neg.shape[0] != c or lhs_neg.shape[2] != d:
+        raise TypeError("Shape doesn't match")
+    if rhs_neg.dim() != 3 or rhs_neg.shape[0] != c or rhs_neg.shape[2] != d:
+        raise TypeError("Shape doesn't match")
+    if name in ("dot", "cos"):
+        pos = (_f32(lhs_pos) * _f32(rhs_pos)).sum(-1)
+        lneg = torch.bmm(rhs_pos, lhs_neg.transpose(-1, -2))
+        rneg = torch.bmm(lhs_pos, rhs_neg.transpose(-1, -2))
+        return pos, lneg, rneg
+    if name == "l2":
+        pos = (_f32(lhs_pos) - _f32(rhs_pos)).pow(2).sum(dim=-1).clamp_min(1e-30).sqrt().neg()
+        lneg = _all_pairs_l2(rhs_pos, lhs_neg).neg()
+        rneg = _all_pairs_l2(lhs_pos, rhs_neg).neg()
+        return pos, lneg, rneg
+    raise NotImplementedError(f"Unknown comparator {name}")
+
+
+# --------------------------------------------------------------------------
+# losses (losses.py:53-161)
+# --------------------------------------------------------------------------
+
+def loss_value(
+    name: str,
+    pos: torch.Tensor,
+    neg: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    margin: float = 0.1,
+) -> torch.Tensor:
+    num_pos = pos.shape[0]
+    if pos.dim() != 1 or neg.dim() != 2 or neg.shape[0] != num_pos:
+        raise TypeError("Shape doesn't match")
+    num_neg = neg.shape[1]
+    if name == "logistic":  # losses.py:55-82
+        neg_weight = 1 / num_neg if num_neg > 0 else 0
+        pos_loss = F.binary_cross_entropy_with_logits(
+            pos, pos.new_ones(()).expand(num_pos), reduction="sum", weight=weight
+        )
+        neg_loss = F.binary_cross_entropy_with_logits(
+            neg,
+            neg.new_zeros(()).expand(num_pos, num_neg),
+            reduction="sum",
+            weight=weight.unsqueeze(-1) if weight is not None else None,
+        )
+        return pos_loss + neg_weight * neg_loss
+    if name == "ranking":  # losses.py:91-124
+        if num_pos == 0 or num_neg == 0:
+            return torch.zeros((), requires_grad=True)
+        per = F.margin_ranking_loss(
+            neg,
+            pos.unsqueeze(1),
+            target=pos.new_full((1, 1), -1, dtype=torch.float),
+            margin=margin,
+            reduction="none",
+        )
+        if weight is not None:
+            per = per * weight.unsqueeze(-1)
+        return per.sum()
+    if name == "softmax":  # losses.py:129-161
+        if num_pos == 0 or num_neg == 0:
+            return torch.zeros((), requires_grad=True)
+        scores = torch.cat([pos.unsqueeze(1), neg.logsumexp(dim=1, keepdim=True)], dim=1)
+        per = F.cross_entropy(scores, pos.new_zeros((num_pos,), dtype=torch.long), reduction="none")
+        if weight is not None:
+            per = per * weight
+        return per.sum()
+    raise NotImplementedError(f"Unknown loss {name}")
+
+
+# --------------------------------------------------------------------------
+# the model forward (model.py:478-856)
+# --------------------------------------------------------------------------
+
+@dataclass
+class Scores:
+    lhs_pos: torch.Tensor
+    rhs_pos: torch.Tensor
+    lhs_neg: torch.Tensor
+    rhs_neg: torch.Tensor
+
+
+def _adjust(cfg: StepConfig, embs, rel, op_params) -> torch.Tensor:
+    """model.py:478-506 without global_emb / half precision: operator then
+    comparator.prepare.  ``op_params is None`` means "no operator"."""
+    if op_params is not None:
+        embs = apply_operator(cfg.operator, embs, op_params, rel)
+    return comparator_prepare(cfg.comparator, embs)
+
+
+def _direction_agnostic(
+    cfg: StepConfig,
+    num_pos: int,
+    src_pos: torch.Tensor,
+    dst_pos: torch.Tensor,
+    src_uniform: Optional[torch.Tensor],
+    dst_uniform: Optional[torch.Tensor],
+    rel,
+    dst_op_params,
+    chunk_size: int,
+    src_method: str,
+    dst_method: str,
+):
+    """model.py:764-856.  ``src_uniform`` / ``dst_uniform`` are the raw rows
+    of the uniformly sampled entities, [C,U,D] (model.py:544,550)."""
+    dim = src_pos.shape[-1]
+    src_pos = _adjust(cfg, src_pos, rel, None)
+    dst_pos = _adjust(cfg, dst_pos, rel, dst_op_params)
+    num_chunks = (num_pos - 1) // chunk_size + 1
+    pad = num_chunks * chunk_size - num_pos
+    if pad > 0:
+        src_pos = torch.cat((src_pos, src_pos.new_zeros(()).expand(pad, dim)), dim=0)
+        dst_pos = torch.cat((dst_pos, dst_pos.new_zeros(()).expand(pad, dim)), dim=0)
+    src_pos = src_pos.view(num_chunks, chunk_size, dim)
+    dst_pos = dst_pos.view(num_chunks, chunk_size, dim)
+    last = num_pos - (num_chunks - 1) * chunk_size
+
+    def negatives(pos_embs, uniform, method, op_params):
+        # model.py:508-622 (NONE / UNIFORM / BATCH_UNIFORM branches)
+        masked_batch = False
+        if method == "none":
+            neg = pos_embs.new_empty((num_chunks, 0, dim))
+        elif method == "uniform":
+            neg = _adjust(cfg, uniform, rel_for_uniform, op_params)
+        elif method == "batch_uniform":
+            neg = pos_embs
+            if uniform is not None and uniform.shape[1] > 0:
+                neg = torch.cat([pos_embs, _adjust(cfg, uniform, rel_for_uniform, op_params)], dim=1)
+            masked_batch = True
+        else:
+            raise NotImplementedError(method)
+        return neg, masked_batch
+
+    # The operator is only ever applied to uniform negatives in standard mode,
+    # where rel is an int; dynamic mode passes no operator for the negatives.
+    rel_for_uniform = rel
+    src_neg, src_masked = negatives(src_pos, src_uniform, src_method, None)
+    dst_neg, dst_masked = negatives(dst_pos, dst_uniform, dst_method, dst_op_params)
+
+    pos_scores, src_neg_scores, dst_neg_scores = comparator_scores(
+        cfg.comparator, src_pos, dst_pos, src_neg, dst_neg
+    )
+    pos_scores = _f32(pos_scores)
+    src_neg_scores = _f32(src_neg_scores)
+    dst_neg_scores = _f32(dst_neg_scores)
+
+    idx = torch.arange(chunk_size, dtype=torch.long)
+    for scores, masked in ((src_neg_scores, src_masked), (dst_neg_scores, dst_masked)):
+        if masked:  # model.py:566-580 and :836-839
+            scores[: num_chunks - 1, idx, idx] = -1e9
+            scores[-1, idx[:last], idx[:last]] = -1e9
+            scores[-1, :last, last:chunk_size] = -1e9
+
+    pos_scores = pos_scores.flatten(0, 1)[:num_pos]
+    src_neg_scores = src_neg_scores.flatten(0, 1)[:num_pos]
+    dst_neg_scores = dst_neg_scores.flatten(0, 1)[:num_pos]
+    return pos_scores, src_neg_scores, dst_neg_scores
+
+
+def model_forward(
+    cfg: StepConfig,
+    lhs_pos: torch.Tensor,
+    rhs_pos: torch.Tensor,
+    lhs_uniform: Optional[torch.Tensor],
+    rhs_uniform: Optional[torch.Tensor],
+    rel,
+    lhs_op_params: Optional[Dict[str, torch.Tensor]],
+    rhs_op_params: Optional[Dict[str, torch.Tensor]],
+) -> Scores:
+    """MultiRelationEmbedder.forward (model.py:624-762) on already gathered
+    rows.  lhs_pos/rhs_pos: [B,D] raw rows; *_uniform: [C,U,D] raw rows of the
+    uniform negatives (None when U == 0 or the side is disabled); rel: int in
+    standard mode, LongTensor[B] in dynamic mode."""
+    num_pos = lhs_pos.shape[0]
+    chunk_size, _, mode = cfg.chunking(num_pos)
+    lhs_method = "none" if cfg.disable_lhs_negs else mode
+    rhs_method = "none" if cfg.disable_rhs_negs else mode
+    if not cfg.dynamic:
+        if lhs_op_params:
+            raise RuntimeError(
+                "In non-dynamic relation mode there should be only a right-hand side operator"
+            )
+        if not isinstance(rel, int):
+            raise TypeError("All positive pairs must come from the same relation")
+        pos, lneg, rneg = _direction_agnostic(
+            cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, rhs_uniform, rel,
+            rhs_op_params if cfg.operator != "none" else None,
+            chunk_size, lhs_method, rhs_method,
+        )
+        return Scores(pos, pos, lneg, rneg)
+    if isinstance(rel, int):
+        raise TypeError("Need relation for each positive pair")
+    # model.py:721-754: forward edges (operator on rhs, negatives on lhs),
+    # then reverse edges (operator on lhs, negatives on rhs).
+    lpos, lneg, _ = _direction_agnostic(
+        cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, None, rel,
+        rhs_op_params if cfg.operator != "none" else None,
+        chunk_size, lhs_method, "none",
+    )
+    rpos, rneg, _ = _direction_agnostic(
+        cfg, num_pos, rhs_pos, lhs_pos, rhs_uniform, None, rel,
+        lhs_op_params if cfg.operator != "none" else None,
+        chunk_size, rhs_method, "none",
+    )
+    return Scores(lpos, rpos, lneg, rneg)
+
+
+# --------------------------------------------------------------------------
+# optimizers (row_adagrad.py:80-107, async_adagrad.py:51-85)
+# --------------------------------------------------------------------------
+
+def row_adagrad_sparse(weight: torch.Tensor, state_sum: torch.Tensor, grad: torch.Tensor, lr: float) -> None:
+    """row_adagrad.py:80-96 on a sparse COO gradient, in place."""
+    if grad._indices().numel() == 0:
+        return
+    grad = grad.coalesce()
+    idx = grad._indices()[0]
+    vals = grad._values()
+    local_g = state_sum[idx]
+    delta = (vals * vals).mean(1)
+    state_sum.index_add_(0, idx, delta)
+    local_g += delta
+    std = local_g.sqrt_().add_(1e-10).unsqueeze(1)
+    weight.index_add_(0, idx, -lr * vals / std)
+
+
+def row_adagrad_dense(weight: torch.Tensor, state_sum: torch.Tensor, grad: torch.Tensor, lr: float) -> None:
+    """row_adagrad.py:97-107, in place."""
+    local_g = state_sum.clone()
+    delta = (grad * grad).mean(1)
+    state_sum += delta
+    local_g += delta
+    std = local_g.sqrt().add_(1e-10)
+    weight.addcdiv_(grad, std.unsqueeze(1), value=-lr)
+
+
+def async_adagrad_dense(param: torch.Tensor, state_sum: torch.Tensor, grad: torch.Tensor, lr: float, eps: float = 1e-10) -> None:
+    """async_adagrad.py:75-85 with lr_decay = 0, in place."""
+    local_g = state_sum.clone()
+    delta = grad * grad
+    state_sum.add_(delta)
+    local_g += delta
+    std = local_g.sqrt().add_(eps)
+    param.addcdiv_(grad, std, value=-lr)
+
+
+# --------------------------------------------------------------------------
+# one training step (train_cpu.py:86-112 + batching.py:139-150)
+# --------------------------------------------------------------------------
+
+@dataclass
+class TrainState:
+    """Tables and optimizer state the step mutates.  ``w_rhs is w_lhs`` when
+    both sides share one entity type (model.py:454-472 wraps the same
+    Parameter for both sides)."""
+
+    w_lhs: torch.Tensor
+    g_lhs: torch.Tensor
+    w_rhs: torch.Tensor
+    g_rhs: torch.Tensor
+    lhs_op: Dict[str, torch.Tensor] = field(default_factory=dict)
+    rhs_op: Dict[str, torch.Tensor] = field(default_factory=dict)
+    lhs_op_sum: Dict[str, torch.Tensor] = field(default_factory=dict)
+    rhs_op_sum: Dict[str, torch.Tensor] = field(default_factory=dict)
+
+    @property
+    def shared(self) -> bool:
+        return self.w_lhs is self.w_rhs
+
+
+def make_state(cfg: StepConfig, w_lhs: torch.Tensor, w_rhs: Optional[torch.Tensor] = None) -> TrainState:
+    shared = w_rhs is None
+    g_lhs = torch.zeros(w_lhs.shape[0])
+    st = TrainState(
+        w_lhs=w_lhs,
+        g_lhs=g_lhs,
+        w_rhs=w_lhs if shared else w_rhs,
+        g_rhs=g_lhs if shared else torch.zeros(w_rhs.shape[0]),
+    )
+    st.rhs_op = init_operator_params(cfg.operator, cfg.dim, cfg.num_relations)
+    st.rhs_op_sum = {k: torch.zeros_like(v) for k, v in st.rhs_op.items()}
+    if cfg.dynamic:
+        st.lhs_op = init_operator_params(cfg.operator, cfg.dim, cfg.num_relations)
+        st.lhs_op_sum = {k: torch.zeros_like(v) for k, v in st.lhs_op.items()}
+    return st
+
+
+@dataclass
+class StepOutput:
+    loss: float
+    violators_lhs: int
+    violators_rhs: int
+    count: int
+    scores: Optional[Scores] = None
+
+
+@dataclass
+class StepGrads:
+    """Gradients of one batch, before any update is applied."""
+
+    sparse_lhs: Optional[torch.Tensor]  # sparse COO on w_lhs (also carries rhs grads when shared)
+    sparse_rhs: Optional[torch.Tensor]
+    lhs_op: Dict[str, torch.Tensor]
+    rhs_op: Dict[str, torch.Tensor]
+
+
+def forward_backward(
+    cfg: StepConfig,
+    st: TrainState,
+    lhs: torch.Tensor,
+    rhs: torch.Tensor,
+    rel,
+    uniform_lhs: Optional[torch.Tensor],
+    uniform_rhs: Optional[torch.Tensor],
+    weight: Optional[torch.Tensor] = None,
+    keep_scores: bool = False,
+) -> Tuple[StepOutput, StepGrads]:
+    """zero_grad -> forward -> calc_loss -> stats -> backward
+    (train_cpu.py:89-105).  uniform_*: LongTensor[C,U] entity indices."""
+    w_l = st.w_lhs.detach().requires_grad_(True)
+    w_r = w_l if st.shared else st.w_rhs.detach().requires_grad_(True)
+    lhs_op = {k: v.detach().requires_grad_(True) for k, v in st.lhs_op.items()}
+    rhs_op = {k: v.detach().requires_grad_(True) for k, v in st.rhs_op.items()}
+
+    lhs_pos = F.embedding(lhs, w_l, sparse=True)
+    rhs_pos = F.embedding(rhs, w_r, sparse=True)
+    lhs_u = (
+        F.embedding(uniform_lhs, w_l, sparse=True)
+        if uniform_lhs is not None and not cfg.disable_lhs_negs and uniform_lhs.numel() > 0
+        else None
+    )
+    rhs_u = (
+        F.embedding(uniform_rhs, w_r, sparse=True)
+        if uniform_rhs is not None and not cfg.disable_rhs_negs and uniform_rhs.numel() > 0
+        else None
+    )
+    scores = model_forward(cfg, lhs_pos, rhs_pos, lhs_u, rhs_u, rel, lhs_op or None, rhs_op or None)
+
+    # batching.py:139-150
+    lhs_loss = loss_value(cfg.loss, scores.lhs_pos, scores.lhs_neg, weight, cfg.margin)
+    rhs_loss = loss_value(cfg.loss, scores.rhs_pos, scores.rhs_neg, weight, cfg.margin)
+    relation = rel if isinstance(rel, int) else 0
+    loss = cfg.relation_weights[relation] * (lhs_loss + rhs_loss)
+
+    out = StepOutput(
+        loss=float(loss),
+        violators_lhs=int((scores.lhs_neg > scores.lhs_pos.unsqueeze(1)).sum()),
+        violators_rhs=int((scores.rhs_neg > scores.rhs_pos.unsqueeze(1)).sum()),
+        count=int(lhs.shape[0]),
+        scores=Scores(
+            scores.lhs_pos.detach(), scores.rhs_pos.detach(),
+            scores.lhs_neg.detach(), scores.rhs_neg.detach(),
+        ) if keep_scores else None,
+    )
+    loss.backward()
+    grads = StepGrads(
+        sparse_lhs=w_l.grad,
+        sparse_rhs=None if st.shared else w_r.grad,
+        lhs_op={k: (v.grad if v.grad is not None else torch.zeros_like(v)) for k, v in lhs_op.items()},
+        rhs_op={k: (v.grad if v.grad is not None else torch.zeros_like(v)) for k, v in rhs_op.items()},
+    )
+    return out, grads
+
+
+def apply_grads(cfg: StepConfig, st: TrainState, grads: StepGrads) -> None:
+    """model_optimizer.step then the per-entity RowAdagrad steps
+    (train_cpu.py:106-110; lr choice train_cpu.py:224-228)."""
+    rel_lr = cfg.relation_lr if cfg.relation_lr is not None else cfg.lr
+    with torch.no_grad():
+        for params, sums, g in (
+            (st.lhs_op, st.lhs_op_sum, grads.lhs_op),
+            (st.rhs_op, st.rhs_op_sum, grads.rhs_op),
+        ):
+            for name, p in params.items():
+                async_adagrad_dense(p, sums[name], g[name], rel_lr)
+        if grads.sparse_lhs is not None:
+            row_adagrad_sparse(st.w_lhs, st.g_lhs, grads.sparse_lhs, cfg.lr)
+        if grads.sparse_rhs is not None:
+            row_adagrad_sparse(st.w_rhs, st.g_rhs, grads.sparse_rhs, cfg.lr)
+
+
+def train_step(cfg, st, lhs, rhs, rel, uniform_lhs, uniform_rhs, weight=None, keep_scores=False) -> StepOutput:
+    """Trainer._process_one_batch (train_cpu.py:86-112) for one batch."""
+    out, grads = forward_backward(cfg, st, lhs, rhs, rel, uniform_lhs, uniform_rhs, weight, keep_scores)
+    apply_grads(cfg, st, grads)
+    return out
+
+
+def train_lockstep(cfg, st, batches: List[tuple]) -> List[StepOutput]:
+    """K HOGWILD workers (train_cpu.py:849-884) in the one interleaving that is
+    deterministic: every worker reads the tables, then every worker writes, in
+    worker order.  ``batches`` is a list of (lhs, rhs, rel, uniform_lhs,
+    uniform_rhs) tuples, one per worker."""
+    outs, all_grads = [], []
+    for b in batches:
+        out, grads = forward_backward(cfg, st, *b)
+        outs.append(out)
+        all_grads.append(grads)
+    for grads in all_grads:
+        apply_grads(cfg, st, grads)
+    return outs
