@@ -1,0 +1,201 @@
+/*
+ * pbg_hip.h -- C ABI of the MI355X (gfx950) implementation of the
+ * PyTorch-BigGraph per-bucket training step.
+ *
+ * The reference has no C ABI of its own: the path is Python over PyTorch ops,
+ * plus one pybind11 module (`_C`, torchbiggraph/util.cpp:425-460).  Each entry
+ * point below names the reference interface it replaces.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - all floats are fp32, all indices int64, tensors are row-major contiguous;
+ *   - the caller owns every buffer, including workspaces (query the *_bytes
+ *     function, allocate, pass in); the library never allocates device memory;
+ *   - work is enqueued on `stream` (a hipStream_t) and the call returns without
+ *     synchronising;
+ *   - return value: PBG_OK or a negative pbg_status; pbg_last_error() gives the
+ *     message of the last failure on the calling thread.
+ */
+#ifndef PBG_HIP_H
+#define PBG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* pbg_stream_t; /* hipStream_t */
+
+typedef enum pbg_status {
+  PBG_OK = 0,
+  PBG_ERR_INVALID = -1,     /* bad argument (shape, enum, null pointer) */
+  PBG_ERR_WORKSPACE = -2,   /* workspace missing or too small */
+  PBG_ERR_LAUNCH = -3,      /* HIP reported an error at launch */
+  PBG_ERR_UNSUPPORTED = -4  /* a combination this build does not implement */
+} pbg_status;
+
+/* Names follow the reference's registries: OPERATORS / DYNAMIC_OPERATORS
+ * (operators.py:46,194), COMPARATORS (model.py:156), LOSS_FUNCTIONS
+ * (losses.py:50). */
+typedef enum pbg_operator {
+  PBG_OP_NONE = 0,
+  PBG_OP_DIAGONAL = 1,
+  PBG_OP_TRANSLATION = 2,
+  PBG_OP_LINEAR = 3,
+  PBG_OP_COMPLEX_DIAGONAL = 4
+} pbg_operator;
+typedef enum pbg_comparator { PBG_CMP_DOT = 0, PBG_CMP_COS = 1, PBG_CMP_L2 = 2 } pbg_comparator;
+typedef enum pbg_loss { PBG_LOSS_RANKING = 0, PBG_LOSS_LOGISTIC = 1, PBG_LOSS_SOFTMAX = 2 } pbg_loss;
+
+int pbg_version(void);
+const char* pbg_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Row gather.  Replaces SimpleEmbedding.get = F.embedding(idx, W, sparse=True)
+ * (model.py:60-61) and the gather half of sample_entities (model.py:70-75).
+ * out[i, :] = table[idx[i], :], bit-exact.  An index outside [0, num_rows)
+ * writes a zero row and sets *oob_flag (if not null) to 1.
+ * ---------------------------------------------------------------------- */
+int pbg_gather_rows(const float* table, int64_t num_rows, int32_t dim, const int64_t* idx, int64_t n,
+                    float* out, int32_t* oob_flag, pbg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * RowAdagrad.  Replaces RowAdagrad.step (row_adagrad.py:48-109).
+ * Sparse branch (:80-96): `idx[n]` / `grad_rows[n, dim]` are the uncoalesced
+ * COO gradient; duplicates are summed (sort by index, segmented sum) before
+ *   delta = mean_d(g^2); G[r] += delta; W[r] -= lr * g / (sqrt(G_old + delta) + 1e-10).
+ * Dense branch (:97-107): `grad[num_rows, dim]`.
+ * ---------------------------------------------------------------------- */
+size_t pbg_row_adagrad_sparse_workspace_bytes(int64_t n);
+int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
+                           const int64_t* idx, const float* grad_rows, int64_t n, float lr,
+                           void* workspace, size_t workspace_bytes, pbg_stream_t stream);
+int pbg_row_adagrad_dense(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
+                          const float* grad, float lr, pbg_stream_t stream);
+
+/* AsyncAdagrad dense step for operator parameters (async_adagrad.py:75-85,
+ * lr_decay = 0): G += g^2; p -= lr * g / (sqrt(G) + eps). */
+int pbg_async_adagrad_dense(float* param, float* state_sum, const float* grad, int64_t numel,
+                            float lr, float eps, pbg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Batched fp32 matrix product on the matrix cores.  Replaces the torch.bmm /
+ * torch.baddbmm call sites of the comparators (model.py:179-180,209-210,234)
+ * and the matmul of the linear operator (operators.py:94-99).
+ *   C[i] (m x n, row-major, ldc) = alpha * A[i] * B[i] + beta * C[i],  i < batch
+ *   a_kmajor = 0: A(r, x) = a[r * lda + x];  1: A(r, x) = a[x * lda + r]
+ *   b_kmajor = 0: B(x, j) = b[j * ldb + x];  1: B(x, j) = b[x * ldb + j]
+ * stride_* are the distances between consecutive matrices, in floats.
+ * ---------------------------------------------------------------------- */
+int pbg_gemm_f32(const float* a, const float* b, float* c, int32_t batch, int32_t m, int32_t n, int32_t k,
+                 int32_t lda, int32_t ldb, int32_t ldc, int64_t stride_a, int64_t stride_b,
+                 int64_t stride_c, int32_t a_kmajor, int32_t b_kmajor, float alpha, float beta,
+                 pbg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * The training step.  Replaces Trainer._process_one_batch (train_cpu.py:86-112):
+ * MultiRelationEmbedder.forward (model.py:624-856), calc_loss
+ * (batching.py:139-150), the Stats counters, autograd backward, AsyncAdagrad on
+ * the operator parameters and RowAdagrad on the embedding tables.
+ *
+ * One call processes `num_workers` batches of `batch_size` edges each in
+ * lock-step: every batch reads the tables as they are on entry, then the
+ * updates of batch 0, 1, ... are applied in that order.  num_workers = 1 is the
+ * reference's single-process sequence; num_workers = K is K HOGWILD workers
+ * (train_cpu.py:849-884) in the one interleaving that is deterministic.
+ * ---------------------------------------------------------------------- */
+typedef struct pbg_step_desc {
+  int32_t dim;              /* D */
+  int32_t num_workers;      /* K >= 1 */
+  int32_t batch_size;       /* B >= 1, edges per batch */
+  int32_t num_batch_negs;   /* config.num_batch_negs; 0 selects uniform-only negatives (model.py:651-656) */
+  int32_t num_uniform_negs; /* config.num_uniform_negs (U) */
+  int32_t disable_lhs_negs; /* config.disable_lhs_negs */
+  int32_t disable_rhs_negs; /* config.disable_rhs_negs */
+  int32_t op;               /* pbg_operator */
+  int32_t dynamic;          /* 0: one relation per batch, operator on rhs (model.py:666-703);
+                               1: relation per edge, operators on both sides (model.py:705-758) */
+  int32_t num_relations;    /* leading axis of the operator parameters and of relation_weights */
+  int32_t comparator;       /* pbg_comparator */
+  int32_t loss;             /* pbg_loss */
+  float margin;             /* ranking loss margin (config.margin) */
+  float lr;                 /* config.lr, RowAdagrad */
+  float relation_lr;        /* config.relation_lr or config.lr, AsyncAdagrad (train_cpu.py:224-228) */
+  int32_t shared_table;     /* 1: lhs and rhs index the same table (w_rhs == w_lhs, g_rhs == g_lhs) */
+  int64_t num_lhs_rows;     /* rows of w_lhs */
+  int64_t num_rhs_rows;     /* rows of w_rhs */
+} pbg_step_desc;
+
+typedef struct pbg_step_buffers {
+  float* w_lhs;               /* [num_lhs_rows, D] */
+  float* g_lhs;               /* [num_lhs_rows]  RowAdagrad state["sum"] */
+  float* w_rhs;               /* [num_rhs_rows, D] */
+  float* g_rhs;               /* [num_rhs_rows] */
+  const int64_t* lhs;         /* [K, B] */
+  const int64_t* rhs;         /* [K, B] */
+  const int64_t* rel;         /* standard: [K]; dynamic: [K, B] */
+  const int64_t* uniform_lhs; /* [K, C, U] entity indices (model.py:70-75), null if unused */
+  const int64_t* uniform_rhs; /* [K, C, U] */
+  const float* edge_weight;   /* [K, B] or null (EdgeList.weight, edgelist.py:51-95) */
+  const float* relation_weights; /* [num_relations] (batching.py:144-148) */
+  /* Operator parameters, leading axis [num_relations]; p0 = diagonal |
+   * translation | linear_transformation | real, p1 = imag; s0/s1 = AsyncAdagrad
+   * state["sum"] of the same shape.  lhs_* only in dynamic mode. */
+  float* rhs_op_p0; float* rhs_op_p1; float* rhs_op_s0; float* rhs_op_s1;
+  float* lhs_op_p0; float* lhs_op_p1; float* lhs_op_s0; float* lhs_op_s1;
+  float* loss_out;            /* [K] loss of each batch (Stats.loss) */
+  int64_t* violators_out;     /* [K, 2] violators_lhs, violators_rhs */
+  void* workspace;
+  size_t workspace_bytes;
+} pbg_step_buffers;
+
+size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc);
+int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream);
+
+/* MultiRelationEmbedder.forward alone (model.py:624-762): scores only, tables
+ * untouched.  lhs_pos/rhs_pos: [K, B]; lhs_neg: [K, B, Nl]; rhs_neg: [K, B, Nr]
+ * with N = (num_batch_negs ? min(num_batch_negs, B) : 0) + U, or 0 when that
+ * side is disabled; masked entries hold -1e9. */
+int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos,
+                      float* rhs_pos, float* lhs_neg, float* rhs_neg, pbg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Permutation helpers.  Replace the `_C` module (util.cpp:425-460).
+ * ---------------------------------------------------------------------- */
+/* _C.reverse_permutation (util.cpp:104-125): out[perm[i]] = i. */
+int pbg_reverse_permutation(const int64_t* perm, int64_t n, int64_t* out, pbg_stream_t stream);
+
+/* _C.shuffle (util.cpp:127-220): rows[perm[i]] <- rows[i], result left in
+ * `rows`.  `scratch` holds n * row_bytes bytes.  row_bytes must be a multiple
+ * of 4.  An out-of-range perm entry sets *oob_flag and drops that row. */
+int pbg_shuffle_rows(void* rows, int64_t n, int64_t row_bytes, const int64_t* perm, void* scratch,
+                     int32_t* oob_flag, pbg_stream_t stream);
+
+/* _C.randperm (util.cpp:14-102): a uniform random permutation of [0, n).  The
+ * reference's bit pattern depends on its thread count; only the contract is
+ * kept.  Deterministic in (n, seed). */
+size_t pbg_randperm_workspace_bytes(int64_t n);
+int pbg_randperm(int64_t n, uint64_t seed, int64_t* out, void* workspace, size_t workspace_bytes,
+                 pbg_stream_t stream);
+
+/* _C.sub_bucket (util.cpp:260-423): stable partition of a bucket's edges into
+ * num_lhs_parts x num_rhs_parts sub-buckets.  lhs_perm_ptrs / rhs_perm_ptrs:
+ * device arrays of num_relations device pointers to the per-relation entity
+ * permutations; *_part_sizes: device arrays [num_relations] of
+ * ceil(entity_count / parts).  offsets_out[parts_l * parts_r + 1] (device)
+ * receives the start of every sub-bucket in the outputs. */
+size_t pbg_sub_bucket_workspace_bytes(int64_t n);
+int pbg_sub_bucket(const int64_t* lhs_in, const int64_t* rhs_in, const int64_t* rel_in, int64_t n,
+                   int32_t num_relations, const int64_t* const* lhs_perm_ptrs,
+                   const int64_t* const* rhs_perm_ptrs, const int64_t* lhs_part_sizes,
+                   const int64_t* rhs_part_sizes, int32_t num_lhs_parts, int32_t num_rhs_parts,
+                   int32_t dynamic_relations, int64_t* lhs_out, int64_t* rhs_out, int64_t* rel_out,
+                   int64_t* offsets_out, int32_t* error_flag, void* workspace, size_t workspace_bytes,
+                   pbg_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PBG_HIP_H */

@@ -1,0 +1,62 @@
+// Internal declarations shared by the HIP translation units of libpbg_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/pbg_hip.h"
+
+namespace pbg {
+
+constexpr int kWave = 64;
+
+// Records `msg` for pbg_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+// Turns the pending HIP launch error (if any) into a pbg_status.
+int check_launch(const char* what);
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int bits_for(uint64_t max_value) {  // number of bits needed to hold max_value
+  int b = 0;
+  while (b < 64 && (max_value >> b) != 0) ++b;
+  return b;
+}
+
+// ---- device radix sort of (uint64 key, uint32 value) pairs ----------------
+// LSD radix sort, 8 bits per pass, stable.  Sorts on key bits [0, key_bits).
+// The result ends up in (keys_out, vals_out); (keys_in, vals_in) are clobbered.
+// `temp` holds sort_temp_bytes(n) bytes.
+size_t sort_temp_bytes(int64_t n);
+int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n,
+               int key_bits, void* temp, hipStream_t stream);
+
+// ---- segmented RowAdagrad over sorted (row << kbits | worker) keys ---------
+// keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim].  A key's
+// row field addresses table 0 for row < rows0, table 1 (row - rows0) for
+// row < rows0 + rows1, and is ignored beyond.
+int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits,
+                       const float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
+                       float* g1, int64_t rows1, float lr, hipStream_t stream);
+
+// ---- plain fp32 batched GEMM on MFMA ----------------------------------------
+// C[b] (M x N, row-major, ldc) = alpha * A[b] * B[b] + beta * C[b], for b in [0, batch).
+// a_kmajor = 0: A(m,k) = A[m * lda + k];  1: A(m,k) = A[k * lda + m].
+// b_kmajor = 0: B(k,n) = B[n * ldb + k];  1: B(k,n) = B[k * ldb + n].
+struct GemmArgs {
+  const float* a; const float* b; float* c;
+  int64_t stride_a, stride_b, stride_c;  // per-batch strides in floats
+  int lda, ldb, ldc;
+  int m, n, k;
+  int batch;
+  int a_kmajor, b_kmajor;
+  float alpha, beta;
+  // optional gather of the B operand: B[b] starts b_index[b] * b_index_stride
+  // floats further (one operator matrix per relation)
+  const int64_t* b_index = nullptr;
+  int64_t b_index_stride = 0;
+};
+int gemm_f32(const GemmArgs& args, hipStream_t stream);
+
+}  // namespace pbg

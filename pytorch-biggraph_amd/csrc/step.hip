@@ -1,0 +1,1182 @@
+// The per-batch training step of PyTorch-BigGraph on one MI355X.
+//
+// One call handles K batches ("workers") that all read the tables as they are
+// on entry; their updates are then applied in worker order.  Stages, each one
+// kernel (or one batched GEMM) over all K batches:
+//
+//   prep      gather rows, apply the relation operator and comparator.prepare,
+//             lay the results out as per-chunk operand matrices; emit the
+//             (row, worker) sort keys of every gradient row        [HBM bound]
+//   scores    S = A * N^T per chunk and side                        [MFMA]
+//   loss      mask, comparator epilogue (l2), loss, dLoss/dS in place, positive
+//             scores and their gradients, violator counts           [L2 bound]
+//   backward  dA = dS * N, dN = dS^T * A per chunk and side          [MFMA]
+//   rowback   chain rule through prepare and the operator back to raw rows,
+//             one gradient row per gathered row                      [HBM bound]
+//   params    operator-parameter gradients and their Adagrad step
+//   update    radix sort of the keys, then a segmented RowAdagrad    [HBM bound]
+//
+// Layout of a row inside a wave: lane l owns elements {h, H + h} for
+// h = l, l + 64, ... < H with H = ceil(D / 2), i.e. both halves of a complex
+// pair sit in the same lane.
+#include <cstring>
+
+#include "pbg_internal.h"
+
+namespace pbg {
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kWavesPerBlock = kRowThreads / kWave;
+
+struct SideCtx {
+  const float* w;       // embedding table of this side
+  const int64_t* idx;   // [K, B] positive entities
+  const int64_t* uidx;  // [K, C, U] uniform negatives (null if u == 0)
+  int64_t key_base;     // offset of this table in the sort-key row space
+  int64_t num_rows;
+  int nb, u, nn;        // batch-negative / uniform / total negative columns of this side
+  int stride_p;         // rows per chunk of the buffer that holds the positives
+  int alias;            // positives are the first P rows of the negatives matrix
+  float *xn, *xp, *xa;  // prepared negatives matrix, positives, operated positives (dynamic)
+  float *an, *ap, *aa;  // per-row aux of the above: 1/norm (cos) or squared norm (l2)
+  float *dxn, *dxp, *dxa;
+  float* s;             // [K*C, P, nn] scores against this side's negatives, then dLoss/dS
+  float* rs;            // [K*C*P] row sums of dLoss/d(squared distance) (l2)
+  int slot_pos, slot_uni;
+  int has_op;           // an operator acts on this side's positives
+  int op_uniform;       // ... and on its uniform negatives (standard mode)
+  const float *p0, *p1; // operator parameters
+  float *xraw, *z, *dz; // [K, op_rows, D] staging of operator inputs / outputs / output grads
+  int op_rows;
+  int plain_written, opd_written;  // dxp / dxa were produced by a GEMM
+};
+
+struct StepCtx {
+  int D, K, B, P, C, U, last, dynamic, op, cmp, loss, num_relations;
+  float margin;
+  SideCtx side[2];
+  const int64_t* rel;
+  const float* edge_weight;
+  const float* rel_weights;
+  float* pos[2];   // [K*C*P] positive score paired with lhs negatives / rhs negatives
+  float* dpos[2];  // gradients of the above (standard mode: only [0], already summed)
+  float* lossrow;  // [K*C*P]
+  int rk;          // gradient rows per batch
+  int kbits;
+  float* gr;       // [K*rk, D] gradient rows
+  uint64_t* keys;
+  uint32_t* vals;
+  unsigned long long* violators;  // [K, 2]
+  float* loss_out;                // [K]
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+template <int NVH>
+struct RowV {
+  float a[2][NVH];
+};
+
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> row_zero() {
+  RowV<NVH> r;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) r.a[0][v] = r.a[1][v] = 0.f;
+  return r;
+}
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> row_load(const float* __restrict__ p, int D, int H, int lane) {
+  RowV<NVH> r;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    const int h = v * kWave + lane;
+    r.a[0][v] = (h < H) ? p[h] : 0.f;
+    r.a[1][v] = (h < H && H + h < D) ? p[H + h] : 0.f;
+  }
+  return r;
+}
+template <int NVH>
+__device__ __forceinline__ void row_store(float* __restrict__ p, const RowV<NVH>& r, int D, int H, int lane) {
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    const int h = v * kWave + lane;
+    if (h < H) p[h] = r.a[0][v];
+    if (h < H && H + h < D) p[H + h] = r.a[1][v];
+  }
+}
+template <int NVH>
+__device__ __forceinline__ float row_dot(const RowV<NVH>& x, const RowV<NVH>& y) {  // per-lane partial
+  float acc = 0.f;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) acc += x.a[0][v] * y.a[0][v] + x.a[1][v] * y.a[1][v];
+  return acc;
+}
+template <int NVH>
+__device__ __forceinline__ void row_axpy(RowV<NVH>& y, float alpha, const RowV<NVH>& x) {
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    y.a[0][v] += alpha * x.a[0][v];
+    y.a[1][v] += alpha * x.a[1][v];
+  }
+}
+
+// y = op_r(x) for the element-wise operators (operators.py:59-84,128-157 and
+// their dynamic twins :212-249,306-338).  `linear` is a GEMM and not handled here.
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> op_forward(int op, const RowV<NVH>& x, const float* __restrict__ p0,
+                                                const float* __restrict__ p1, int64_t r, int D, int H, int lane) {
+  RowV<NVH> y = x;
+  if (op == PBG_OP_DIAGONAL || op == PBG_OP_TRANSLATION) {
+    const float* p = p0 + r * D;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      const int h = v * kWave + lane;
+      const float q0 = (h < H) ? p[h] : 0.f;
+      const float q1 = (h < H && H + h < D) ? p[H + h] : 0.f;
+      if (op == PBG_OP_DIAGONAL) {
+        y.a[0][v] = q0 * x.a[0][v];
+        y.a[1][v] = q1 * x.a[1][v];
+      } else {
+        y.a[0][v] = x.a[0][v] + q0;
+        y.a[1][v] = x.a[1][v] + q1;
+      }
+    }
+  } else if (op == PBG_OP_COMPLEX_DIAGONAL) {
+    const float* re = p0 + r * H;
+    const float* im = p1 + r * H;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      const int h = v * kWave + lane;
+      const float br = (h < H) ? re[h] : 0.f;
+      const float bi = (h < H) ? im[h] : 0.f;
+      y.a[0][v] = x.a[0][v] * br - x.a[1][v] * bi;
+      y.a[1][v] = x.a[0][v] * bi + x.a[1][v] * br;
+    }
+  }
+  return y;
+}
+
+// dx = (d op_r / dx)^T dz for the element-wise operators.
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> op_backward(int op, const RowV<NVH>& dz, const float* __restrict__ p0,
+                                                 const float* __restrict__ p1, int64_t r, int D, int H, int lane) {
+  RowV<NVH> dx = dz;
+  if (op == PBG_OP_DIAGONAL) {
+    const float* p = p0 + r * D;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      const int h = v * kWave + lane;
+      dx.a[0][v] = ((h < H) ? p[h] : 0.f) * dz.a[0][v];
+      dx.a[1][v] = ((h < H && H + h < D) ? p[H + h] : 0.f) * dz.a[1][v];
+    }
+  } else if (op == PBG_OP_COMPLEX_DIAGONAL) {
+    const float* re = p0 + r * H;
+    const float* im = p1 + r * H;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      const int h = v * kWave + lane;
+      const float br = (h < H) ? re[h] : 0.f;
+      const float bi = (h < H) ? im[h] : 0.f;
+      dx.a[0][v] = br * dz.a[0][v] + bi * dz.a[1][v];
+      dx.a[1][v] = br * dz.a[1][v] - bi * dz.a[0][v];
+    }
+  }
+  return dx;
+}
+
+// comparator.prepare (model.py:161-162,187-192,251-252), in place; returns the
+// per-row aux value: 1/norm for cos, norm^2 for l2 (model.py:228-229).
+template <int NVH>
+__device__ __forceinline__ float prepare_row(int cmp, RowV<NVH>& y) {
+  if (cmp == PBG_CMP_DOT) return 0.f;
+  const float nrm = sqrtf(wave_sum(row_dot(y, y)));
+  if (cmp == PBG_CMP_COS) {
+    const float inv = 1.0f / nrm;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      y.a[0][v] *= inv;
+      y.a[1][v] *= inv;
+    }
+    return inv;
+  }
+  return nrm * nrm;
+}
+
+// gradient through comparator.prepare: cos: dz = (dy - y (y . dy)) / norm.
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> prepare_backward(int cmp, const RowV<NVH>& dy, const RowV<NVH>& y, float aux) {
+  if (cmp != PBG_CMP_COS) return dy;
+  const float dot = wave_sum(row_dot(y, dy));
+  RowV<NVH> dz;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    dz.a[0][v] = aux * (dy.a[0][v] - y.a[0][v] * dot);
+    dz.a[1][v] = aux * (dy.a[1][v] - y.a[1][v] * dot);
+  }
+  return dz;
+}
+
+__device__ __forceinline__ int64_t clamp_index(int64_t v, int64_t n) { return v < 0 ? 0 : (v >= n ? n - 1 : v); }
+
+// ---------------------------------------------------------------------------
+// prep
+// ---------------------------------------------------------------------------
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int CP = c.C * c.P;
+  const int J0 = CP + c.C * c.side[0].u;
+  const int J = J0 + CP + c.C * c.side[1].u;
+  if (job >= (int64_t)c.K * J) return;
+  const int k = (int)(job / J);
+  int r = (int)(job % J);
+  const int s = r >= J0;
+  if (s) r -= J0;
+  const SideCtx& sd = c.side[s];
+  const int D = c.D, H = (D + 1) / 2;
+
+  if (r < CP) {
+    const int cc = r / c.P, i = r % c.P;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    float* xp_row = sd.xp + (kc * sd.stride_p + i) * D;
+    float* ap = sd.ap ? sd.ap + kc * sd.stride_p + i : nullptr;
+    float* xa_row = c.dynamic ? sd.xa + (kc * c.P + i) * D : nullptr;
+    float* aa = (c.dynamic && sd.aa) ? sd.aa + kc * c.P + i : nullptr;
+    if (r >= c.B) {  // padding of an incomplete last chunk (model.py:790-798)
+      const RowV<NVH> zero = row_zero<NVH>();
+      row_store<NVH>(xp_row, zero, D, H, lane);
+      if (ap && lane == 0) *ap = 0.f;
+      if (xa_row) row_store<NVH>(xa_row, zero, D, H, lane);
+      if (aa && lane == 0) *aa = 0.f;
+      return;
+    }
+    const int64_t e = (int64_t)k * c.B + r;
+    const int64_t id = clamp_index(sd.idx[e], sd.num_rows);
+    const int64_t rel = clamp_index(c.dynamic ? c.rel[e] : c.rel[k], c.num_relations);
+    const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+    if (lane == 0) {
+      const int64_t slot = (int64_t)k * c.rk + sd.slot_pos + r;
+      c.keys[slot] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
+      c.vals[slot] = (uint32_t)slot;
+    }
+    if (c.dynamic || !sd.has_op) {
+      RowV<NVH> y = x;
+      const float aux = prepare_row<NVH>(c.cmp, y);
+      row_store<NVH>(xp_row, y, D, H, lane);
+      if (ap && lane == 0) *ap = aux;
+    }
+    if (sd.has_op) {
+      if (c.op == PBG_OP_LINEAR) {
+        row_store<NVH>(sd.xraw + ((int64_t)k * sd.op_rows + r) * D, x, D, H, lane);
+      } else {
+        RowV<NVH> y = op_forward<NVH>(c.op, x, sd.p0, sd.p1, rel, D, H, lane);
+        const float aux = prepare_row<NVH>(c.cmp, y);
+        row_store<NVH>(c.dynamic ? xa_row : xp_row, y, D, H, lane);
+        float* auxdst = c.dynamic ? aa : ap;
+        if (auxdst && lane == 0) *auxdst = aux;
+      }
+    }
+  } else {
+    const int r2 = r - CP;
+    const int cc = r2 / sd.u, uu = r2 % sd.u;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    const int64_t id = clamp_index(sd.uidx[kc * c.U + uu], sd.num_rows);
+    const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+    if (lane == 0) {
+      const int64_t slot = (int64_t)k * c.rk + sd.slot_uni + r2;
+      c.keys[slot] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
+      c.vals[slot] = (uint32_t)slot;
+    }
+    if (sd.op_uniform && c.op == PBG_OP_LINEAR) {
+      row_store<NVH>(sd.xraw + ((int64_t)k * sd.op_rows + c.B + r2) * D, x, D, H, lane);
+      return;
+    }
+    RowV<NVH> y = x;
+    if (sd.op_uniform) {
+      const int64_t rel = clamp_index(c.rel[k], c.num_relations);
+      y = op_forward<NVH>(c.op, x, sd.p0, sd.p1, rel, D, H, lane);
+    }
+    const float aux = prepare_row<NVH>(c.cmp, y);
+    row_store<NVH>(sd.xn + (kc * sd.nn + sd.nb + uu) * D, y, D, H, lane);
+    if (sd.an && lane == 0) sd.an[kc * sd.nn + sd.nb + uu] = aux;
+  }
+}
+
+// comparator.prepare on the rows a `linear` operator produced (staging z), moved
+// to their operand positions.
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, int s) {
+  const int lane = threadIdx.x & 63;
+  const SideCtx& sd = c.side[s];
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * sd.op_rows) return;
+  const int k = (int)(job / sd.op_rows), r = (int)(job % sd.op_rows);
+  const int D = c.D, H = (D + 1) / 2;
+  RowV<NVH> y = row_load<NVH>(sd.z + job * D, D, H, lane);
+  const float aux = prepare_row<NVH>(c.cmp, y);
+  if (r < c.B) {
+    const int cc = r / c.P, i = r % c.P;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    if (c.dynamic) {
+      row_store<NVH>(sd.xa + (kc * c.P + i) * D, y, D, H, lane);
+      if (sd.aa && lane == 0) sd.aa[kc * c.P + i] = aux;
+    } else {
+      row_store<NVH>(sd.xp + (kc * sd.stride_p + i) * D, y, D, H, lane);
+      if (sd.ap && lane == 0) sd.ap[kc * sd.stride_p + i] = aux;
+    }
+  } else {
+    const int r2 = r - c.B;
+    const int cc = r2 / sd.u, uu = r2 % sd.u;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    row_store<NVH>(sd.xn + (kc * sd.nn + sd.nb + uu) * D, y, D, H, lane);
+    if (sd.an && lane == 0) sd.an[kc * sd.nn + sd.nb + uu] = aux;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// loss
+// ---------------------------------------------------------------------------
+// comparator on a matched pair (model.py:177,207,267-274)
+__device__ __forceinline__ float kappa(int cmp, const float* __restrict__ a, const float* __restrict__ b, int D,
+                                       int lane) {
+  float acc = 0.f;
+  if (cmp == PBG_CMP_L2) {
+    for (int d = lane; d < D; d += kWave) {
+      const float t = a[d] - b[d];
+      acc += t * t;
+    }
+    return -sqrtf(fmaxf(wave_sum(acc), 1e-30f));
+  }
+  for (int d = lane; d < D; d += kWave) acc += a[d] * b[d];
+  return wave_sum(acc);
+}
+
+__device__ __forceinline__ float softplusf(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float sigmoidf(float z) {
+  if (z >= 0.f) return 1.0f / (1.0f + expf(-z));
+  const float e = expf(z);
+  return e / (1.0f + e);
+}
+
+struct ScoreRow {
+  const float* raw;  // chunk score row, a.b for every comparator
+  const float* bn;   // squared norms of the negatives (l2)
+  float a2;          // squared norm of the positive operand (l2)
+  int cmp, nb, i, masked_from;  // batch-negative columns; own column; first padded column
+
+  // score of column j as the model returns it (model.py:234-246,836-839); `live`
+  // is false where the value is a constant with no gradient
+  __device__ __forceinline__ float at(int j, bool* live) const {
+    float t = raw[j];
+    bool ok = true;
+    if (cmp == PBG_CMP_L2) {
+      const float qd = fmaf(-2.0f, t, bn[j]) + a2;
+      ok = qd >= 1e-30f;
+      t = -sqrtf(fmaxf(qd, 1e-30f));
+    }
+    if (j < nb && (j == i || j >= masked_from)) {
+      t = -1e9f;
+      ok = false;
+    }
+    *live = ok;
+    return t;
+  }
+};
+
+__device__ __forceinline__ void positive_scores(const StepCtx& c, int64_t kc, int i, int lane, float* posv) {
+  const int D = c.D;
+  const float* lp = c.side[0].xp + (kc * c.side[0].stride_p + i) * D;
+  const float* rp = c.side[1].xp + (kc * c.side[1].stride_p + i) * D;
+  if (!c.dynamic) {
+    posv[0] = posv[1] = kappa(c.cmp, lp, rp, D, lane);
+  } else {
+    posv[0] = kappa(c.cmp, lp, c.side[1].xa + (kc * c.P + i) * D, D, lane);
+    posv[1] = kappa(c.cmp, rp, c.side[0].xa + (kc * c.P + i) * D, D, lane);
+  }
+}
+
+__device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t kc, int cc, int i) {
+  const SideCtx& sd = c.side[s];
+  const SideCtx& so = c.side[1 - s];
+  ScoreRow sr;
+  sr.raw = sd.s + (kc * c.P + i) * sd.nn;
+  sr.cmp = c.cmp;
+  sr.bn = nullptr;
+  sr.a2 = 0.f;
+  if (c.cmp == PBG_CMP_L2) {
+    sr.bn = sd.an + kc * sd.nn;
+    sr.a2 = c.dynamic ? so.aa[kc * c.P + i] : so.ap[kc * so.stride_p + i];
+  }
+  sr.nb = sd.nb;
+  sr.i = i;
+  sr.masked_from = (cc == c.C - 1) ? c.last : c.P;
+  return sr;
+}
+
+__global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int CP = c.C * c.P;
+  if (job >= (int64_t)c.K * CP) return;
+  const int k = (int)(job / CP), q = (int)(job % CP);
+  const int cc = q / c.P, i = q % c.P;
+  const int64_t kc = (int64_t)k * c.C + cc;
+  if (q >= c.B) {  // padded positive: its rows of dLoss/dS are zero
+    for (int s = 0; s < 2; ++s) {
+      const SideCtx& sd = c.side[s];
+      float* row = sd.s + (kc * c.P + i) * sd.nn;
+      for (int j = lane; j < sd.nn; j += kWave) row[j] = 0.f;
+      if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = 0.f;
+    }
+    if (lane == 0) {
+      c.lossrow[job] = 0.f;
+      c.dpos[0][job] = 0.f;
+      if (c.dynamic) c.dpos[1][job] = 0.f;
+      c.pos[0][job] = 0.f;
+      if (c.dynamic) c.pos[1][job] = 0.f;
+    }
+    return;
+  }
+  float posv[2];
+  positive_scores(c, kc, i, lane, posv);
+  const int64_t e = (int64_t)k * c.B + q;
+  float w = c.rel_weights[c.dynamic ? 0 : clamp_index(c.rel[k], c.num_relations)];
+  if (c.edge_weight) w *= c.edge_weight[e];
+
+  float loss_acc = 0.f;  // per-lane partial, unweighted
+  float dposv[2] = {0.f, 0.f};
+  for (int s = 0; s < 2; ++s) {
+    const SideCtx& sd = c.side[s];
+    const int nn = sd.nn;
+    const float pos = posv[s];
+    if (nn == 0) {
+      // losses.py:63,101-102,140-141: only the logistic loss keeps its positive term
+      if (c.loss == PBG_LOSS_LOGISTIC) {
+        if (lane == 0) loss_acc += softplusf(-pos);
+        dposv[s] = (sigmoidf(pos) - 1.0f) * w;
+      }
+      continue;
+    }
+    ScoreRow sr = score_row(c, s, kc, cc, i);
+    float* out = sd.s + (kc * c.P + i) * nn;
+    float dpos_part = 0.f, rowsum = 0.f;
+    int viol = 0;
+    float mx = pos, inv_z = 0.f;
+    const float inv_nn = 1.0f / (float)nn;
+    if (c.loss == PBG_LOSS_SOFTMAX) {
+      bool live;
+      for (int j = lane; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
+      mx = wave_max(mx);
+      float z = 0.f;
+      for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
+      z = wave_sum(z) + expf(pos - mx);
+      inv_z = 1.0f / z;
+      if (lane == 0) {
+        loss_acc += (mx + logf(z)) - pos;
+        dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+      }
+    } else if (c.loss == PBG_LOSS_LOGISTIC) {
+      if (lane == 0) {
+        loss_acc += softplusf(-pos);
+        dpos_part += (sigmoidf(pos) - 1.0f) * w;
+      }
+    }
+    for (int j = lane; j < nn; j += kWave) {
+      bool live;
+      const float t = sr.at(j, &live);
+      float g;
+      if (c.loss == PBG_LOSS_RANKING) {
+        // F.margin_ranking_loss(neg, pos, target=-1): max(0, (t - pos) + margin); the
+        // clamp lets the gradient through at exactly 0
+        const float x = (t - pos) + c.margin;
+        if (x > 0.f) loss_acc += x;
+        g = (x >= 0.f) ? w : 0.f;
+        dpos_part -= g;
+      } else if (c.loss == PBG_LOSS_LOGISTIC) {
+        loss_acc += softplusf(t) * inv_nn;
+        g = sigmoidf(t) * inv_nn * w;
+      } else {
+        g = expf(t - mx) * inv_z * w;
+      }
+      if (t > pos) ++viol;
+      if (!live) g = 0.f;
+      if (c.cmp == PBG_CMP_L2) {
+        // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq so that the
+        // backward GEMMs produce the cross terms of ||a||^2 - 2ab + ||b||^2
+        const float dq = live ? g * 0.5f / t : 0.f;
+        rowsum += dq;
+        out[j] = -2.0f * dq;
+      } else {
+        out[j] = g;
+      }
+    }
+    dposv[s] = wave_sum(dpos_part);
+    if (sd.rs) {
+      rowsum = wave_sum(rowsum);
+      if (lane == 0) sd.rs[kc * c.P + i] = rowsum;
+    }
+    int vtot = viol;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) vtot += __shfl_xor(vtot, off, 64);
+    if (lane == 0 && vtot > 0) atomicAdd(&c.violators[k * 2 + s], (unsigned long long)vtot);
+  }
+  const float loss_row = wave_sum(loss_acc) * w;
+  if (lane == 0) {
+    c.lossrow[job] = loss_row;
+    c.pos[0][job] = posv[0];
+    if (c.dynamic) {
+      c.pos[1][job] = posv[1];
+      c.dpos[0][job] = dposv[0];
+      c.dpos[1][job] = dposv[1];
+    } else {
+      c.dpos[0][job] = dposv[0] + dposv[1];
+    }
+  }
+}
+
+// loss_out[k] = sum of the batch's per-edge losses, in a fixed order
+__global__ __launch_bounds__(256) void loss_reduce_kernel(StepCtx c) {
+  __shared__ float sh[256];
+  const int CP = c.C * c.P;
+  const float* rows = c.lossrow + (int64_t)blockIdx.x * CP;
+  float acc = 0.f;
+  for (int q = threadIdx.x; q < CP; q += 256) acc += rows[q];
+  sh[threadIdx.x] = acc;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) sh[threadIdx.x] += sh[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) c.loss_out[blockIdx.x] = sh[0];
+}
+
+__global__ void zero_violators_kernel(unsigned long long* v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[i] = 0ull;
+}
+
+// forward-only output: de-chunked, masked scores (model.py:842-844)
+__global__ __launch_bounds__(kRowThreads) void scores_out_kernel(StepCtx c, float* __restrict__ lhs_pos,
+                                                                 float* __restrict__ rhs_pos,
+                                                                 float* __restrict__ lhs_neg,
+                                                                 float* __restrict__ rhs_neg) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.B) return;
+  const int k = (int)(job / c.B), q = (int)(job % c.B);
+  const int cc = q / c.P, i = q % c.P;
+  const int64_t kc = (int64_t)k * c.C + cc;
+  float posv[2];
+  positive_scores(c, kc, i, lane, posv);
+  if (lane == 0) {
+    lhs_pos[job] = posv[0];
+    rhs_pos[job] = posv[1];
+  }
+  for (int s = 0; s < 2; ++s) {
+    const int nn = c.side[s].nn;
+    if (nn == 0) continue;
+    ScoreRow sr = score_row(c, s, kc, cc, i);
+    float* out = (s == 0 ? lhs_neg : rhs_neg) + job * nn;
+    bool live;
+    for (int j = lane; j < nn; j += kWave) out[j] = sr.at(j, &live);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// rowback
+// ---------------------------------------------------------------------------
+// sum over the P rows of a chunk of column `col` of the stored -2 dLoss/dq
+__device__ __forceinline__ float column_sum(const float* __restrict__ s, int64_t kc, int P, int nn, int col, int lane) {
+  const float* base = s + kc * P * nn + col;
+  float acc = 0.f;
+  for (int r = lane; r < P; r += kWave) acc += base[(int64_t)r * nn];
+  return wave_sum(acc);
+}
+
+// dy += dpos * d kappa(self, other) / d self
+template <int NVH>
+__device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos, const RowV<NVH>& self,
+                                             const RowV<NVH>& other, float pos) {
+  if (cmp == PBG_CMP_L2) {
+    // kappa = -sqrt(max(sum (a-b)^2, 1e-30)); no gradient where the clamp is active
+    if (pos * pos <= 1e-30f) return;
+    const float coef = dpos / pos;
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      dy.a[0][v] += coef * (self.a[0][v] - other.a[0][v]);
+      dy.a[1][v] += coef * (self.a[1][v] - other.a[1][v]);
+    }
+  } else {
+    row_axpy<NVH>(dy, dpos, other);
+  }
+}
+
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int CP = c.C * c.P;
+  const int J0 = c.B + c.C * c.side[0].u;
+  const int J = J0 + c.B + c.C * c.side[1].u;
+  if (job >= (int64_t)c.K * J) return;
+  const int k = (int)(job / J);
+  int r = (int)(job % J);
+  const int s = r >= J0;
+  if (s) r -= J0;
+  const SideCtx& sd = c.side[s];
+  const SideCtx& so = c.side[1 - s];
+  const int D = c.D, H = (D + 1) / 2;
+  const bool l2 = c.cmp == PBG_CMP_L2;
+  const bool keep_dz = sd.dz != nullptr;
+
+  if (r < c.B) {
+    const int cc = r / c.P, i = r % c.P;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    const int64_t pq = (int64_t)k * CP + r;
+    const int64_t e = (int64_t)k * c.B + r;
+    const int64_t rel = clamp_index(c.dynamic ? c.rel[e] : c.rel[k], c.num_relations);
+    float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + r) * D;
+    const RowV<NVH> y1 = row_load<NVH>(sd.xp + (kc * sd.stride_p + i) * D, D, H, lane);
+    const float aux1 = sd.ap ? sd.ap[kc * sd.stride_p + i] : 0.f;
+    if (!c.dynamic) {
+      RowV<NVH> dy = sd.plain_written ? row_load<NVH>(sd.dxp + (kc * sd.stride_p + i) * D, D, H, lane)
+                                      : row_zero<NVH>();
+      if (l2) {
+        float coef = 0.f;
+        if (sd.nb > 0) coef -= column_sum(sd.s, kc, c.P, sd.nn, i, lane);
+        if (so.nn > 0) coef += 2.0f * so.rs[kc * c.P + i];
+        row_axpy<NVH>(dy, coef, y1);
+      }
+      const RowV<NVH> other = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq]);
+      const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
+      if (sd.has_op) {
+        if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz, D, H, lane);
+        if (c.op != PBG_OP_LINEAR)
+          row_store<NVH>(out, op_backward<NVH>(c.op, dz, sd.p0, sd.p1, rel, D, H, lane), D, H, lane);
+      } else {
+        row_store<NVH>(out, dz, D, H, lane);
+      }
+    } else {
+      // role 1: the plain row f(x), a batch negative of its own side and the
+      // partner of the other side's operated positive
+      RowV<NVH> dy = row_zero<NVH>();
+      if (sd.alias) {
+        dy = row_load<NVH>(sd.dxp + (kc * sd.stride_p + i) * D, D, H, lane);
+        if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, i, lane), y1);
+      }
+      const RowV<NVH> other = row_load<NVH>(so.xa + (kc * c.P + i) * D, D, H, lane);
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq]);
+      RowV<NVH> dx = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
+      // role 2: the operated row f(op(x)), scored against the other side's negatives
+      const RowV<NVH> y2 = row_load<NVH>(sd.xa + (kc * c.P + i) * D, D, H, lane);
+      const float aux2 = sd.aa ? sd.aa[kc * c.P + i] : 0.f;
+      RowV<NVH> dy2 = row_zero<NVH>();
+      if (sd.opd_written) {
+        dy2 = row_load<NVH>(sd.dxa + (kc * c.P + i) * D, D, H, lane);
+        if (l2) row_axpy<NVH>(dy2, 2.0f * so.rs[kc * c.P + i], y2);
+      }
+      const RowV<NVH> other2 = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
+      add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq]);
+      const RowV<NVH> dz2 = prepare_backward<NVH>(c.cmp, dy2, y2, aux2);
+      if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz2, D, H, lane);
+      if (c.op != PBG_OP_LINEAR) {
+        const RowV<NVH> dx2 = op_backward<NVH>(c.op, dz2, sd.p0, sd.p1, rel, D, H, lane);
+        row_axpy<NVH>(dx, 1.0f, dx2);
+      }
+      row_store<NVH>(out, dx, D, H, lane);
+    }
+  } else {
+    const int r2 = r - c.B;
+    const int cc = r2 / sd.u, uu = r2 % sd.u;
+    const int64_t kc = (int64_t)k * c.C + cc;
+    const int col = sd.nb + uu;
+    float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
+    const RowV<NVH> y = row_load<NVH>(sd.xn + (kc * sd.nn + col) * D, D, H, lane);
+    RowV<NVH> dy = row_load<NVH>(sd.dxn + (kc * sd.nn + col) * D, D, H, lane);
+    if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, col, lane), y);
+    const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y, sd.an ? sd.an[kc * sd.nn + col] : 0.f);
+    if (sd.op_uniform) {
+      const int64_t rel = clamp_index(c.rel[k], c.num_relations);
+      if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D, dz, D, H, lane);
+      if (c.op != PBG_OP_LINEAR)
+        row_store<NVH>(out, op_backward<NVH>(c.op, dz, sd.p0, sd.p1, rel, D, H, lane), D, H, lane);
+    } else {
+      row_store<NVH>(out, dz, D, H, lane);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// operator parameters (standard mode: one relation per batch)
+// ---------------------------------------------------------------------------
+// dth[k, e] = sum over the operator rows of batch k of the parameter gradient of
+// element e: diagonal x.dz, translation dz, complex_diagonal (real | imag).
+__global__ __launch_bounds__(256) void param_grad_kernel(StepCtx c, int s, float* __restrict__ dth) {
+  __shared__ float sh[4][64];
+  const SideCtx& sd = c.side[s];
+  const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int k = blockIdx.y;
+  const int e = blockIdx.x * 64 + lane;
+  const int D = c.D, H = D / 2;
+  float acc = 0.f;
+  if (e < D) {
+    for (int r = rg; r < sd.op_rows; r += 4) {
+      const float* dz = sd.dz + ((int64_t)k * sd.op_rows + r) * D;
+      if (c.op == PBG_OP_TRANSLATION) {
+        acc += dz[e];
+        continue;
+      }
+      int64_t id;
+      if (r < c.B) {
+        id = sd.idx[(int64_t)k * c.B + r];
+      } else {
+        const int r2 = r - c.B;
+        id = sd.uidx[((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u];
+      }
+      const float* x = sd.w + clamp_index(id, sd.num_rows) * D;
+      if (c.op == PBG_OP_DIAGONAL) {
+        acc += x[e] * dz[e];
+      } else if (e < H) {  // d/d real
+        acc += x[e] * dz[e] + x[e + H] * dz[e + H];
+      } else {             // d/d imag
+        const int h = e - H;
+        acc += x[h] * dz[h + H] - x[h + H] * dz[h];
+      }
+    }
+  }
+  sh[rg][lane] = acc;
+  __syncthreads();
+  if (rg == 0 && e < D) dth[(int64_t)k * D + e] = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+}
+
+// AsyncAdagrad (async_adagrad.py:75-85), the K batches' gradients applied in order.
+__global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ dth, int64_t psize, float* p0,
+                                    float* p1, float* s0, float* s1, float lr) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= psize) return;
+  const int H = c.D / 2;
+  for (int k = 0; k < c.K; ++k) {
+    const int64_t r = clamp_index(c.rel[k], c.num_relations);
+    float* p;
+    float* st;
+    if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+      if (e < H) {
+        p = p0 + r * H + e;
+        st = s0 + r * H + e;
+      } else {
+        p = p1 + r * H + (e - H);
+        st = s1 + r * H + (e - H);
+      }
+    } else {
+      p = p0 + r * psize + e;
+      st = s0 + r * psize + e;
+    }
+    const float g = dth[(int64_t)k * psize + e];
+    const float sum = *st + g * g;
+    *st = sum;
+    *p += -lr * (g / (sqrtf(sum) + 1e-10f));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct Plan {
+  StepCtx c;
+  size_t bytes;
+  // buffers that only the host-side orchestration touches
+  float* dth[2];
+  uint64_t* keys_b;
+  uint32_t* vals_b;
+  void* sort_temp;
+  int64_t psize;  // floats of parameter gradient per batch
+  int nvh;
+};
+
+int validate(const pbg_step_desc* d, bool training) {
+  if (!d) return fail(PBG_ERR_INVALID, "step: null descriptor");
+  if (d->dim <= 0 || d->dim > 1024) return fail(PBG_ERR_UNSUPPORTED, "step: dim must be in [1, 1024], got %d", d->dim);
+  if (d->num_workers < 1 || d->num_workers > 256) return fail(PBG_ERR_INVALID, "step: num_workers must be in [1, 256]");
+  if (d->batch_size < 1) return fail(PBG_ERR_INVALID, "step: batch_size must be positive");
+  if (d->num_batch_negs < 0 || d->num_uniform_negs < 0) return fail(PBG_ERR_INVALID, "step: negative negatives count");
+  if (d->num_batch_negs == 0 && d->num_uniform_negs == 0)
+    return fail(PBG_ERR_INVALID, "step: num_batch_negs and num_uniform_negs cannot both be 0");
+  if (d->op < PBG_OP_NONE || d->op > PBG_OP_COMPLEX_DIAGONAL) return fail(PBG_ERR_INVALID, "step: unknown operator %d", d->op);
+  if (d->comparator < PBG_CMP_DOT || d->comparator > PBG_CMP_L2) return fail(PBG_ERR_INVALID, "step: unknown comparator %d", d->comparator);
+  if (d->loss < PBG_LOSS_RANKING || d->loss > PBG_LOSS_SOFTMAX) return fail(PBG_ERR_INVALID, "step: unknown loss %d", d->loss);
+  if (d->op == PBG_OP_COMPLEX_DIAGONAL && d->dim % 2 != 0)
+    return fail(PBG_ERR_INVALID,
+                "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");  // operators.py:132-136
+  if (d->num_relations < 1) return fail(PBG_ERR_INVALID, "step: num_relations must be positive");
+  if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
+  if (d->dynamic && d->op == PBG_OP_LINEAR)
+    return fail(PBG_ERR_UNSUPPORTED, "step: the linear operator with dynamic relations is not implemented");
+  if (training && d->dynamic && d->op != PBG_OP_NONE)
+    return fail(PBG_ERR_UNSUPPORTED, "step: training operator parameters with dynamic relations is not implemented");
+  return PBG_OK;
+}
+
+// Carves the workspace.  With base == nullptr only the size is computed.
+int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
+  StepCtx& c = plan->c;
+  memset(plan, 0, sizeof(*plan));
+  char* base = b ? (char*)b->workspace : nullptr;
+  size_t off = 0;
+  auto take = [&](size_t count, size_t elem) -> void* {
+    const size_t o = off;
+    off += align_up(count * elem, 256);
+    return base ? (void*)(base + o) : nullptr;
+  };
+  auto takef = [&](size_t count) -> float* { return (float*)take(count, sizeof(float)); };
+
+  c.D = d->dim;
+  c.K = d->num_workers;
+  c.B = d->batch_size;
+  c.U = d->num_uniform_negs;
+  const bool batch_mode = d->num_batch_negs > 0;
+  c.P = batch_mode ? (d->num_batch_negs < c.B ? d->num_batch_negs : c.B) : (c.U < c.B ? c.U : c.B);
+  c.C = (c.B - 1) / c.P + 1;
+  c.last = c.B - (c.C - 1) * c.P;
+  c.dynamic = d->dynamic;
+  c.op = d->op;
+  c.cmp = d->comparator;
+  c.loss = d->loss;
+  c.margin = d->margin;
+  c.num_relations = d->num_relations;
+  const int D = c.D, K = c.K, C = c.C, P = c.P;
+  const int64_t KC = (int64_t)K * C;
+  const bool need_aux = c.cmp != PBG_CMP_DOT;
+
+  int slot = 0;
+  for (int s = 0; s < 2; ++s) {
+    SideCtx& sd = c.side[s];
+    const bool enabled = s == 0 ? !d->disable_lhs_negs : !d->disable_rhs_negs;
+    sd.nb = (enabled && batch_mode) ? P : 0;
+    sd.u = enabled ? c.U : 0;
+    sd.nn = sd.nb + sd.u;
+    sd.alias = sd.nb > 0;
+    sd.stride_p = sd.alias ? sd.nn : P;
+    sd.num_rows = s == 0 ? d->num_lhs_rows : d->num_rhs_rows;
+    sd.key_base = (s == 1 && !d->shared_table) ? d->num_lhs_rows : 0;
+    sd.slot_pos = slot;
+    slot += c.B;
+    sd.slot_uni = slot;
+    slot += C * sd.u;
+    if (c.dynamic) {
+      sd.has_op = 1;
+      sd.op_uniform = 0;
+    } else {
+      sd.has_op = (s == 1 && c.op != PBG_OP_NONE) ? 1 : 0;
+      sd.op_uniform = sd.has_op;
+    }
+    sd.op_rows = sd.has_op ? c.B + (sd.op_uniform ? C * sd.u : 0) : 0;
+  }
+  c.rk = slot;
+  c.kbits = bits_for((uint64_t)(K - 1));
+
+  for (int s = 0; s < 2; ++s) {
+    SideCtx& sd = c.side[s];
+    const SideCtx& so = c.side[1 - s];
+    // prepared operands and their gradients
+    if (sd.nn > 0) {
+      sd.xn = takef(KC * sd.nn * D);
+      sd.dxn = takef(KC * sd.nn * D);
+      if (need_aux) sd.an = takef(KC * sd.nn);
+      sd.s = takef(KC * P * sd.nn);
+      if (c.cmp == PBG_CMP_L2) sd.rs = takef(KC * P);
+    }
+    if (sd.alias) {
+      sd.xp = sd.xn;
+      sd.dxp = sd.dxn;
+      sd.ap = sd.an;
+    } else {
+      sd.xp = takef(KC * P * D);
+      sd.dxp = takef(KC * P * D);
+      if (need_aux) sd.ap = takef(KC * P);
+    }
+    if (c.dynamic) {
+      sd.xa = takef(KC * P * D);
+      sd.dxa = takef(KC * P * D);
+      if (need_aux) sd.aa = takef(KC * P);
+    }
+    // which gradient buffers a GEMM fills (see run_backward)
+    sd.plain_written = sd.alias || (!c.dynamic && (s == 0 ? (d->disable_rhs_negs == 0) : (d->disable_lhs_negs == 0)));
+    sd.opd_written = c.dynamic && (s == 0 ? (d->disable_rhs_negs == 0) : (d->disable_lhs_negs == 0));
+    (void)so;
+    if (sd.has_op && c.op != PBG_OP_NONE) {
+      sd.dz = takef((size_t)K * sd.op_rows * D);
+      if (c.op == PBG_OP_LINEAR) {
+        sd.xraw = takef((size_t)K * sd.op_rows * D);
+        sd.z = takef((size_t)K * sd.op_rows * D);
+      }
+    }
+  }
+  const int64_t CP = (int64_t)C * P;
+  c.pos[0] = takef(K * CP);
+  c.dpos[0] = takef(K * CP);
+  if (c.dynamic) {
+    c.pos[1] = takef(K * CP);
+    c.dpos[1] = takef(K * CP);
+  } else {
+    c.pos[1] = c.pos[0];
+    c.dpos[1] = c.dpos[0];
+  }
+  c.lossrow = takef(K * CP);
+
+  plan->psize = 0;
+  if (c.op == PBG_OP_LINEAR) plan->psize = (int64_t)D * D;
+  else if (c.op != PBG_OP_NONE) plan->psize = D;
+  for (int s = 0; s < 2; ++s)
+    if (c.side[s].has_op && plan->psize > 0) plan->dth[s] = takef((size_t)K * plan->psize);
+
+  const int64_t npairs = (int64_t)K * c.rk;
+  c.gr = takef((size_t)npairs * D);
+  c.keys = (uint64_t*)take(npairs, 8);
+  plan->keys_b = (uint64_t*)take(npairs, 8);
+  c.vals = (uint32_t*)take(npairs, 4);
+  plan->vals_b = (uint32_t*)take(npairs, 4);
+  plan->sort_temp = take(sort_temp_bytes(npairs), 1);
+  plan->bytes = off;
+  plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
+
+  if (b) {
+    c.side[0].w = b->w_lhs;
+    c.side[1].w = b->w_rhs;
+    c.side[0].idx = b->lhs;
+    c.side[1].idx = b->rhs;
+    c.side[0].uidx = b->uniform_lhs;
+    c.side[1].uidx = b->uniform_rhs;
+    c.side[0].p0 = b->lhs_op_p0;
+    c.side[0].p1 = b->lhs_op_p1;
+    c.side[1].p0 = b->rhs_op_p0;
+    c.side[1].p1 = b->rhs_op_p1;
+    c.rel = b->rel;
+    c.edge_weight = b->edge_weight;
+    c.rel_weights = b->relation_weights;
+    c.violators = (unsigned long long*)b->violators_out;
+    c.loss_out = b->loss_out;
+  }
+  return PBG_OK;
+}
+
+int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, bool training) {
+  if (!b) return fail(PBG_ERR_INVALID, "step: null buffers");
+  if (!b->w_lhs || !b->w_rhs || !b->lhs || !b->rhs || !b->rel || !b->relation_weights)
+    return fail(PBG_ERR_INVALID, "step: null table / edge / relation pointer");
+  if (training && (!b->g_lhs || !b->g_rhs || !b->loss_out || !b->violators_out))
+    return fail(PBG_ERR_INVALID, "step: null optimizer state or statistics pointer");
+  if (d->shared_table && (b->w_lhs != b->w_rhs || d->num_lhs_rows != d->num_rhs_rows))
+    return fail(PBG_ERR_INVALID, "step: shared_table needs w_lhs == w_rhs");
+  if (!d->shared_table && b->w_lhs == b->w_rhs)
+    return fail(PBG_ERR_INVALID, "step: w_lhs == w_rhs needs shared_table = 1");
+  if ((uintptr_t)b->w_lhs % 16 != 0 || (uintptr_t)b->w_rhs % 16 != 0)
+    return fail(PBG_ERR_INVALID, "step: tables must be 16-byte aligned");
+  if (plan.c.side[0].u > 0 && !b->uniform_lhs) return fail(PBG_ERR_INVALID, "step: uniform_lhs is null");
+  if (plan.c.side[1].u > 0 && !b->uniform_rhs) return fail(PBG_ERR_INVALID, "step: uniform_rhs is null");
+  for (int s = 0; s < 2; ++s) {
+    if (!plan.c.side[s].has_op || d->op == PBG_OP_NONE) continue;
+    const float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
+    const float* p1 = s == 0 ? b->lhs_op_p1 : b->rhs_op_p1;
+    const float* s0 = s == 0 ? b->lhs_op_s0 : b->rhs_op_s0;
+    const float* s1 = s == 0 ? b->lhs_op_s1 : b->rhs_op_s1;
+    const bool two = d->op == PBG_OP_COMPLEX_DIAGONAL;
+    if (!p0 || (two && !p1)) return fail(PBG_ERR_INVALID, "step: null operator parameter");
+    if (training && (!s0 || (two && !s1))) return fail(PBG_ERR_INVALID, "step: null operator optimizer state");
+  }
+  if (!b->workspace || b->workspace_bytes < plan.bytes)
+    return fail(PBG_ERR_WORKSPACE, "step: workspace needs %zu bytes, got %zu", plan.bytes, b->workspace_bytes);
+  if ((uintptr_t)b->workspace % 256 != 0) return fail(PBG_ERR_WORKSPACE, "step: workspace must be 256-byte aligned");
+  const uint64_t rows = (uint64_t)d->num_lhs_rows + (d->shared_table ? 0 : (uint64_t)d->num_rhs_rows);
+  if (bits_for(rows) + plan.c.kbits > 62) return fail(PBG_ERR_UNSUPPORTED, "step: tables too large for the sort key");
+  if ((int64_t)plan.c.K * plan.c.rk >= ((int64_t)1 << 32))
+    return fail(PBG_ERR_UNSUPPORTED, "step: too many gradient rows per call");
+  return PBG_OK;
+}
+
+#define PBG_DISPATCH_NVH(nvh, KERNEL, grid, stream, ...)                                                      \
+  do {                                                                                                       \
+    if ((nvh) <= 1) hipLaunchKernelGGL((KERNEL<1>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);          \
+    else if ((nvh) <= 2) hipLaunchKernelGGL((KERNEL<2>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);     \
+    else if ((nvh) <= 4) hipLaunchKernelGGL((KERNEL<4>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);     \
+    else hipLaunchKernelGGL((KERNEL<8>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);                     \
+  } while (0)
+
+dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 1, kWavesPerBlock)); }
+
+// prep + operator GEMM (linear) + score GEMMs
+int run_forward(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int D = c.D, K = c.K, C = c.C, P = c.P;
+  const int64_t jobs = (int64_t)K * (2 * C * P + C * c.side[0].u + C * c.side[1].u);
+  PBG_DISPATCH_NVH(plan.nvh, prep_kernel, wave_grid(jobs), stream, c);
+  int rc;
+  if (c.op == PBG_OP_LINEAR) {
+    for (int s = 0; s < 2; ++s) {
+      const SideCtx& sd = c.side[s];
+      if (!sd.has_op) continue;
+      GemmArgs g{};  // z[k] = xraw[k] * W[rel[k]]^T   (operators.py:94-99)
+      g.a = sd.xraw; g.stride_a = (int64_t)sd.op_rows * D; g.lda = D; g.a_kmajor = 0;
+      g.b = sd.p0; g.stride_b = 0; g.ldb = D; g.b_kmajor = 0;
+      g.b_index = c.rel; g.b_index_stride = (int64_t)D * D;
+      g.c = sd.z; g.stride_c = (int64_t)sd.op_rows * D; g.ldc = D;
+      g.m = sd.op_rows; g.n = D; g.k = D; g.batch = K; g.alpha = 1.f; g.beta = 0.f;
+      if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
+      PBG_DISPATCH_NVH(plan.nvh, prepare_staged_kernel, wave_grid((int64_t)K * sd.op_rows), stream, c, s);
+    }
+  }
+  for (int s = 0; s < 2; ++s) {
+    const SideCtx& sd = c.side[s];
+    const SideCtx& so = c.side[1 - s];
+    if (sd.nn == 0) continue;
+    GemmArgs g{};  // S = A * N^T   (model.py:179-180, 234)
+    g.a = c.dynamic ? so.xa : so.xp;
+    g.stride_a = (int64_t)(c.dynamic ? P : so.stride_p) * D; g.lda = D; g.a_kmajor = 0;
+    g.b = sd.xn; g.stride_b = (int64_t)sd.nn * D; g.ldb = D; g.b_kmajor = 0;
+    g.c = sd.s; g.stride_c = (int64_t)P * sd.nn; g.ldc = sd.nn;
+    g.m = P; g.n = sd.nn; g.k = D; g.batch = K * C; g.alpha = 1.f; g.beta = 0.f;
+    if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
+  }
+  return check_launch("step forward");
+}
+
+int run_backward(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int D = c.D, K = c.K, C = c.C, P = c.P;
+  int rc;
+  for (int s = 0; s < 2; ++s) {  // dN = dS^T * A  -> dxn (all nn rows, first writer)
+    const SideCtx& sd = c.side[s];
+    const SideCtx& so = c.side[1 - s];
+    if (sd.nn == 0) continue;
+    GemmArgs g{};
+    g.a = sd.s; g.stride_a = (int64_t)P * sd.nn; g.lda = sd.nn; g.a_kmajor = 1;  // A(m = col, k = row)
+    g.b = c.dynamic ? so.xa : so.xp;
+    g.stride_b = (int64_t)(c.dynamic ? P : so.stride_p) * D; g.ldb = D; g.b_kmajor = 1;
+    g.c = sd.dxn; g.stride_c = (int64_t)sd.nn * D; g.ldc = D;
+    g.m = sd.nn; g.n = D; g.k = P; g.batch = K * C; g.alpha = 1.f; g.beta = 0.f;
+    if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
+  }
+  for (int s = 0; s < 2; ++s) {  // dA = dS * N -> the other side's positives (operated ones in dynamic mode)
+    const SideCtx& sd = c.side[s];
+    const SideCtx& so = c.side[1 - s];
+    if (sd.nn == 0) continue;
+    GemmArgs g{};
+    g.a = sd.s; g.stride_a = (int64_t)P * sd.nn; g.lda = sd.nn; g.a_kmajor = 0;
+    g.b = sd.xn; g.stride_b = (int64_t)sd.nn * D; g.ldb = D; g.b_kmajor = 1;
+    if (c.dynamic) {
+      g.c = so.dxa; g.stride_c = (int64_t)P * D; g.beta = 0.f;
+    } else {
+      g.c = so.dxp; g.stride_c = (int64_t)so.stride_p * D; g.beta = so.alias ? 1.f : 0.f;
+    }
+    g.ldc = D;
+    g.m = P; g.n = D; g.k = sd.nn; g.batch = K * C; g.alpha = 1.f;
+    if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
+  }
+  const int64_t jobs = (int64_t)K * (2 * c.B + C * c.side[0].u + C * c.side[1].u);
+  PBG_DISPATCH_NVH(plan.nvh, rowback_kernel, wave_grid(jobs), stream, c);
+  return check_launch("step backward");
+}
+
+int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  if (c.op == PBG_OP_NONE) return PBG_OK;
+  const int D = c.D, K = c.K;
+  int rc;
+  for (int s = 0; s < 2; ++s) {
+    const SideCtx& sd = c.side[s];
+    if (!sd.has_op) continue;
+    float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
+    float* p1 = s == 0 ? b->lhs_op_p1 : b->rhs_op_p1;
+    float* s0 = s == 0 ? b->lhs_op_s0 : b->rhs_op_s0;
+    float* s1 = s == 0 ? b->lhs_op_s1 : b->rhs_op_s1;
+    if (c.op == PBG_OP_LINEAR) {
+      GemmArgs g{};  // dx = dz * W  -> gradient rows of this side (positives, then uniform negatives)
+      g.a = sd.dz; g.stride_a = (int64_t)sd.op_rows * D; g.lda = D; g.a_kmajor = 0;
+      g.b = sd.p0; g.stride_b = 0; g.ldb = D; g.b_kmajor = 1;
+      g.b_index = c.rel; g.b_index_stride = (int64_t)D * D;
+      g.c = c.gr + (int64_t)sd.slot_pos * D; g.stride_c = (int64_t)c.rk * D; g.ldc = D;
+      g.m = sd.op_rows; g.n = D; g.k = D; g.batch = K; g.alpha = 1.f; g.beta = 0.f;
+      if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
+      GemmArgs h{};  // dW = dz^T * x
+      h.a = sd.dz; h.stride_a = (int64_t)sd.op_rows * D; h.lda = D; h.a_kmajor = 1;
+      h.b = sd.xraw; h.stride_b = (int64_t)sd.op_rows * D; h.ldb = D; h.b_kmajor = 1;
+      h.c = plan.dth[s]; h.stride_c = (int64_t)D * D; h.ldc = D;
+      h.m = D; h.n = D; h.k = sd.op_rows; h.batch = K; h.alpha = 1.f; h.beta = 0.f;
+      if ((rc = gemm_f32(h, stream)) != PBG_OK) return rc;
+    } else {
+      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K), dim3(256), 0, stream, c, s,
+                         plan.dth[s]);
+    }
+    hipLaunchKernelGGL(param_update_kernel, dim3((unsigned)ceil_div(plan.psize, 256)), dim3(256), 0, stream, c, s,
+                       plan.dth[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
+  }
+  return check_launch("step params");
+}
+
+}  // namespace
+}  // namespace pbg
+
+using namespace pbg;
+
+extern "C" size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc) {
+  if (validate(desc, false) != PBG_OK) return 0;
+  Plan plan;
+  make_plan(desc, nullptr, &plan);
+  return plan.bytes;
+}
+
+extern "C" int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream) {
+  int rc = validate(desc, true);
+  if (rc != PBG_OK) return rc;
+  Plan plan;
+  make_plan(desc, bufs, &plan);
+  if ((rc = check_buffers(desc, bufs, plan, true)) != PBG_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const StepCtx& c = plan.c;
+  hipLaunchKernelGGL(zero_violators_kernel, dim3((unsigned)ceil_div(c.K * 2, 64)), dim3(64), 0, s, c.violators, c.K * 2);
+  if ((rc = run_forward(plan, s)) != PBG_OK) return rc;
+  hipLaunchKernelGGL(loss_kernel, wave_grid((int64_t)c.K * c.C * c.P), dim3(kRowThreads), 0, s, c);
+  hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+  if ((rc = run_backward(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_params(desc, bufs, plan, s)) != PBG_OK) return rc;
+  const int64_t npairs = (int64_t)c.K * c.rk;
+  const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
+  rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, bits_for(rows - 1) + c.kbits, plan.sort_temp, s);
+  if (rc != PBG_OK) return rc;
+  if (desc->shared_table) {
+    rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
+                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s);
+  } else {
+    rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
+                            desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s);
+  }
+  return rc;
+}
+
+extern "C" int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos,
+                                 float* rhs_pos, float* lhs_neg, float* rhs_neg, pbg_stream_t stream) {
+  int rc = validate(desc, false);
+  if (rc != PBG_OK) return rc;
+  Plan plan;
+  make_plan(desc, bufs, &plan);
+  if ((rc = check_buffers(desc, bufs, plan, false)) != PBG_OK) return rc;
+  const StepCtx& c = plan.c;
+  if (!lhs_pos || !rhs_pos || (c.side[0].nn > 0 && !lhs_neg) || (c.side[1].nn > 0 && !rhs_neg))
+    return fail(PBG_ERR_INVALID, "pbg_model_forward: null output");
+  hipStream_t s = (hipStream_t)stream;
+  if ((rc = run_forward(plan, s)) != PBG_OK) return rc;
+  hipLaunchKernelGGL(scores_out_kernel, wave_grid((int64_t)c.K * c.B), dim3(kRowThreads), 0, s, c, lhs_pos, rhs_pos,
+                     lhs_neg, rhs_neg);
+  return check_launch("pbg_model_forward");
+}

@@ -1,0 +1,173 @@
+"""GPU parity of the stand-alone kernels, called through the C ABI: gather and
+permutations bit-exact, RowAdagrad / GEMM within 1e-5 relative of the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import perm as operm
+from oracle import step as ostep
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dim,n_rows,n", [(100, 1000, 4000), (3, 7, 20), (1024, 300, 513), (400, 64, 1), (6, 5, 0)])
+def test_gather_bit_exact(pbg, dim, n_rows, n):
+    say("gather", dim, n_rows, n)
+    g = torch.Generator().manual_seed(dim)
+    w = torch.randn(n_rows, dim, generator=g)
+    idx = torch.randint(0, n_rows, (n,), generator=g)
+    out = pbg.native.gather_rows(w.to(DEV), idx.to(DEV))
+    assert torch.equal(out.cpu(), w[idx])
+    # two-dimensional index (sample_entities' [C, U] layout)
+    if n >= 4:
+        idx2 = idx[: n // 2 * 2].view(2, -1)
+        assert torch.equal(pbg.native.gather_rows(w.to(DEV), idx2.to(DEV)).cpu(), w[idx2])
+
+
+def test_gather_out_of_range(pbg):
+    w = torch.randn(5, 4, device=DEV)
+    with pytest.raises(IndexError):
+        pbg.native.gather_rows(w, torch.tensor([0, 5], device=DEV))
+
+
+@pytest.mark.parametrize("m,n,k,batch,akm,bkm", [
+    (50, 100, 100, 7, 0, 0), (100, 100, 50, 5, 1, 1), (50, 100, 100, 5, 0, 1),
+    (130, 200, 33, 3, 0, 0), (1, 1, 1, 1, 0, 0), (200, 131, 257, 2, 1, 1), (17, 300, 64, 2, 0, 1),
+    (256, 256, 300, 2, 1, 1), (64, 64, 16, 1, 0, 0),
+])
+def test_gemm_against_float64(pbg, m, n, k, batch, akm, bkm):
+    say("gemm", m, n, k, batch, akm, bkm)
+    g = torch.Generator().manual_seed(m * 1000 + n)
+    a = torch.randn((batch, k, m) if akm else (batch, m, k), generator=g)
+    b = torch.randn((batch, k, n) if bkm else (batch, n, k), generator=g)
+    c0 = torch.randn(batch, m, n, generator=g)
+    am = a.transpose(1, 2) if akm else a
+    bm = b if bkm else b.transpose(1, 2)
+    for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+        want = alpha * torch.bmm(am.double(), bm.double()) + beta * c0.double()
+        c = c0.clone().to(DEV)
+        pbg.native.gemm(a.to(DEV), b.to(DEV), c, batch, m, n, k, m if akm else k, n if bkm else k, n,
+                        a[0].numel(), b[0].numel(), m * n, akm, bkm, alpha, beta)
+        got = c.cpu().double()
+        scale = want.abs().max().item() + 1e-30
+        assert (got - want).abs().max().item() <= 2e-6 * scale * max(1, k ** 0.5), (alpha, beta)
+
+
+def test_bmm_nt_unaligned_dim(pbg):
+    a = torch.randn(3, 5, 7)
+    b = torch.randn(3, 6, 7)
+    got = pbg.native.bmm_nt(a.to(DEV), b.to(DEV)).cpu()
+    assert torch.allclose(got, torch.bmm(a, b.transpose(1, 2)), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dim,n_rows,n", [(100, 500, 4000), (1, 9, 30), (4, 50, 1), (1024, 40, 300), (10, 100000, 5000),
+                                          (400, 3, 700)])
+def test_row_adagrad_sparse(pbg, dim, n_rows, n):
+    say("row_adagrad_sparse", dim, n_rows, n)
+    g = torch.Generator().manual_seed(n)
+    w = torch.randn(n_rows, dim, generator=g)
+    gs = torch.rand(n_rows, generator=g)
+    idx = torch.randint(0, n_rows, (n,), generator=g)
+    vals = torch.randn(n, dim, generator=g)
+    wd, gd = w.clone().to(DEV), gs.clone().to(DEV)
+    pbg.native.row_adagrad_sparse(wd, gd, idx.to(DEV), vals.to(DEV), 0.1)
+    ostep.row_adagrad_sparse(w, gs, torch.sparse_coo_tensor(idx.unsqueeze(0), vals, (n_rows, dim)), 0.1)
+    assert torch.allclose(wd.cpu(), w, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(gd.cpu(), gs, rtol=1e-5, atol=1e-7)
+    # a second step on top of the first (state carries over)
+    pbg.native.row_adagrad_sparse(wd, gd, idx.to(DEV), vals.to(DEV), 0.1)
+    ostep.row_adagrad_sparse(w, gs, torch.sparse_coo_tensor(idx.unsqueeze(0), vals, (n_rows, dim)), 0.1)
+    assert torch.allclose(wd.cpu(), w, rtol=1e-5, atol=1e-6)
+
+
+def test_row_adagrad_empty_and_dense(pbg):
+    w = torch.randn(6, 5)
+    gs = torch.rand(6)
+    wd, gd = w.clone().to(DEV), gs.clone().to(DEV)
+    pbg.native.row_adagrad_sparse(wd, gd, torch.empty(0, dtype=torch.int64, device=DEV),
+                                  torch.empty(0, 5, device=DEV), 0.1)
+    assert torch.equal(wd.cpu(), w)
+    grad = torch.randn(6, 5)
+    pbg.native.row_adagrad_dense(wd, gd, grad.to(DEV), 0.05)
+    ostep.row_adagrad_dense(w, gs, grad, 0.05)
+    assert torch.allclose(wd.cpu(), w, rtol=1e-6, atol=1e-7) and torch.allclose(gd.cpu(), gs, rtol=1e-6)
+    p, s, gr = torch.randn(37), torch.rand(37), torch.randn(37)
+    pd, sd = p.clone().to(DEV), s.clone().to(DEV)
+    pbg.native.async_adagrad_dense(pd, sd, gr.to(DEV), 0.01)
+    ostep.async_adagrad_dense(p, s, gr, 0.01)
+    assert torch.allclose(pd.cpu(), p, rtol=1e-6, atol=1e-7) and torch.allclose(sd.cpu(), s, rtol=1e-6)
+
+
+@pytest.mark.parametrize("n", [1, 2, 1000, 70001])
+def test_permutation_helpers_bit_exact(pbg, n):
+    say("perm", n)
+    p = np.random.default_rng(n).permutation(n).astype(np.int64)
+    tp = torch.from_numpy(p).to(DEV)
+    assert np.array_equal(pbg.native.reverse_permutation(tp).cpu().numpy(), operm.reverse_permutation(p))
+    for shape, dtype in (((n, 100), torch.float32), ((n,), torch.float32), ((n,), torch.int64), ((n, 3), torch.float32),
+                         ((n, 2, 2), torch.float64)):
+        t = (torch.randn(shape) * 1000).to(dtype)
+        want = operm.shuffle(t.numpy(), p)
+        td = t.to(DEV)
+        pbg.native.shuffle_rows(td, tp)
+        assert np.array_equal(td.cpu().numpy(), want), (shape, dtype)
+    # undo with the reverse permutation (train_gpu.py:627-632)
+    t = torch.randn(n, 8)
+    td = t.to(DEV)
+    pbg.native.shuffle_rows(td, tp)
+    pbg.native.shuffle_rows(td, pbg.native.reverse_permutation(tp))
+    assert torch.equal(td.cpu(), t)
+
+
+def test_shuffle_rejects_bad_permutation(pbg):
+    t = torch.randn(4, 4, device=DEV)
+    with pytest.raises(ValueError):
+        pbg.native.shuffle_rows(t, torch.tensor([0, 1, 2, 4], device=DEV))
+
+
+@pytest.mark.parametrize("n", [1, 5000, 200003])
+def test_randperm_contract(pbg, n):
+    a = pbg.native.randperm(n, 7, DEV).cpu().numpy()
+    assert operm.is_permutation(a)
+    assert np.array_equal(a, pbg.native.randperm(n, 7, DEV).cpu().numpy())
+    if n > 1000:
+        b = pbg.native.randperm(n, 8, DEV).cpu().numpy()
+        assert (a != b).mean() > 0.99
+        # first-order uniformity: where element 0..n/10 land, in 10 bins (chi-square, 9 dof)
+        inv = operm.reverse_permutation(a)
+        counts = np.bincount(inv[: n // 10] * 10 // n, minlength=10)
+        expected = (n // 10) / 10
+        assert ((counts - expected) ** 2 / expected).sum() < 40
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+@pytest.mark.parametrize("parts", [(1, 1), (2, 3), (8, 8)])
+def test_sub_bucket_bit_exact(pbg, dynamic, parts):
+    say("sub_bucket", dynamic, parts)
+    rng = np.random.default_rng(5)
+    n, n_rel = 20000, 3
+    cl = [int(c) for c in rng.integers(50, 400, n_rel)]
+    cr = [int(c) for c in rng.integers(50, 400, n_rel)]
+    rel = rng.integers(0, n_rel, n).astype(np.int64)
+    look = np.zeros(n, dtype=np.int64) if dynamic else rel
+    lhs = (rng.random(n) * np.array(cl)[look]).astype(np.int64)
+    rhs = (rng.random(n) * np.array(cr)[look]).astype(np.int64)
+    pl = [rng.permutation(c).astype(np.int64) for c in cl]
+    pr = [rng.permutation(c).astype(np.int64) for c in cr]
+    lo, ro, relo, ranges = operm.sub_bucket(lhs, rhs, rel, cl, pl, cr, pr, parts[0], parts[1], dynamic)
+    d = lambda x: torch.from_numpy(x).to(DEV)
+    outs = [torch.empty(n, dtype=torch.int64, device=DEV) for _ in range(3)]
+    offs = pbg.native.sub_bucket(
+        d(lhs), d(rhs), d(rel), [d(x) for x in pl], [d(x) for x in pr],
+        [-(-c // parts[0]) for c in cl], [-(-c // parts[1]) for c in cr], parts[0], parts[1], dynamic, *outs)
+    assert np.array_equal(outs[0].cpu().numpy(), lo)
+    assert np.array_equal(outs[1].cpu().numpy(), ro)
+    assert np.array_equal(outs[2].cpu().numpy(), relo)
+    offs = offs.cpu().numpy()
+    for (i, j), (a, b) in ranges.items():
+        assert (offs[i * parts[1] + j], offs[i * parts[1] + j + 1]) == (a, b)
