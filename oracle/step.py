@@ -539,14 +539,14 @@ def train_step(cfg, st, lhs, rhs, rel, uniform_lhs, uniform_rhs, weight=None, ke
     return out
 
 
-def train_lockstep(cfg, st, batches: List[tuple]) -> List[StepOutput]:
+def train_lockstep(cfg, st, batches: List[tuple], keep_scores: bool = False) -> List[StepOutput]:
     """K HOGWILD workers (train_cpu.py:849-884) in the one interleaving that is
     deterministic: every worker reads the tables, then every worker writes, in
     worker order.  ``batches`` is a list of (lhs, rhs, rel, uniform_lhs,
     uniform_rhs) tuples, one per worker."""
     outs, all_grads = [], []
     for b in batches:
-        out, grads = forward_backward(cfg, st, *b)
+        out, grads = forward_backward(cfg, st, *b, keep_scores=keep_scores)
         outs.append(out)
         all_grads.append(grads)
     for grads in all_grads:
