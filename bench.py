@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Throughput of the PBG training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1] [--workers 40]
+
+A "step" is one batch of `batch_size` edges through the whole hot path (gather,
+operator, scoring against batch + uniform negatives, loss, backward, RowAdagrad
+and operator Adagrad).  Batches are issued `workers` at a time through
+pbg_train_step, which processes them like `workers` HOGWILD processes in
+lock-step (all read, then all write in order); `--workers 1` is the strictly
+sequential single-process order.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+# name -> the fields of BASELINE.json's configs
+WORKLOADS = {
+    "cfg1": dict(desc="single relation, identity/dot/ranking(0.1), dim 100, 100k entities, B=1000, 50 batch + 50 uniform negatives",
+                 entities=100_000, edges=1_000_000, dim=100, batch=1000, batch_negs=50, uniform_negs=50,
+                 operator="none", comparator="dot", loss="ranking", relations=1, dynamic=False,
+                 init_scale=1e-3, zipf=None, two_tables=False),
+    "cfg2": dict(desc="1345 relations, complex_diagonal/dot/softmax, dim 400, 14951 entities, B=1000, chunk 50 + 1000 uniform negatives, single-relation batches",
+                 entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=1000,
+                 operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=False,
+                 init_scale=1e-3, zipf=1.1, two_tables=False),
+    "cfg3": dict(desc="single relation, identity/dot/softmax, dim 1024, 4.85M entities, B=10000, 1000 batch + 100 uniform negatives",
+                 entities=4_847_571, edges=4_000_000, dim=1024, batch=10_000, batch_negs=1000, uniform_negs=100,
+                 operator="none", comparator="dot", loss="softmax", relations=1, dynamic=False,
+                 init_scale=1e-3, zipf=2.0, two_tables=False),
+    "cfg4": dict(desc="one bucket of 4x4: translation/l2/ranking, dim 100, two resident partitions of 10.4M entities, B=1000, 50 + 50 negatives",
+                 entities=10_413_058, edges=4_000_000, dim=100, batch=1000, batch_negs=50, uniform_negs=50,
+                 operator="translation", comparator="l2", loss="ranking", relations=1, dynamic=False,
+                 init_scale=1e-3, zipf=1.8, two_tables=True),
+    "cfg5": dict(desc="500 relations, linear/cos/logistic, dim 256, 2M entities, B=2000, 100 batch + 100 uniform negatives, single-relation batches",
+                 entities=2_000_000, edges=4_000_000, dim=256, batch=2000, batch_negs=100, uniform_negs=100,
+                 operator="linear", comparator="cos", loss="logistic", relations=500, dynamic=False,
+                 init_scale=1e-3, zipf=None, rel_zipf=1.2, two_tables=False),
+}
+
+
+def power_law_ids(n, num, s, gen, device):
+    """ids in [0, num) with P(rank r) ~ r^-s, ranks mapped through a shuffle."""
+    u = torch.rand(n, generator=gen, device=device, dtype=torch.float64)
+    if abs(s - 1.0) < 1e-9:
+        r = torch.exp(u * math.log(num))
+    else:
+        a = 1.0 - s
+        r = ((num ** a - 1.0) * u + 1.0) ** (1.0 / a)
+    ranks = (r.floor().long() - 1).clamp_(0, num - 1)
+    shuffle = torch.randperm(num, generator=gen, device=device)
+    return shuffle[ranks]
+
+
+def make_workload(w, device, seed=0):
+    gen = torch.Generator(device=device).manual_seed(seed)
+    e, d = w["entities"], w["dim"]
+    tables = [torch.randn(e, d, generator=gen, device=device) * w["init_scale"]]
+    if w["two_tables"]:
+        tables.append(torch.randn(e, d, generator=gen, device=device) * w["init_scale"])
+    n = w["edges"]
+    if w["zipf"]:
+        lhs = power_law_ids(n, e, w["zipf"], gen, device)
+        rhs = power_law_ids(n, e, w["zipf"], gen, device)
+    else:
+        lhs = torch.randint(0, e, (n,), generator=gen, device=device)
+        rhs = torch.randint(0, e, (n,), generator=gen, device=device)
+    return tables, lhs, rhs
+
+
+def algorithmic(w, spec):
+    """Per-batch algorithmic bytes and flops of each stage."""
+    b, d = w["batch"], w["dim"]
+    p, c, u = spec.chunk_size, spec.num_chunks, w["uniform_negs"]
+    n = p + u
+    rows = 2 * b + 2 * c * u
+    gemm = 2.0 * 2 * c * p * n * d  # both sides, multiply-add
+    out = {
+        "prep": ("hbm", rows * (2 * 4 * d + 8)),          # gather: read row, write row, read index
+        "scores": ("mfma", gemm),
+        "loss": ("hbm", 2 * 2 * c * p * n * 4),           # read S, write dS, both sides
+        "backward_dn": ("mfma", gemm),
+        "backward_da": ("mfma", gemm),
+        "rowback": ("hbm", rows * (3 * 4 * d)),           # read prepared grad + prepared row, write raw grad
+        "sort": ("hbm", rows * 12 * 2),
+        "update": ("hbm", rows * (3 * 4 * d + 8) + rows * 8),  # grad read + W read/write + G r/w + key (duplicates not credited)
+    }
+    if w["operator"] == "linear":
+        op_rows = b + c * u
+        out["operator"] = ("mfma", 2.0 * op_rows * d * d)
+        out["params"] = ("mfma", 2.0 * 2 * op_rows * d * d)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed batches")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed batches")
+    ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
+    ap.add_argument("--workers", type=int, default=40, help="batches in flight per call (HOGWILD workers)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="length of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-sequential", action="store_true", help="skip the workers=1 measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (one process, no collectives); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__
+
+    pkg = __graft_entry__.load_package()
+    w = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tables, lhs_all, rhs_all = make_workload(w, dev)
+    e, d, b = w["entities"], w["dim"], w["batch"]
+
+    def make_runner(workers):
+        spec = pkg.StepSpec(dim=d, batch_size=b, num_workers=workers, num_batch_negs=w["batch_negs"],
+                            num_uniform_negs=w["uniform_negs"], operator=w["operator"], dynamic=w["dynamic"],
+                            num_relations=w["relations"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
+                            lr=0.1)
+        ws = [t.clone() for t in tables]
+        gs = [torch.zeros(t.shape[0], device=dev) for t in tables]
+        rhs_op, rhs_sum = {}, {}
+        r = w["relations"]
+        if w["operator"] == "complex_diagonal":
+            rhs_op = {"real": torch.ones(r, d // 2, device=dev), "imag": torch.zeros(r, d // 2, device=dev)}
+        elif w["operator"] == "translation":
+            rhs_op = {"translation": torch.zeros(r, d, device=dev)}
+        elif w["operator"] == "diagonal":
+            rhs_op = {"diagonal": torch.ones(r, d, device=dev)}
+        elif w["operator"] == "linear":
+            rhs_op = {"linear_transformation": torch.eye(d, device=dev).repeat(r, 1, 1).contiguous()}
+        rhs_sum = {k: torch.zeros_like(v) for k, v in rhs_op.items()}
+        runner = pkg.StepRunner(spec, ws[0], gs[0], ws[1] if len(ws) > 1 else None, gs[1] if len(gs) > 1 else None,
+                                rhs_op, rhs_sum)
+        return spec, runner
+
+    gen = torch.Generator(device=dev).manual_seed(1)
+    n_edges = lhs_all.shape[0]
+    if w["relations"] > 1:
+        if w.get("rel_zipf"):
+            rel_pool = power_law_ids(4096, w["relations"], w["rel_zipf"], gen, dev)
+        elif w["zipf"]:
+            rel_pool = power_law_ids(4096, w["relations"], w["zipf"], gen, dev)
+        else:
+            rel_pool = torch.randint(0, w["relations"], (4096,), generator=gen, device=dev)
+    else:
+        rel_pool = torch.zeros(4096, dtype=torch.int64, device=dev)
+
+    def run(workers, batches, warm, profile_calls=0):
+        spec, runner = make_runner(workers)
+        c, u = spec.num_chunks, w["uniform_negs"]
+        per_call = workers * b
+        calls = max(1, batches // workers)
+        warm_calls = max(1, warm // workers)
+        n_r = tables[-1].shape[0]
+
+        def one_call(i, profiled=False):
+            off = (i * per_call) % (n_edges - per_call + 1)
+            lhs = lhs_all[off:off + per_call]
+            rhs = rhs_all[off:off + per_call]
+            rel = rel_pool[(i * workers) % (4096 - workers + 1):][:workers]
+            # the uniform negatives of model.py:70-75, drawn on the device inside the timed loop
+            ul = torch.randint(0, e, (workers, c, u), generator=gen, device=dev)
+            ur = torch.randint(0, n_r, (workers, c, u), generator=gen, device=dev)
+            if profiled:
+                return runner.train_profiled(lhs, rhs, rel, ul, ur)
+            runner.train(lhs, rhs, rel, ul, ur)
+            return None
+
+        for i in range(warm_calls):
+            one_call(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(calls):
+            one_call(warm_calls + i)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        stages = None
+        if profile_calls:
+            acc = None
+            for i in range(profile_calls):
+                ms = one_call(warm_calls + calls + i, profiled=True)
+                acc = ms if acc is None else [a + m for a, m in zip(acc, ms)]
+            stages = dict(zip(runner.STAGES, [a / profile_calls for a in acc]))
+        loss = float(runner.loss_out.mean().item()) / b
+        return spec, calls * per_call / dt, dt / (calls * workers) * 1e3, calls * workers, stages, loss
+
+    default_steps = {"cfg1": 8000, "cfg2": 400, "cfg3": 40, "cfg4": 8000, "cfg5": 800}[args.workload]
+    steps = args.steps if args.steps is not None else default_steps
+    warmup = args.warmup if args.warmup is not None else max(args.workers, steps // 10)
+    workers = max(1, min(args.workers, steps))
+    spec, eps, ms_per_step, timed, stages, loss = run(workers, steps, warmup, profile_calls=10)
+
+    seq = None
+    if not args.no_sequential and workers > 1:
+        _, seq_eps, seq_ms, seq_timed, _, _ = run(1, max(50, min(steps // 8, 1000)), 20)
+        seq = {"value": seq_eps, "ms_per_step": seq_ms, "steps": seq_timed, "workers": 1}
+
+    # roofline of the dominant stage (HIP events around each stage of pbg_train_step, on its stream)
+    alg = algorithmic(w, spec)
+    dominant = max((k for k in stages if k in alg), key=lambda k: stages[k])
+    bound, units_per_batch = alg[dominant]
+    launches = {"scores": 2, "backward_dn": 2, "backward_da": 2}.get(dominant, 1)
+    seconds = stages[dominant] * 1e-3
+    units = units_per_batch * workers
+    if bound == "hbm":
+        achieved, peak, unit = units / seconds / 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = units / seconds / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+    roofline = {
+        "kernel": dominant, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
+        "frac": achieved / peak, "traffic": None, "launches_in_stage": launches,
+        "avg_launch_ms": stages[dominant] / launches,
+        "stages_ms": stages,
+        "all": {k: {"bound": alg[k][0],
+                    "achieved": (alg[k][1] * workers / (stages[k] * 1e-3) / (1e9 if alg[k][0] == "hbm" else 1e12)) if stages[k] > 0 else None}
+                for k in stages if k in alg},
+    }
+
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import hogwild, step as ostep
+
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        cfg = ostep.StepConfig(dim=d, operator=w["operator"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
+                               num_batch_negs=w["batch_negs"], num_uniform_negs=w["uniform_negs"], dynamic=w["dynamic"],
+                               num_relations=w["relations"], lr=0.1, relation_weights=[1.0] * w["relations"])
+        n_cpu = min(n_edges, max(cores * 4 * b, 200_000))
+        cpu_rows = min(e, 2_000_000)  # bounded sample of the table for the host-memory copy
+        w_cpu = tables[0][:cpu_rows].cpu()
+        w_cpu_r = tables[1][:cpu_rows].cpu() if len(tables) > 1 else None
+        rel_cpu = rel_pool.cpu()[torch.arange(n_cpu) // b % 4096]
+        cpu_eps, cpu_edges, cpu_wall = hogwild.run(
+            cfg, w_cpu, (lhs_all[:n_cpu] % cpu_rows).cpu(), (rhs_all[:n_cpu] % cpu_rows).cpu(), rel_cpu, b, cores,
+            args.cpu_seconds, w_rhs=w_cpu_r)
+        cpu = {"value": cpu_eps, "unit": "edges/s", "cores": cores, "kind": "port",
+               "sample": f"{cpu_edges} edges in {cpu_wall:.1f} s, {cores} HOGWILD processes (oracle.hogwild over shared-memory tables"
+                         f"{'' if cpu_rows == e else f', first {cpu_rows} table rows'})"}
+
+    line = {
+        "metric": "train edges/sec (100 negs/edge) on 1 MI355X",
+        "value": eps, "unit": "edges/s", "n_gpus": 1, "steps": timed, "warmup": warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
+                   "hogwild_workers": workers, "uniform_negative_draw": "torch.randint on device, inside the timed loop",
+                   "mean_loss_per_edge_last_call": loss},
+        "sequential": seq,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -154,6 +154,17 @@ typedef struct pbg_step_buffers {
 size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc);
 int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream);
 
+/* The same step with HIP events recorded on `stream` between its stages; waits
+ * for the step to finish and writes the pbg_train_step_num_stages() stage
+ * durations in milliseconds to stage_ms (HOST memory).  Stages: 0 gather +
+ * element-wise operator + prepare, 1 linear operator, 2 score GEMMs, 3 loss,
+ * 4 dN GEMMs, 5 dA GEMMs, 6 chain rule to raw rows, 7 operator parameters,
+ * 8 key sort, 9 RowAdagrad update.  No counterpart in the reference (it logs wall-clock per bucket,
+ * train_cpu.py:696-703). */
+int pbg_train_step_num_stages(void);
+int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,
+                           float* stage_ms);
+
 /* MultiRelationEmbedder.forward alone (model.py:624-762): scores only, tables
  * untouched.  lhs_pos/rhs_pos: [K, B]; lhs_neg: [K, B, Nl]; rhs_neg: [K, B, Nr]
  * with N = (num_batch_negs ? min(num_batch_negs, B) : 0) + U, or 0 when that

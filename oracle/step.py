@@ -496,7 +496,7 @@ def forward_backward(
     loss = cfg.relation_weights[relation] * (lhs_loss + rhs_loss)
 
     out = StepOutput(
-        loss=float(loss),
+        loss=float(loss.detach()),
         violators_lhs=int((scores.lhs_neg > scores.lhs_pos.unsqueeze(1)).sum()),
         violators_rhs=int((scores.rhs_neg > scores.rhs_pos.unsqueeze(1)).sum()),
         count=int(lhs.shape[0]),

@@ -75,6 +75,8 @@ SIGNATURES = {
                                c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_float, c_float, c_void_p]),
     "pbg_train_step_workspace_bytes": (c_size_t, [POINTER(StepDesc)]),
     "pbg_train_step": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p]),
+    "pbg_train_step_num_stages": (c_int32, []),
+    "pbg_train_step_profile": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, POINTER(c_float)]),
     "pbg_model_forward": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),
     "pbg_reverse_permutation": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p]),

@@ -1015,12 +1015,17 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
 
 dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 1, kWavesPerBlock)); }
 
-// prep + operator GEMM (linear) + score GEMMs
-int run_forward(const Plan& plan, hipStream_t stream) {
+int run_prep(const Plan& plan, hipStream_t stream) {
   const StepCtx& c = plan.c;
-  const int D = c.D, K = c.K, C = c.C, P = c.P;
-  const int64_t jobs = (int64_t)K * (2 * C * P + C * c.side[0].u + C * c.side[1].u);
+  const int64_t jobs = (int64_t)c.K * (2 * c.C * c.P + c.C * c.side[0].u + c.C * c.side[1].u);
   PBG_DISPATCH_NVH(plan.nvh, prep_kernel, wave_grid(jobs), stream, c);
+  return check_launch("step prep");
+}
+
+// the `linear` operator: one GEMM per side that has it, then comparator.prepare
+int run_operator_forward(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int D = c.D, K = c.K;
   int rc;
   if (c.op == PBG_OP_LINEAR) {
     for (int s = 0; s < 2; ++s) {
@@ -1036,6 +1041,14 @@ int run_forward(const Plan& plan, hipStream_t stream) {
       PBG_DISPATCH_NVH(plan.nvh, prepare_staged_kernel, wave_grid((int64_t)K * sd.op_rows), stream, c, s);
     }
   }
+  return check_launch("step operator");
+}
+
+// score GEMMs
+int run_scores(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int D = c.D, K = c.K, C = c.C, P = c.P;
+  int rc;
   for (int s = 0; s < 2; ++s) {
     const SideCtx& sd = c.side[s];
     const SideCtx& so = c.side[1 - s];
@@ -1051,7 +1064,7 @@ int run_forward(const Plan& plan, hipStream_t stream) {
   return check_launch("step forward");
 }
 
-int run_backward(const Plan& plan, hipStream_t stream) {
+int run_backward_dn(const Plan& plan, hipStream_t stream) {
   const StepCtx& c = plan.c;
   const int D = c.D, K = c.K, C = c.C, P = c.P;
   int rc;
@@ -1067,6 +1080,13 @@ int run_backward(const Plan& plan, hipStream_t stream) {
     g.m = sd.nn; g.n = D; g.k = P; g.batch = K * C; g.alpha = 1.f; g.beta = 0.f;
     if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
   }
+  return check_launch("step backward dN");
+}
+
+int run_backward_da(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int D = c.D, K = c.K, C = c.C, P = c.P;
+  int rc;
   for (int s = 0; s < 2; ++s) {  // dA = dS * N -> the other side's positives (operated ones in dynamic mode)
     const SideCtx& sd = c.side[s];
     const SideCtx& so = c.side[1 - s];
@@ -1083,9 +1103,14 @@ int run_backward(const Plan& plan, hipStream_t stream) {
     g.m = P; g.n = D; g.k = sd.nn; g.batch = K * C; g.alpha = 1.f;
     if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
   }
-  const int64_t jobs = (int64_t)K * (2 * c.B + C * c.side[0].u + C * c.side[1].u);
-  PBG_DISPATCH_NVH(plan.nvh, rowback_kernel, wave_grid(jobs), stream, c);
   return check_launch("step backward");
+}
+
+int run_rowback(const Plan& plan, hipStream_t stream) {
+  const StepCtx& c = plan.c;
+  const int64_t jobs = (int64_t)c.K * (2 * c.B + c.C * c.side[0].u + c.C * c.side[1].u);
+  PBG_DISPATCH_NVH(plan.nvh, rowback_kernel, wave_grid(jobs), stream, c);
+  return check_launch("step rowback");
 }
 
 int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, hipStream_t stream) {
@@ -1136,24 +1161,44 @@ extern "C" size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc) {
   return plan.bytes;
 }
 
-extern "C" int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream) {
+namespace {
+// prep | operator forward | score GEMMs | loss | dN GEMMs | dA GEMMs | rowback | params | sort | update
+constexpr int kStages = 10;
+
+int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_t s, hipEvent_t* ev) {
   int rc = validate(desc, true);
   if (rc != PBG_OK) return rc;
   Plan plan;
   make_plan(desc, bufs, &plan);
   if ((rc = check_buffers(desc, bufs, plan, true)) != PBG_OK) return rc;
-  hipStream_t s = (hipStream_t)stream;
   const StepCtx& c = plan.c;
+  auto mark = [&](int i) {
+    if (ev) hipEventRecord(ev[i], s);
+  };
+  mark(0);
   hipLaunchKernelGGL(zero_violators_kernel, dim3((unsigned)ceil_div(c.K * 2, 64)), dim3(64), 0, s, c.violators, c.K * 2);
-  if ((rc = run_forward(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
+  mark(1);
+  if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
+  mark(2);
+  if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
+  mark(3);
   hipLaunchKernelGGL(loss_kernel, wave_grid((int64_t)c.K * c.C * c.P), dim3(kRowThreads), 0, s, c);
   hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
-  if ((rc = run_backward(plan, s)) != PBG_OK) return rc;
+  mark(4);
+  if ((rc = run_backward_dn(plan, s)) != PBG_OK) return rc;
+  mark(5);
+  if ((rc = run_backward_da(plan, s)) != PBG_OK) return rc;
+  mark(6);
+  if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
+  mark(7);
   if ((rc = run_params(desc, bufs, plan, s)) != PBG_OK) return rc;
+  mark(8);
   const int64_t npairs = (int64_t)c.K * c.rk;
   const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
   rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, bits_for(rows - 1) + c.kbits, plan.sort_temp, s);
   if (rc != PBG_OK) return rc;
+  mark(9);
   if (desc->shared_table) {
     rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s);
@@ -1161,6 +1206,33 @@ extern "C" int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers*
     rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s);
   }
+  mark(10);
+  return rc;
+}
+}  // namespace
+
+extern "C" int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream) {
+  return run_step(desc, bufs, (hipStream_t)stream, nullptr);
+}
+
+extern "C" int pbg_train_step_num_stages(void) { return kStages; }
+
+extern "C" int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,
+                                      float* stage_ms) {
+  if (!stage_ms) return fail(PBG_ERR_INVALID, "pbg_train_step_profile: null output");
+  hipEvent_t ev[kStages + 1];
+  for (int i = 0; i <= kStages; ++i) {
+    if (hipEventCreate(&ev[i]) != hipSuccess) return fail(PBG_ERR_LAUNCH, "pbg_train_step_profile: hipEventCreate failed");
+  }
+  int rc = run_step(desc, bufs, (hipStream_t)stream, ev);
+  if (rc == PBG_OK) {
+    if (hipEventSynchronize(ev[kStages]) != hipSuccess) rc = fail(PBG_ERR_LAUNCH, "pbg_train_step_profile: sync failed");
+  }
+  for (int i = 0; i < kStages && rc == PBG_OK; ++i) {
+    if (hipEventElapsedTime(&stage_ms[i], ev[i], ev[i + 1]) != hipSuccess)
+      rc = fail(PBG_ERR_LAUNCH, "pbg_train_step_profile: elapsed time failed");
+  }
+  for (int i = 0; i <= kStages; ++i) hipEventDestroy(ev[i]);
   return rc;
 }
 
@@ -1175,7 +1247,9 @@ extern "C" int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffe
   if (!lhs_pos || !rhs_pos || (c.side[0].nn > 0 && !lhs_neg) || (c.side[1].nn > 0 && !rhs_neg))
     return fail(PBG_ERR_INVALID, "pbg_model_forward: null output");
   hipStream_t s = (hipStream_t)stream;
-  if ((rc = run_forward(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
   hipLaunchKernelGGL(scores_out_kernel, wave_grid((int64_t)c.K * c.B), dim3(kRowThreads), 0, s, c, lhs_pos, rhs_pos,
                      lhs_neg, rhs_neg);
   return check_launch("pbg_model_forward");

@@ -314,6 +314,17 @@ class StepRunner:
         bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
         check(_lib.lib().pbg_train_step(ctypes.byref(self.desc), ctypes.byref(bufs), _stream()))
 
+    STAGES = ("prep", "operator", "scores", "loss", "backward_dn", "backward_da", "rowback", "params", "sort", "update")
+
+    def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> List[float]:
+        """train() with HIP events between the stages; synchronises and returns
+        the stage durations in milliseconds (order: StepRunner.STAGES)."""
+        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
+        n = _lib.lib().pbg_train_step_num_stages()
+        out = (ctypes.c_float * n)()
+        check(_lib.lib().pbg_train_step_profile(ctypes.byref(self.desc), ctypes.byref(bufs), _stream(), out))
+        return [float(x) for x in out]
+
     def forward(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None):
         """Scores only: (lhs_pos[K,B], rhs_pos[K,B], lhs_neg[K,B,Nl], rhs_neg[K,B,Nr])."""
         s = self.spec
