@@ -20,6 +20,10 @@ from . import step as ostep
 
 def _worker(rank: int, cfg, shared: Dict[str, torch.Tensor], lhs, rhs, rel, batch_size: int, max_seconds: float,
             barrier, out_queue) -> None:
+    # CPU workers must never open the GPU (autograd's first backward() would
+    # otherwise ask the HIP runtime for its device count)
+    os.environ["HIP_VISIBLE_DEVICES"] = ""
+    os.environ["ROCR_VISIBLE_DEVICES"] = ""
     torch.set_num_threads(1)
     torch.manual_seed(os.getpid())
     st = ostep.TrainState(
@@ -81,6 +85,9 @@ def run(cfg, w_lhs: torch.Tensor, lhs: torch.Tensor, rhs: torch.Tensor, rel: tor
     # split_almost_equally (util.py:227-236)
     per = lhs.shape[0] // workers + (1 if lhs.shape[0] % workers else 0)
     procs = []
+    saved_env = {k: os.environ.get(k) for k in ("HIP_VISIBLE_DEVICES", "ROCR_VISIBLE_DEVICES")}
+    os.environ["HIP_VISIBLE_DEVICES"] = ""
+    os.environ["ROCR_VISIBLE_DEVICES"] = ""
     for r in range(workers):
         sl = perm[min(r * per, lhs.shape[0]):min((r + 1) * per, lhs.shape[0])]
         if not cfg.dynamic:
@@ -89,6 +96,11 @@ def run(cfg, w_lhs: torch.Tensor, lhs: torch.Tensor, rhs: torch.Tensor, rel: tor
                                               batch_size, max_seconds, barrier, queue))
         p.start()
         procs.append(p)
+    for k, v in saved_env.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
     # fail fast when a worker dies (util.py:320-347 polls the same way)
     import queue as queue_mod
 
