@@ -64,13 +64,14 @@ int pbg_gather_rows(const float* table, int64_t num_rows, int32_t dim, const int
 /* ------------------------------------------------------------------------
  * RowAdagrad.  Replaces RowAdagrad.step (row_adagrad.py:48-109).
  * Sparse branch (:80-96): `idx[n]` / `grad_rows[n, dim]` are the uncoalesced
- * COO gradient; duplicates are summed (sort by index, segmented sum) before
+ * COO gradient; duplicates are summed (sort by index, segmented sum, formed in
+ * place: grad_rows is CLOBBERED) before
  *   delta = mean_d(g^2); G[r] += delta; W[r] -= lr * g / (sqrt(G_old + delta) + 1e-10).
  * Dense branch (:97-107): `grad[num_rows, dim]`.
  * ---------------------------------------------------------------------- */
 size_t pbg_row_adagrad_sparse_workspace_bytes(int64_t n);
 int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
-                           const int64_t* idx, const float* grad_rows, int64_t n, float lr,
+                           const int64_t* idx, float* grad_rows, int64_t n, float lr,
                            void* workspace, size_t workspace_bytes, pbg_stream_t stream);
 int pbg_row_adagrad_dense(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
                           const float* grad, float lr, pbg_stream_t stream);

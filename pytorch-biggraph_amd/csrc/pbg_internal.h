@@ -33,11 +33,11 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
                int key_bits, void* temp, hipStream_t stream);
 
 // ---- segmented RowAdagrad over sorted (row << kbits | worker) keys ---------
-// keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim].  A key's
-// row field addresses table 0 for row < rows0, table 1 (row - rows0) for
+// keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim], which is
+// clobbered (duplicate sums are formed in place).  A key's row field addresses table 0 for row < rows0, table 1 (row - rows0) for
 // row < rows0 + rows1, and is ignored beyond.
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits,
-                       const float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
+                       float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
                        float* g1, int64_t rows1, float lr, hipStream_t stream);
 
 // ---- plain fp32 batched GEMM on MFMA ----------------------------------------

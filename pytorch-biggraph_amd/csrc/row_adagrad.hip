@@ -43,12 +43,134 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const float* _
 }
 
 // ---- segmented RowAdagrad over sorted keys -----------------------------------
-// One wave per sorted position; only the wave sitting on the first key of a row
-// works.  It walks the row's keys: equal keys (same worker) are summed, then one
-// Adagrad update is applied per worker in ascending worker order, exactly as if
-// the workers' sparse steps had been applied one after another.
+// Keys are (row << kbits | worker), sorted.  Equal keys form a "run" (the
+// duplicates of one row inside one worker's batch, to be summed); the runs of
+// one row are applied one Adagrad update after another in worker order, exactly
+// as if the workers' sparse steps had been applied in sequence.  Power-law
+// graphs make single runs hundreds of rows long, so the summation is spread
+// over three kernels, all deterministic and in place in grad_rows:
+//   tile_reduce   one wave per tile of kTile sorted positions sums every piece
+//                 (maximal stretch of equal keys inside the tile) longer than 1
+//                 into the gradient row of the piece's first position;
+//   run_combine   one wave per run that crosses tile borders adds the pieces of
+//                 the later tiles into the row of the run's first position;
+//   row_update    one wave per row walks its runs (one gradient row each).
+constexpr int kTile = 32;
+
 template <int NV, bool VEC>
-__global__ __launch_bounds__(kRowThreads) void row_adagrad_sorted_kernel(
+struct RowRegs {
+  static constexpr int W = VEC ? 4 : 1;
+  float v[NV * W];
+
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int q = 0; q < NV * W; ++q) v[q] = 0.f;
+  }
+  __device__ __forceinline__ void load(const float* __restrict__ p, int nv, int lane) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = i * kWave + lane;
+      if (VEC) {
+        const float4 x = (e < nv) ? reinterpret_cast<const float4*>(p)[e] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[i * W + 0] = x.x; v[i * W + 1] = x.y; v[i * W + 2] = x.z; v[i * W + 3] = x.w;
+      } else {
+        v[i] = (e < nv) ? p[e] : 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void add(const float* __restrict__ p, int nv, int lane) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = i * kWave + lane;
+      if (e < nv) {
+        if (VEC) {
+          const float4 x = reinterpret_cast<const float4*>(p)[e];
+          v[i * W + 0] += x.x; v[i * W + 1] += x.y; v[i * W + 2] += x.z; v[i * W + 3] += x.w;
+        } else {
+          v[i] += p[e];
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float* __restrict__ p, int nv, int lane) const {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = i * kWave + lane;
+      if (e < nv) {
+        if (VEC) {
+          reinterpret_cast<float4*>(p)[e] = make_float4(v[i * W + 0], v[i * W + 1], v[i * W + 2], v[i * W + 3]);
+        } else {
+          p[e] = v[i];
+        }
+      }
+    }
+  }
+};
+
+// First position in (start, n) whose key, shifted right by `shift`, differs from
+// `want`; all 64 lanes scan together.
+__device__ __forceinline__ int64_t scan_end(const uint64_t* __restrict__ keys, int64_t start, int64_t n,
+                                            uint64_t want, int shift, int lane) {
+  int64_t base = start + 1;
+  while (true) {
+    const int64_t j = base + lane;
+    const bool same = (j < n) && ((keys[j] >> shift) == want);
+    const uint64_t m = __ballot(same);
+    if (m != ~0ull) return base + (__ffsll((unsigned long long)~m) - 1);
+    base += kWave;
+  }
+}
+
+template <int NV, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t* __restrict__ keys,
+                                                                  const uint32_t* __restrict__ vals, int64_t n,
+                                                                  float* __restrict__ grad_rows, int dim) {
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  const int64_t begin = tile * kTile;
+  if (begin >= n) return;
+  const int64_t end = (begin + kTile < n) ? begin + kTile : n;
+  const int nv = VEC ? (dim >> 2) : dim;
+  // one key per lane for the whole tile, then pieces are found with ballots
+  const int64_t mine = begin + lane;
+  const uint64_t key = (mine < end) ? keys[mine] : 0ull;
+  const uint64_t prev = __shfl_up(key, 1, 64);
+  const bool starts = (mine < end) && (lane == 0 || prev != key);
+  uint64_t heads = __ballot(starts);  // bit l set: a piece starts at begin + l
+  while (heads != 0ull) {
+    const int a = __ffsll((unsigned long long)heads) - 1;
+    heads &= heads - 1;
+    const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
+    if (b - a < 2) continue;
+    RowRegs<NV, VEC> acc;
+    acc.load(grad_rows + (int64_t)vals[begin + a] * dim, nv, lane);
+    for (int j = a + 1; j < b; ++j) acc.add(grad_rows + (int64_t)vals[begin + j] * dim, nv, lane);
+    acc.store(grad_rows + (int64_t)vals[begin + a] * dim, nv, lane);
+  }
+}
+
+template <int NV, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t* __restrict__ keys,
+                                                                  const uint32_t* __restrict__ vals, int64_t n,
+                                                                  float* __restrict__ grad_rows, int dim) {
+  const int lane = threadIdx.x & 63;
+  const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const uint64_t key = keys[i];
+  if (i > 0 && keys[i - 1] == key) return;             // not the head of a run
+  const int64_t tile_end = (i / kTile + 1) * kTile;
+  if (tile_end >= n || keys[tile_end] != key) return;  // the run ends inside its first tile
+  const int64_t end = scan_end(keys, tile_end, n, key, 0, lane);
+  const int nv = VEC ? (dim >> 2) : dim;
+  RowRegs<NV, VEC> acc;
+  float* head = grad_rows + (int64_t)vals[i] * dim;
+  acc.load(head, nv, lane);
+  for (int64_t p = tile_end; p < end; p += kTile) acc.add(grad_rows + (int64_t)vals[p] * dim, nv, lane);
+  acc.store(head, nv, lane);
+}
+
+template <int NV, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
     const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
     float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
@@ -68,63 +190,28 @@ __global__ __launch_bounds__(kRowThreads) void row_adagrad_sorted_kernel(
     wrow = w1 + ((int64_t)row - rows0) * dim;
     gptr = g1 + ((int64_t)row - rows0);
   }
-  constexpr int W = VEC ? 4 : 1;
-  float w[NV * W];
   const int nv = VEC ? (dim >> 2) : dim;
-#pragma unroll
-  for (int v = 0; v < NV; ++v) {
-    const int e = v * kWave + lane;
-    if (VEC) {
-      float4 x = (e < nv) ? reinterpret_cast<const float4*>(wrow)[e] : make_float4(0.f, 0.f, 0.f, 0.f);
-      w[v * 4 + 0] = x.x; w[v * 4 + 1] = x.y; w[v * 4 + 2] = x.z; w[v * 4 + 3] = x.w;
-    } else {
-      w[v] = (e < nv) ? wrow[e] : 0.f;
-    }
-  }
+  RowRegs<NV, VEC> w;
+  w.load(wrow, nv, lane);
   float gsum = *gptr;
   const float fdim = (float)dim;
   int64_t j = i;
   while (j < n && (keys[j] >> kbits) == row) {
     const uint64_t key = keys[j];
-    float g[NV * W];
-#pragma unroll
-    for (int q = 0; q < NV * W; ++q) g[q] = 0.f;
-    while (j < n && keys[j] == key) {
-      const float* grow = grad_rows + (int64_t)vals[j] * dim;
-#pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const int e = v * kWave + lane;
-        if (e < nv) {
-          if (VEC) {
-            float4 x = reinterpret_cast<const float4*>(grow)[e];
-            g[v * 4 + 0] += x.x; g[v * 4 + 1] += x.y; g[v * 4 + 2] += x.z; g[v * 4 + 3] += x.w;
-          } else {
-            g[v] += grow[e];
-          }
-        }
-      }
-      ++j;
-    }
+    RowRegs<NV, VEC> g;
+    g.load(grad_rows + (int64_t)vals[j] * dim, nv, lane);  // the run's sum (tile_reduce / run_combine)
+    // a single-worker call has one run per row: no need to look for its end
+    j = (kbits == 0) ? n : scan_end(keys, j, n, key, 0, lane);
     float sq = 0.f;
 #pragma unroll
-    for (int q = 0; q < NV * W; ++q) sq += g[q] * g[q];
+    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) sq += g.v[q] * g.v[q];
     const float delta = wave_sum(sq) / fdim;
     gsum += delta;
     const float stdv = sqrtf(gsum) + 1e-10f;
 #pragma unroll
-    for (int q = 0; q < NV * W; ++q) w[q] += (-lr * g[q]) / stdv;
+    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) w.v[q] += (-lr * g.v[q]) / stdv;
   }
-#pragma unroll
-  for (int v = 0; v < NV; ++v) {
-    const int e = v * kWave + lane;
-    if (e < nv) {
-      if (VEC) {
-        reinterpret_cast<float4*>(wrow)[e] = make_float4(w[v * 4 + 0], w[v * 4 + 1], w[v * 4 + 2], w[v * 4 + 3]);
-      } else {
-        wrow[e] = w[v];
-      }
-    }
-  }
+  w.store(wrow, nv, lane);
   if (lane == 0) *gptr = gsum;
 }
 
@@ -168,13 +255,19 @@ __global__ void async_adagrad_dense_kernel(float* __restrict__ p, float* __restr
 }
 
 template <bool VEC>
-int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, const float* grad_rows,
+int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                   int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
                   hipStream_t stream) {
-  const dim3 grid((unsigned)ceil_div(n, kRowThreads / kWave)), block(kRowThreads);
-#define PBG_LAUNCH(NV)                                                                                          \
-  hipLaunchKernelGGL((row_adagrad_sorted_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, kbits, grad_rows, \
-                     dim, w0, g0, rows0, w1, g1, rows1, lr)
+  const int wpb = kRowThreads / kWave;
+  const dim3 grid((unsigned)ceil_div(n, wpb)), block(kRowThreads);
+  const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
+#define PBG_LAUNCH(NV)                                                                                             \
+  do {                                                                                                             \
+    hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim);  \
+    hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, grad_rows, dim);       \
+    hipLaunchKernelGGL((row_update_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, kbits, grad_rows, dim,  \
+                       w0, g0, rows0, w1, g1, rows1, lr);                                                          \
+  } while (0)
   if (nvec <= 1) PBG_LAUNCH(1);
   else if (nvec <= 2) PBG_LAUNCH(2);
   else if (nvec <= 4) PBG_LAUNCH(4);
@@ -187,7 +280,7 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 
 }  // namespace
 
-int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, const float* grad_rows,
+int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                        int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
                        hipStream_t stream) {
   if (n <= 0) return PBG_OK;
@@ -246,7 +339,7 @@ SparseWs carve_sparse(void* base, int64_t n) {
 extern "C" size_t pbg_row_adagrad_sparse_workspace_bytes(int64_t n) { return carve_sparse(nullptr, n).total; }
 
 extern "C" int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
-                                      const int64_t* idx, const float* grad_rows, int64_t n, float lr,
+                                      const int64_t* idx, float* grad_rows, int64_t n, float lr,
                                       void* workspace, size_t workspace_bytes, pbg_stream_t stream) {
   if (n < 0 || dim <= 0 || num_rows < 0) return fail(PBG_ERR_INVALID, "pbg_row_adagrad_sparse: bad sizes");
   if (n == 0) return PBG_OK;  // row_adagrad.py:81-82

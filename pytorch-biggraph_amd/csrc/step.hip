@@ -721,18 +721,21 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
 // ---------------------------------------------------------------------------
 // operator parameters (standard mode: one relation per batch)
 // ---------------------------------------------------------------------------
-// dth[k, e] = sum over the operator rows of batch k of the parameter gradient of
-// element e: diagonal x.dz, translation dz, complex_diagonal (real | imag).
-__global__ __launch_bounds__(256) void param_grad_kernel(StepCtx c, int s, float* __restrict__ dth) {
-  __shared__ float sh[4][64];
+// dth[k, slice, e] = sum over the operator rows r = slice (mod slices) of batch k
+// of the parameter gradient of element e: diagonal x.dz, translation dz,
+// complex_diagonal (real | imag).  Fixed summation order, no atomics.
+constexpr int kParamGroups = 16;
+__global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c, int s, float* __restrict__ dth,
+                                                                        int slices) {
+  __shared__ float sh[kParamGroups][64];
   const SideCtx& sd = c.side[s];
   const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
-  const int k = blockIdx.y;
+  const int k = blockIdx.y, slice = blockIdx.z;
   const int e = blockIdx.x * 64 + lane;
   const int D = c.D, H = D / 2;
   float acc = 0.f;
   if (e < D) {
-    for (int r = rg; r < sd.op_rows; r += 4) {
+    for (int r = slice * kParamGroups + rg; r < sd.op_rows; r += slices * kParamGroups) {
       const float* dz = sd.dz + ((int64_t)k * sd.op_rows + r) * D;
       if (c.op == PBG_OP_TRANSLATION) {
         acc += dz[e];
@@ -758,12 +761,17 @@ __global__ __launch_bounds__(256) void param_grad_kernel(StepCtx c, int s, float
   }
   sh[rg][lane] = acc;
   __syncthreads();
-  if (rg == 0 && e < D) dth[(int64_t)k * D + e] = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+  if (rg == 0 && e < D) {
+    float total = 0.f;
+#pragma unroll
+    for (int g = 0; g < kParamGroups; ++g) total += sh[g][lane];
+    dth[((int64_t)k * slices + slice) * D + e] = total;
+  }
 }
 
 // AsyncAdagrad (async_adagrad.py:75-85), the K batches' gradients applied in order.
-__global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ dth, int64_t psize, float* p0,
-                                    float* p1, float* s0, float* s1, float lr) {
+__global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ dth, int slices, int64_t psize,
+                                    float* p0, float* p1, float* s0, float* s1, float lr) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= psize) return;
   const int H = c.D / 2;
@@ -783,7 +791,8 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
       p = p0 + r * psize + e;
       st = s0 + r * psize + e;
     }
-    const float g = dth[(int64_t)k * psize + e];
+    float g = 0.f;
+    for (int sl = 0; sl < slices; ++sl) g += dth[((int64_t)k * slices + sl) * psize + e];
     const float sum = *st + g * g;
     *st = sum;
     *p += -lr * (g / (sqrtf(sum) + 1e-10f));
@@ -802,6 +811,7 @@ struct Plan {
   uint32_t* vals_b;
   void* sort_temp;
   int64_t psize;  // floats of parameter gradient per batch
+  int pslices[2]; // partial sums per batch of the element-wise parameter gradients
   int nvh;
 };
 
@@ -938,8 +948,15 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->psize = 0;
   if (c.op == PBG_OP_LINEAR) plan->psize = (int64_t)D * D;
   else if (c.op != PBG_OP_NONE) plan->psize = D;
-  for (int s = 0; s < 2; ++s)
-    if (c.side[s].has_op && plan->psize > 0) plan->dth[s] = takef((size_t)K * plan->psize);
+  for (int s = 0; s < 2; ++s) {
+    plan->pslices[s] = 1;
+    if (!c.side[s].has_op || plan->psize == 0) continue;
+    if (c.op != PBG_OP_LINEAR) {
+      int sl = (int)ceil_div(c.side[s].op_rows, 32 * kParamGroups);
+      plan->pslices[s] = sl < 1 ? 1 : (sl > 16 ? 16 : sl);
+    }
+    plan->dth[s] = takef((size_t)K * plan->pslices[s] * plan->psize);
+  }
 
   const int64_t npairs = (int64_t)K * c.rk;
   c.gr = takef((size_t)npairs * D);
@@ -1140,11 +1157,11 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
       h.m = D; h.n = D; h.k = sd.op_rows; h.batch = K; h.alpha = 1.f; h.beta = 0.f;
       if ((rc = gemm_f32(h, stream)) != PBG_OK) return rc;
     } else {
-      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K), dim3(256), 0, stream, c, s,
-                         plan.dth[s]);
+      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
+                         dim3(kParamGroups * 64), 0, stream, c, s, plan.dth[s], plan.pslices[s]);
     }
     hipLaunchKernelGGL(param_update_kernel, dim3((unsigned)ceil_div(plan.psize, 256)), dim3(256), 0, stream, c, s,
-                       plan.dth[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
+                       plan.dth[s], plan.pslices[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
   }
   return check_launch("step params");
 }
