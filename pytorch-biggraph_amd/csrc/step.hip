@@ -62,6 +62,7 @@ struct StepCtx {
   float* pos[2];   // [K*C*P] positive score paired with lhs negatives / rhs negatives
   float* dpos[2];  // gradients of the above (standard mode: only [0], already summed)
   float* lossrow;  // [K*C*P]
+  int* violrow;    // [K*C*P, 2] violators of each edge (lhs, rhs)
   int rk;          // gradient rows per batch
   int kbits;
   float* gr;       // [K*rk, D] gradient rows
@@ -441,6 +442,8 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     }
     if (lane == 0) {
       c.lossrow[job] = 0.f;
+      c.violrow[job * 2] = 0;
+      c.violrow[job * 2 + 1] = 0;
       c.dpos[0][job] = 0.f;
       if (c.dynamic) c.dpos[1][job] = 0.f;
       c.pos[0][job] = 0.f;
@@ -456,6 +459,7 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
 
   float loss_acc = 0.f;  // per-lane partial, unweighted
   float dposv[2] = {0.f, 0.f};
+  int violv[2] = {0, 0};
   for (int s = 0; s < 2; ++s) {
     const SideCtx& sd = c.side[s];
     const int nn = sd.nn;
@@ -529,11 +533,13 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     int vtot = viol;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) vtot += __shfl_xor(vtot, off, 64);
-    if (lane == 0 && vtot > 0) atomicAdd(&c.violators[k * 2 + s], (unsigned long long)vtot);
+    violv[s] = vtot;
   }
   const float loss_row = wave_sum(loss_acc) * w;
   if (lane == 0) {
     c.lossrow[job] = loss_row;
+    c.violrow[job * 2] = violv[0];
+    c.violrow[job * 2 + 1] = violv[1];
     c.pos[0][job] = posv[0];
     if (c.dynamic) {
       c.pos[1][job] = posv[1];
@@ -545,25 +551,37 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
   }
 }
 
-// loss_out[k] = sum of the batch's per-edge losses, in a fixed order
+// loss_out[k] = sum of the batch's per-edge losses, in a fixed order; violators likewise
 __global__ __launch_bounds__(256) void loss_reduce_kernel(StepCtx c) {
   __shared__ float sh[256];
+  __shared__ long long shv[2][256];
   const int CP = c.C * c.P;
   const float* rows = c.lossrow + (int64_t)blockIdx.x * CP;
+  const int* viol = c.violrow + (int64_t)blockIdx.x * CP * 2;
   float acc = 0.f;
-  for (int q = threadIdx.x; q < CP; q += 256) acc += rows[q];
+  long long v0 = 0, v1 = 0;
+  for (int q = threadIdx.x; q < CP; q += 256) {
+    acc += rows[q];
+    v0 += viol[q * 2];
+    v1 += viol[q * 2 + 1];
+  }
   sh[threadIdx.x] = acc;
+  shv[0][threadIdx.x] = v0;
+  shv[1][threadIdx.x] = v1;
   __syncthreads();
   for (int off = 128; off > 0; off >>= 1) {
-    if ((int)threadIdx.x < off) sh[threadIdx.x] += sh[threadIdx.x + off];
+    if ((int)threadIdx.x < off) {
+      sh[threadIdx.x] += sh[threadIdx.x + off];
+      shv[0][threadIdx.x] += shv[0][threadIdx.x + off];
+      shv[1][threadIdx.x] += shv[1][threadIdx.x + off];
+    }
     __syncthreads();
   }
-  if (threadIdx.x == 0) c.loss_out[blockIdx.x] = sh[0];
-}
-
-__global__ void zero_violators_kernel(unsigned long long* v, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) v[i] = 0ull;
+  if (threadIdx.x == 0) {
+    c.loss_out[blockIdx.x] = sh[0];
+    c.violators[blockIdx.x * 2] = (unsigned long long)shv[0][0];
+    c.violators[blockIdx.x * 2 + 1] = (unsigned long long)shv[1][0];
+  }
 }
 
 // forward-only output: de-chunked, masked scores (model.py:842-844)
@@ -944,6 +962,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     c.dpos[1] = c.dpos[0];
   }
   c.lossrow = takef(K * CP);
+  c.violrow = (int*)take(K * CP * 2, sizeof(int));
 
   plan->psize = 0;
   if (c.op == PBG_OP_LINEAR) plan->psize = (int64_t)D * D;
@@ -1193,7 +1212,6 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if (ev) hipEventRecord(ev[i], s);
   };
   mark(0);
-  hipLaunchKernelGGL(zero_violators_kernel, dim3((unsigned)ceil_div(c.K * 2, 64)), dim3(64), 0, s, c.violators, c.K * 2);
   if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
   mark(1);
   if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
