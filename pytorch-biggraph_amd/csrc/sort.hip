@@ -63,10 +63,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
   // offset of digit t for this block = keys with a smaller digit anywhere
   //                                  + keys with digit t in earlier blocks
   uint32_t total = 0, before = 0;
-  for (int b = 0; b < nblocks; ++b) {
-    const uint32_t cnt = counts[(int64_t)b * kRadix + t];
-    total += cnt;
-    if (b < (int)blockIdx.x) before += cnt;
+  for (int b0 = 0; b0 < nblocks; b0 += 8) {  // eight independent loads in flight
+    uint32_t cnt[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cnt[u] = (b0 + u < nblocks) ? counts[(int64_t)(b0 + u) * kRadix + t] : 0u;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      total += cnt[u];
+      if (b0 + u < (int)blockIdx.x) before += cnt[u];
+    }
   }
   scan[t] = total;
   __syncthreads();
