@@ -174,6 +174,58 @@ int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, f
                       float* rhs_pos, float* lhs_neg, float* rhs_neg, pbg_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Plugin-level entry points: one operator / comparator / loss at a time, forward
+ * and backward, for code that calls the plugin classes directly (the reference's
+ * unit tests do).  The training step above does not go through these.
+ * ---------------------------------------------------------------------- */
+/* AbstractOperator.forward / AbstractDynamicOperator.forward (operators.py:49-157,
+ * 197-338): y[i] = op(x[i]).  rel == NULL: one operator, parameters p0 (diagonal
+ * | translation | linear_transformation | real) and p1 (imag).  rel != NULL:
+ * rel[n_rows] selects one of num_ops parameter rows per input row. */
+int pbg_operator_forward(int32_t op, int32_t dim, int64_t n_rows, const float* x, const float* p0,
+                         const float* p1, const int64_t* rel, int64_t num_ops, float* y, pbg_stream_t stream);
+/* Its gradient: dx is written; dp0 / dp1 are ACCUMULATED into (zero them first). */
+int pbg_operator_backward(int32_t op, int32_t dim, int64_t n_rows, const float* x, const float* dy,
+                          const float* p0, const float* p1, const int64_t* rel, int64_t num_ops, float* dx,
+                          float* dp0, float* dp1, pbg_stream_t stream);
+
+/* AbstractComparator.prepare (model.py:161-162,187-192,251-252): y = x for dot
+ * and l2, x / ||x|| for cos.  aux[n] (optional) receives 1/||x|| (cos) or
+ * ||x||^2 (l2). */
+int pbg_comparator_prepare(int32_t cmp, int32_t dim, int64_t n, const float* x, float* y, float* aux,
+                           pbg_stream_t stream);
+int pbg_comparator_prepare_backward(int32_t cmp, int32_t dim, int64_t n, const float* dy, const float* y,
+                                    const float* aux, float* dx, pbg_stream_t stream);
+
+/* AbstractComparator.forward (model.py:164-182,194-212,254-278):
+ * lhs_pos, rhs_pos [chunks, p, dim]; lhs_neg [chunks, ln, dim]; rhs_neg [chunks, rn, dim]
+ * -> pos [chunks, p], lhs_neg_scores [chunks, p, ln] = rhs_pos x lhs_neg,
+ *    rhs_neg_scores [chunks, p, rn] = lhs_pos x rhs_neg.
+ * The workspace is only needed by l2. */
+size_t pbg_comparator_workspace_bytes(int32_t chunks, int32_t p, int32_t ln, int32_t rn);
+int pbg_comparator_forward(int32_t cmp, int32_t chunks, int32_t p, int32_t ln, int32_t rn, int32_t dim,
+                           const float* lhs_pos, const float* rhs_pos, const float* lhs_neg,
+                           const float* rhs_neg, float* pos, float* lhs_neg_scores, float* rhs_neg_scores,
+                           void* workspace, size_t workspace_bytes, pbg_stream_t stream);
+int pbg_comparator_backward(int32_t cmp, int32_t chunks, int32_t p, int32_t ln, int32_t rn, int32_t dim,
+                            const float* lhs_pos, const float* rhs_pos, const float* lhs_neg,
+                            const float* rhs_neg, const float* pos, const float* lhs_neg_scores,
+                            const float* rhs_neg_scores, const float* dpos, const float* dlhs_neg_scores,
+                            const float* drhs_neg_scores, float* dlhs_pos, float* drhs_pos, float* dlhs_neg,
+                            float* drhs_neg, void* workspace, size_t workspace_bytes, pbg_stream_t stream);
+
+/* AbstractLossFunction.forward (losses.py:53-161): pos [num_pos], neg [num_pos,
+ * num_neg], weight [num_pos] or NULL -> *out (device scalar).  row_workspace
+ * holds num_pos floats. */
+int pbg_loss_forward(int32_t loss, float margin, int64_t num_pos, int32_t num_neg, const float* pos,
+                     const float* neg, const float* weight, float* out, float* row_workspace,
+                     pbg_stream_t stream);
+/* Its gradient, scaled by *upstream (device scalar). */
+int pbg_loss_backward(int32_t loss, float margin, int64_t num_pos, int32_t num_neg, const float* pos,
+                      const float* neg, const float* weight, const float* upstream, float* dpos,
+                      float* dneg, pbg_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Permutation helpers.  Replace the `_C` module (util.cpp:425-460).
  * ---------------------------------------------------------------------- */
 /* _C.reverse_permutation (util.cpp:104-125): out[perm[i]] = i. */

@@ -79,6 +79,20 @@ SIGNATURES = {
     "pbg_train_step_profile": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, POINTER(c_float)]),
     "pbg_model_forward": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),
+    "pbg_operator_forward": (c_int32, [c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                       c_void_p, c_void_p]),
+    "pbg_operator_backward": (c_int32, [c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "pbg_comparator_prepare": (c_int32, [c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "pbg_comparator_prepare_backward": (c_int32, [c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                  c_void_p]),
+    "pbg_comparator_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "pbg_comparator_forward": (c_int32, [c_int32] * 6 + [c_void_p] * 8 + [c_size_t, c_void_p]),
+    "pbg_comparator_backward": (c_int32, [c_int32] * 6 + [c_void_p] * 15 + [c_size_t, c_void_p]),
+    "pbg_loss_forward": (c_int32, [c_int32, c_float, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p]),
+    "pbg_loss_backward": (c_int32, [c_int32, c_float, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_void_p, c_void_p]),
     "pbg_reverse_permutation": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p]),
     "pbg_shuffle_rows": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "pbg_randperm_workspace_bytes": (c_size_t, [c_int64]),

@@ -22,6 +22,7 @@
 #include <cstring>
 
 #include "pbg_internal.h"
+#include "row_ops.h"
 
 namespace pbg {
 namespace {
@@ -71,163 +72,6 @@ struct StepCtx {
   unsigned long long* violators;  // [K, 2]
   float* loss_out;                // [K]
 };
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
-}
-
-template <int NVH>
-struct RowV {
-  float a[2][NVH];
-};
-
-template <int NVH>
-__device__ __forceinline__ RowV<NVH> row_zero() {
-  RowV<NVH> r;
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) r.a[0][v] = r.a[1][v] = 0.f;
-  return r;
-}
-template <int NVH>
-__device__ __forceinline__ RowV<NVH> row_load(const float* __restrict__ p, int D, int H, int lane) {
-  RowV<NVH> r;
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) {
-    const int h = v * kWave + lane;
-    r.a[0][v] = (h < H) ? p[h] : 0.f;
-    r.a[1][v] = (h < H && H + h < D) ? p[H + h] : 0.f;
-  }
-  return r;
-}
-template <int NVH>
-__device__ __forceinline__ void row_store(float* __restrict__ p, const RowV<NVH>& r, int D, int H, int lane) {
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) {
-    const int h = v * kWave + lane;
-    if (h < H) p[h] = r.a[0][v];
-    if (h < H && H + h < D) p[H + h] = r.a[1][v];
-  }
-}
-template <int NVH>
-__device__ __forceinline__ float row_dot(const RowV<NVH>& x, const RowV<NVH>& y) {  // per-lane partial
-  float acc = 0.f;
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) acc += x.a[0][v] * y.a[0][v] + x.a[1][v] * y.a[1][v];
-  return acc;
-}
-template <int NVH>
-__device__ __forceinline__ void row_axpy(RowV<NVH>& y, float alpha, const RowV<NVH>& x) {
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) {
-    y.a[0][v] += alpha * x.a[0][v];
-    y.a[1][v] += alpha * x.a[1][v];
-  }
-}
-
-// y = op_r(x) for the element-wise operators (operators.py:59-84,128-157 and
-// their dynamic twins :212-249,306-338).  `linear` is a GEMM and not handled here.
-template <int NVH>
-__device__ __forceinline__ RowV<NVH> op_forward(int op, const RowV<NVH>& x, const float* __restrict__ p0,
-                                                const float* __restrict__ p1, int64_t r, int D, int H, int lane) {
-  RowV<NVH> y = x;
-  if (op == PBG_OP_DIAGONAL || op == PBG_OP_TRANSLATION) {
-    const float* p = p0 + r * D;
-#pragma unroll
-    for (int v = 0; v < NVH; ++v) {
-      const int h = v * kWave + lane;
-      const float q0 = (h < H) ? p[h] : 0.f;
-      const float q1 = (h < H && H + h < D) ? p[H + h] : 0.f;
-      if (op == PBG_OP_DIAGONAL) {
-        y.a[0][v] = q0 * x.a[0][v];
-        y.a[1][v] = q1 * x.a[1][v];
-      } else {
-        y.a[0][v] = x.a[0][v] + q0;
-        y.a[1][v] = x.a[1][v] + q1;
-      }
-    }
-  } else if (op == PBG_OP_COMPLEX_DIAGONAL) {
-    const float* re = p0 + r * H;
-    const float* im = p1 + r * H;
-#pragma unroll
-    for (int v = 0; v < NVH; ++v) {
-      const int h = v * kWave + lane;
-      const float br = (h < H) ? re[h] : 0.f;
-      const float bi = (h < H) ? im[h] : 0.f;
-      y.a[0][v] = x.a[0][v] * br - x.a[1][v] * bi;
-      y.a[1][v] = x.a[0][v] * bi + x.a[1][v] * br;
-    }
-  }
-  return y;
-}
-
-// dx = (d op_r / dx)^T dz for the element-wise operators.
-template <int NVH>
-__device__ __forceinline__ RowV<NVH> op_backward(int op, const RowV<NVH>& dz, const float* __restrict__ p0,
-                                                 const float* __restrict__ p1, int64_t r, int D, int H, int lane) {
-  RowV<NVH> dx = dz;
-  if (op == PBG_OP_DIAGONAL) {
-    const float* p = p0 + r * D;
-#pragma unroll
-    for (int v = 0; v < NVH; ++v) {
-      const int h = v * kWave + lane;
-      dx.a[0][v] = ((h < H) ? p[h] : 0.f) * dz.a[0][v];
-      dx.a[1][v] = ((h < H && H + h < D) ? p[H + h] : 0.f) * dz.a[1][v];
-    }
-  } else if (op == PBG_OP_COMPLEX_DIAGONAL) {
-    const float* re = p0 + r * H;
-    const float* im = p1 + r * H;
-#pragma unroll
-    for (int v = 0; v < NVH; ++v) {
-      const int h = v * kWave + lane;
-      const float br = (h < H) ? re[h] : 0.f;
-      const float bi = (h < H) ? im[h] : 0.f;
-      dx.a[0][v] = br * dz.a[0][v] + bi * dz.a[1][v];
-      dx.a[1][v] = br * dz.a[1][v] - bi * dz.a[0][v];
-    }
-  }
-  return dx;
-}
-
-// comparator.prepare (model.py:161-162,187-192,251-252), in place; returns the
-// per-row aux value: 1/norm for cos, norm^2 for l2 (model.py:228-229).
-template <int NVH>
-__device__ __forceinline__ float prepare_row(int cmp, RowV<NVH>& y) {
-  if (cmp == PBG_CMP_DOT) return 0.f;
-  const float nrm = sqrtf(wave_sum(row_dot(y, y)));
-  if (cmp == PBG_CMP_COS) {
-    const float inv = 1.0f / nrm;
-#pragma unroll
-    for (int v = 0; v < NVH; ++v) {
-      y.a[0][v] *= inv;
-      y.a[1][v] *= inv;
-    }
-    return inv;
-  }
-  return nrm * nrm;
-}
-
-// gradient through comparator.prepare: cos: dz = (dy - y (y . dy)) / norm.
-template <int NVH>
-__device__ __forceinline__ RowV<NVH> prepare_backward(int cmp, const RowV<NVH>& dy, const RowV<NVH>& y, float aux) {
-  if (cmp != PBG_CMP_COS) return dy;
-  const float dot = wave_sum(row_dot(y, dy));
-  RowV<NVH> dz;
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) {
-    dz.a[0][v] = aux * (dy.a[0][v] - y.a[0][v] * dot);
-    dz.a[1][v] = aux * (dy.a[1][v] - y.a[1][v] * dot);
-  }
-  return dz;
-}
-
-__device__ __forceinline__ int64_t clamp_index(int64_t v, int64_t n) { return v < 0 ? 0 : (v >= n ? n - 1 : v); }
 
 // ---------------------------------------------------------------------------
 // prep
@@ -361,13 +205,6 @@ __device__ __forceinline__ float kappa(int cmp, const float* __restrict__ a, con
   }
   for (int d = lane; d < D; d += kWave) acc += a[d] * b[d];
   return wave_sum(acc);
-}
-
-__device__ __forceinline__ float softplusf(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
-__device__ __forceinline__ float sigmoidf(float z) {
-  if (z >= 0.f) return 1.0f / (1.0f + expf(-z));
-  const float e = expf(z);
-  return e / (1.0f + e);
 }
 
 struct ScoreRow {

@@ -1,0 +1,385 @@
+"""Embeddings, comparators and the multi-relation model (reference:
+torchbiggraph/model.py).
+
+``COMPARATORS`` holds ``dot``, ``cos`` and ``l2`` with the reference's
+``prepare`` / ``forward`` contract (differentiable, computed by
+pbg_comparator_*).  ``MultiRelationEmbedder`` keeps the reference's constructor,
+``set_embeddings`` / ``set_all_embeddings`` / ``clear_all_embeddings`` and
+``forward(edges) -> (Scores, reg)``; its forward is ONE call into libpbg_hip
+(pbg_model_forward) and additionally accepts the uniform-negative indices from
+outside, so that two implementations can be fed the same negatives.  Training
+goes through ``train.Trainer`` (one pbg_train_step call per batch), not through
+autograd on these scores.
+
+Not provided (outside the accelerated path): FeaturizedEmbedding, squared_l2,
+BiasedComparator, all_negs, global embeddings, max_norm, half precision,
+regularizers.
+"""
+from abc import ABC, abstractmethod
+from enum import Enum
+from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple, Union
+
+import torch
+import torch.nn as nn
+
+from . import _lib, native
+from ._lib import COMPARATOR_CODES, check
+from .config import EntitySchema, RelationSchema
+from .edgelist import EdgeList
+from .entitylist import EntityList
+from .native import _need, _ptr, _stream
+from .operators import AbstractDynamicOperator, AbstractOperator
+from .plugin import PluginRegistry
+from .types import Bucket, FloatTensorType, LongTensorType, Side
+from .util import match_shape
+
+
+class AbstractEmbedding(nn.Module, ABC):
+    @abstractmethod
+    def forward(self, input_: EntityList) -> FloatTensorType:
+        pass
+
+    @abstractmethod
+    def get_all_entities(self) -> FloatTensorType:
+        pass
+
+    @abstractmethod
+    def sample_entities(self, *dims: int) -> FloatTensorType:
+        pass
+
+
+class _GatherFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, weight, idx):
+        ctx.save_for_backward(idx)
+        ctx.shape = weight.shape
+        return native.gather_rows(weight.detach().contiguous(), idx.contiguous())
+
+    @staticmethod
+    def backward(ctx, grad):
+        (idx,) = ctx.saved_tensors
+        # a sparse COO gradient, as F.embedding(sparse=True) produces
+        flat = idx.reshape(1, -1)
+        sparse = torch.sparse_coo_tensor(flat, grad.reshape(-1, ctx.shape[1]), ctx.shape)
+        return sparse, None
+
+
+class SimpleEmbedding(AbstractEmbedding):
+    """Row gather from one table (model.py:51-75)."""
+
+    def __init__(self, weight: nn.Parameter, max_norm: Optional[float] = None):
+        super().__init__()
+        if max_norm is not None:
+            raise NotImplementedError("max_norm is not supported")
+        self.weight: nn.Parameter = weight
+        self.max_norm = None
+
+    def forward(self, input_: EntityList) -> FloatTensorType:
+        return self.get(input_.to_tensor())
+
+    def get(self, input_: LongTensorType) -> FloatTensorType:
+        if input_.numel() == 0:
+            return self.weight.new_empty((*input_.shape, self.weight.shape[1]))
+        return _GatherFunction.apply(self.weight, input_)
+
+    def get_all_entities(self) -> FloatTensorType:
+        return self.get(torch.arange(self.weight.size(0), dtype=torch.long, device=self.weight.device))
+
+    def sample_indices(self, *dims: int) -> LongTensorType:
+        return torch.randint(low=0, high=self.weight.size(0), size=dims, device=self.weight.device)
+
+    def sample_entities(self, *dims: int) -> FloatTensorType:
+        return self.get(self.sample_indices(*dims))
+
+
+# ---------------------------------------------------------------------------
+class _PrepareFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, code, embs):
+        x = embs.contiguous()
+        _need(x, torch.float32, "embs")
+        dim = x.shape[-1]
+        n = x.numel() // dim if dim else 0
+        y = torch.empty_like(x)
+        aux = torch.empty(max(n, 1), dtype=torch.float32, device=x.device)
+        check(_lib.lib().pbg_comparator_prepare(code, dim, n, _ptr(x), _ptr(y), _ptr(aux), _stream()))
+        ctx.code, ctx.dim, ctx.n = code, dim, n
+        ctx.save_for_backward(y, aux)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        y, aux = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = torch.empty_like(y)
+        check(_lib.lib().pbg_comparator_prepare_backward(ctx.code, ctx.dim, ctx.n, _ptr(dy), _ptr(y), _ptr(aux),
+                                                         _ptr(dx), _stream()))
+        return None, dx
+
+
+class _ScoresFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, code, lhs_pos, rhs_pos, lhs_neg, rhs_neg):
+        ts = [t.contiguous() for t in (lhs_pos, rhs_pos, lhs_neg, rhs_neg)]
+        for t, name in zip(ts, ("lhs_pos", "rhs_pos", "lhs_neg", "rhs_neg")):
+            _need(t, torch.float32, name)
+        c, p, d = ts[0].shape
+        ln, rn = ts[2].shape[1], ts[3].shape[1]
+        dev = ts[0].device
+        pos = torch.empty((c, p), dtype=torch.float32, device=dev)
+        lneg = torch.empty((c, p, ln), dtype=torch.float32, device=dev)
+        rneg = torch.empty((c, p, rn), dtype=torch.float32, device=dev)
+        nbytes = _lib.lib().pbg_comparator_workspace_bytes(c, p, ln, rn)
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        check(_lib.lib().pbg_comparator_forward(code, c, p, ln, rn, d, *[_ptr(t) for t in ts], _ptr(pos), _ptr(lneg),
+                                                _ptr(rneg), _ptr(ws), ws.numel(), _stream()))
+        ctx.code, ctx.dims = code, (c, p, ln, rn, d)
+        ctx.save_for_backward(*ts, pos, lneg, rneg)
+        return pos, lneg, rneg
+
+    @staticmethod
+    def backward(ctx, dpos, dlneg, drneg):
+        lp, rp, ln_, rn_, pos, lneg, rneg = ctx.saved_tensors
+        c, p, ln, rn, d = ctx.dims
+        dev = lp.device
+        grads = [g.contiguous() if g is not None else torch.zeros_like(ref)
+                 for g, ref in ((dpos, pos), (dlneg, lneg), (drneg, rneg))]
+        outs = [torch.empty_like(t) for t in (lp, rp, ln_, rn_)]
+        nbytes = _lib.lib().pbg_comparator_workspace_bytes(c, p, ln, rn)
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        check(_lib.lib().pbg_comparator_backward(
+            ctx.code, c, p, ln, rn, d, _ptr(lp), _ptr(rp), _ptr(ln_), _ptr(rn_), _ptr(pos), _ptr(lneg), _ptr(rneg),
+            *[_ptr(g) for g in grads], *[_ptr(o) for o in outs], _ptr(ws), ws.numel(), _stream()))
+        return (None, *outs)
+
+
+class AbstractComparator(nn.Module, ABC):
+    """Scores between sets of vectors chunked alike:
+    L+ [C,P,D], R+ [C,P,D], L- [C,L,D], R- [C,R,D] ->
+    <L+,R+> [C,P], R+ x L- [C,P,L], L+ x R- [C,P,R]   (model.py:105-153)."""
+
+    comparator_name: str = ""
+
+    @property
+    def comparator_code(self) -> int:
+        return COMPARATOR_CODES[self.comparator_name]
+
+    def prepare(self, embs: FloatTensorType) -> FloatTensorType:
+        return embs
+
+    def forward(self, lhs_pos, rhs_pos, lhs_neg, rhs_neg) -> Tuple[FloatTensorType, FloatTensorType, FloatTensorType]:
+        num_chunks, num_pos_per_chunk, dim = match_shape(lhs_pos, -1, -1, -1)
+        match_shape(rhs_pos, num_chunks, num_pos_per_chunk, dim)
+        match_shape(lhs_neg, num_chunks, -1, dim)
+        match_shape(rhs_neg, num_chunks, -1, dim)
+        return _ScoresFunction.apply(self.comparator_code, lhs_pos, rhs_pos, lhs_neg, rhs_neg)
+
+
+COMPARATORS = PluginRegistry[AbstractComparator]()
+
+
+@COMPARATORS.register_as("dot")
+class DotComparator(AbstractComparator):
+    comparator_name = "dot"
+
+
+@COMPARATORS.register_as("cos")
+class CosComparator(AbstractComparator):
+    comparator_name = "cos"
+
+    def prepare(self, embs: FloatTensorType) -> FloatTensorType:
+        return _PrepareFunction.apply(self.comparator_code, embs)
+
+
+@COMPARATORS.register_as("l2")
+class L2Comparator(AbstractComparator):
+    comparator_name = "l2"
+
+
+# ---------------------------------------------------------------------------
+def ceil_of_ratio(num: int, den: int) -> int:
+    return (num - 1) // den + 1
+
+
+class Negatives(Enum):
+    NONE = "none"
+    UNIFORM = "uniform"
+    BATCH_UNIFORM = "batch_uniform"
+    ALL = "all"
+
+
+class Scores(NamedTuple):
+    lhs_pos: FloatTensorType
+    rhs_pos: FloatTensorType
+    lhs_neg: FloatTensorType
+    rhs_neg: FloatTensorType
+
+
+class MultiRelationEmbedder(nn.Module):
+    """A multi-relation embedding model scored against batch and uniform
+    negatives (model.py:368-856)."""
+
+    EMB_PREFIX = "emb_"
+
+    def __init__(
+        self,
+        default_dim: int,
+        relations: List[RelationSchema],
+        entities: Dict[str, EntitySchema],
+        num_batch_negs: int,
+        num_uniform_negs: int,
+        disable_lhs_negs: bool,
+        disable_rhs_negs: bool,
+        lhs_operators: Sequence[Optional[Union[AbstractOperator, AbstractDynamicOperator]]],
+        rhs_operators: Sequence[Optional[Union[AbstractOperator, AbstractDynamicOperator]]],
+        comparator: AbstractComparator,
+        regularizer=None,
+        global_emb: bool = False,
+        max_norm: Optional[float] = None,
+        num_dynamic_rels: int = 0,
+        half_precision: bool = False,
+    ) -> None:
+        super().__init__()
+        if regularizer is not None:
+            raise NotImplementedError("Regularizers are not supported")
+        if global_emb:
+            raise NotImplementedError("Global embeddings are not supported")
+        if max_norm is not None:
+            raise NotImplementedError("max_norm is not supported")
+        if half_precision:
+            raise NotImplementedError("Half precision is not supported")
+        if any(e.featurized for e in entities.values()):
+            raise NotImplementedError("Featurized entities are not supported")
+        if any(r.all_negs for r in relations):
+            raise NotImplementedError("all_negs is not supported")
+        self.default_dim = default_dim
+        self.relations: List[RelationSchema] = relations
+        self.entities: Dict[str, EntitySchema] = entities
+        self.num_dynamic_rels: int = num_dynamic_rels
+        if num_dynamic_rels > 0:
+            assert len(relations) == 1
+        self.lhs_operators: nn.ModuleList = nn.ModuleList(lhs_operators)
+        self.rhs_operators: nn.ModuleList = nn.ModuleList(rhs_operators)
+        self.num_batch_negs: int = num_batch_negs
+        self.num_uniform_negs: int = num_uniform_negs
+        self.disable_lhs_negs = disable_lhs_negs
+        self.disable_rhs_negs = disable_rhs_negs
+        self.comparator = comparator
+        self.lhs_embs: nn.ModuleDict = nn.ModuleDict()
+        self.rhs_embs: nn.ModuleDict = nn.ModuleDict()
+        self.global_embs = None
+        self.max_norm = None
+        self.half_precision = False
+        self.regularizer = None
+        self._runners: Dict[tuple, native.StepRunner] = {}
+
+    # --- embeddings ---------------------------------------------------------
+    def set_embeddings(self, entity: str, side: Side, weights: nn.Parameter) -> None:
+        emb = SimpleEmbedding(weights)
+        side.pick(self.lhs_embs, self.rhs_embs)[self.EMB_PREFIX + entity] = emb
+        self._runners.clear()
+
+    def set_all_embeddings(self, holder, bucket: Bucket) -> None:
+        for entity in holder.lhs_unpartitioned_types:
+            self.set_embeddings(entity, Side.LHS, holder.unpartitioned_embeddings[entity])
+        for entity in holder.rhs_unpartitioned_types:
+            self.set_embeddings(entity, Side.RHS, holder.unpartitioned_embeddings[entity])
+        for entity in holder.lhs_partitioned_types:
+            self.set_embeddings(entity, Side.LHS, holder.partitioned_embeddings[entity, bucket.lhs])
+        for entity in holder.rhs_partitioned_types:
+            self.set_embeddings(entity, Side.RHS, holder.partitioned_embeddings[entity, bucket.rhs])
+
+    def clear_all_embeddings(self) -> None:
+        self.lhs_embs.clear()
+        self.rhs_embs.clear()
+        self._runners.clear()
+
+    # --- the fused path -------------------------------------------------------
+    def resolve(self, edges: EdgeList):
+        """Validates the batch as model.py:633-646,674-678 does and returns
+        (relation_idx, lhs table module, rhs table module)."""
+        if self.num_dynamic_rels > 0:
+            if edges.has_scalar_relation_type():
+                raise TypeError("Need relation for each positive pair")
+            relation_idx = 0
+        else:
+            if not edges.has_scalar_relation_type():
+                raise TypeError("All positive pairs must come from the same relation")
+            relation_idx = edges.get_relation_type_as_scalar()
+            if self.lhs_operators[relation_idx] is not None:
+                raise RuntimeError(
+                    "In non-dynamic relation mode there should be only a right-hand side operator"
+                )
+        relation = self.relations[relation_idx]
+        lhs_module = self.lhs_embs[self.EMB_PREFIX + relation.lhs]
+        rhs_module = self.rhs_embs[self.EMB_PREFIX + relation.rhs]
+        return relation_idx, lhs_module, rhs_module
+
+    def step_spec(self, relation_idx: int, num_pos: int, dim: int, **training) -> native.StepSpec:
+        rhs_op = self.rhs_operators[relation_idx]
+        dynamic = self.num_dynamic_rels > 0
+        return native.StepSpec(
+            dim=dim, batch_size=num_pos, num_workers=1, num_batch_negs=self.num_batch_negs,
+            num_uniform_negs=self.num_uniform_negs, disable_lhs_negs=bool(self.disable_lhs_negs),
+            disable_rhs_negs=bool(self.disable_rhs_negs),
+            operator=rhs_op.op_name if rhs_op is not None else "none", dynamic=dynamic,
+            num_relations=self.num_dynamic_rels if dynamic else 1,
+            comparator=self.comparator.comparator_name, **training)
+
+    def operator_tensors(self, relation_idx: int):
+        """({name: tensor} of the rhs operator, of the lhs operator) in the
+        layout pbg_step_buffers expects."""
+        def pack(op):
+            if op is None:
+                return {}
+            p0, p1 = op.fused_params()
+            if p0 is None:
+                return {}
+            return {"real": p0.data, "imag": p1.data} if p1 is not None else {"p0": p0.data}
+        lhs = pack(self.lhs_operators[relation_idx]) if self.num_dynamic_rels > 0 else {}
+        return pack(self.rhs_operators[relation_idx]), lhs
+
+    def sample_uniform(self, lhs_module, rhs_module, num_chunks: int):
+        """torch.randint(0, E, (C, U)) per side, left-hand side first, as
+        SimpleEmbedding.sample_entities draws them (model.py:70-75,802-821)."""
+        u = self.num_uniform_negs
+        ul = lhs_module.sample_indices(num_chunks, u) if (u > 0 and not self.disable_lhs_negs) else None
+        ur = rhs_module.sample_indices(num_chunks, u) if (u > 0 and not self.disable_rhs_negs) else None
+        return ul, ur
+
+    def forward(self, edges: EdgeList, uniform_negs=None) -> Tuple[Scores, None]:
+        """Scores of a batch (model.py:624-762).  `uniform_negs` = (lhs [C,U],
+        rhs [C,U]) entity indices; drawn with torch.randint when omitted."""
+        num_pos = len(edges)
+        relation_idx, lhs_module, rhs_module = self.resolve(edges)
+        if self.num_batch_negs == 0 and self.num_uniform_negs == 0:
+            raise ValueError("num_batch_negs and num_uniform_negs cannot both be 0")
+        w_l, w_r = lhs_module.weight, rhs_module.weight
+        dim = w_l.shape[1]
+        dev = w_l.device
+        nl = 0 if self.disable_lhs_negs else None
+        if num_pos == 0:
+            spec = self.step_spec(relation_idx, 1, dim)
+            z = torch.empty((0,), dtype=torch.float32, device=dev)
+            return Scores(z, z.clone(), z.new_empty((0, spec.num_negs(self.disable_lhs_negs))),
+                          z.new_empty((0, spec.num_negs(self.disable_rhs_negs)))), None
+        spec = self.step_spec(relation_idx, num_pos, dim)
+        key = ("fwd", relation_idx, num_pos, w_l.data_ptr(), w_r.data_ptr())
+        runner = self._runners.get(key)
+        if runner is None:
+            rhs_op, lhs_op = self.operator_tensors(relation_idx)
+            runner = native.StepRunner(spec, w_l.data, torch.empty(0, device=dev), w_r.data, torch.empty(0, device=dev),
+                                       rhs_op, None, lhs_op, None)
+            self._runners[key] = runner
+        if uniform_negs is None:
+            uniform_negs = self.sample_uniform(lhs_module, rhs_module, spec.num_chunks)
+        ul, ur = uniform_negs
+        lhs = edges.lhs.to_tensor().to(dev).contiguous()
+        rhs = edges.rhs.to_tensor().to(dev).contiguous()
+        if self.num_dynamic_rels > 0:
+            rel = edges.get_relation_type_as_vector().to(dev).contiguous()
+        else:
+            rel = torch.zeros(1, dtype=torch.int64, device=dev)  # the runner holds this relation's operator only
+        lp, rp, ln, rn = runner.forward(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
+                                        ur.contiguous() if ur is not None else None)
+        return Scores(lp[0], rp[0], ln[0], rn[0]), None
