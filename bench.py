@@ -141,10 +141,21 @@ def main():
     ap.add_argument("--workers", type=int, default=40, help="batches in flight per call (HOGWILD workers)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="length of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-sequential", action="store_true", help="skip the workers=1 measurement")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU (one process, no collectives); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "5 device copies", "bytes_read_each": src.numel() * 4, "bytes_written_each": src.numel() * 4}))
+        return
 
     w = WORKLOADS[args.workload]
     # The CPU baseline runs first, before this process opens the GPU: its worker
