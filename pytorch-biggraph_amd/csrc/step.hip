@@ -655,6 +655,205 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------
+// operator parameters, dynamic relations (one relation per edge)
+// ---------------------------------------------------------------------------
+// `linear` with a relation per row: z_e = W[rel_e] x_e, one wave per positive
+// (operators.py:259-269).  Reads the raw rows staged by prep.
+__global__ __launch_bounds__(kRowThreads) void dyn_linear_forward_kernel(StepCtx c, int s) {
+  const SideCtx& sd = c.side[s];
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.B) return;
+  const int D = c.D;
+  const float* m = sd.p0 + clamp_index(c.rel[job], c.num_relations) * D * D;
+  const float* x = sd.xraw + job * D;
+  float* z = sd.z + job * D;
+  for (int o = 0; o < D; ++o) {
+    float acc = 0.f;
+    for (int d = lane; d < D; d += kWave) acc += m[(int64_t)o * D + d] * x[d];
+    acc = wave_sum(acc);
+    if (lane == 0) z[o] = acc;
+  }
+}
+
+// gr[row of e] += W[rel_e]^T dz_e
+__global__ __launch_bounds__(kRowThreads) void dyn_linear_backward_kernel(StepCtx c, int s) {
+  const SideCtx& sd = c.side[s];
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.B) return;
+  const int D = c.D;
+  const int k = (int)(job / c.B), q = (int)(job % c.B);
+  const float* m = sd.p0 + clamp_index(c.rel[job], c.num_relations) * D * D;
+  const float* g = sd.dz + job * D;
+  float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
+  for (int d = lane; d < D; d += kWave) {
+    float acc = 0.f;
+    for (int o = 0; o < D; ++o) acc += m[(int64_t)o * D + d] * g[o];
+    out[d] += acc;
+  }
+}
+
+// sort keys (relation << kbits | batch) of every positive, value = k * B + q
+__global__ void rel_keys_kernel(StepCtx c, uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)c.K * c.B) return;
+  const int64_t r = clamp_index(c.rel[e], c.num_relations);
+  keys[e] = ((uint64_t)r << c.kbits) | (uint64_t)(e / c.B);
+  vals[e] = (uint32_t)e;
+}
+
+// First position after `start` whose key >> shift differs from `want` (block-wide, 256 threads).
+__device__ __forceinline__ int64_t block_scan_end(const uint64_t* __restrict__ keys, int64_t start, int64_t n,
+                                                  uint64_t want, int shift, int64_t* sh_end) {
+  int64_t base = start + 1;
+  while (true) {
+    if (threadIdx.x == 0) *sh_end = -1;
+    __syncthreads();
+    const int64_t j = base + threadIdx.x;
+    const bool same = (j < n) && ((keys[j] >> shift) == want);
+    const bool prev_same = (j == base) || ((j - 1 < n) && ((keys[j - 1] >> shift) == want));
+    if (!same && prev_same && j <= n) *sh_end = j;  // exactly one thread sees the first mismatch
+    __syncthreads();
+    const int64_t found = *sh_end;
+    __syncthreads();
+    if (found >= 0) return found;
+    base += blockDim.x;
+  }
+}
+
+// Element-wise operators: one workgroup per (relation present in the call, 64-element slice).
+// It walks the relation's runs (one per batch, ascending), sums each run's parameter
+// gradient over the run's edges in a fixed order and applies AsyncAdagrad
+// (async_adagrad.py:75-85) before the next run: the K batches' updates in order.
+__global__ __launch_bounds__(256) void dyn_param_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
+                                                        const uint32_t* __restrict__ vals, float* p0, float* p1,
+                                                        float* s0, float* s1, float lr) {
+  __shared__ float sh[4][64];
+  __shared__ int64_t sh_end;
+  const SideCtx& sd = c.side[s];
+  const int64_t n = (int64_t)c.K * c.B;
+  const int64_t i = blockIdx.x;
+  const uint64_t rel = keys[i] >> c.kbits;
+  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;
+  const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int e = blockIdx.y * 64 + lane;
+  const int D = c.D, H = D / 2;
+  float* p;
+  float* st;
+  if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+    p = (e < H) ? p0 + rel * H + e : p1 + rel * H + (e - H);
+    st = (e < H) ? s0 + rel * H + e : s1 + rel * H + (e - H);
+  } else {
+    p = p0 + rel * D + e;
+    st = s0 + rel * D + e;
+  }
+  int64_t j = i;
+  while (j < n && (keys[j] >> c.kbits) == rel) {
+    const int64_t end = block_scan_end(keys, j, n, keys[j], 0, &sh_end);
+    float acc = 0.f;
+    if (e < D) {
+      for (int64_t r = j + rg; r < end; r += 4) {
+        const int64_t edge = vals[r];
+        const float* dz = sd.dz + edge * D;
+        if (c.op == PBG_OP_TRANSLATION) {
+          acc += dz[e];
+          continue;
+        }
+        const float* x = sd.w + clamp_index(sd.idx[edge], sd.num_rows) * D;
+        if (c.op == PBG_OP_DIAGONAL) {
+          acc += x[e] * dz[e];
+        } else if (e < H) {
+          acc += x[e] * dz[e] + x[e + H] * dz[e + H];
+        } else {
+          const int h = e - H;
+          acc += x[h] * dz[h + H] - x[h + H] * dz[h];
+        }
+      }
+    }
+    sh[rg][lane] = acc;
+    __syncthreads();
+    if (rg == 0 && e < D) {
+      const float g = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+      const float sum = *st + g * g;
+      *st = sum;
+      *p += -lr * (g / (sqrtf(sum) + 1e-10f));
+    }
+    __syncthreads();
+    j = end;
+  }
+}
+
+// `linear`: one workgroup per (relation present, 64 x 64 tile of its matrix); thread
+// (ty, tx) owns a 4 x 4 block of dW[o, i] = sum over the run's edges of dz[o] x[i].
+__global__ __launch_bounds__(256) void dyn_linear_param_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
+                                                               const uint32_t* __restrict__ vals, float* w,
+                                                               float* wsum, float lr) {
+  constexpr int kRows = 16;
+  __shared__ float sh_dz[kRows][64];
+  __shared__ float sh_x[kRows][64];
+  __shared__ int64_t sh_end;
+  const SideCtx& sd = c.side[s];
+  const int64_t n = (int64_t)c.K * c.B;
+  const int64_t i = blockIdx.x;
+  const uint64_t rel = keys[i] >> c.kbits;
+  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;
+  const int D = c.D;
+  const int tiles = (D + 63) / 64;
+  const int o0 = (blockIdx.y / tiles) * 64, i0 = (blockIdx.y % tiles) * 64;
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+  float* wr = w + (int64_t)rel * D * D;
+  float* sr = wsum + (int64_t)rel * D * D;
+  int64_t j = i;
+  while (j < n && (keys[j] >> c.kbits) == rel) {
+    const int64_t end = block_scan_end(keys, j, n, keys[j], 0, &sh_end);
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+    for (int64_t r0 = j; r0 < end; r0 += kRows) {
+      // stage up to kRows edges: 64 values of dz (rows of the tile) and of x (columns of the tile) each
+      for (int t = threadIdx.x; t < kRows * 64; t += 256) {
+        const int rr = t >> 6, col = t & 63;
+        float vdz = 0.f, vx = 0.f;
+        if (r0 + rr < end) {
+          const int64_t edge = vals[r0 + rr];
+          if (o0 + col < D) vdz = sd.dz[edge * D + o0 + col];
+          if (i0 + col < D) vx = sd.xraw[edge * D + i0 + col];
+        }
+        sh_dz[rr][col] = vdz;
+        sh_x[rr][col] = vx;
+      }
+      __syncthreads();
+#pragma unroll 4
+      for (int rr = 0; rr < kRows; ++rr) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) acc[a][b] += sh_dz[rr][ty * 4 + a] * sh_x[rr][tx * 4 + b];
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int o = o0 + ty * 4 + a, ii = i0 + tx * 4 + b;
+        if (o < D && ii < D) {
+          const int64_t at = (int64_t)o * D + ii;
+          const float g = acc[a][b];
+          const float sum = sr[at] + g * g;
+          sr[at] = sum;
+          wr[at] += -lr * (g / (sqrtf(sum) + 1e-10f));
+        }
+      }
+    }
+    j = end;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 struct Plan {
@@ -667,6 +866,10 @@ struct Plan {
   void* sort_temp;
   int64_t psize;  // floats of parameter gradient per batch
   int pslices[2]; // partial sums per batch of the element-wise parameter gradients
+  // dynamic relations: (relation, batch) keys of the positives and their sort buffers
+  uint64_t *rkeys_a, *rkeys_b;
+  uint32_t *rvals_a, *rvals_b;
+  void* rsort_temp;
   int nvh;
 };
 
@@ -686,10 +889,6 @@ int validate(const pbg_step_desc* d, bool training) {
                 "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");  // operators.py:132-136
   if (d->num_relations < 1) return fail(PBG_ERR_INVALID, "step: num_relations must be positive");
   if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
-  if (d->dynamic && d->op == PBG_OP_LINEAR)
-    return fail(PBG_ERR_UNSUPPORTED, "step: the linear operator with dynamic relations is not implemented");
-  if (training && d->dynamic && d->op != PBG_OP_NONE)
-    return fail(PBG_ERR_UNSUPPORTED, "step: training operator parameters with dynamic relations is not implemented");
   return PBG_OK;
 }
 
@@ -804,9 +1003,17 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->psize = 0;
   if (c.op == PBG_OP_LINEAR) plan->psize = (int64_t)D * D;
   else if (c.op != PBG_OP_NONE) plan->psize = D;
+  if (c.dynamic && plan->psize > 0) {
+    const int64_t ne = (int64_t)K * c.B;
+    plan->rkeys_a = (uint64_t*)take(ne, 8);
+    plan->rkeys_b = (uint64_t*)take(ne, 8);
+    plan->rvals_a = (uint32_t*)take(ne, 4);
+    plan->rvals_b = (uint32_t*)take(ne, 4);
+    plan->rsort_temp = take(sort_temp_bytes(ne), 1);
+  }
   for (int s = 0; s < 2; ++s) {
     plan->pslices[s] = 1;
-    if (!c.side[s].has_op || plan->psize == 0) continue;
+    if (!c.side[s].has_op || plan->psize == 0 || c.dynamic) continue;
     if (c.op != PBG_OP_LINEAR) {
       int sl = (int)ceil_div(c.side[s].op_rows, 32 * kParamGroups);
       plan->pslices[s] = sl < 1 ? 1 : (sl > 16 ? 16 : sl);
@@ -900,6 +1107,13 @@ int run_operator_forward(const Plan& plan, hipStream_t stream) {
   const StepCtx& c = plan.c;
   const int D = c.D, K = c.K;
   int rc;
+  if (c.op == PBG_OP_LINEAR && c.dynamic) {
+    for (int s = 0; s < 2; ++s) {
+      hipLaunchKernelGGL(dyn_linear_forward_kernel, wave_grid((int64_t)K * c.B), dim3(kRowThreads), 0, stream, c, s);
+      PBG_DISPATCH_NVH(plan.nvh, prepare_staged_kernel, wave_grid((int64_t)K * c.B), stream, c, s);
+    }
+    return check_launch("step operator");
+  }
   if (c.op == PBG_OP_LINEAR) {
     for (int s = 0; s < 2; ++s) {
       const SideCtx& sd = c.side[s];
@@ -991,6 +1205,30 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
   if (c.op == PBG_OP_NONE) return PBG_OK;
   const int D = c.D, K = c.K;
   int rc;
+  if (c.dynamic) {
+    const int64_t ne = (int64_t)K * c.B;
+    hipLaunchKernelGGL(rel_keys_kernel, dim3((unsigned)ceil_div(ne, 256)), dim3(256), 0, stream, c, plan.rkeys_a,
+                       plan.rvals_a);
+    rc = sort_pairs(plan.rkeys_a, plan.rvals_a, plan.rkeys_b, plan.rvals_b, ne,
+                    bits_for((uint64_t)(c.num_relations - 1)) + c.kbits, plan.rsort_temp, stream);
+    if (rc != PBG_OK) return rc;
+    for (int s = 0; s < 2; ++s) {
+      float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
+      float* p1 = s == 0 ? b->lhs_op_p1 : b->rhs_op_p1;
+      float* s0 = s == 0 ? b->lhs_op_s0 : b->rhs_op_s0;
+      float* s1 = s == 0 ? b->lhs_op_s1 : b->rhs_op_s1;
+      if (c.op == PBG_OP_LINEAR) {
+        hipLaunchKernelGGL(dyn_linear_backward_kernel, wave_grid(ne), dim3(kRowThreads), 0, stream, c, s);
+        const int tiles = (D + 63) / 64;
+        hipLaunchKernelGGL(dyn_linear_param_kernel, dim3((unsigned)ne, (unsigned)(tiles * tiles)), dim3(256), 0, stream,
+                           c, s, plan.rkeys_b, plan.rvals_b, p0, s0, d->relation_lr);
+      } else {
+        hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
+                           plan.rkeys_b, plan.rvals_b, p0, p1, s0, s1, d->relation_lr);
+      }
+    }
+    return check_launch("step params (dynamic)");
+  }
   for (int s = 0; s < 2; ++s) {
     const SideCtx& sd = c.side[s];
     if (!sd.has_op) continue;

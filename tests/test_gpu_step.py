@@ -100,8 +100,6 @@ def compare_scores(cfg, got, want_scores):
 
 FORWARD_CASES = []
 for op, cmp_, dyn in itertools.product(ostep.OPERATOR_NAMES, ostep.COMPARATOR_NAMES, (False, True)):
-    if dyn and op == "linear":
-        continue
     FORWARD_CASES.append(dict(operator=op, comparator=cmp_, dynamic=dyn, num_batch_negs=4, num_uniform_negs=3,
                               num_pos=10, dim=6))
 FORWARD_CASES += [
@@ -149,8 +147,8 @@ for op, cmp_, loss in itertools.product(("none", "diagonal", "translation", "com
                                         ostep.COMPARATOR_NAMES, ostep.LOSS_NAMES):
     TRAIN_CASES.append(dict(operator=op, comparator=cmp_, loss=loss, dynamic=False, num_batch_negs=4,
                             num_uniform_negs=3, num_pos=10, dim=6))
-for cmp_, loss in itertools.product(ostep.COMPARATOR_NAMES, ostep.LOSS_NAMES):
-    TRAIN_CASES.append(dict(operator="none", comparator=cmp_, loss=loss, dynamic=True, num_batch_negs=4,
+for op, cmp_, loss in itertools.product(ostep.OPERATOR_NAMES, ostep.COMPARATOR_NAMES, ostep.LOSS_NAMES):
+    TRAIN_CASES.append(dict(operator=op, comparator=cmp_, loss=loss, dynamic=True, num_batch_negs=4,
                             num_uniform_negs=3, num_pos=10, dim=6))
 TRAIN_CASES += [
     dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50,
@@ -175,6 +173,14 @@ TRAIN_CASES += [
          num_pos=9, dim=8, disable_rhs_negs=True),
     dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=16, num_uniform_negs=2,
          num_pos=5, dim=7),
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=50,
+         num_uniform_negs=100, num_pos=200, dim=400),
+    dict(operator="linear", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=100,
+         num_uniform_negs=100, num_pos=300, dim=130),
+    dict(operator="translation", comparator="l2", loss="ranking", dynamic=True, num_batch_negs=50,
+         num_uniform_negs=50, num_pos=173, dim=100),
+    dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=0,
+         num_uniform_negs=9, num_pos=40, dim=9, disable_lhs_negs=True),
 ]
 
 
