@@ -43,10 +43,18 @@ WORKLOADS = {
                  entities=10_413_058, edges=4_000_000, dim=100, batch=1000, batch_negs=50, uniform_negs=50,
                  operator="translation", comparator="l2", loss="ranking", relations=1, dynamic=False,
                  init_scale=1e-3, zipf=1.8, two_tables=True),
-    "cfg5": dict(desc="500 relations, linear/cos/logistic, dim 256, 2M entities, B=2000, 100 batch + 100 uniform negatives, single-relation batches",
+    "cfg5": dict(desc="500 relations (dynamic: one per edge), linear/cos/logistic, dim 256, 2M entities, B=2000, 100 batch + 100 uniform negatives, mixed batches sorted by relation",
                  entities=2_000_000, edges=4_000_000, dim=256, batch=2000, batch_negs=100, uniform_negs=100,
-                 operator="linear", comparator="cos", loss="logistic", relations=500, dynamic=False,
+                 operator="linear", comparator="cos", loss="logistic", relations=500, dynamic=True,
                  init_scale=1e-3, zipf=None, rel_zipf=1.2, two_tables=False),
+    "cfg5s": dict(desc="500 relations, linear/cos/logistic, dim 256, 2M entities, B=2000, 100 batch + 100 uniform negatives, single-relation batches",
+                  entities=2_000_000, edges=4_000_000, dim=256, batch=2000, batch_negs=100, uniform_negs=100,
+                  operator="linear", comparator="cos", loss="logistic", relations=500, dynamic=False,
+                  init_scale=1e-3, zipf=None, rel_zipf=1.2, two_tables=False),
+    "cfg2d": dict(desc="1345 relations (dynamic: one per edge), complex_diagonal/dot/softmax, dim 400, 14951 entities, B=1000, chunk 50 + 1000 uniform negatives",
+                  entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=1000,
+                  operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=True,
+                  init_scale=1e-3, zipf=1.1, two_tables=False),
 }
 
 
@@ -98,6 +106,9 @@ def cpu_baseline(w, seconds):
     else:
         pool = torch.zeros(4096, dtype=torch.int64)
     rel = pool[torch.arange(n) // b % 4096]
+    if w["dynamic"]:
+        s_rel = w.get("rel_zipf") or w["zipf"]
+        rel = power_law_ids(n, w["relations"], s_rel, gen, "cpu") if s_rel else torch.randint(0, w["relations"], (n,), generator=gen)
     cfg = ostep.StepConfig(dim=d, operator=w["operator"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
                            num_batch_negs=w["batch_negs"], num_uniform_negs=w["uniform_negs"], dynamic=w["dynamic"],
                            num_relations=w["relations"], lr=0.1, relation_weights=[1.0] * w["relations"])
@@ -189,8 +200,10 @@ def main():
         elif w["operator"] == "linear":
             rhs_op = {"linear_transformation": torch.eye(d, device=dev).repeat(r, 1, 1).contiguous()}
         rhs_sum = {k: torch.zeros_like(v) for k, v in rhs_op.items()}
+        lhs_op = {k: v.clone() for k, v in rhs_op.items()} if w["dynamic"] else {}
+        lhs_sum = {k: torch.zeros_like(v) for k, v in lhs_op.items()}
         runner = pkg.StepRunner(spec, ws[0], gs[0], ws[1] if len(ws) > 1 else None, gs[1] if len(gs) > 1 else None,
-                                rhs_op, rhs_sum)
+                                rhs_op, rhs_sum, lhs_op, lhs_sum)
         return spec, runner
 
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -204,6 +217,14 @@ def main():
             rel_pool = torch.randint(0, w["relations"], (4096,), generator=gen, device=dev)
     else:
         rel_pool = torch.zeros(4096, dtype=torch.int64, device=dev)
+    rel_edges = None
+    if w["dynamic"]:
+        # one relation per edge, sorted inside every batch-sized slice ("mixed batches sorted by relation")
+        s_rel = w.get("rel_zipf") or w["zipf"]
+        rel_edges = power_law_ids(n_edges, w["relations"], s_rel, gen, dev) if s_rel else \
+            torch.randint(0, w["relations"], (n_edges,), generator=gen, device=dev)
+        full = n_edges // b * b
+        rel_edges[:full] = rel_edges[:full].view(-1, b).sort(dim=1).values.reshape(-1)
 
     def run(workers, batches, warm, profile_calls=0):
         spec, runner = make_runner(workers)
@@ -214,10 +235,13 @@ def main():
         n_r = tables[-1].shape[0]
 
         def one_call(i, profiled=False):
-            off = (i * per_call) % (n_edges - per_call + 1)
+            off = (i * per_call) % (n_edges - per_call + 1) // b * b
             lhs = lhs_all[off:off + per_call]
             rhs = rhs_all[off:off + per_call]
-            rel = rel_pool[(i * workers) % (4096 - workers + 1):][:workers]
+            if rel_edges is not None:
+                rel = rel_edges[off:off + per_call]
+            else:
+                rel = rel_pool[(i * workers) % (4096 - workers + 1):][:workers]
             # the uniform negatives of model.py:70-75, drawn on the device inside the timed loop
             ul = torch.randint(0, e, (workers, c, u), generator=gen, device=dev)
             ur = torch.randint(0, n_r, (workers, c, u), generator=gen, device=dev)
@@ -244,7 +268,7 @@ def main():
         loss = float(runner.loss_out.mean().item()) / b
         return spec, calls * per_call / dt, dt / (calls * workers) * 1e3, calls * workers, stages, loss
 
-    default_steps = {"cfg1": 8000, "cfg2": 400, "cfg3": 40, "cfg4": 8000, "cfg5": 800}[args.workload]
+    default_steps = {"cfg1": 8000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 8000, "cfg5": 400, "cfg5s": 800}[args.workload]
     steps = args.steps if args.steps is not None else default_steps
     warmup = args.warmup if args.warmup is not None else max(args.workers, steps // 10)
     workers = max(1, min(args.workers, steps))

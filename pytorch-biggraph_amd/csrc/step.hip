@@ -19,6 +19,7 @@
 // Layout of a row inside a wave: lane l owns elements {h, H + h} for
 // h = l, l + 64, ... < H with H = ceil(D / 2), i.e. both halves of a complex
 // pair sit in the same lane.
+#include <cstdlib>
 #include <cstring>
 
 #include "pbg_internal.h"
@@ -262,6 +263,72 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   return sr;
 }
 
+// Loss of one positive against one side's nn negatives (one wave): adds the
+// unweighted per-lane loss partial to *loss_acc, overwrites the score row with
+// dLoss/dscore (l2: -2 dLoss/d squared distance) and returns the wave-reduced
+// dLoss/dpos, violator count and (l2) row sum of dLoss/d squared distance.
+__device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
+                                          float pos, float w, int lane, float* loss_acc, float* dpos_out,
+                                          int* viol_out, float* rowsum_out) {
+  float dpos_part = 0.f, rowsum = 0.f;
+  int viol = 0;
+  float mx = pos, inv_z = 0.f;
+  const float inv_nn = 1.0f / (float)nn;
+  if (loss == PBG_LOSS_SOFTMAX) {
+    bool live;
+    for (int j = lane; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
+    mx = wave_max(mx);
+    float z = 0.f;
+    for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
+    z = wave_sum(z) + expf(pos - mx);
+    inv_z = 1.0f / z;
+    if (lane == 0) {
+      *loss_acc += (mx + logf(z)) - pos;
+      dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+    }
+  } else if (loss == PBG_LOSS_LOGISTIC) {
+    if (lane == 0) {
+      *loss_acc += softplusf(-pos);
+      dpos_part += (sigmoidf(pos) - 1.0f) * w;
+    }
+  }
+  for (int j = lane; j < nn; j += kWave) {
+    bool live;
+    const float t = sr.at(j, &live);
+    float g;
+    if (loss == PBG_LOSS_RANKING) {
+      // F.margin_ranking_loss(neg, pos, target=-1): max(0, (t - pos) + margin); the
+      // clamp lets the gradient through at exactly 0
+      const float x = (t - pos) + margin;
+      if (x > 0.f) *loss_acc += x;
+      g = (x >= 0.f) ? w : 0.f;
+      dpos_part -= g;
+    } else if (loss == PBG_LOSS_LOGISTIC) {
+      *loss_acc += softplusf(t) * inv_nn;
+      g = sigmoidf(t) * inv_nn * w;
+    } else {
+      g = expf(t - mx) * inv_z * w;
+    }
+    if (t > pos) ++viol;
+    if (!live) g = 0.f;
+    if (cmp == PBG_CMP_L2) {
+      // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq so that the
+      // backward GEMMs produce the cross terms of ||a||^2 - 2ab + ||b||^2
+      const float dq = live ? g * 0.5f / t : 0.f;
+      rowsum += dq;
+      out[j] = -2.0f * dq;
+    } else {
+      out[j] = g;
+    }
+  }
+  *dpos_out = wave_sum(dpos_part);
+  *rowsum_out = wave_sum(rowsum);
+  int vtot = viol;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) vtot += __shfl_xor(vtot, off, 64);
+  *viol_out = vtot;
+}
+
 __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
   const int lane = threadIdx.x & 63;
   const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
@@ -311,66 +378,9 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     }
     ScoreRow sr = score_row(c, s, kc, cc, i);
     float* out = sd.s + (kc * c.P + i) * nn;
-    float dpos_part = 0.f, rowsum = 0.f;
-    int viol = 0;
-    float mx = pos, inv_z = 0.f;
-    const float inv_nn = 1.0f / (float)nn;
-    if (c.loss == PBG_LOSS_SOFTMAX) {
-      bool live;
-      for (int j = lane; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
-      mx = wave_max(mx);
-      float z = 0.f;
-      for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
-      z = wave_sum(z) + expf(pos - mx);
-      inv_z = 1.0f / z;
-      if (lane == 0) {
-        loss_acc += (mx + logf(z)) - pos;
-        dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
-      }
-    } else if (c.loss == PBG_LOSS_LOGISTIC) {
-      if (lane == 0) {
-        loss_acc += softplusf(-pos);
-        dpos_part += (sigmoidf(pos) - 1.0f) * w;
-      }
-    }
-    for (int j = lane; j < nn; j += kWave) {
-      bool live;
-      const float t = sr.at(j, &live);
-      float g;
-      if (c.loss == PBG_LOSS_RANKING) {
-        // F.margin_ranking_loss(neg, pos, target=-1): max(0, (t - pos) + margin); the
-        // clamp lets the gradient through at exactly 0
-        const float x = (t - pos) + c.margin;
-        if (x > 0.f) loss_acc += x;
-        g = (x >= 0.f) ? w : 0.f;
-        dpos_part -= g;
-      } else if (c.loss == PBG_LOSS_LOGISTIC) {
-        loss_acc += softplusf(t) * inv_nn;
-        g = sigmoidf(t) * inv_nn * w;
-      } else {
-        g = expf(t - mx) * inv_z * w;
-      }
-      if (t > pos) ++viol;
-      if (!live) g = 0.f;
-      if (c.cmp == PBG_CMP_L2) {
-        // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq so that the
-        // backward GEMMs produce the cross terms of ||a||^2 - 2ab + ||b||^2
-        const float dq = live ? g * 0.5f / t : 0.f;
-        rowsum += dq;
-        out[j] = -2.0f * dq;
-      } else {
-        out[j] = g;
-      }
-    }
-    dposv[s] = wave_sum(dpos_part);
-    if (sd.rs) {
-      rowsum = wave_sum(rowsum);
-      if (lane == 0) sd.rs[kc * c.P + i] = rowsum;
-    }
-    int vtot = viol;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) vtot += __shfl_xor(vtot, off, 64);
-    violv[s] = vtot;
+    float rowsum;
+    side_loss(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum);
+    if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = rowsum;
   }
   const float loss_row = wave_sum(loss_acc) * w;
   if (lane == 0) {
@@ -655,6 +665,325 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------
+// fused chunk kernel: the whole chain from gather to raw-row gradients for one
+// chunk in one workgroup, operands resident in LDS
+// ---------------------------------------------------------------------------
+// Eligible shapes (standard mode, operator none / translation / diagonal,
+// comparator dot / l2, batch + uniform negatives on both sides, D <= 128,
+// P <= 64, U <= 64) keep a chunk's 2(P+U) prepared rows and its two score
+// matrices in LDS (132 KB at P = U = 50, D = 100).  Eight waves: phase 0 gathers
+// and applies the operator; phase 1 forms S = A N^T with fp32 MFMA (one row tile
+// per wave, all column tiles in registers); phase 2 is the per-edge loss, in
+// place in LDS; phase 3 forms the four gradient matrices
+//   dL = dS_R N_R + dS_L[:, :P]^T R      dU_L = dS_L[:, P:]^T R     (and L <-> R)
+// with MFMA straight from LDS and writes the raw-row gradients to HBM.
+typedef float float4v __attribute__((ext_vector_type(4)));
+constexpr int kFusedThreads = 512;
+
+struct FusedLayout {
+  int ldx, lds;                  // row strides (floats) of the operand rows and of the score rows
+  int xn[2], sc[2], sq[2], rs[2], cs[2], pos, dpos;  // offsets in floats
+  int total;                     // floats
+};
+
+__global__ __launch_bounds__(kFusedThreads) void fused_chunk_kernel(StepCtx c, FusedLayout f) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t kc = blockIdx.x;
+  const int k = (int)(kc / c.C), cc = (int)(kc % c.C);
+  const int D = c.D, P = c.P, U = c.U, N = P + U, CP = c.C * c.P;
+  const int valid = (cc == c.C - 1) ? c.last : P;
+  float* xn[2] = {lds + f.xn[0], lds + f.xn[1]};
+  float* sc[2] = {lds + f.sc[0], lds + f.sc[1]};
+  float* sq[2] = {lds + f.sq[0], lds + f.sq[1]};
+  float* rs[2] = {lds + f.rs[0], lds + f.rs[1]};
+  float* cs[2] = {lds + f.cs[0], lds + f.cs[1]};
+  float* pos_ = lds + f.pos;
+  float* dpos_ = lds + f.dpos;
+  const int64_t rel = clamp_index(c.rel[k], c.num_relations);
+  const bool l2 = c.cmp == PBG_CMP_L2;
+
+  // ---- phase 0: gather, operator, squared norms; clear the score matrices ----
+  for (int t = threadIdx.x; t < 2 * P * f.lds; t += kFusedThreads) sc[0][t] = 0.f;  // sc[1] follows sc[0]
+  for (int slot = wave; slot < 2 * N; slot += kFusedThreads / kWave) {
+    const int s = slot / N, j = slot % N;
+    const SideCtx& sd = c.side[s];
+    float* dst = xn[s] + j * f.ldx;
+    int64_t id = -1, pair = 0;
+    if (j < P) {
+      const int q = cc * P + j;
+      if (q < c.B) {
+        id = sd.idx[(int64_t)k * c.B + q];
+        pair = (int64_t)k * c.rk + sd.slot_pos + q;
+      }
+    } else {
+      const int u = j - P;
+      id = sd.uidx[kc * U + u];
+      pair = (int64_t)k * c.rk + sd.slot_uni + cc * U + u;
+    }
+    const bool live = id >= 0;
+    if (live) id = clamp_index(id, sd.num_rows);
+    float sumsq = 0.f;
+    for (int d = lane; d < f.ldx; d += kWave) {
+      float v = 0.f;
+      if (live && d < D) {
+        v = sd.w[id * D + d];
+        if (s == 1 && c.op == PBG_OP_DIAGONAL) v = sd.p0[rel * D + d] * v;
+        else if (s == 1 && c.op == PBG_OP_TRANSLATION) v = v + sd.p0[rel * D + d];
+      }
+      dst[d] = v;
+      sumsq += v * v;
+    }
+    if (l2) {
+      const float nrm = sqrtf(wave_sum(sumsq));
+      if (lane == 0) sq[s][j] = nrm * nrm;
+    }
+    if (live && lane == 0) {
+      c.keys[pair] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
+      c.vals[pair] = (uint32_t)pair;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 1: S_s = A_(1-s) N_s^T ----
+  {
+    const int s = wave >> 2, rt = wave & 3;
+    const int TN = (N + 15) >> 4;
+    if (rt * 16 < P) {
+      float4v acc[8];
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const float* A = xn[1 - s];
+      const float* Bm = xn[s];
+      const int ar = rt * 16 + (lane & 15);
+      const int ksteps = (D + 3) >> 2;
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const int kk = ks * 4 + (lane >> 4);
+        const float a = (ar < P) ? A[ar * f.ldx + kk] : 0.f;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+          if (ct < TN) {
+            const int br = ct * 16 + (lane & 15);
+            const float b = (br < N) ? Bm[br * f.ldx + kk] : 0.f;
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) {
+        if (ct < TN) {
+          const int col = ct * 16 + (lane & 15);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = rt * 16 + 4 * (lane >> 4) + r;
+            if (row < P && col < N) sc[s][row * f.lds + col] = acc[ct][r];
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: loss, dLoss/dS in place ----
+  const float w_rel = c.rel_weights[rel];
+  for (int i = wave; i < P; i += kFusedThreads / kWave) {
+    const int q = cc * P + i;
+    const int64_t job = (int64_t)k * CP + q;
+    if (i >= valid) {  // padded positive: its score rows were cleared in phase 0 and phase 1 skipped nothing there
+      for (int j = lane; j < f.lds; j += kWave) {
+        sc[0][i * f.lds + j] = 0.f;
+        sc[1][i * f.lds + j] = 0.f;
+      }
+      if (lane == 0) {
+        rs[0][i] = rs[1][i] = 0.f;
+        pos_[i] = dpos_[i] = 0.f;
+        c.lossrow[job] = 0.f;
+        c.violrow[job * 2] = 0;
+        c.violrow[job * 2 + 1] = 0;
+      }
+      continue;
+    }
+    const float posv = kappa(c.cmp, xn[0] + i * f.ldx, xn[1] + i * f.ldx, D, lane);
+    float w = w_rel;
+    if (c.edge_weight) w *= c.edge_weight[(int64_t)k * c.B + q];
+    float loss_acc = 0.f, dposv[2], rowsum[2];
+    int violv[2];
+    for (int s = 0; s < 2; ++s) {
+      ScoreRow sr;
+      sr.raw = sc[s] + i * f.lds;
+      sr.bn = sq[s];
+      sr.a2 = l2 ? sq[1 - s][i] : 0.f;
+      sr.cmp = c.cmp;
+      sr.nb = P;
+      sr.i = i;
+      sr.masked_from = valid;
+      side_loss(c.loss, c.margin, c.cmp, sr, sc[s] + i * f.lds, N, posv, w, lane, &loss_acc, &dposv[s], &violv[s],
+                &rowsum[s]);
+    }
+    const float loss_row = wave_sum(loss_acc) * w;
+    if (lane == 0) {
+      rs[0][i] = rowsum[0];
+      rs[1][i] = rowsum[1];
+      pos_[i] = posv;
+      dpos_[i] = dposv[0] + dposv[1];
+      c.lossrow[job] = loss_row;
+      c.violrow[job * 2] = violv[0];
+      c.violrow[job * 2 + 1] = violv[1];
+    }
+  }
+  __syncthreads();
+  if (l2) {  // column sums of the stored -2 dLoss/dq
+    for (int t = threadIdx.x; t < 2 * N; t += kFusedThreads) {
+      const int s = t / N, j = t % N;
+      float acc = 0.f;
+      for (int i = 0; i < P; ++i) acc += sc[s][i * f.lds + j];
+      cs[s][j] = acc;
+    }
+    __syncthreads();
+  }
+
+  // ---- phase 3: gradients of the 2(P+U) rows, written to HBM ----
+  {
+    const int m = wave >> 2, rt = wave & 3;  // m: side whose rows' gradients this wave forms
+    const int TD = (D + 15) >> 4;
+    const SideCtx& sd = c.side[m];
+    const float* ds_a = sc[1 - m];  // scores in which this side's positives were the A operand
+    const float* ds_n = sc[m];      // scores against this side's negatives
+    const float* bx = xn[1 - m];    // the other side's rows: the B operand of every product here
+    const bool has_op = m == 1 && c.op != PBG_OP_NONE;
+    if (rt * 16 < P) {
+      float4v acc[8];
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const int ar = rt * 16 + (lane & 15);
+      for (int ks = 0; ks < ((N + 3) >> 2); ++ks) {  // dS_a (P x N) times the other side's N rows
+        const int kk = ks * 4 + (lane >> 4);
+        const float a = (ar < P && kk < N) ? ds_a[ar * f.lds + kk] : 0.f;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+          if (ct < TD) {
+            const int dc = ct * 16 + (lane & 15);
+            const float b = (kk < N && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+          }
+        }
+      }
+      for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {  // (dS_n[:, :P])^T (P x P) times the other side's positives
+        const int kk = ks * 4 + (lane >> 4);
+        const float a = (ar < P && kk < P) ? ds_n[kk * f.lds + ar] : 0.f;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+          if (ct < TD) {
+            const int dc = ct * 16 + (lane & 15);
+            const float b = (kk < P && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) {
+        if (ct < TD) {
+          const int d = ct * 16 + (lane & 15);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int i = rt * 16 + 4 * (lane >> 4) + r;
+            if (i < valid && d < D) {
+              const float self = xn[m][i * f.ldx + d], other = bx[i * f.ldx + d];
+              float v = acc[ct][r];
+              if (l2) {
+                v += (2.0f * rs[1 - m][i] - cs[m][i]) * self;
+                const float pz = pos_[i];
+                if (pz * pz > 1e-30f) v += dpos_[i] / pz * (self - other);
+              } else {
+                v += dpos_[i] * other;
+              }
+              const int q = cc * P + i;
+              if (has_op) {
+                if (sd.dz) sd.dz[((int64_t)k * sd.op_rows + q) * D + d] = v;
+                if (c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
+              }
+              c.gr[((int64_t)k * c.rk + sd.slot_pos + q) * D + d] = v;
+            }
+          }
+        }
+      }
+    }
+    if (rt * 16 < U) {  // uniform negatives of side m: (dS_n[:, P:])^T (U x P) times the other side's positives
+      float4v acc[8];
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const int au = rt * 16 + (lane & 15);
+      for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {
+        const int kk = ks * 4 + (lane >> 4);
+        const float a = (au < U && kk < P) ? ds_n[kk * f.lds + P + au] : 0.f;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+          if (ct < TD) {
+            const int dc = ct * 16 + (lane & 15);
+            const float b = (kk < P && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) {
+        if (ct < TD) {
+          const int d = ct * 16 + (lane & 15);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int u = rt * 16 + 4 * (lane >> 4) + r;
+            if (u < U && d < D) {
+              float v = acc[ct][r];
+              if (l2) v -= cs[m][P + u] * xn[m][(P + u) * f.ldx + d];
+              const int r2 = cc * U + u;
+              if (has_op) {
+                if (sd.dz) sd.dz[((int64_t)k * sd.op_rows + c.B + r2) * D + d] = v;
+                if (c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
+              }
+              c.gr[((int64_t)k * c.rk + sd.slot_uni + r2) * D + d] = v;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Row stride >= n (a multiple of 4) that keeps both MFMA access patterns
+// (16 rows x 4 columns, and 4 rows x 16 columns) at most 3-way bank conflicted.
+int lds_stride(int n) {
+  int ld = (n + 3) / 4 * 4;
+  while (ld % 32 != 12 && ld % 32 != 20) ld += 4;
+  return ld;
+}
+
+bool fused_layout(const StepCtx& c, FusedLayout* f) {
+  if (c.dynamic) return false;
+  if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
+  if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2) return false;
+  if (c.D > 128 || c.P > 64 || c.U > 64) return false;
+  for (int s = 0; s < 2; ++s)
+    if (c.side[s].nb != c.P || c.side[s].u != c.U) return false;
+  const int N = c.P + c.U;
+  f->ldx = lds_stride(c.D);
+  f->lds = lds_stride(N);
+  int off = 0;
+  auto take = [&](int count) { int o = off; off += (count + 3) / 4 * 4; return o; };
+  f->xn[0] = take(N * f->ldx);
+  f->xn[1] = take(N * f->ldx + 16);
+  f->sc[0] = take(c.P * f->lds);
+  f->sc[1] = take(c.P * f->lds + 16);
+  if (f->sc[1] != f->sc[0] + c.P * f->lds) return false;  // phase 0 clears both as one block
+  for (int s = 0; s < 2; ++s) f->sq[s] = take(N);
+  for (int s = 0; s < 2; ++s) f->rs[s] = take(c.P);
+  for (int s = 0; s < 2; ++s) f->cs[s] = take(N);
+  f->pos = take(c.P);
+  f->dpos = take(c.P);
+  f->total = off;
+  return (size_t)off * sizeof(float) <= 160 * 1024 - 512;
+}
+
+// ---------------------------------------------------------------------------
 // operator parameters, dynamic relations (one relation per edge)
 // ---------------------------------------------------------------------------
 // `linear` with a relation per row: z_e = W[rel_e] x_e, one wave per positive
@@ -866,6 +1195,8 @@ struct Plan {
   void* sort_temp;
   int64_t psize;  // floats of parameter gradient per batch
   int pslices[2]; // partial sums per batch of the element-wise parameter gradients
+  bool fused;          // the chunk fits the LDS-resident kernel
+  FusedLayout fl;
   // dynamic relations: (relation, batch) keys of the positives and their sort buffers
   uint64_t *rkeys_a, *rkeys_b;
   uint32_t *rvals_a, *rvals_b;
@@ -1030,6 +1361,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->sort_temp = take(sort_temp_bytes(npairs), 1);
   plan->bytes = off;
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
+  plan->fused = fused_layout(c, &plan->fl) && getenv("PBG_DISABLE_FUSED") == nullptr;
 
   if (b) {
     c.side[0].w = b->w_lhs;
@@ -1287,21 +1619,42 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if (ev) hipEventRecord(ev[i], s);
   };
   mark(0);
-  if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
-  mark(1);
-  if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
-  mark(2);
-  if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
-  mark(3);
-  hipLaunchKernelGGL(loss_kernel, wave_grid((int64_t)c.K * c.C * c.P), dim3(kRowThreads), 0, s, c);
-  hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
-  mark(4);
-  if ((rc = run_backward_dn(plan, s)) != PBG_OK) return rc;
-  mark(5);
-  if ((rc = run_backward_da(plan, s)) != PBG_OK) return rc;
-  mark(6);
-  if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
-  mark(7);
+  if (plan.fused) {
+    // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
+    const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
+    static size_t lds_allowed = 0;
+    if (lds_bytes > lds_allowed) {
+      if (hipFuncSetAttribute((const void*)fused_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes) != hipSuccess)
+        return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
+      lds_allowed = lds_bytes;
+    }
+    hipLaunchKernelGGL(fused_chunk_kernel, dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c, plan.fl);
+    mark(1);
+    mark(2);
+    mark(3);
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+    mark(4);
+    mark(5);
+    mark(6);
+    mark(7);
+  } else {
+    if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
+    mark(1);
+    if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
+    mark(2);
+    if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
+    mark(3);
+    hipLaunchKernelGGL(loss_kernel, wave_grid((int64_t)c.K * c.C * c.P), dim3(kRowThreads), 0, s, c);
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+    mark(4);
+    if ((rc = run_backward_dn(plan, s)) != PBG_OK) return rc;
+    mark(5);
+    if ((rc = run_backward_da(plan, s)) != PBG_OK) return rc;
+    mark(6);
+    if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
+    mark(7);
+  }
   if ((rc = run_params(desc, bufs, plan, s)) != PBG_OK) return rc;
   mark(8);
   const int64_t npairs = (int64_t)c.K * c.rk;
