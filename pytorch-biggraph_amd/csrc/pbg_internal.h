@@ -25,12 +25,14 @@ inline int bits_for(uint64_t max_value) {  // number of bits needed to hold max_
 }
 
 // ---- device radix sort of (uint64 key, uint32 value) pairs ----------------
-// LSD radix sort, 8 bits per pass, stable.  Sorts on key bits [0, key_bits).
-// The result ends up in (keys_out, vals_out); (keys_in, vals_in) are clobbered.
+// LSD radix sort, up to 9 bits per pass, stable.  Sorts on key bits
+// [low_bit, key_bits): an input already ordered by the bits below low_bit comes
+// out ordered by all bits below key_bits.  Both buffer pairs are clobbered; the
+// result is in whichever pair *keys_sorted / *vals_sorted name on return.
 // `temp` holds sort_temp_bytes(n) bytes.
 size_t sort_temp_bytes(int64_t n);
-int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n,
-               int key_bits, void* temp, hipStream_t stream);
+int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
+               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted);
 
 // ---- segmented RowAdagrad over sorted (row << kbits | worker) keys ---------
 // keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim], which is

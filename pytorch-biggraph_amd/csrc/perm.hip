@@ -208,9 +208,11 @@ extern "C" int pbg_randperm(int64_t n, uint64_t seed, int64_t* out, void* worksp
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(random_keys_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, n, seed, ws.keys_a,
                      ws.vals_a);
-  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, kRandKeyBits, ws.temp, s);
+  uint64_t* skeys;
+  uint32_t* svals;
+  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, 0, kRandKeyBits, ws.temp, s, &skeys, &svals);
   if (rc != PBG_OK) return rc;
-  hipLaunchKernelGGL(widen_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, ws.vals_b, n, out);
+  hipLaunchKernelGGL(widen_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, svals, n, out);
   return check_launch("pbg_randperm");
 }
 
@@ -245,9 +247,12 @@ extern "C" int pbg_sub_bucket(const int64_t* lhs_in, const int64_t* rhs_in, cons
                   n, num_relations, num_lhs_parts, num_rhs_parts, dynamic_relations};
   const dim3 grid((unsigned)ceil_div(n, 256)), block(256);
   hipLaunchKernelGGL(sub_bucket_keys_kernel, grid, block, 0, s, a, ws.keys_a, ws.vals_a, error_flag);
-  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, bits_for((uint64_t)(nb - 1)), ws.temp, s);
+  uint64_t* skeys;
+  uint32_t* svals;
+  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, 0, bits_for((uint64_t)(nb - 1)), ws.temp, s,
+                      &skeys, &svals);
   if (rc != PBG_OK) return rc;
-  hipLaunchKernelGGL(sub_bucket_emit_kernel, grid, block, 0, s, a, ws.keys_b, ws.vals_b, lhs_out, rhs_out, rel_out,
+  hipLaunchKernelGGL(sub_bucket_emit_kernel, grid, block, 0, s, a, skeys, svals, lhs_out, rhs_out, rel_out,
                      offsets_out);
   return check_launch("pbg_sub_bucket");
 }

@@ -5,6 +5,7 @@
 // (dim 100) is one coalesced request of 25 lanes and a 4 KiB row (dim 1024) is
 // four full-wave requests.
 #include "pbg_internal.h"
+#include "row_ops.h"
 
 namespace pbg {
 namespace {
@@ -12,11 +13,6 @@ namespace {
 constexpr int kRowThreads = 256;  // 4 waves per block, one row per wave
 constexpr int kMaxV4 = 4;         // float4 per lane: covers dim <= 1024
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
 
 // ---- gather ----------------------------------------------------------------
 template <bool VEC>
@@ -52,9 +48,11 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const float* _
 //   tile_reduce   one wave per tile of kTile sorted positions sums every piece
 //                 (maximal stretch of equal keys inside the tile) longer than 1
 //                 into the gradient row of the piece's first position;
-//   run_combine   one wave per run that crosses tile borders adds the pieces of
-//                 the later tiles into the row of the run's first position;
-//   row_update    one wave per row walks its runs (one gradient row each).
+//   run_combine   one wave per tile border; the first border a run crosses adds
+//                 the pieces of the later tiles into the row of the run's first
+//                 position;
+//   row_update    one wave per row walks its runs (one gradient row each), the
+//                 keys of the next 64 positions held in registers.
 constexpr int kTile = 32;
 
 template <int NV, bool VEC>
@@ -92,6 +90,10 @@ struct RowRegs {
       }
     }
   }
+  __device__ __forceinline__ void add(const RowRegs& o) {
+#pragma unroll
+    for (int q = 0; q < NV * W; ++q) v[q] += o.v[q];
+  }
   __device__ __forceinline__ void store(float* __restrict__ p, int nv, int lane) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -121,6 +123,15 @@ __device__ __forceinline__ int64_t scan_end(const uint64_t* __restrict__ keys, i
   }
 }
 
+// value of lane `l` (uniform) of a per-lane 32-bit / 64-bit quantity
+__device__ __forceinline__ uint32_t lane_u32(uint32_t v, int l) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, l);
+}
+__device__ __forceinline__ uint64_t lane_u64(uint64_t v, int l) {
+  const uint32_t lo = lane_u32((uint32_t)v, l), hi = lane_u32((uint32_t)(v >> 32), l);
+  return ((uint64_t)hi << 32) | lo;
+}
+
 template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
@@ -131,9 +142,10 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
   if (begin >= n) return;
   const int64_t end = (begin + kTile < n) ? begin + kTile : n;
   const int nv = VEC ? (dim >> 2) : dim;
-  // one key per lane for the whole tile, then pieces are found with ballots
+  // one key and one value per lane for the whole tile, then pieces are found with ballots
   const int64_t mine = begin + lane;
   const uint64_t key = (mine < end) ? keys[mine] : 0ull;
+  const uint32_t val = (mine < end) ? vals[mine] : 0u;
   const uint64_t prev = __shfl_up(key, 1, 64);
   const bool starts = (mine < end) && (lane == 0 || prev != key);
   uint64_t heads = __ballot(starts);  // bit l set: a piece starts at begin + l
@@ -143,30 +155,74 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
     const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
     if (b - a < 2) continue;
     RowRegs<NV, VEC> acc;
-    acc.load(grad_rows + (int64_t)vals[begin + a] * dim, nv, lane);
-    for (int j = a + 1; j < b; ++j) acc.add(grad_rows + (int64_t)vals[begin + j] * dim, nv, lane);
-    acc.store(grad_rows + (int64_t)vals[begin + a] * dim, nv, lane);
+    float* head = grad_rows + (int64_t)lane_u32(val, a) * dim;
+    acc.load(head, nv, lane);
+    int j = a + 1;
+    for (; j + 1 < b; j += 2) {  // two rows in flight
+      RowRegs<NV, VEC> x, y;
+      x.load(grad_rows + (int64_t)lane_u32(val, j) * dim, nv, lane);
+      y.load(grad_rows + (int64_t)lane_u32(val, j + 1) * dim, nv, lane);
+      acc.add(x);
+      acc.add(y);
+    }
+    if (j < b) acc.add(grad_rows + (int64_t)lane_u32(val, j) * dim, nv, lane);
+    acc.store(head, nv, lane);
   }
 }
 
+// One wave per tile border: if a run crosses the border and this is the first
+// border it crosses, add the pieces of all later tiles into the run's head row.
 template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
                                                                   float* __restrict__ grad_rows, int dim) {
   const int lane = threadIdx.x & 63;
-  const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
-  if (i >= n) return;
-  const uint64_t key = keys[i];
-  if (i > 0 && keys[i - 1] == key) return;             // not the head of a run
-  const int64_t tile_end = (i / kTile + 1) * kTile;
-  if (tile_end >= n || keys[tile_end] != key) return;  // the run ends inside its first tile
-  const int64_t end = scan_end(keys, tile_end, n, key, 0, lane);
+  const int64_t b = ((int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6) + 1) * kTile;
+  if (b >= n) return;
+  // window of the tile before the border (lanes 0..31) and the tile after it (lanes 32..63)
+  const int64_t p = b - kTile + lane;
+  const uint64_t kk = keys[p < n ? p : n - 1];
+  const uint64_t key = lane_u64(kk, kTile);
+  if (lane_u64(kk, kTile - 1) != key) return;  // no run crosses this border
+  const uint64_t same = __ballot(p < n && kk == key);
+  const uint32_t not_before = ~(uint32_t)same;  // zero bits: positions of the run in the tile before the border
+  const int head_lane = not_before ? 32 - __clz(not_before) : 0;
+  if (head_lane == 0 && b - kTile > 0 && keys[b - kTile - 1] == key) return;  // an earlier border owns this run
+  const uint32_t not_after = ~(uint32_t)(same >> 32);
+  const int64_t end = not_after ? b + (__ffs(not_after) - 1) : scan_end(keys, b + kTile - 1, n, key, 0, lane);
   const int nv = VEC ? (dim >> 2) : dim;
   RowRegs<NV, VEC> acc;
-  float* head = grad_rows + (int64_t)vals[i] * dim;
+  float* head = grad_rows + (int64_t)vals[b - kTile + head_lane] * dim;
   acc.load(head, nv, lane);
-  for (int64_t p = tile_end; p < end; p += kTile) acc.add(grad_rows + (int64_t)vals[p] * dim, nv, lane);
+  for (int64_t base = b; base < end; base += (int64_t)kTile * kWave) {  // 64 pieces' first positions per round
+    const int64_t q = base + (int64_t)lane * kTile;
+    const uint32_t v = q < end ? vals[q] : 0u;
+    const int64_t left = (end - base + kTile - 1) / kTile;
+    const int count = left < kWave ? (int)left : kWave;
+    int j = 0;
+    for (; j + 1 < count; j += 2) {
+      RowRegs<NV, VEC> x, y;
+      x.load(grad_rows + (int64_t)lane_u32(v, j) * dim, nv, lane);
+      y.load(grad_rows + (int64_t)lane_u32(v, j + 1) * dim, nv, lane);
+      acc.add(x);
+      acc.add(y);
+    }
+    if (j < count) acc.add(grad_rows + (int64_t)lane_u32(v, j) * dim, nv, lane);
+  }
   acc.store(head, nv, lane);
+}
+
+template <int NV, bool VEC>
+__device__ __forceinline__ float adagrad_apply(RowRegs<NV, VEC>& w, const RowRegs<NV, VEC>& g, float gsum, float fdim,
+                                               float lr) {
+  float sq = 0.f;
+#pragma unroll
+  for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) sq += g.v[q] * g.v[q];
+  gsum += wave_sum(sq) / fdim;
+  const float stdv = sqrtf(gsum) + 1e-10f;
+#pragma unroll
+  for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) w.v[q] += (-lr * g.v[q]) / stdv;
+  return gsum;
 }
 
 template <int NV, bool VEC>
@@ -177,7 +233,11 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   const int lane = threadIdx.x & 63;
   const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
   if (i >= n) return;
-  const uint64_t row = keys[i] >> kbits;
+  // one coalesced look at this and the next 63 sorted positions
+  const int64_t p = i + lane;
+  const uint64_t kk = keys[p < n ? p : n - 1];
+  const uint32_t vv = vals[p < n ? p : n - 1];
+  const uint64_t row = lane_u64(kk, 0) >> kbits;
   if (i > 0 && (keys[i - 1] >> kbits) == row) return;
   if ((int64_t)row >= rows0 + rows1) return;  // out-of-range indices are parked past both tables
 
@@ -191,25 +251,39 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     gptr = g1 + ((int64_t)row - rows0);
   }
   const int nv = VEC ? (dim >> 2) : dim;
+  const float fdim = (float)dim;
   RowRegs<NV, VEC> w;
   w.load(wrow, nv, lane);
   float gsum = *gptr;
-  const float fdim = (float)dim;
-  int64_t j = i;
-  while (j < n && (keys[j] >> kbits) == row) {
-    const uint64_t key = keys[j];
+
+  const uint64_t in_row = __ballot(p < n && (kk >> kbits) == row);
+  if (~in_row != 0ull) {
+    // the row ends inside the window: its runs are known from the keys in registers
+    const int len = __ffsll((unsigned long long)~in_row) - 1;
+    const uint64_t up = __shfl_up(kk, 1, 64);
+    uint64_t heads = __ballot(lane < len && (lane == 0 || up != kk));  // first position of every run
     RowRegs<NV, VEC> g;
-    g.load(grad_rows + (int64_t)vals[j] * dim, nv, lane);  // the run's sum (tile_reduce / run_combine)
-    // a single-worker call has one run per row: no need to look for its end
-    j = (kbits == 0) ? n : scan_end(keys, j, n, key, 0, lane);
-    float sq = 0.f;
-#pragma unroll
-    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) sq += g.v[q] * g.v[q];
-    const float delta = wave_sum(sq) / fdim;
-    gsum += delta;
-    const float stdv = sqrtf(gsum) + 1e-10f;
-#pragma unroll
-    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) w.v[q] += (-lr * g.v[q]) / stdv;
+    g.load(grad_rows + (int64_t)lane_u32(vv, 0) * dim, nv, lane);  // each run's sum sits in its first row
+    heads &= heads - 1;
+    while (heads != 0ull) {  // the next run's row is in flight while this one is applied
+      const int a = __ffsll((unsigned long long)heads) - 1;
+      heads &= heads - 1;
+      RowRegs<NV, VEC> next;
+      next.load(grad_rows + (int64_t)lane_u32(vv, a) * dim, nv, lane);
+      gsum = adagrad_apply(w, g, gsum, fdim, lr);
+      g = next;
+    }
+    gsum = adagrad_apply(w, g, gsum, fdim, lr);
+  } else {
+    int64_t j = i;
+    while (j < n && (keys[j] >> kbits) == row) {
+      const uint64_t key = keys[j];
+      RowRegs<NV, VEC> g;
+      g.load(grad_rows + (int64_t)vals[j] * dim, nv, lane);
+      // a single-worker call has one run per row: no need to look for its end
+      j = (kbits == 0) ? n : scan_end(keys, j, n, key, 0, lane);
+      gsum = adagrad_apply(w, g, gsum, fdim, lr);
+    }
   }
   w.store(wrow, nv, lane);
   if (lane == 0) *gptr = gsum;
@@ -261,10 +335,13 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   const int wpb = kRowThreads / kWave;
   const dim3 grid((unsigned)ceil_div(n, wpb)), block(kRowThreads);
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
+  const int64_t borders = ceil_div(n, kTile) - 1;
+  const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim);  \
-    hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, grad_rows, dim);       \
+    if (borders > 0)                                                                                              \
+      hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
     hipLaunchKernelGGL((row_update_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, kbits, grad_rows, dim,  \
                        w0, g0, rows0, w1, g1, rows1, lr);                                                          \
   } while (0)
@@ -352,10 +429,13 @@ extern "C" int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t n
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(make_keys_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, idx, n, num_rows, ws.keys_a,
                      ws.vals_a);
-  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, bits_for((uint64_t)num_rows), ws.temp, s);
+  uint64_t* skeys;
+  uint32_t* svals;
+  int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, 0, bits_for((uint64_t)num_rows), ws.temp, s,
+                      &skeys, &svals);
   if (rc != PBG_OK) return rc;
   // out-of-range indices were parked at key == num_rows and are skipped by the update
-  return row_adagrad_sorted(ws.keys_b, ws.vals_b, n, 0, grad_rows, dim, weight, state_sum, num_rows, nullptr,
+  return row_adagrad_sorted(skeys, svals, n, 0, grad_rows, dim, weight, state_sum, num_rows, nullptr,
                             nullptr, 0, lr, s);
 }
 

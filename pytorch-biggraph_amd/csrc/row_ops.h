@@ -10,16 +10,95 @@
 
 namespace pbg {
 
+// Cross-lane reductions with DPP moves (ALU-rate) instead of LDS permutes: four
+// steps fold a row of 16 lanes onto itself (quad swaps, half-row mirror, row
+// mirror), two row broadcasts carry the row sums into lane 63, which is then
+// read back as a scalar.  Every lane returns the total.
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ int dpp_i(int old, int v) {
+  return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, BANK_MASK, false);
+}
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf>
+__device__ __forceinline__ float dpp_f(float old, float v) {
+  return __int_as_float(dpp_i<CTRL, ROW_MASK, BANK_MASK>(__float_as_int(old), __float_as_int(v)));
+}
+constexpr int kDppQuadSwap1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kDppQuadSwap2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+constexpr int kDppRowBcast15 = 0x142;   // lane 15 of each row -> the next row
+constexpr int kDppRowBcast31 = 0x143;   // lane 31 -> rows 2 and 3
+
+// sum over each row of 16 lanes, left in every lane of the row
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f<kDppQuadSwap1>(0.f, v);
+  v += dpp_f<kDppQuadSwap2>(0.f, v);
+  v += dpp_f<kDppRowHalfMirror>(0.f, v);
+  v += dpp_f<kDppRowMirror>(0.f, v);
+  return v;
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  v = row16_sum(v);
+  v += dpp_f<kDppRowBcast15, 0xa>(0.f, v);
+  v += dpp_f<kDppRowBcast31, 0xc>(0.f, v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+// sums of lanes 0..31 and of lanes 32..63: valid in lane 31 and lane 63 respectively
+__device__ __forceinline__ float half_sum_at_31(float v) {
+  v = row16_sum(v);
+  v += dpp_f<kDppRowBcast15, 0xa>(0.f, v);
   return v;
 }
+__device__ __forceinline__ int wave_sum_int(int v) {
+  v += dpp_i<kDppQuadSwap1, 0xf, 0xf>(0, v);
+  v += dpp_i<kDppQuadSwap2, 0xf, 0xf>(0, v);
+  v += dpp_i<kDppRowHalfMirror, 0xf, 0xf>(0, v);
+  v += dpp_i<kDppRowMirror, 0xf, 0xf>(0, v);
+  v += dpp_i<kDppRowBcast15, 0xa, 0xf>(0, v);
+  v += dpp_i<kDppRowBcast31, 0xc, 0xf>(0, v);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+// reductions over the 4 lanes of a quad, result in all 4
+__device__ __forceinline__ float quad_sum(float v) {
+  v += dpp_f<kDppQuadSwap1>(0.f, v);
+  v += dpp_f<kDppQuadSwap2>(0.f, v);
+  return v;
+}
+__device__ __forceinline__ float quad_max(float v) {
+  v = fmaxf(v, dpp_f<kDppQuadSwap1>(v, v));
+  v = fmaxf(v, dpp_f<kDppQuadSwap2>(v, v));
+  return v;
+}
+__device__ __forceinline__ int quad_sum_int(int v) {
+  v += dpp_i<kDppQuadSwap1, 0xf, 0xf>(0, v);
+  v += dpp_i<kDppQuadSwap2, 0xf, 0xf>(0, v);
+  return v;
+}
+struct WaveReduce {  // a row spread over the 64 lanes of a wave
+  static constexpr int kStep = 64;
+  static __device__ __forceinline__ float sum(float v);
+  static __device__ __forceinline__ float max(float v);
+  static __device__ __forceinline__ int sum_int(int v);
+};
+struct QuadReduce {  // a row spread over the 4 lanes of a quad
+  static constexpr int kStep = 4;
+  static __device__ __forceinline__ float sum(float v) { return quad_sum(v); }
+  static __device__ __forceinline__ float max(float v) { return quad_max(v); }
+  static __device__ __forceinline__ int sum_int(int v) { return quad_sum_int(v); }
+};
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+  v = fmaxf(v, dpp_f<kDppQuadSwap1>(v, v));
+  v = fmaxf(v, dpp_f<kDppQuadSwap2>(v, v));
+  v = fmaxf(v, dpp_f<kDppRowHalfMirror>(v, v));
+  v = fmaxf(v, dpp_f<kDppRowMirror>(v, v));
+  v = fmaxf(v, dpp_f<kDppRowBcast15, 0xa>(v, v));
+  v = fmaxf(v, dpp_f<kDppRowBcast31, 0xc>(v, v));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
+
+__device__ __forceinline__ float WaveReduce::sum(float v) { return wave_sum(v); }
+__device__ __forceinline__ float WaveReduce::max(float v) { return wave_max(v); }
+__device__ __forceinline__ int WaveReduce::sum_int(int v) { return wave_sum_int(v); }
 
 template <int NVH>
 struct RowV {

@@ -1,27 +1,31 @@
-// Stable LSD radix sort of (uint64 key, uint32 value) pairs, 8 bits per pass.
+// Stable LSD radix sort of (uint64 key, uint32 value) pairs on a bit range of the
+// key, up to 9 bits per pass.
 //
 // Every block owns a contiguous power-of-two tile of positions.  One histogram
 // kernel counts the first digit per tile; after that each pass is ONE kernel:
 // a block derives its digit offsets from the per-tile counts of all tiles (at
-// most 256 of them), ranks its keys slice by slice (ballot matching inside a
-// wave, LDS counts across the 4 waves, a running per-digit cursor across
-// slices), scatters them, and counts the next pass's digit of every key into the
-// tile the key lands in, so the next pass needs no histogram kernel of its own.
-// Stability makes the order of equal keys the order of the input, which keeps
-// segmented gradient sums deterministic.
+// most 256 of them, stored digit-major so that a thread reads its digit's counts
+// with a few independent 128-bit loads), ranks its keys slice by slice (ballot
+// matching inside a wave, LDS counts across the 4 waves, a running per-digit
+// cursor across slices), scatters them, and counts the next pass's digit of
+// every key into the tile the key lands in, so the next pass needs no histogram
+// kernel of its own.  Stability makes the order of equal keys the order of the
+// input, which keeps segmented gradient sums deterministic and lets a caller
+// whose input is already ordered by the low bits leave those bits out.
 #include "pbg_internal.h"
 
 namespace pbg {
 namespace {
 
 constexpr int kSortThreads = 256;
-constexpr int kRadix = 256;
+constexpr int kMaxDigitBits = 9;
 constexpr int kMaxSortBlocks = 256;
-constexpr int kMaxPasses = 9;
+constexpr int kMaxPasses = 8;
 
 struct SortPlan {
   int tile_shift;  // keys per block = 1 << tile_shift
   int blocks;
+  int stride;      // blocks rounded up to a multiple of 4: row length of the digit-major counts
 };
 
 SortPlan plan_sort(int64_t n) {
@@ -29,62 +33,103 @@ SortPlan plan_sort(int64_t n) {
   p.tile_shift = 9;
   while (ceil_div(n, (int64_t)1 << p.tile_shift) > kMaxSortBlocks) ++p.tile_shift;
   p.blocks = (int)ceil_div(n > 0 ? n : 1, (int64_t)1 << p.tile_shift);
+  p.stride = (p.blocks + 3) / 4 * 4;
   return p;
 }
 
-// counts[pass][block][digit]; this kernel fills pass 0 and clears the others
+// counts[pass][digit][stride]; this kernel fills pass 0 and clears the others
 __global__ __launch_bounds__(kSortThreads) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n,
-                                                                 int tile_shift, int passes,
+                                                                 int tile_shift, int shift, int digit_bits,
+                                                                 int passes, int stride,
                                                                  uint32_t* __restrict__ counts) {
-  __shared__ uint32_t hist[kRadix];
-  const int nblocks = gridDim.x;
-  hist[threadIdx.x] = 0;
-  for (int p = 1; p < passes; ++p) counts[((int64_t)p * nblocks + blockIdx.x) * kRadix + threadIdx.x] = 0;
+  __shared__ uint32_t hist[1 << kMaxDigitBits];
+  const int digits = 1 << digit_bits;
+  const uint32_t mask = (uint32_t)digits - 1u;
+  for (int d = threadIdx.x; d < digits; d += kSortThreads) hist[d] = 0;
+  for (int p = 1; p < passes; ++p)
+    for (int d = threadIdx.x; d < digits; d += kSortThreads)
+      counts[((int64_t)p * digits + d) * stride + blockIdx.x] = 0;
+  if (blockIdx.x == 0)  // the padding columns of every pass
+    for (int p = 0; p < passes; ++p)
+      for (int d = threadIdx.x; d < digits; d += kSortThreads)
+        for (int b = gridDim.x; b < stride; ++b) counts[((int64_t)p * digits + d) * stride + b] = 0;
   __syncthreads();
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kSortThreads) atomicAdd(&hist[keys[i] & 0xff], 1u);
+  for (int64_t i = begin + threadIdx.x; i < end; i += kSortThreads)
+    atomicAdd(&hist[(uint32_t)(keys[i] >> shift) & mask], 1u);
   __syncthreads();
-  counts[(int64_t)blockIdx.x * kRadix + threadIdx.x] = hist[threadIdx.x];
+  for (int d = threadIdx.x; d < digits; d += kSortThreads) counts[(int64_t)d * stride + blockIdx.x] = hist[d];
 }
 
+// DPT digits per thread: 1 (up to 8 digit bits) or 2 (9 digit bits); digit d belongs to thread d % 256.
+template <int DPT>
 __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
-    uint32_t* __restrict__ vals_out, int64_t n, int tile_shift, int shift, const uint32_t* __restrict__ counts,
-    uint32_t* __restrict__ next_counts) {
-  __shared__ uint32_t cursor[kRadix];         // next output slot of each digit for this block
-  __shared__ uint32_t wave_count[4][kRadix];  // per-wave digit counts of the current slice
-  __shared__ uint32_t scan[kRadix];
+    uint32_t* __restrict__ vals_out, int64_t n, int tile_shift, int shift, int digit_bits, int next_shift,
+    int next_digit_bits, int stride, const uint32_t* __restrict__ counts, uint32_t* __restrict__ next_counts) {
+  constexpr int kDigits = DPT * kSortThreads;
+  constexpr int kBits = DPT == 1 ? 8 : 9;
+  __shared__ uint32_t cursor[kDigits];         // next output slot of each digit for this block
+  __shared__ uint32_t wave_count[4][kDigits];  // per-wave digit counts of the current slice
+  __shared__ uint32_t wave_total[4];
   const int t = threadIdx.x;
   const int wave = t >> 6;
   const int lane = t & 63;
-  const int nblocks = gridDim.x;
-  // offset of digit t for this block = keys with a smaller digit anywhere
-  //                                  + keys with digit t in earlier blocks
-  uint32_t total = 0, before = 0;
-  for (int b0 = 0; b0 < nblocks; b0 += 8) {  // eight independent loads in flight
-    uint32_t cnt[8];
+  const int me = blockIdx.x;
+  // offset of digit d for this block = keys with a smaller digit anywhere
+  //                                  + keys with digit d in earlier blocks
+  uint32_t total[DPT], before[DPT];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) cnt[u] = (b0 + u < nblocks) ? counts[(int64_t)(b0 + u) * kRadix + t] : 0u;
+  for (int d = 0; d < DPT; ++d) total[d] = before[d] = 0;
+  const int quads = stride >> 2;
+  for (int q0 = 0; q0 < quads; q0 += 16) {  // 16 x DPT independent 128-bit loads in flight
+    uint4 cnt[DPT][16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      total += cnt[u];
-      if (b0 + u < (int)blockIdx.x) before += cnt[u];
+    for (int d = 0; d < DPT; ++d) {
+      const uint4* row = reinterpret_cast<const uint4*>(counts + (int64_t)(t + d * kSortThreads) * stride);
+      const bool has = ((t + d * kSortThreads) >> digit_bits) == 0;  // digits past the pass's width hold no keys
+#pragma unroll
+      for (int u = 0; u < 16; ++u) cnt[d][u] = (has && q0 + u < quads) ? row[q0 + u] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int d = 0; d < DPT; ++d) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int b = (q0 + u) * 4;
+        const uint4 c4 = cnt[d][u];
+        total[d] += c4.x + c4.y + c4.z + c4.w;
+        before[d] += (b < me ? c4.x : 0u) + (b + 1 < me ? c4.y : 0u) + (b + 2 < me ? c4.z : 0u) +
+                     (b + 3 < me ? c4.w : 0u);
+      }
     }
   }
-  scan[t] = total;
-  __syncthreads();
-  for (int off = 1; off < kRadix; off <<= 1) {  // inclusive scan over the 256 digit totals
-    const uint32_t v = (t >= off) ? scan[t - off] : 0;
+  // exclusive scan of the digit totals in digit order (digit = t + d * 256)
+  uint32_t carry = 0;
+#pragma unroll
+  for (int d = 0; d < DPT; ++d) {
+    uint32_t incl = total[d];
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
+    }
+    if (lane == 63) wave_total[wave] = incl;
     __syncthreads();
-    scan[t] += v;
+    uint32_t ahead = carry;
+    for (int w = 0; w < wave; ++w) ahead += wave_total[w];
+    carry += wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    cursor[t + d * kSortThreads] = ahead + incl - total[d] + before[d];
     __syncthreads();
   }
-  cursor[t] = scan[t] - total + before;
-  for (int w = 0; w < 4; ++w) wave_count[w][t] = 0;
+#pragma unroll
+  for (int d = 0; d < DPT; ++d)
+    for (int w = 0; w < 4; ++w) wave_count[w][t + d * kSortThreads] = 0;
   __syncthreads();
 
+  const uint32_t mask = (1u << digit_bits) - 1u;
+  const uint32_t next_mask = (1u << next_digit_bits) - 1u;
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
@@ -104,11 +149,11 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
       key_next = keys_in[i + kSortThreads];
       val_next = vals_in[i + kSortThreads];
     }
-    const uint32_t digit = shift < 64 ? (uint32_t)((key >> shift) & 0xff) : 0u;
+    const uint32_t digit = (uint32_t)(key >> shift) & mask;
     // lanes of this wave holding the same digit
     uint64_t peers = __ballot(valid);
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < kBits; ++b) {
       const bool bit = (digit >> b) & 1u;
       const uint64_t m = __ballot(valid && bit);
       peers &= bit ? m : ~m;
@@ -124,18 +169,21 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
       keys_out[pos] = key;
       vals_out[pos] = val;
       if (next_counts) {
-        const uint32_t next_digit = shift + 8 < 64 ? (uint32_t)((key >> (shift + 8)) & 0xff) : 0u;
-        atomicAdd(&next_counts[(int64_t)(pos >> tile_shift) * kRadix + next_digit], 1u);
+        const uint32_t next_digit = (uint32_t)(key >> next_shift) & next_mask;
+        atomicAdd(&next_counts[(int64_t)next_digit * stride + (pos >> tile_shift)], 1u);
       }
     }
     __syncthreads();
-    uint32_t slice_total = 0;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      slice_total += wave_count[w][t];
-      wave_count[w][t] = 0;
+    for (int d = 0; d < DPT; ++d) {
+      uint32_t slice_total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        slice_total += wave_count[w][t + d * kSortThreads];
+        wave_count[w][t + d * kSortThreads] = 0;
+      }
+      cursor[t + d * kSortThreads] += slice_total;
     }
-    cursor[t] += slice_total;
     __syncthreads();
   }
 }
@@ -144,37 +192,52 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
 
 size_t sort_temp_bytes(int64_t n) {
   SortPlan p = plan_sort(n);
-  return align_up((size_t)kMaxPasses * p.blocks * kRadix * sizeof(uint32_t), 256);
+  return align_up((size_t)kMaxPasses * (1 << kMaxDigitBits) * p.stride * sizeof(uint32_t), 256);
 }
 
-int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n,
-               int key_bits, void* temp, hipStream_t stream) {
+int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
+               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted) {
+  *keys_sorted = keys_in;
+  *vals_sorted = vals_in;
   if (n <= 0) return PBG_OK;
   if (n >= (int64_t)1 << 32)
     return fail(PBG_ERR_UNSUPPORTED, "sort_pairs: n=%lld does not fit 32-bit offsets", (long long)n);
+  if (low_bit < 0 || key_bits > 64 || low_bit > key_bits) return fail(PBG_ERR_INVALID, "sort_pairs: bad bit range");
   SortPlan p = plan_sort(n);
   uint32_t* counts = (uint32_t*)temp;
-  int passes = (key_bits + 7) / 8;
-  if (passes < 1) passes = 1;
-  // an odd number of ping-pong passes ends in the "out" buffers; pad an even
-  // count with one more pass over a zero digit
-  if (passes % 2 == 0) passes += 1;
+  int bits = key_bits - low_bit;
+  if (bits < 1) bits = 1;
+  const int passes = (bits + kMaxDigitBits - 1) / kMaxDigitBits;
   if (passes > kMaxPasses) return fail(PBG_ERR_INVALID, "sort_pairs: too many key bits");
-  hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kSortThreads), 0, stream, keys_in, n, p.tile_shift, passes,
-                     counts);
+  // digits of equal width, the last one possibly narrower; shifts stay below 64
+  const int width = (bits + passes - 1) / passes;
+  const int digits = 1 << width;
+  auto pass_bits = [&](int pass) { int left = bits - pass * width; return left < width ? left : width; };
+  hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kSortThreads), 0, stream, keys_in, n, p.tile_shift,
+                     low_bit, width, passes, p.stride, counts);
   uint64_t* ksrc = keys_in;
   uint32_t* vsrc = vals_in;
   uint64_t* kdst = keys_out;
   uint32_t* vdst = vals_out;
   for (int pass = 0; pass < passes; ++pass) {
-    const int shift = pass * 8;
-    uint32_t* cur = counts + (size_t)pass * p.blocks * kRadix;
-    uint32_t* next = (pass + 1 < passes) ? counts + (size_t)(pass + 1) * p.blocks * kRadix : nullptr;
-    hipLaunchKernelGGL(sort_scatter_kernel, dim3(p.blocks), dim3(kSortThreads), 0, stream, ksrc, vsrc, kdst, vdst, n,
-                       p.tile_shift, shift, cur, next);
+    const int shift = low_bit + pass * width;
+    const bool last = pass + 1 == passes;
+    uint32_t* cur = counts + (size_t)pass * digits * p.stride;
+    uint32_t* next = last ? nullptr : counts + (size_t)(pass + 1) * digits * p.stride;
+    const int nshift = last ? 0 : shift + width;
+    const int nbits = last ? 1 : pass_bits(pass + 1);
+    if (width <= 8) {
+      hipLaunchKernelGGL(sort_scatter_kernel<1>, dim3(p.blocks), dim3(kSortThreads), 0, stream, ksrc, vsrc, kdst, vdst,
+                         n, p.tile_shift, shift, pass_bits(pass), nshift, nbits, p.stride, cur, next);
+    } else {
+      hipLaunchKernelGGL(sort_scatter_kernel<2>, dim3(p.blocks), dim3(kSortThreads), 0, stream, ksrc, vsrc, kdst, vdst,
+                         n, p.tile_shift, shift, pass_bits(pass), nshift, nbits, p.stride, cur, next);
+    }
     uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
     uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
   }
+  *keys_sorted = ksrc;
+  *vals_sorted = vsrc;
   return check_launch("sort_pairs");
 }
 

@@ -263,12 +263,15 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   return sr;
 }
 
-// Loss of one positive against one side's nn negatives (one wave): adds the
-// unweighted per-lane loss partial to *loss_acc, overwrites the score row with
-// dLoss/dscore (l2: -2 dLoss/d squared distance) and returns the wave-reduced
-// dLoss/dpos, violator count and (l2) row sum of dLoss/d squared distance.
+// Loss of one positive against one side's nn negatives, computed by the group
+// of lanes R describes (a wave, or a quad); `first` is the lane's index in the
+// group.  Adds the unweighted per-lane loss partial to *loss_acc, overwrites the
+// score row with dLoss/dscore (l2: -2 dLoss/d squared distance) and returns the
+// group-reduced dLoss/dpos, violator count and (l2) row sum of dLoss/d squared
+// distance.
+template <class R>
 __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
-                                          float pos, float w, int lane, float* loss_acc, float* dpos_out,
+                                          float pos, float w, int first, float* loss_acc, float* dpos_out,
                                           int* viol_out, float* rowsum_out) {
   float dpos_part = 0.f, rowsum = 0.f;
   int viol = 0;
@@ -276,23 +279,23 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
   const float inv_nn = 1.0f / (float)nn;
   if (loss == PBG_LOSS_SOFTMAX) {
     bool live;
-    for (int j = lane; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
-    mx = wave_max(mx);
+    for (int j = first; j < nn; j += R::kStep) mx = fmaxf(mx, sr.at(j, &live));
+    mx = R::max(mx);
     float z = 0.f;
-    for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
-    z = wave_sum(z) + expf(pos - mx);
+    for (int j = first; j < nn; j += R::kStep) z += expf(sr.at(j, &live) - mx);
+    z = R::sum(z) + expf(pos - mx);
     inv_z = 1.0f / z;
-    if (lane == 0) {
+    if (first == 0) {
       *loss_acc += (mx + logf(z)) - pos;
       dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
     }
   } else if (loss == PBG_LOSS_LOGISTIC) {
-    if (lane == 0) {
+    if (first == 0) {
       *loss_acc += softplusf(-pos);
       dpos_part += (sigmoidf(pos) - 1.0f) * w;
     }
   }
-  for (int j = lane; j < nn; j += kWave) {
+  for (int j = first; j < nn; j += R::kStep) {
     bool live;
     const float t = sr.at(j, &live);
     float g;
@@ -321,12 +324,9 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
       out[j] = g;
     }
   }
-  *dpos_out = wave_sum(dpos_part);
-  *rowsum_out = wave_sum(rowsum);
-  int vtot = viol;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) vtot += __shfl_xor(vtot, off, 64);
-  *viol_out = vtot;
+  *dpos_out = R::sum(dpos_part);
+  *rowsum_out = R::sum(rowsum);
+  *viol_out = R::sum_int(viol);
 }
 
 __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     ScoreRow sr = score_row(c, s, kc, cc, i);
     float* out = sd.s + (kc * c.P + i) * nn;
     float rowsum;
-    side_loss(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum);
+    side_loss<WaveReduce>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum);
     if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = rowsum;
   }
   const float loss_row = wave_sum(loss_acc) * w;
@@ -683,161 +683,209 @@ constexpr int kFusedThreads = 512;
 struct FusedLayout {
   int ldx, lds;                  // row strides (floats) of the operand rows and of the score rows
   int xn[2], sc[2], sq[2], rs[2], cs[2], pos, dpos;  // offsets in floats
+  int part;                      // [2 sides][dLoss/dpos, weighted loss, violators][P] per-side results of the loss phase
+  int ids;                       // int32 row ids of the 2N operand rows (-1: padding); last block
   int total;                     // floats
 };
 
+template <int TN, int TD>  // column tiles of the score matrices (N / 16) and of the gradient matrices (D / 16)
 __global__ __launch_bounds__(kFusedThreads) void fused_chunk_kernel(StepCtx c, FusedLayout f) {
+  // All LDS accesses index `lds` directly (no pointer tables), so that they
+  // compile to ds_read / ds_write rather than flat accesses.
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // Everything indexed by the wave number or by a side must reach the kernel
+  // arguments through scalar registers (readfirstlane) or selects: a per-lane
+  // index into an argument array turns into a global load.
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t kc = blockIdx.x;
   const int k = (int)(kc / c.C), cc = (int)(kc % c.C);
   const int D = c.D, P = c.P, U = c.U, N = P + U, CP = c.C * c.P;
+  const int sq0 = f.sq[0], sq1 = f.sq[1], rs0 = f.rs[0], rs1 = f.rs[1], cs0 = f.cs[0], cs1 = f.cs[1];
+  const int ldx = f.ldx, lds_ = f.lds;
   const int valid = (cc == c.C - 1) ? c.last : P;
-  float* xn[2] = {lds + f.xn[0], lds + f.xn[1]};
-  float* sc[2] = {lds + f.sc[0], lds + f.sc[1]};
-  float* sq[2] = {lds + f.sq[0], lds + f.sq[1]};
-  float* rs[2] = {lds + f.rs[0], lds + f.rs[1]};
-  float* cs[2] = {lds + f.cs[0], lds + f.cs[1]};
-  float* pos_ = lds + f.pos;
-  float* dpos_ = lds + f.dpos;
+  const int xn0 = f.xn[0], xn1 = f.xn[1];  // operand rows of side 0 / 1: [N][ldx]
+  const int sc0 = f.sc[0], sc1 = f.sc[1];  // score rows against side 0 / 1's negatives: [P][lds_]
   const int64_t rel = clamp_index(c.rel[k], c.num_relations);
   const bool l2 = c.cmp == PBG_CMP_L2;
+  int* ids = reinterpret_cast<int*>(lds + f.ids);
 
-  // ---- phase 0: gather, operator, squared norms; clear the score matrices ----
-  for (int t = threadIdx.x; t < 2 * P * f.lds; t += kFusedThreads) sc[0][t] = 0.f;  // sc[1] follows sc[0]
-  for (int slot = wave; slot < 2 * N; slot += kFusedThreads / kWave) {
-    const int s = slot / N, j = slot % N;
-    const SideCtx& sd = c.side[s];
-    float* dst = xn[s] + j * f.ldx;
+  // ---- phase 0a: row ids and sort keys; clear operand and score storage ----
+  for (int t = threadIdx.x * 4; t < f.sq[0] - sc0; t += kFusedThreads * 4)  // both score blocks, pads included
+    *reinterpret_cast<float4*>(&lds[sc0 + t]) = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int t = threadIdx.x; t < f.ids - f.sq[0]; t += kFusedThreads) lds[f.sq[0] + t] = 0.f;
+  for (int t = threadIdx.x; t < 4 * ldx; t += kFusedThreads) lds[xn1 + N * ldx + t] = 0.f;  // slack rows read by the k loops
+  for (int slot = threadIdx.x; slot < 2 * N; slot += kFusedThreads) {
+    const int s = slot >= N, j = slot - s * N;
     int64_t id = -1, pair = 0;
+    bool real = true;  // false: a padded position of the last chunk
     if (j < P) {
       const int q = cc * P + j;
-      if (q < c.B) {
-        id = sd.idx[(int64_t)k * c.B + q];
-        pair = (int64_t)k * c.rk + sd.slot_pos + q;
+      real = q < c.B;
+      if (real) {
+        id = (s ? c.side[1].idx : c.side[0].idx)[(int64_t)k * c.B + q];
+        pair = (int64_t)k * c.rk + (s ? c.side[1].slot_pos : c.side[0].slot_pos) + q;
       }
     } else {
       const int u = j - P;
-      id = sd.uidx[kc * U + u];
-      pair = (int64_t)k * c.rk + sd.slot_uni + cc * U + u;
+      id = (s ? c.side[1].uidx : c.side[0].uidx)[kc * U + u];
+      pair = (int64_t)k * c.rk + (s ? c.side[1].slot_uni : c.side[0].slot_uni) + cc * U + u;
     }
-    const bool live = id >= 0;
-    if (live) id = clamp_index(id, sd.num_rows);
-    float sumsq = 0.f;
-    for (int d = lane; d < f.ldx; d += kWave) {
-      float v = 0.f;
-      if (live && d < D) {
-        v = sd.w[id * D + d];
-        if (s == 1 && c.op == PBG_OP_DIAGONAL) v = sd.p0[rel * D + d] * v;
-        else if (s == 1 && c.op == PBG_OP_TRANSLATION) v = v + sd.p0[rel * D + d];
-      }
-      dst[d] = v;
-      sumsq += v * v;
-    }
-    if (l2) {
-      const float nrm = sqrtf(wave_sum(sumsq));
-      if (lane == 0) sq[s][j] = nrm * nrm;
-    }
-    if (live && lane == 0) {
-      c.keys[pair] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
+    if (real) {
+      id = clamp_index(id, s ? c.side[1].num_rows : c.side[0].num_rows);
+      c.keys[pair] = ((uint64_t)((s ? c.side[1].key_base : c.side[0].key_base) + id) << c.kbits) | (uint64_t)k;
       c.vals[pair] = (uint32_t)pair;
+    }
+    ids[slot] = (int)id;
+  }
+  __syncthreads();
+
+  // ---- phase 0b: gather + operator into LDS; half a wave per row, 128-bit loads, all of a wave's rows in flight ----
+  {
+    constexpr int kPairs = 16;  // 8 waves x 16 x 2 half-waves = 256 >= 2N rows
+    const int half = lane >> 5, c4 = (lane & 31) << 2;
+    const bool col_ok = c4 < D;
+    float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c.op != PBG_OP_NONE && col_ok) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + c4);
+    float4 v[kPairs];
+    int idv[kPairs];
+#pragma unroll
+    for (int u = 0; u < kPairs; ++u) {  // all row ids first: one LDS round trip
+      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
+      const int id = ids[min(slot, 2 * N - 1)];
+      idv[u] = slot < 2 * N ? id : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kPairs; ++u) {
+      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
+      v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (idv[u] >= 0 && col_ok) {
+        const float* w = slot >= N ? c.side[1].w : c.side[0].w;
+        v[u] = *reinterpret_cast<const float4*>(w + (int64_t)idv[u] * D + c4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPairs; ++u) {
+      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
+      if (slot >= 2 * N) continue;  // uniform per half-wave; the reduction below stays inside a half
+      const int s = slot >= N, j = slot - s * N;
+      float4 y = v[u];
+      if (s == 1 && idv[u] >= 0) {
+        if (c.op == PBG_OP_DIAGONAL) {
+          y.x *= par.x; y.y *= par.y; y.z *= par.z; y.w *= par.w;
+        } else if (c.op == PBG_OP_TRANSLATION && col_ok) {
+          y.x += par.x; y.y += par.y; y.z += par.z; y.w += par.w;
+        }
+      }
+      if (c4 < ldx) *reinterpret_cast<float4*>(&lds[(s ? xn1 : xn0) + j * ldx + c4]) = y;  // pads get zeros
+      if (l2) {
+        const float sumsq = half_sum_at_31(y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w);
+        const float nrm = sqrtf(sumsq);
+        if ((lane & 31) == 31) lds[(s ? sq1 : sq0) + j] = nrm * nrm;
+      }
     }
   }
   __syncthreads();
 
   // ---- phase 1: S_s = A_(1-s) N_s^T ----
+  // Row / column indices past the matrix are clamped instead of guarded: they
+  // only feed output rows / columns that are never stored, and the loop body
+  // stays free of branches (loads of a k-step issue together, then the MFMAs).
   {
     const int s = wave >> 2, rt = wave & 3;
-    const int TN = (N + 15) >> 4;
     if (rt * 16 < P) {
-      float4v acc[8];
+      float4v acc[TN];
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const float* A = xn[1 - s];
-      const float* Bm = xn[s];
-      const int ar = rt * 16 + (lane & 15);
+      for (int ct = 0; ct < TN; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const int ar = min(rt * 16 + (lane & 15), P - 1);
+      const int a_at = (s ? xn0 : xn1) + ar * ldx + (lane >> 4);
+      int b_at[TN];
+#pragma unroll
+      for (int ct = 0; ct < TN; ++ct) b_at[ct] = (s ? xn1 : xn0) + min(ct * 16 + (lane & 15), N - 1) * ldx + (lane >> 4);
       const int ksteps = (D + 3) >> 2;
       for (int ks = 0; ks < ksteps; ++ks) {
-        const int kk = ks * 4 + (lane >> 4);
-        const float a = (ar < P) ? A[ar * f.ldx + kk] : 0.f;
+        const float a = lds[a_at + ks * 4];
+        float b[TN];
 #pragma unroll
-        for (int ct = 0; ct < 8; ++ct) {
-          if (ct < TN) {
-            const int br = ct * 16 + (lane & 15);
-            const float b = (br < N) ? Bm[br * f.ldx + kk] : 0.f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
-          }
-        }
+        for (int ct = 0; ct < TN; ++ct) b[ct] = lds[b_at[ct] + ks * 4];
+#pragma unroll
+        for (int ct = 0; ct < TN; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
       }
+      const int s_off = s ? sc1 : sc0;
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) {
-        if (ct < TN) {
-          const int col = ct * 16 + (lane & 15);
+      for (int ct = 0; ct < TN; ++ct) {
+        const int col = ct * 16 + (lane & 15);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int row = rt * 16 + 4 * (lane >> 4) + r;
-            if (row < P && col < N) sc[s][row * f.lds + col] = acc[ct][r];
-          }
+        for (int r = 0; r < 4; ++r) {
+          const int row = rt * 16 + 4 * (lane >> 4) + r;
+          if (row < P && col < N) lds[s_off + row * lds_ + col] = acc[ct][r];
         }
       }
     }
   }
   __syncthreads();
 
-  // ---- phase 2: loss, dLoss/dS in place ----
-  const float w_rel = c.rel_weights[rel];
-  for (int i = wave; i < P; i += kFusedThreads / kWave) {
-    const int q = cc * P + i;
-    const int64_t job = (int64_t)k * CP + q;
-    if (i >= valid) {  // padded positive: its score rows were cleared in phase 0 and phase 1 skipped nothing there
-      for (int j = lane; j < f.lds; j += kWave) {
-        sc[0][i * f.lds + j] = 0.f;
-        sc[1][i * f.lds + j] = 0.f;
+  // ---- phase 2: loss, dLoss/dS in place; one quad of lanes per (edge, side), columns interleaved ----
+  {
+    const int t = threadIdx.x, qd = t & 3;
+    if (t < 4 * P) {  // positive scores (model.py:177,207,267-274)
+      const int i = t >> 2;
+      float acc = 0.f;
+      for (int d = qd; d < D; d += 4) {
+        const float a = lds[xn0 + i * ldx + d], b = lds[xn1 + i * ldx + d];
+        acc += l2 ? (a - b) * (a - b) : a * b;
       }
-      if (lane == 0) {
-        rs[0][i] = rs[1][i] = 0.f;
-        pos_[i] = dpos_[i] = 0.f;
-        c.lossrow[job] = 0.f;
-        c.violrow[job * 2] = 0;
-        c.violrow[job * 2 + 1] = 0;
+      acc = quad_sum(acc);
+      if (qd == 0) lds[f.pos + i] = l2 ? -sqrtf(fmaxf(acc, 1e-30f)) : acc;
+    }
+    __syncthreads();
+    if (t < 8 * P) {
+      const int pair = t >> 2;
+      const int s = pair >= P, i = pair - s * P;
+      const int row_at = (s ? sc1 : sc0) + i * lds_;
+      float loss_w = 0.f, dpos_s = 0.f, rowsum = 0.f;
+      int viol = 0;
+      if (i >= valid) {  // padded positive: no loss, zero gradient rows
+        for (int j = qd; j < lds_; j += 4) lds[row_at + j] = 0.f;
+      } else {
+        float w = c.rel_weights[rel];
+        if (c.edge_weight) w *= c.edge_weight[(int64_t)k * c.B + cc * P + i];
+        ScoreRow sr;
+        sr.raw = lds + row_at;
+        sr.bn = lds + (s ? sq1 : sq0);
+        sr.a2 = l2 ? lds[(s ? sq0 : sq1) + i] : 0.f;
+        sr.cmp = c.cmp;
+        sr.nb = P;
+        sr.i = i;
+        sr.masked_from = valid;
+        float loss_acc = 0.f;
+        side_loss<QuadReduce>(c.loss, c.margin, c.cmp, sr, lds + row_at, N, lds[f.pos + i], w, qd, &loss_acc, &dpos_s,
+                              &viol, &rowsum);
+        loss_w = quad_sum(loss_acc) * w;
       }
-      continue;
+      if (qd == 0) {
+        lds[(s ? rs1 : rs0) + i] = rowsum;
+        lds[f.part + (s * 3 + 0) * P + i] = dpos_s;
+        lds[f.part + (s * 3 + 1) * P + i] = loss_w;
+        lds[f.part + (s * 3 + 2) * P + i] = __int_as_float(viol);
+      }
     }
-    const float posv = kappa(c.cmp, xn[0] + i * f.ldx, xn[1] + i * f.ldx, D, lane);
-    float w = w_rel;
-    if (c.edge_weight) w *= c.edge_weight[(int64_t)k * c.B + q];
-    float loss_acc = 0.f, dposv[2], rowsum[2];
-    int violv[2];
-    for (int s = 0; s < 2; ++s) {
-      ScoreRow sr;
-      sr.raw = sc[s] + i * f.lds;
-      sr.bn = sq[s];
-      sr.a2 = l2 ? sq[1 - s][i] : 0.f;
-      sr.cmp = c.cmp;
-      sr.nb = P;
-      sr.i = i;
-      sr.masked_from = valid;
-      side_loss(c.loss, c.margin, c.cmp, sr, sc[s] + i * f.lds, N, posv, w, lane, &loss_acc, &dposv[s], &violv[s],
-                &rowsum[s]);
-    }
-    const float loss_row = wave_sum(loss_acc) * w;
-    if (lane == 0) {
-      rs[0][i] = rowsum[0];
-      rs[1][i] = rowsum[1];
-      pos_[i] = posv;
-      dpos_[i] = dposv[0] + dposv[1];
-      c.lossrow[job] = loss_row;
-      c.violrow[job * 2] = violv[0];
-      c.violrow[job * 2 + 1] = violv[1];
+    __syncthreads();
+    if (t < P) {  // both sides of an edge together: statistics out, dLoss/dpos for phase 3
+      const int64_t job = (int64_t)k * CP + cc * P + t;
+      lds[f.dpos + t] = lds[f.part + 0 * P + t] + lds[f.part + 3 * P + t];
+      c.lossrow[job] = lds[f.part + 1 * P + t] + lds[f.part + 4 * P + t];
+      c.violrow[job * 2] = __float_as_int(lds[f.part + 2 * P + t]);
+      c.violrow[job * 2 + 1] = __float_as_int(lds[f.part + 5 * P + t]);
     }
   }
   __syncthreads();
   if (l2) {  // column sums of the stored -2 dLoss/dq
     for (int t = threadIdx.x; t < 2 * N; t += kFusedThreads) {
-      const int s = t / N, j = t % N;
+      const int s = t >= N, j = t - s * N;
+      const int s_off = s ? sc1 : sc0;
       float acc = 0.f;
-      for (int i = 0; i < P; ++i) acc += sc[s][i * f.lds + j];
-      cs[s][j] = acc;
+      for (int i = 0; i < P; ++i) acc += lds[s_off + i * lds_ + j];
+      lds[(s ? cs1 : cs0) + j] = acc;
     }
     __syncthreads();
   }
@@ -845,103 +893,100 @@ __global__ __launch_bounds__(kFusedThreads) void fused_chunk_kernel(StepCtx c, F
   // ---- phase 3: gradients of the 2(P+U) rows, written to HBM ----
   {
     const int m = wave >> 2, rt = wave & 3;  // m: side whose rows' gradients this wave forms
-    const int TD = (D + 15) >> 4;
     const SideCtx& sd = c.side[m];
-    const float* ds_a = sc[1 - m];  // scores in which this side's positives were the A operand
-    const float* ds_n = sc[m];      // scores against this side's negatives
-    const float* bx = xn[1 - m];    // the other side's rows: the B operand of every product here
+    const int dsa = m ? sc0 : sc1;  // scores in which this side's positives were the A operand
+    const int dsn = m ? sc1 : sc0;  // scores against this side's negatives
+    const int bx = m ? xn0 : xn1;   // the other side's rows: the B operand of every product here
+    const int xs = m ? xn1 : xn0;   // this side's rows
+    const int rs_o = m ? rs0 : rs1, cs_m = m ? cs1 : cs0;
     const bool has_op = m == 1 && c.op != PBG_OP_NONE;
     if (rt * 16 < P) {
-      float4v acc[8];
+      // The k index runs past N (resp. P) up to the next multiple of 4: the score
+      // blocks keep zero pad columns and zero pad rows there, so those terms vanish.
+      float4v acc[TD];
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const int ar = rt * 16 + (lane & 15);
-      for (int ks = 0; ks < ((N + 3) >> 2); ++ks) {  // dS_a (P x N) times the other side's N rows
-        const int kk = ks * 4 + (lane >> 4);
-        const float a = (ar < P && kk < N) ? ds_a[ar * f.lds + kk] : 0.f;
+      for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const int ar = min(rt * 16 + (lane & 15), P - 1);
+      const int b_at = bx + (lane >> 4) * ldx + (lane & 15);
+      {
+        const int a_at = dsa + ar * lds_ + (lane >> 4);
+        for (int ks = 0; ks < ((N + 3) >> 2); ++ks) {  // dS_a (P x N) times the other side's N rows
+          const float a = lds[a_at + ks * 4];
+          float b[TD];
 #pragma unroll
-        for (int ct = 0; ct < 8; ++ct) {
-          if (ct < TD) {
-            const int dc = ct * 16 + (lane & 15);
-            const float b = (kk < N && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
-          }
+          for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
+#pragma unroll
+          for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
         }
       }
-      for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {  // (dS_n[:, :P])^T (P x P) times the other side's positives
-        const int kk = ks * 4 + (lane >> 4);
-        const float a = (ar < P && kk < P) ? ds_n[kk * f.lds + ar] : 0.f;
+      {
+        const int a_at = dsn + (lane >> 4) * lds_ + ar;
+        for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {  // (dS_n[:, :P])^T (P x P) times the other side's positives
+          const float a = lds[a_at + ks * 4 * lds_];
+          float b[TD];
 #pragma unroll
-        for (int ct = 0; ct < 8; ++ct) {
-          if (ct < TD) {
-            const int dc = ct * 16 + (lane & 15);
-            const float b = (kk < P && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
-          }
+          for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
+#pragma unroll
+          for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
         }
       }
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) {
-        if (ct < TD) {
+      for (int r = 0; r < 4; ++r) {
+        const int i = rt * 16 + 4 * (lane >> 4) + r;
+        if (i >= valid) continue;
+        const int q = cc * P + i;
+        const float dpz = lds[f.dpos + i], pz = lds[f.pos + i];
+        const float coef = l2 ? 2.0f * lds[rs_o + i] - lds[cs_m + i] : 0.f;
+        const float pcoef = (l2 && pz * pz > 1e-30f) ? dpz / pz : 0.f;
+        float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
+        float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + q) * D : nullptr;
+#pragma unroll
+        for (int ct = 0; ct < TD; ++ct) {
           const int d = ct * 16 + (lane & 15);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int i = rt * 16 + 4 * (lane >> 4) + r;
-            if (i < valid && d < D) {
-              const float self = xn[m][i * f.ldx + d], other = bx[i * f.ldx + d];
-              float v = acc[ct][r];
-              if (l2) {
-                v += (2.0f * rs[1 - m][i] - cs[m][i]) * self;
-                const float pz = pos_[i];
-                if (pz * pz > 1e-30f) v += dpos_[i] / pz * (self - other);
-              } else {
-                v += dpos_[i] * other;
-              }
-              const int q = cc * P + i;
-              if (has_op) {
-                if (sd.dz) sd.dz[((int64_t)k * sd.op_rows + q) * D + d] = v;
-                if (c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
-              }
-              c.gr[((int64_t)k * c.rk + sd.slot_pos + q) * D + d] = v;
-            }
+          if (d < D) {
+            const float self = lds[xs + i * ldx + d], other = lds[bx + i * ldx + d];
+            float v = acc[ct][r];
+            if (l2) v += coef * self + pcoef * (self - other);
+            else v += dpz * other;
+            if (dzo) dzo[d] = v;
+            if (has_op && c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
+            out[d] = v;
           }
         }
       }
     }
     if (rt * 16 < U) {  // uniform negatives of side m: (dS_n[:, P:])^T (U x P) times the other side's positives
-      float4v acc[8];
+      float4v acc[TD];
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const int au = rt * 16 + (lane & 15);
+      for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      const int au = min(rt * 16 + (lane & 15), U - 1);
+      const int a_at = dsn + (lane >> 4) * lds_ + P + au;
+      const int b_at = bx + (lane >> 4) * ldx + (lane & 15);
       for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {
-        const int kk = ks * 4 + (lane >> 4);
-        const float a = (au < U && kk < P) ? ds_n[kk * f.lds + P + au] : 0.f;
+        const float a = lds[a_at + ks * 4 * lds_];
+        float b[TD];
 #pragma unroll
-        for (int ct = 0; ct < 8; ++ct) {
-          if (ct < TD) {
-            const int dc = ct * 16 + (lane & 15);
-            const float b = (kk < P && dc < f.ldx) ? bx[kk * f.ldx + dc] : 0.f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
-          }
-        }
+        for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
+#pragma unroll
+        for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
       }
 #pragma unroll
-      for (int ct = 0; ct < 8; ++ct) {
-        if (ct < TD) {
-          const int d = ct * 16 + (lane & 15);
+      for (int r = 0; r < 4; ++r) {
+        const int u = rt * 16 + 4 * (lane >> 4) + r;
+        if (u >= U) continue;
+        const int r2 = cc * U + u;
+        const float coef = l2 ? lds[cs_m + P + u] : 0.f;
+        float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
+        float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D : nullptr;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int u = rt * 16 + 4 * (lane >> 4) + r;
-            if (u < U && d < D) {
-              float v = acc[ct][r];
-              if (l2) v -= cs[m][P + u] * xn[m][(P + u) * f.ldx + d];
-              const int r2 = cc * U + u;
-              if (has_op) {
-                if (sd.dz) sd.dz[((int64_t)k * sd.op_rows + c.B + r2) * D + d] = v;
-                if (c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
-              }
-              c.gr[((int64_t)k * c.rk + sd.slot_uni + r2) * D + d] = v;
-            }
+        for (int ct = 0; ct < TD; ++ct) {
+          const int d = ct * 16 + (lane & 15);
+          if (d < D) {
+            float v = acc[ct][r];
+            if (l2) v -= coef * lds[xs + (P + u) * ldx + d];
+            if (dzo) dzo[d] = v;
+            if (has_op && c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
+            out[d] = v;
           }
         }
       }
@@ -961,7 +1006,8 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.dynamic) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2) return false;
-  if (c.D > 128 || c.P > 64 || c.U > 64) return false;
+  if (c.D > 128 || c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
+  if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;
   for (int s = 0; s < 2; ++s)
     if (c.side[s].nb != c.P || c.side[s].u != c.U) return false;
   const int N = c.P + c.U;
@@ -969,16 +1015,18 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   f->lds = lds_stride(N);
   int off = 0;
   auto take = [&](int count) { int o = off; off += (count + 3) / 4 * 4; return o; };
+  const int p4 = (c.P + 3) / 4 * 4;
   f->xn[0] = take(N * f->ldx);
-  f->xn[1] = take(N * f->ldx + 16);
-  f->sc[0] = take(c.P * f->lds);
-  f->sc[1] = take(c.P * f->lds + 16);
-  if (f->sc[1] != f->sc[0] + c.P * f->lds) return false;  // phase 0 clears both as one block
+  f->xn[1] = take(N * f->ldx + 4 * f->ldx);  // slack: k-steps and column tiles may read past the last row
+  f->sc[0] = take(p4 * f->lds);              // pad rows and pad columns stay zero
+  f->sc[1] = take(p4 * f->lds + 4 * f->lds);
   for (int s = 0; s < 2; ++s) f->sq[s] = take(N);
   for (int s = 0; s < 2; ++s) f->rs[s] = take(c.P);
   for (int s = 0; s < 2; ++s) f->cs[s] = take(N);
   f->pos = take(c.P);
   f->dpos = take(c.P);
+  f->part = take(6 * c.P);
+  f->ids = take(2 * N);
   f->total = off;
   return (size_t)off * sizeof(float) <= 160 * 1024 - 512;
 }
@@ -1541,8 +1589,10 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
     const int64_t ne = (int64_t)K * c.B;
     hipLaunchKernelGGL(rel_keys_kernel, dim3((unsigned)ceil_div(ne, 256)), dim3(256), 0, stream, c, plan.rkeys_a,
                        plan.rvals_a);
-    rc = sort_pairs(plan.rkeys_a, plan.rvals_a, plan.rkeys_b, plan.rvals_b, ne,
-                    bits_for((uint64_t)(c.num_relations - 1)) + c.kbits, plan.rsort_temp, stream);
+    uint64_t* rkeys;  // the edges arrive in batch order, so sorting on the relation bits orders by (relation, batch)
+    uint32_t* rvals;
+    rc = sort_pairs(plan.rkeys_a, plan.rvals_a, plan.rkeys_b, plan.rvals_b, ne, c.kbits,
+                    bits_for((uint64_t)(c.num_relations - 1)) + c.kbits, plan.rsort_temp, stream, &rkeys, &rvals);
     if (rc != PBG_OK) return rc;
     for (int s = 0; s < 2; ++s) {
       float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
@@ -1553,10 +1603,10 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
         hipLaunchKernelGGL(dyn_linear_backward_kernel, wave_grid(ne), dim3(kRowThreads), 0, stream, c, s);
         const int tiles = (D + 63) / 64;
         hipLaunchKernelGGL(dyn_linear_param_kernel, dim3((unsigned)ne, (unsigned)(tiles * tiles)), dim3(256), 0, stream,
-                           c, s, plan.rkeys_b, plan.rvals_b, p0, s0, d->relation_lr);
+                           c, s, rkeys, rvals, p0, s0, d->relation_lr);
       } else {
         hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
-                           plan.rkeys_b, plan.rvals_b, p0, p1, s0, s1, d->relation_lr);
+                           rkeys, rvals, p0, p1, s0, s1, d->relation_lr);
       }
     }
     return check_launch("step params (dynamic)");
@@ -1622,14 +1672,20 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
     const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
-    static size_t lds_allowed = 0;
-    if (lds_bytes > lds_allowed) {
-      if (hipFuncSetAttribute((const void*)fused_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)lds_bytes) != hipSuccess)
+    const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
+    const void* fn = small_tiles ? (const void*)fused_chunk_kernel<7, 7> : (const void*)fused_chunk_kernel<8, 8>;
+    static size_t lds_allowed[2] = {0, 0};
+    if (lds_bytes > lds_allowed[small_tiles]) {
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
         return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
-      lds_allowed = lds_bytes;
+      lds_allowed[small_tiles] = lds_bytes;
     }
-    hipLaunchKernelGGL(fused_chunk_kernel, dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c, plan.fl);
+    if (small_tiles)
+      hipLaunchKernelGGL((fused_chunk_kernel<7, 7>), dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c,
+                         plan.fl);
+    else
+      hipLaunchKernelGGL((fused_chunk_kernel<8, 8>), dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c,
+                         plan.fl);
     mark(1);
     mark(2);
     mark(3);
@@ -1659,14 +1715,18 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   mark(8);
   const int64_t npairs = (int64_t)c.K * c.rk;
   const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
-  rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, bits_for(rows - 1) + c.kbits, plan.sort_temp, s);
+  // gradient rows are numbered batch by batch, so a stable sort on the row bits alone orders them by (row, batch)
+  uint64_t* skeys;
+  uint32_t* svals;
+  rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, bits_for(rows - 1) + c.kbits,
+                  plan.sort_temp, s, &skeys, &svals);
   if (rc != PBG_OK) return rc;
   mark(9);
   if (desc->shared_table) {
-    rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
+    rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s);
   } else {
-    rc = row_adagrad_sorted(plan.keys_b, plan.vals_b, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
+    rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s);
   }
   mark(10);
