@@ -677,167 +677,353 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
 // place in LDS; phase 3 forms the four gradient matrices
 //   dL = dS_R N_R + dS_L[:, :P]^T R      dU_L = dS_L[:, P:]^T R     (and L <-> R)
 // with MFMA straight from LDS and writes the raw-row gradients to HBM.
+//
+// The kernel is instantiated per comparator and loss and keeps its straight-line
+// parts short: a workgroup runs every instruction once, so code that does not
+// fit the instruction cache is paid for in fetch stalls by every workgroup.
 typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kFusedThreads = 512;
+constexpr int kFusedIds = 256;  // slots of the row id array: 8 waves x 16 rounds x 2 half-waves
+constexpr int kQuadCols = 32;   // score columns per lane of a quad: N <= 128
 
 struct FusedLayout {
   int ldx, lds;                  // row strides (floats) of the operand rows and of the score rows
   int xn[2], sc[2], sq[2], rs[2], cs[2], pos, dpos;  // offsets in floats
   int part;                      // [2 sides][dLoss/dpos, weighted loss, violators][P] per-side results of the loss phase
-  int ids;                       // int32 row ids of the 2N operand rows (-1: padding); last block
+  int ids;                       // int32 row ids of the 2N operand rows (-1: padding), kFusedIds slots; last block
   int total;                     // floats
 };
 
-template <int TN, int TD>  // column tiles of the score matrices (N / 16) and of the gradient matrices (D / 16)
-__global__ __launch_bounds__(kFusedThreads) void fused_chunk_kernel(StepCtx c, FusedLayout f) {
-  // All LDS accesses index `lds` directly (no pointer tables), so that they
-  // compile to ds_read / ds_write rather than flat accesses.
-  extern __shared__ __attribute__((aligned(16))) float lds[];
-  // Everything indexed by the wave number or by a side must reach the kernel
-  // arguments through scalar registers (readfirstlane) or selects: a per-lane
-  // index into an argument array turns into a global load.
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t kc = blockIdx.x;
-  const int k = (int)(kc / c.C), cc = (int)(kc % c.C);
-  const int D = c.D, P = c.P, U = c.U, N = P + U, CP = c.C * c.P;
-  const int sq0 = f.sq[0], sq1 = f.sq[1], rs0 = f.rs[0], rs1 = f.rs[1], cs0 = f.cs[0], cs1 = f.cs[1];
-  const int ldx = f.ldx, lds_ = f.lds;
-  const int valid = (cc == c.C - 1) ? c.last : P;
-  const int xn0 = f.xn[0], xn1 = f.xn[1];  // operand rows of side 0 / 1: [N][ldx]
-  const int sc0 = f.sc[0], sc1 = f.sc[1];  // score rows against side 0 / 1's negatives: [P][lds_]
-  const int64_t rel = clamp_index(c.rel[k], c.num_relations);
-  const bool l2 = c.cmp == PBG_CMP_L2;
-  int* ids = reinterpret_cast<int*>(lds + f.ids);
+// Loss of one positive against one side's N negatives for a score row held in
+// LDS and spread over the four lanes of a quad (lane qd owns columns qd, qd + 4,
+// ...).  The lane's columns live in registers from the first read on, so the LDS
+// latency is paid once and the passes of the softmax run over registers.
+// Columns at or past N act as scores of -inf: they add nothing to any loss and
+// are never written back.  Overwrites the row with dLoss/dscore (l2: -2 dLoss/d
+// squared distance); the outputs are quad-reduced.
+template <int CMP, int LOSS>
+__device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at, float a2, float margin, int N, int nb,
+                                               int i, int masked_from, float pos, float w, int qd, float* loss_w,
+                                               float* dpos_out, int* viol_out, float* rowsum_out) {
+  constexpr bool l2 = CMP == PBG_CMP_L2;
+  float t[kQuadCols];
+  uint32_t live = 0xffffffffu;  // bit e clear: column qd + 4e is a constant with no gradient
+#pragma unroll
+  for (int e = 0; e < kQuadCols; ++e) t[e] = lds[row_at + min(qd + 4 * e, N - 1)];
+  if (l2) {
+#pragma unroll
+    for (int e = 0; e < kQuadCols; ++e) {
+      const float q = fmaf(-2.0f, t[e], lds[bn_at + min(qd + 4 * e, N - 1)]) + a2;
+      if (!(q >= 1e-30f)) live &= ~(1u << e);
+      t[e] = -sqrtf(fmaxf(q, 1e-30f));
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kQuadCols; ++e) {
+    const int j = qd + 4 * e;
+    if (j < nb && (j == i || j >= masked_from)) {
+      t[e] = -1e9f;
+      live &= ~(1u << e);
+    }
+    if (j >= N) {
+      t[e] = -INFINITY;
+      live &= ~(1u << e);
+    }
+  }
+  float loss_acc = 0.f, dpos_part = 0.f, rowsum = 0.f, mx = pos, inv_z = 0.f;
+  int viol = 0;
+  const float inv_nn = 1.0f / (float)N;
+  if (LOSS == PBG_LOSS_SOFTMAX) {
+#pragma unroll
+    for (int e = 0; e < kQuadCols; ++e) mx = fmaxf(mx, t[e]);
+    mx = quad_max(mx);
+    float z = 0.f;
+#pragma unroll
+    for (int e = 0; e < kQuadCols; ++e) z += expf(t[e] - mx);
+    z = quad_sum(z) + expf(pos - mx);
+    inv_z = 1.0f / z;
+    if (qd == 0) {
+      loss_acc += (mx + logf(z)) - pos;
+      dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+    }
+  } else if (LOSS == PBG_LOSS_LOGISTIC) {
+    if (qd == 0) {
+      loss_acc += softplusf(-pos);
+      dpos_part += (sigmoidf(pos) - 1.0f) * w;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kQuadCols; ++e) {
+    const int j = qd + 4 * e;
+    const float te = t[e];
+    float g;
+    if (LOSS == PBG_LOSS_RANKING) {
+      // F.margin_ranking_loss(neg, pos, target=-1): max(0, (t - pos) + margin); the
+      // clamp lets the gradient through at exactly 0
+      const float x = (te - pos) + margin;
+      if (x > 0.f) loss_acc += x;
+      g = (x >= 0.f) ? w : 0.f;
+      dpos_part -= g;
+    } else if (LOSS == PBG_LOSS_LOGISTIC) {
+      loss_acc += softplusf(te) * inv_nn;
+      g = sigmoidf(te) * inv_nn * w;
+    } else {
+      g = expf(te - mx) * inv_z * w;
+    }
+    if (te > pos) ++viol;
+    const bool lv = (live >> e) & 1u;
+    if (!lv) g = 0.f;
+    if (l2) {
+      // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq so that the
+      // backward products give the cross terms of ||a||^2 - 2ab + ||b||^2
+      const float dq = lv ? g * 0.5f / te : 0.f;
+      rowsum += dq;
+      g = -2.0f * dq;
+    }
+    if (j < N) lds[row_at + j] = g;
+  }
+  *loss_w = quad_sum(loss_acc) * w;
+  *dpos_out = quad_sum(dpos_part);
+  *rowsum_out = quad_sum(rowsum);
+  *viol_out = quad_sum_int(viol);
+}
 
-  // ---- phase 0a: row ids and sort keys; clear operand and score storage ----
-  for (int t = threadIdx.x * 4; t < f.sq[0] - sc0; t += kFusedThreads * 4)  // both score blocks, pads included
-    *reinterpret_cast<float4*>(&lds[sc0 + t]) = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int t = threadIdx.x; t < f.ids - f.sq[0]; t += kFusedThreads) lds[f.sq[0] + t] = 0.f;
-  for (int t = threadIdx.x; t < 4 * ldx; t += kFusedThreads) lds[xn1 + N * ldx + t] = 0.f;  // slack rows read by the k loops
-  for (int slot = threadIdx.x; slot < 2 * N; slot += kFusedThreads) {
-    const int s = slot >= N, j = slot - s * N;
-    int64_t id = -1, pair = 0;
-    bool real = true;  // false: a padded position of the last chunk
-    if (j < P) {
-      const int q = cc * P + j;
+// acc[ct] += A(16 x 4 per k-step, element (lane & 15, lane >> 4) at a_at + ks * a_step)
+//          * B(4 x 16 per column tile, at b_at + ks * b_step + ct * b_tile)
+// over `ksteps` k-steps; the operands of the next k-step are in flight while the
+// MFMAs of the current one issue.  Reads one k-step past the end (the caller's
+// buffers keep slack there).
+template <int T>
+__device__ __forceinline__ void mfma_sweep(const float* lds, int a_at, int a_step, int b_at, int b_step, int b_tile,
+                                           int ksteps, float4v* acc) {
+  float a = lds[a_at];
+  float b[T];
+#pragma unroll
+  for (int ct = 0; ct < T; ++ct) b[ct] = lds[b_at + ct * b_tile];
+  for (int ks = 0; ks < ksteps; ++ks) {
+    a_at += a_step;
+    b_at += b_step;
+    const float an = lds[a_at];
+    float bn[T];
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) bn[ct] = lds[b_at + ct * b_tile];
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
+    a = an;
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) b[ct] = bn[ct];
+  }
+}
+
+// Geometry of one chunk, the same for both roles.
+struct FusedGeom {
+  int D, P, U, N, ldx, lds, xn0, xn1, sc0, sc1, sq0, sq1, rs0, rs1, cs0, cs1;
+};
+
+// ---- loader role: waves 8..15 ----
+// Row ids and sort keys of chunk kc; thread t < kFusedIds owns slot t of the id array.
+__device__ __forceinline__ void fused_load_ids(const StepCtx& c, const FusedGeom& g, int64_t kc, int t, int* ids) {
+  if (t >= kFusedIds) return;
+  const int k = (int)(kc / c.C), cc = (int)(kc % c.C);
+  const int slot = t;
+  const int s = slot >= g.N, j = slot - s * g.N;
+  int64_t id = -1, pair = 0;
+  bool real = slot < 2 * g.N;  // false: a slot past the operand rows or a padded position of the last chunk
+  if (real) {
+    if (j < g.P) {
+      const int q = cc * g.P + j;
       real = q < c.B;
       if (real) {
         id = (s ? c.side[1].idx : c.side[0].idx)[(int64_t)k * c.B + q];
         pair = (int64_t)k * c.rk + (s ? c.side[1].slot_pos : c.side[0].slot_pos) + q;
       }
     } else {
-      const int u = j - P;
-      id = (s ? c.side[1].uidx : c.side[0].uidx)[kc * U + u];
-      pair = (int64_t)k * c.rk + (s ? c.side[1].slot_uni : c.side[0].slot_uni) + cc * U + u;
+      const int u = j - g.P;
+      id = (s ? c.side[1].uidx : c.side[0].uidx)[kc * g.U + u];
+      pair = (int64_t)k * c.rk + (s ? c.side[1].slot_uni : c.side[0].slot_uni) + cc * g.U + u;
     }
-    if (real) {
-      id = clamp_index(id, s ? c.side[1].num_rows : c.side[0].num_rows);
-      c.keys[pair] = ((uint64_t)((s ? c.side[1].key_base : c.side[0].key_base) + id) << c.kbits) | (uint64_t)k;
-      c.vals[pair] = (uint32_t)pair;
-    }
-    ids[slot] = (int)id;
   }
-  __syncthreads();
+  if (real) {
+    id = clamp_index(id, s ? c.side[1].num_rows : c.side[0].num_rows);
+    c.keys[pair] = ((uint64_t)((s ? c.side[1].key_base : c.side[0].key_base) + id) << c.kbits) | (uint64_t)k;
+    c.vals[pair] = (uint32_t)pair;
+  }
+  ids[slot] = (int)id;
+}
 
-  // ---- phase 0b: gather + operator into LDS; half a wave per row, 128-bit loads, all of a wave's rows in flight ----
-  {
-    constexpr int kPairs = 16;  // 8 waves x 16 x 2 half-waves = 256 >= 2N rows
-    const int half = lane >> 5, c4 = (lane & 31) << 2;
-    const bool col_ok = c4 < D;
-    float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (c.op != PBG_OP_NONE && col_ok) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + c4);
-    float4 v[kPairs];
-    int idv[kPairs];
+constexpr int kFusedRounds = kFusedIds / 16;  // rows per half-wave of the 8 loader waves
+
+// Half a wave per row, 128-bit loads, all of a wave's rows in flight.
+__device__ __forceinline__ void fused_issue_rows(const StepCtx& c, const FusedGeom& g, const int* ids, int lwave, int lane,
+                                                 float4* v, int* idv) {
+  const int half = lane >> 5, c4 = (lane & 31) << 2;
+  const int slot0 = half * 8 + lwave;  // this half-wave's rows: slot0 + 16 u
 #pragma unroll
-    for (int u = 0; u < kPairs; ++u) {  // all row ids first: one LDS round trip
-      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
-      const int id = ids[min(slot, 2 * N - 1)];
-      idv[u] = slot < 2 * N ? id : -1;
+  for (int u = 0; u < kFusedRounds; ++u) idv[u] = ids[slot0 + 16 * u];
+#pragma unroll
+  for (int u = 0; u < kFusedRounds; ++u) {
+    v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (idv[u] >= 0 && c4 < g.D) {
+      const float* w = slot0 + 16 * u >= g.N ? c.side[1].w : c.side[0].w;
+      v[u] = *reinterpret_cast<const float4*>(w + (int64_t)idv[u] * g.D + c4);
     }
+  }
+}
+
+// Operator (rhs side) and, for l2, the squared norms; rows land in LDS.
+template <int CMP>
+__device__ __forceinline__ void fused_store_rows(const StepCtx& c, const FusedGeom& g, float* lds, int64_t rel, int lwave,
+                                                 int lane, const float4* v, const int* idv) {
+  const int half = lane >> 5, c4 = (lane & 31) << 2;
+  const bool col_ok = c4 < g.D;
+  float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (c.op != PBG_OP_NONE && col_ok) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * g.D + c4);
+  const int slot0 = half * 8 + lwave;
 #pragma unroll
-    for (int u = 0; u < kPairs; ++u) {
-      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
-      v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (idv[u] >= 0 && col_ok) {
-        const float* w = slot >= N ? c.side[1].w : c.side[0].w;
-        v[u] = *reinterpret_cast<const float4*>(w + (int64_t)idv[u] * D + c4);
+  for (int u = 0; u < kFusedRounds; ++u) {
+    const int slot = slot0 + 16 * u;
+    if (slot >= 2 * g.N) break;  // uniform per half-wave; the reduction below stays inside a half
+    const int s = slot >= g.N, j = slot - s * g.N;
+    float4 y = v[u];
+    if (s == 1 && idv[u] >= 0) {
+      if (c.op == PBG_OP_DIAGONAL) {
+        y.x *= par.x; y.y *= par.y; y.z *= par.z; y.w *= par.w;
+      } else if (c.op == PBG_OP_TRANSLATION && col_ok) {
+        y.x += par.x; y.y += par.y; y.z += par.z; y.w += par.w;
       }
     }
+    if (c4 < g.ldx) *reinterpret_cast<float4*>(&lds[(s ? g.xn1 : g.xn0) + j * g.ldx + c4]) = y;  // pads get zeros
+    if (CMP == PBG_CMP_L2) {
+      const float sumsq = half_sum_at_31(y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w);
+      const float nrm = sqrtf(sumsq);
+      if ((lane & 31) == 31) lds[(s ? g.sq1 : g.sq0) + j] = nrm * nrm;
+    }
+  }
+}
+
+// Persistent kernel: workgroup b takes chunks b, b + gridDim.x, ...  Waves 0..7
+// compute (phases 1-3); waves 8..15 load: while chunk n is being computed they
+// fetch the ids of chunk n + 1 and hold its rows in registers, and as soon as
+// phase 3 of chunk n has let go of the operand rows they write them to LDS.  The
+// two roles run different code between the same sequence of barriers.
+template <int TN, int TD, int CMP, int LOSS>  // column tiles of the score matrices (N / 16) and of the gradient matrices (D / 16)
+__global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
+  // All LDS accesses index `lds` directly (no pointer tables), so that they
+  // compile to ds_read / ds_write rather than flat accesses.  Everything indexed
+  // by the wave number or by a side reaches the kernel arguments through scalar
+  // registers (readfirstlane) or selects: a per-lane index into an argument
+  // array turns into a global load.
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr bool l2 = CMP == PBG_CMP_L2;
+  const int lane = threadIdx.x & 63;
+  const int wave16 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = wave16 & 7, tid = threadIdx.x & (kFusedThreads - 1);
+  FusedGeom g;
+  g.D = c.D; g.P = c.P; g.U = c.U; g.N = c.P + c.U; g.ldx = f.ldx; g.lds = f.lds;
+  g.xn0 = f.xn[0]; g.xn1 = f.xn[1];  // operand rows of side 0 / 1: [N][ldx]
+  g.sc0 = f.sc[0]; g.sc1 = f.sc[1];  // score rows against side 0 / 1's negatives: [P][lds]
+  g.sq0 = f.sq[0]; g.sq1 = f.sq[1]; g.rs0 = f.rs[0]; g.rs1 = f.rs[1]; g.cs0 = f.cs[0]; g.cs1 = f.cs[1];
+  const int D = g.D, P = g.P, U = g.U, N = g.N, ldx = g.ldx, lds_ = g.lds, CP = c.C * c.P;
+  const int xn0 = g.xn0, xn1 = g.xn1, sc0 = g.sc0, sc1 = g.sc1;
+  int* ids = reinterpret_cast<int*>(lds + f.ids);
+
+  if (wave16 >= 8) {
+    // ================= loader role =================
+    float4 v[kFusedRounds];
+    int idv[kFusedRounds];
+    fused_load_ids(c, g, blockIdx.x, tid, ids);
+    __syncthreads();  // ids visible; the compute waves have cleared the storage behind the operand rows
+    fused_issue_rows(c, g, ids, wave, lane, v, idv);
+    for (int64_t kc = blockIdx.x; kc < num_chunks; kc += gridDim.x) {
+      const int64_t kn = kc + gridDim.x;
+      const int64_t rel = clamp_index(c.rel[kc / c.C], c.num_relations);
+      // The thread-to-cell mapping is the same for every chunk; hiding the thread's
+      // indices from the optimiser once per chunk keeps it from hoisting every
+      // address of the loop body into registers that stay live (and spill).
+      int ln = lane, t = tid;
+      asm volatile("" : "+v"(ln), "+v"(t));
+      fused_store_rows<CMP>(c, g, lds, rel, wave, ln, v, idv);
+      __syncthreads();  // (a) operand rows of chunk kc in LDS
+      if (kn < num_chunks) fused_load_ids(c, g, kn, t, ids);
+      __syncthreads();  // (b)
+      __syncthreads();  // (c)
+      __syncthreads();  // (d)
+      __syncthreads();  // (e)
+      __syncthreads();  // (f)
+      // Issued here, the loads have the whole of phase 3 (no barriers inside) to
+      // enter the memory pipeline; issued earlier, the loader waves would sit in
+      // the issue queue and hold up the barriers of the loss phase.
+      if (kn < num_chunks) fused_issue_rows(c, g, ids, wave, ln, v, idv);
+      __syncthreads();  // (g) phase 3 has let go of the operand rows
+    }
+    return;
+  }
+
+  // ================= compute role =================
+  for (int t = tid * 4; t < f.ids - sc0; t += kFusedThreads * 4)  // score blocks (pads included), small arrays
+    *reinterpret_cast<float4*>(&lds[sc0 + t]) = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int t = tid; t < 4 * ldx; t += kFusedThreads) lds[xn1 + N * ldx + t] = 0.f;  // slack rows read by the k loops
+  __syncthreads();
+  // Pad rows and pad columns of the score blocks are never written again, and
+  // every other cell is rewritten by each chunk before it is read.
+
+  for (int64_t kc = blockIdx.x; kc < num_chunks; kc += gridDim.x) {
+    const int k = (int)(kc / c.C), cc = (int)(kc % c.C);
+    const int valid = (cc == c.C - 1) ? c.last : P;
+    const int64_t rel = clamp_index(c.rel[k], c.num_relations);
+    int lane_ = threadIdx.x & 63, t = tid;  // opaque per chunk, see the loader loop
+    asm volatile("" : "+v"(lane_), "+v"(t));
+    __syncthreads();  // (a)
+
+    // ---- phase 1: S_s = A_(1-s) N_s^T ----
+    // Row / column indices past the matrix are clamped or left to run into the
+    // storage behind it instead of guarded: they only feed output rows / columns
+    // that are never stored, and the loop body stays free of branches.
+    {
+      const int s = wave >> 2, rt = wave & 3;
+      if (rt * 16 < P) {
+        float4v acc[TN];
 #pragma unroll
-    for (int u = 0; u < kPairs; ++u) {
-      const int slot = (u * 2 + half) * (kFusedThreads / kWave) + wave;
-      if (slot >= 2 * N) continue;  // uniform per half-wave; the reduction below stays inside a half
-      const int s = slot >= N, j = slot - s * N;
-      float4 y = v[u];
-      if (s == 1 && idv[u] >= 0) {
-        if (c.op == PBG_OP_DIAGONAL) {
-          y.x *= par.x; y.y *= par.y; y.z *= par.z; y.w *= par.w;
-        } else if (c.op == PBG_OP_TRANSLATION && col_ok) {
-          y.x += par.x; y.y += par.y; y.z += par.z; y.w += par.w;
+        for (int ct = 0; ct < TN; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+        const int ar = min(rt * 16 + (lane_ & 15), P - 1);
+        const int a_at = (s ? xn0 : xn1) + ar * ldx + (lane_ >> 4);
+        const int b_at = (s ? xn1 : xn0) + (lane_ & 15) * ldx + (lane_ >> 4);  // column tile ct: 16 rows further down
+        mfma_sweep<TN>(lds, a_at, 4, b_at, 4, 16 * ldx, (D + 3) >> 2, acc);
+        const int s_off = s ? sc1 : sc0;
+#pragma unroll
+        for (int ct = 0; ct < TN; ++ct) {
+          const int col = ct * 16 + (lane_ & 15);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = rt * 16 + 4 * (lane_ >> 4) + r;
+            if (row < P && col < N) lds[s_off + row * lds_ + col] = acc[ct][r];
+          }
         }
       }
-      if (c4 < ldx) *reinterpret_cast<float4*>(&lds[(s ? xn1 : xn0) + j * ldx + c4]) = y;  // pads get zeros
-      if (l2) {
-        const float sumsq = half_sum_at_31(y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w);
-        const float nrm = sqrtf(sumsq);
-        if ((lane & 31) == 31) lds[(s ? sq1 : sq0) + j] = nrm * nrm;
-      }
     }
-  }
-  __syncthreads();
+    __syncthreads();  // (b)
 
-  // ---- phase 1: S_s = A_(1-s) N_s^T ----
-  // Row / column indices past the matrix are clamped instead of guarded: they
-  // only feed output rows / columns that are never stored, and the loop body
-  // stays free of branches (loads of a k-step issue together, then the MFMAs).
-  {
-    const int s = wave >> 2, rt = wave & 3;
-    if (rt * 16 < P) {
-      float4v acc[TN];
-#pragma unroll
-      for (int ct = 0; ct < TN; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const int ar = min(rt * 16 + (lane & 15), P - 1);
-      const int a_at = (s ? xn0 : xn1) + ar * ldx + (lane >> 4);
-      int b_at[TN];
-#pragma unroll
-      for (int ct = 0; ct < TN; ++ct) b_at[ct] = (s ? xn1 : xn0) + min(ct * 16 + (lane & 15), N - 1) * ldx + (lane >> 4);
-      const int ksteps = (D + 3) >> 2;
-      for (int ks = 0; ks < ksteps; ++ks) {
-        const float a = lds[a_at + ks * 4];
-        float b[TN];
-#pragma unroll
-        for (int ct = 0; ct < TN; ++ct) b[ct] = lds[b_at[ct] + ks * 4];
-#pragma unroll
-        for (int ct = 0; ct < TN; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
-      }
-      const int s_off = s ? sc1 : sc0;
-#pragma unroll
-      for (int ct = 0; ct < TN; ++ct) {
-        const int col = ct * 16 + (lane & 15);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = rt * 16 + 4 * (lane >> 4) + r;
-          if (row < P && col < N) lds[s_off + row * lds_ + col] = acc[ct][r];
-        }
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- phase 2: loss, dLoss/dS in place; one quad of lanes per (edge, side), columns interleaved ----
-  {
-    const int t = threadIdx.x, qd = t & 3;
+    // ---- phase 2: loss, dLoss/dS in place; one quad of lanes per (edge, side), columns interleaved ----
+    const int qd = t & 3;
     if (t < 4 * P) {  // positive scores (model.py:177,207,267-274)
       const int i = t >> 2;
       float acc = 0.f;
-      for (int d = qd; d < D; d += 4) {
-        const float a = lds[xn0 + i * ldx + d], b = lds[xn1 + i * ldx + d];
-        acc += l2 ? (a - b) * (a - b) : a * b;
+      for (int d0 = qd; d0 < D; d0 += 32) {  // eight columns of both rows in flight
+        float a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int d = min(d0 + 4 * u, D - 1);
+          a[u] = lds[xn0 + i * ldx + d];
+          b[u] = lds[xn1 + i * ldx + d];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (d0 + 4 * u < D) acc += l2 ? (a[u] - b[u]) * (a[u] - b[u]) : a[u] * b[u];
       }
       acc = quad_sum(acc);
       if (qd == 0) lds[f.pos + i] = l2 ? -sqrtf(fmaxf(acc, 1e-30f)) : acc;
     }
-    __syncthreads();
+    __syncthreads();  // (c)
     if (t < 8 * P) {
       const int pair = t >> 2;
       const int s = pair >= P, i = pair - s * P;
@@ -849,148 +1035,136 @@ __global__ __launch_bounds__(kFusedThreads) void fused_chunk_kernel(StepCtx c, F
       } else {
         float w = c.rel_weights[rel];
         if (c.edge_weight) w *= c.edge_weight[(int64_t)k * c.B + cc * P + i];
-        ScoreRow sr;
-        sr.raw = lds + row_at;
-        sr.bn = lds + (s ? sq1 : sq0);
-        sr.a2 = l2 ? lds[(s ? sq0 : sq1) + i] : 0.f;
-        sr.cmp = c.cmp;
-        sr.nb = P;
-        sr.i = i;
-        sr.masked_from = valid;
-        float loss_acc = 0.f;
-        side_loss<QuadReduce>(c.loss, c.margin, c.cmp, sr, lds + row_at, N, lds[f.pos + i], w, qd, &loss_acc, &dpos_s,
-                              &viol, &rowsum);
-        loss_w = quad_sum(loss_acc) * w;
+        quad_side_loss<CMP, LOSS>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f, c.margin, N, P,
+                                  i, valid, lds[f.pos + i], w, qd, &loss_w, &dpos_s, &viol, &rowsum);
       }
       if (qd == 0) {
-        lds[(s ? rs1 : rs0) + i] = rowsum;
+        lds[(s ? g.rs1 : g.rs0) + i] = rowsum;
         lds[f.part + (s * 3 + 0) * P + i] = dpos_s;
         lds[f.part + (s * 3 + 1) * P + i] = loss_w;
         lds[f.part + (s * 3 + 2) * P + i] = __int_as_float(viol);
       }
     }
-    __syncthreads();
+    __syncthreads();  // (d)
     if (t < P) {  // both sides of an edge together: statistics out, dLoss/dpos for phase 3
       const int64_t job = (int64_t)k * CP + cc * P + t;
-      lds[f.dpos + t] = lds[f.part + 0 * P + t] + lds[f.part + 3 * P + t];
+      const float dpos = lds[f.part + 0 * P + t] + lds[f.part + 3 * P + t];
       c.lossrow[job] = lds[f.part + 1 * P + t] + lds[f.part + 4 * P + t];
       c.violrow[job * 2] = __float_as_int(lds[f.part + 2 * P + t]);
       c.violrow[job * 2 + 1] = __float_as_int(lds[f.part + 5 * P + t]);
+      if (l2) {
+        lds[f.dpos + t] = dpos;
+      } else {
+        // dot: dLoss/dpos_i goes onto the (masked, so far zero) diagonal of the
+        // scores against the rhs negatives, whose i-th batch negative is the i-th
+        // positive's own rhs row: the products of phase 3 then carry
+        // dpos_i * rhs_i into the lhs gradient and dpos_i * lhs_i into the rhs one.
+        lds[sc1 + t * lds_ + t] = dpos;
+      }
     }
-  }
-  __syncthreads();
-  if (l2) {  // column sums of the stored -2 dLoss/dq
-    for (int t = threadIdx.x; t < 2 * N; t += kFusedThreads) {
-      const int s = t >= N, j = t - s * N;
-      const int s_off = s ? sc1 : sc0;
-      float acc = 0.f;
-      for (int i = 0; i < P; ++i) acc += lds[s_off + i * lds_ + j];
-      lds[(s ? cs1 : cs0) + j] = acc;
+    if (l2) {  // column sums of the stored -2 dLoss/dq
+      for (int t2 = t; t2 < 2 * N; t2 += kFusedThreads) {
+        const int s = t2 >= N, j = t2 - s * N;
+        const int s_off = s ? sc1 : sc0;
+        float acc = 0.f;
+        for (int i = 0; i < P; ++i) acc += lds[s_off + i * lds_ + j];
+        lds[(s ? g.cs1 : g.cs0) + j] = acc;
+      }
     }
-    __syncthreads();
-  }
+    __syncthreads();  // (e)
+    // Both score blocks carry a P x P part against the batch negatives, and the
+    // batch negatives of one side are the positives of that side: the gradient of
+    // positive row i of the lhs is  sum_j dS_R[i][j] rhs_j + sum_j dS_L[j][i] rhs_j,
+    // so the two parts fold into G = dS_R[:, :P] + dS_L[:, :P]^T (and G^T for the
+    // rhs rows), kept in place, and phase 3 needs one product per row block.
+    for (int e = t; e < P * P; e += kFusedThreads) {
+      const int i = e / P, j = e - i * P;
+      const float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
+      lds[sc1 + i * lds_ + j] = sum;
+      lds[sc0 + j * lds_ + i] = sum;
+    }
+    __syncthreads();  // (f)
 
-  // ---- phase 3: gradients of the 2(P+U) rows, written to HBM ----
-  {
-    const int m = wave >> 2, rt = wave & 3;  // m: side whose rows' gradients this wave forms
-    const SideCtx& sd = c.side[m];
-    const int dsa = m ? sc0 : sc1;  // scores in which this side's positives were the A operand
-    const int dsn = m ? sc1 : sc0;  // scores against this side's negatives
-    const int bx = m ? xn0 : xn1;   // the other side's rows: the B operand of every product here
-    const int xs = m ? xn1 : xn0;   // this side's rows
-    const int rs_o = m ? rs0 : rs1, cs_m = m ? cs1 : cs0;
-    const bool has_op = m == 1 && c.op != PBG_OP_NONE;
-    if (rt * 16 < P) {
-      // The k index runs past N (resp. P) up to the next multiple of 4: the score
-      // blocks keep zero pad columns and zero pad rows there, so those terms vanish.
-      float4v acc[TD];
+    // ---- phase 3: gradients of the 2(P+U) rows, written to HBM ----
+    {
+      const int m = wave >> 2, rt = wave & 3;  // m: side whose rows' gradients this wave forms
+      const SideCtx& sd = c.side[m];
+      const int dsa = m ? sc0 : sc1;  // scores in which this side's positives were the A operand
+      const int dsn = m ? sc1 : sc0;  // scores against this side's negatives
+      const int bx = m ? xn0 : xn1;   // the other side's rows: the B operand of every product here
+      const int xs = m ? xn1 : xn0;   // this side's rows
+      const int rs_o = m ? g.rs0 : g.rs1, cs_m = m ? g.cs1 : g.cs0;
+      const bool has_op = m == 1 && c.op != PBG_OP_NONE;
+      const bool diag = has_op && c.op == PBG_OP_DIAGONAL;
+      const int b_at = bx + (lane_ >> 4) * ldx + (lane_ & 15);
+      const int pk = (P + 3) >> 2;
+      if (rt * 16 < P) {
+        // The k index runs past N (resp. P) up to the next multiple of 4: the score
+        // blocks keep zero pad columns and zero pad rows there, so those terms vanish.
+        float4v acc[TD];
 #pragma unroll
-      for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const int ar = min(rt * 16 + (lane & 15), P - 1);
-      const int b_at = bx + (lane >> 4) * ldx + (lane & 15);
-      {
-        const int a_at = dsa + ar * lds_ + (lane >> 4);
-        for (int ks = 0; ks < ((N + 3) >> 2); ++ks) {  // dS_a (P x N) times the other side's N rows
-          const float a = lds[a_at + ks * 4];
-          float b[TD];
+        for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+        const int ar = min(rt * 16 + (lane_ & 15), P - 1);
+        // [G | dS_a[:, P:]] (P x N) times the other side's N rows
+        mfma_sweep<TD>(lds, dsa + ar * lds_ + (lane_ >> 4), 4, b_at, 4 * ldx, 16, (N + 3) >> 2, acc);
 #pragma unroll
-          for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
+        for (int r = 0; r < 4; ++r) {
+          const int i = rt * 16 + 4 * (lane_ >> 4) + r;
+          if (i >= valid) continue;
+          const int q = cc * P + i;
+          float coef = 0.f, pcoef = 0.f;
+          if (l2) {
+            const float dpz = lds[f.dpos + i], pz = lds[f.pos + i];
+            coef = 2.0f * lds[rs_o + i] - lds[cs_m + i];
+            pcoef = pz * pz > 2e-30f ? dpz / pz : 0.f;
+          }
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
+          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + q) * D : nullptr;
 #pragma unroll
-          for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
+          for (int ct = 0; ct < TD; ++ct) {
+            const int d = ct * 16 + (lane_ & 15);
+            if (d < D) {
+              float v = acc[ct][r];
+              if (l2) {
+                const float self = lds[xs + i * ldx + d], other = lds[bx + i * ldx + d];
+                v += coef * self + pcoef * (self - other);
+              }
+              if (dzo) dzo[d] = v;
+              if (diag) v *= sd.p0[rel * D + d];
+              out[d] = v;
+            }
+          }
         }
       }
-      {
-        const int a_at = dsn + (lane >> 4) * lds_ + ar;
-        for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {  // (dS_n[:, :P])^T (P x P) times the other side's positives
-          const float a = lds[a_at + ks * 4 * lds_];
-          float b[TD];
+      if (rt * 16 < U) {  // uniform negatives of side m: (dS_n[:, P:])^T (U x P) times the other side's positives
+        float4v acc[TD];
 #pragma unroll
-          for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
+        for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+        const int au = min(rt * 16 + (lane_ & 15), U - 1);
+        mfma_sweep<TD>(lds, dsn + (lane_ >> 4) * lds_ + P + au, 4 * lds_, b_at, 4 * ldx, 16, pk, acc);
 #pragma unroll
-          for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
-        }
-      }
+        for (int r = 0; r < 4; ++r) {
+          const int u = rt * 16 + 4 * (lane_ >> 4) + r;
+          if (u >= U) continue;
+          const int r2 = cc * U + u;
+          const float coef = l2 ? lds[cs_m + P + u] : 0.f;
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
+          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D : nullptr;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = rt * 16 + 4 * (lane >> 4) + r;
-        if (i >= valid) continue;
-        const int q = cc * P + i;
-        const float dpz = lds[f.dpos + i], pz = lds[f.pos + i];
-        const float coef = l2 ? 2.0f * lds[rs_o + i] - lds[cs_m + i] : 0.f;
-        const float pcoef = (l2 && pz * pz > 1e-30f) ? dpz / pz : 0.f;
-        float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
-        float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + q) * D : nullptr;
-#pragma unroll
-        for (int ct = 0; ct < TD; ++ct) {
-          const int d = ct * 16 + (lane & 15);
-          if (d < D) {
-            const float self = lds[xs + i * ldx + d], other = lds[bx + i * ldx + d];
-            float v = acc[ct][r];
-            if (l2) v += coef * self + pcoef * (self - other);
-            else v += dpz * other;
-            if (dzo) dzo[d] = v;
-            if (has_op && c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
-            out[d] = v;
+          for (int ct = 0; ct < TD; ++ct) {
+            const int d = ct * 16 + (lane_ & 15);
+            if (d < D) {
+              float v = acc[ct][r];
+              if (l2) v -= coef * lds[xs + (P + u) * ldx + d];
+              if (dzo) dzo[d] = v;
+              if (diag) v *= sd.p0[rel * D + d];
+              out[d] = v;
+            }
           }
         }
       }
     }
-    if (rt * 16 < U) {  // uniform negatives of side m: (dS_n[:, P:])^T (U x P) times the other side's positives
-      float4v acc[TD];
-#pragma unroll
-      for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
-      const int au = min(rt * 16 + (lane & 15), U - 1);
-      const int a_at = dsn + (lane >> 4) * lds_ + P + au;
-      const int b_at = bx + (lane >> 4) * ldx + (lane & 15);
-      for (int ks = 0; ks < ((P + 3) >> 2); ++ks) {
-        const float a = lds[a_at + ks * 4 * lds_];
-        float b[TD];
-#pragma unroll
-        for (int ct = 0; ct < TD; ++ct) b[ct] = lds[b_at + ks * 4 * ldx + ct * 16];
-#pragma unroll
-        for (int ct = 0; ct < TD; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int u = rt * 16 + 4 * (lane >> 4) + r;
-        if (u >= U) continue;
-        const int r2 = cc * U + u;
-        const float coef = l2 ? lds[cs_m + P + u] : 0.f;
-        float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
-        float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D : nullptr;
-#pragma unroll
-        for (int ct = 0; ct < TD; ++ct) {
-          const int d = ct * 16 + (lane & 15);
-          if (d < D) {
-            float v = acc[ct][r];
-            if (l2) v -= coef * lds[xs + (P + u) * ldx + d];
-            if (dzo) dzo[d] = v;
-            if (has_op && c.op == PBG_OP_DIAGONAL) v *= sd.p0[rel * D + d];
-            out[d] = v;
-          }
-        }
-      }
-    }
+    __syncthreads();  // (g)
   }
 }
 
@@ -1658,6 +1832,52 @@ namespace {
 // prep | operator forward | score GEMMs | loss | dN GEMMs | dA GEMMs | rowback | params | sort | update
 constexpr int kStages = 10;
 
+// One instantiation of the fused kernel per (tile count, comparator, loss); each
+// raises its dynamic LDS limit the first time it needs more than it was given.
+template <int T, int CMP, int LOSS>
+int launch_fused_as(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+  static size_t lds_allowed = 0;
+  if (lds_bytes > lds_allowed) {
+    if (hipFuncSetAttribute((const void*)fused_chunk_kernel<T, T, CMP, LOSS>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+      return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
+    lds_allowed = lds_bytes;
+  }
+  // one persistent workgroup per compute unit (the LDS footprint allows no more)
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+  }
+  const int chunks = plan.c.K * plan.c.C;
+  hipLaunchKernelGGL((fused_chunk_kernel<T, T, CMP, LOSS>), dim3((unsigned)(chunks < cus ? chunks : cus)),
+                     dim3(2 * kFusedThreads), lds_bytes, s, plan.c, plan.fl, chunks);
+  return PBG_OK;
+}
+
+template <int T, int CMP>
+int launch_fused_loss(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+  switch (plan.c.loss) {
+    case PBG_LOSS_RANKING: return launch_fused_as<T, CMP, PBG_LOSS_RANKING>(plan, lds_bytes, s);
+    case PBG_LOSS_LOGISTIC: return launch_fused_as<T, CMP, PBG_LOSS_LOGISTIC>(plan, lds_bytes, s);
+    default: return launch_fused_as<T, CMP, PBG_LOSS_SOFTMAX>(plan, lds_bytes, s);
+  }
+}
+
+int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+  const StepCtx& c = plan.c;
+  const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
+  const bool l2 = c.cmp == PBG_CMP_L2;
+  if (small_tiles) {
+    return l2 ? launch_fused_loss<7, PBG_CMP_L2>(plan, lds_bytes, s)
+              : launch_fused_loss<7, PBG_CMP_DOT>(plan, lds_bytes, s);
+  }
+  return l2 ? launch_fused_loss<8, PBG_CMP_L2>(plan, lds_bytes, s)
+            : launch_fused_loss<8, PBG_CMP_DOT>(plan, lds_bytes, s);
+}
+
 int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_t s, hipEvent_t* ev) {
   int rc = validate(desc, true);
   if (rc != PBG_OK) return rc;
@@ -1672,20 +1892,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
     const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
-    const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
-    const void* fn = small_tiles ? (const void*)fused_chunk_kernel<7, 7> : (const void*)fused_chunk_kernel<8, 8>;
-    static size_t lds_allowed[2] = {0, 0};
-    if (lds_bytes > lds_allowed[small_tiles]) {
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-        return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
-      lds_allowed[small_tiles] = lds_bytes;
-    }
-    if (small_tiles)
-      hipLaunchKernelGGL((fused_chunk_kernel<7, 7>), dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c,
-                         plan.fl);
-    else
-      hipLaunchKernelGGL((fused_chunk_kernel<8, 8>), dim3((unsigned)(c.K * c.C)), dim3(kFusedThreads), lds_bytes, s, c,
-                         plan.fl);
+    if ((rc = launch_fused(plan, lds_bytes, s)) != PBG_OK) return rc;
     mark(1);
     mark(2);
     mark(3);

@@ -196,6 +196,28 @@ def compare_state(cfg, runner, st, rtol, tag):
             assert_close(got[k], want[k], rtol, f"{tag} {name}.{k}")
 
 
+def hinge_ties(cfg, scores, eps=2e-6):
+    """Number of negatives whose hinge argument (neg - pos) + margin lies within
+    eps of 0 (GPU and CPU scores agree to about 1e-7)."""
+    n = 0
+    for pos, neg in ((scores.lhs_pos, scores.lhs_neg), (scores.rhs_pos, scores.rhs_neg)):
+        x = (neg - pos.unsqueeze(1)) + cfg.margin
+        n += int((x.abs() < eps).sum())
+    return n
+
+
+def copy_state(runner, st):
+    runner.w_lhs.copy_(st.w_lhs)
+    runner.g_lhs.copy_(st.g_lhs)
+    if not st.shared:
+        runner.w_rhs.copy_(st.w_rhs)
+        runner.g_rhs.copy_(st.g_rhs)
+    for got, want in ((runner.rhs_op, st.rhs_op), (runner.rhs_op_sum, st.rhs_op_sum),
+                      (runner.lhs_op, st.lhs_op), (runner.lhs_op_sum, st.lhs_op_sum)):
+        for k in want:
+            got[k].copy_(want[k])
+
+
 @pytest.mark.parametrize("case", TRAIN_CASES, ids=ids)
 @pytest.mark.parametrize("workers", [1, 3])
 def test_train_step(pbg, case, workers):
@@ -240,8 +262,20 @@ def test_hundred_steps(pbg, case):
     cfg = ostep.StepConfig(dim=dim, num_relations=2, relation_weights=[1.0, 1.0], lr=0.1, dynamic=False, **case)
     st, batches = make_inputs(cfg, num_pos, 2000, 100, seed=1, scale=1e-3 if case["operator"] == "none" else 0.1)
     runner = to_runner(pbg, cfg, st, num_pos, 1)
-    for b in batches:
+    resyncs = 0
+    for n, b in enumerate(batches):
         runner.train(*pack(cfg, [b]))
-        ostep.train_step(cfg, st, *b)
+        out = ostep.train_step(cfg, st, *b, keep_scores=cfg.loss == "ranking")
+        if cfg.loss == "ranking" and hinge_ties(cfg, out.scores) > 0:
+            # A negative within rounding distance of the hinge: max(0, x) has a
+            # gradient of 0 on one side and 1 on the other, so two correct fp32
+            # evaluations may take different sides and then drift apart for good.
+            # Such a step is checked on its own at a tolerance that admits one
+            # flipped hinge per row, then the GPU state restarts from the oracle's.
+            torch.cuda.synchronize()
+            compare_state(cfg, runner, st, 5e-2, f"step {n} (hinge tie)")
+            copy_state(runner, st)
+            resyncs += 1
     torch.cuda.synchronize()
+    assert resyncs <= 10, resyncs
     compare_state(cfg, runner, st, 1e-4, "100 steps")
