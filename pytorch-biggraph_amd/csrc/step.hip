@@ -788,11 +788,13 @@ __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at
   *viol_out = quad_sum_int(viol);
 }
 
-// acc[ct] += A(16 x 4 per k-step, element (lane & 15, lane >> 4) at a_at + ks * a_step)
-//          * B(4 x 16 per column tile, at b_at + ks * b_step + ct * b_tile)
+// acc[ct] += (A(16 x 4 per k-step, element (lane & 15, lane >> 4) at a_at + ks * a_step)
+//          * B(4 x 16 per column tile, at b_at + ks * b_step + ct * b_tile))^T
 // over `ksteps` k-steps; the operands of the next k-step are in flight while the
 // MFMAs of the current one issue.  Reads one k-step past the end (the caller's
-// buffers keep slack there).
+// buffers keep slack there).  The product is formed as B^T A^T, so a lane ends up
+// with four consecutive columns of ONE row of A B: acc[ct][r] is element
+// (lane & 15, ct * 16 + 4 * (lane >> 4) + r), which stores as one 128-bit word.
 template <int T>
 __device__ __forceinline__ void mfma_sweep(const float* lds, int a_at, int a_step, int b_at, int b_step, int b_tile,
                                            int ksteps, float4v* acc) {
@@ -808,7 +810,7 @@ __device__ __forceinline__ void mfma_sweep(const float* lds, int a_at, int a_ste
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) bn[ct] = lds[b_at + ct * b_tile];
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct], a, acc[ct], 0, 0, 0);
     a = an;
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) b[ct] = bn[ct];
@@ -989,14 +991,16 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         const int a_at = (s ? xn0 : xn1) + ar * ldx + (lane_ >> 4);
         const int b_at = (s ? xn1 : xn0) + (lane_ & 15) * ldx + (lane_ >> 4);  // column tile ct: 16 rows further down
         mfma_sweep<TN>(lds, a_at, 4, b_at, 4, 16 * ldx, (D + 3) >> 2, acc);
-        const int s_off = s ? sc1 : sc0;
+        const int row = rt * 16 + (lane_ & 15);
+        if (row < P) {
+          const int at = (s ? sc1 : sc0) + row * lds_ + 4 * (lane_ >> 4);
 #pragma unroll
-        for (int ct = 0; ct < TN; ++ct) {
-          const int col = ct * 16 + (lane_ & 15);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int row = rt * 16 + 4 * (lane_ >> 4) + r;
-            if (row < P && col < N) lds[s_off + row * lds_ + col] = acc[ct][r];
+          for (int ct = 0; ct < TN; ++ct) {
+            const int col = ct * 16 + 4 * (lane_ >> 4);
+            if (col < N)  // pad columns stay zero
+              *reinterpret_cast<float4*>(&lds[at + ct * 16]) =
+                  make_float4(acc[ct][0], col + 1 < N ? acc[ct][1] : 0.f, col + 2 < N ? acc[ct][2] : 0.f,
+                              col + 3 < N ? acc[ct][3] : 0.f);
           }
         }
       }
@@ -1107,10 +1111,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         const int ar = min(rt * 16 + (lane_ & 15), P - 1);
         // [G | dS_a[:, P:]] (P x N) times the other side's N rows
         mfma_sweep<TD>(lds, dsa + ar * lds_ + (lane_ >> 4), 4, b_at, 4 * ldx, 16, (N + 3) >> 2, acc);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = rt * 16 + 4 * (lane_ >> 4) + r;
-          if (i >= valid) continue;
+        const int i = rt * 16 + (lane_ & 15), d0 = 4 * (lane_ >> 4);
+        if (i < valid) {
           const int q = cc * P + i;
           float coef = 0.f, pcoef = 0.f;
           if (l2) {
@@ -1118,20 +1120,27 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
             coef = 2.0f * lds[rs_o + i] - lds[cs_m + i];
             pcoef = pz * pz > 2e-30f ? dpz / pz : 0.f;
           }
-          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
-          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + q) * D : nullptr;
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D + d0;
+          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + q) * D + d0 : nullptr;
 #pragma unroll
           for (int ct = 0; ct < TD; ++ct) {
-            const int d = ct * 16 + (lane_ & 15);
-            if (d < D) {
-              float v = acc[ct][r];
+            const int d = ct * 16 + d0;
+            if (d < D) {  // D is a multiple of 4
+              float4 v = make_float4(acc[ct][0], acc[ct][1], acc[ct][2], acc[ct][3]);
               if (l2) {
-                const float self = lds[xs + i * ldx + d], other = lds[bx + i * ldx + d];
-                v += coef * self + pcoef * (self - other);
+                const float4 self = *reinterpret_cast<const float4*>(&lds[xs + i * ldx + d]);
+                const float4 other = *reinterpret_cast<const float4*>(&lds[bx + i * ldx + d]);
+                v.x += coef * self.x + pcoef * (self.x - other.x);
+                v.y += coef * self.y + pcoef * (self.y - other.y);
+                v.z += coef * self.z + pcoef * (self.z - other.z);
+                v.w += coef * self.w + pcoef * (self.w - other.w);
               }
-              if (dzo) dzo[d] = v;
-              if (diag) v *= sd.p0[rel * D + d];
-              out[d] = v;
+              if (dzo) *reinterpret_cast<float4*>(dzo + ct * 16) = v;
+              if (diag) {
+                const float4 p = *reinterpret_cast<const float4*>(sd.p0 + rel * D + d);
+                v.x *= p.x; v.y *= p.y; v.z *= p.z; v.w *= p.w;
+              }
+              *reinterpret_cast<float4*>(out + ct * 16) = v;
             }
           }
         }
@@ -1142,23 +1151,27 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         for (int ct = 0; ct < TD; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int au = min(rt * 16 + (lane_ & 15), U - 1);
         mfma_sweep<TD>(lds, dsn + (lane_ >> 4) * lds_ + P + au, 4 * lds_, b_at, 4 * ldx, 16, pk, acc);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int u = rt * 16 + 4 * (lane_ >> 4) + r;
-          if (u >= U) continue;
+        const int u = rt * 16 + (lane_ & 15), d0 = 4 * (lane_ >> 4);
+        if (u < U) {
           const int r2 = cc * U + u;
           const float coef = l2 ? lds[cs_m + P + u] : 0.f;
-          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
-          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D : nullptr;
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D + d0;
+          float* dzo = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D + d0 : nullptr;
 #pragma unroll
           for (int ct = 0; ct < TD; ++ct) {
-            const int d = ct * 16 + (lane_ & 15);
+            const int d = ct * 16 + d0;
             if (d < D) {
-              float v = acc[ct][r];
-              if (l2) v -= coef * lds[xs + (P + u) * ldx + d];
-              if (dzo) dzo[d] = v;
-              if (diag) v *= sd.p0[rel * D + d];
-              out[d] = v;
+              float4 v = make_float4(acc[ct][0], acc[ct][1], acc[ct][2], acc[ct][3]);
+              if (l2) {
+                const float4 self = *reinterpret_cast<const float4*>(&lds[xs + (P + u) * ldx + d]);
+                v.x -= coef * self.x; v.y -= coef * self.y; v.z -= coef * self.z; v.w -= coef * self.w;
+              }
+              if (dzo) *reinterpret_cast<float4*>(dzo + ct * 16) = v;
+              if (diag) {
+                const float4 p = *reinterpret_cast<const float4*>(sd.p0 + rel * D + d);
+                v.x *= p.x; v.y *= p.y; v.z *= p.z; v.w *= p.w;
+              }
+              *reinterpret_cast<float4*>(out + ct * 16) = v;
             }
           }
         }
