@@ -51,7 +51,8 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const float* _
 //   run_combine   one wave per tile border; the first border a run crosses adds
 //                 the pieces of the later tiles into the row of the run's first
 //                 position;
-//   row_update    one wave per row walks its runs (one gradient row each), the
+//   row_update    a wave per few sorted positions; at each position that starts
+//                 a row it walks the row's runs (one gradient row each), the
 //                 keys of the next 64 positions held in registers.
 constexpr int kTile = 32;
 
@@ -225,68 +226,89 @@ __device__ __forceinline__ float adagrad_apply(RowRegs<NV, VEC>& w, const RowReg
   return gsum;
 }
 
-template <int NV, bool VEC>
+// One wave looks at R consecutive sorted positions; a position that starts a row
+// gets the row's update.  All loads that do not depend on each other (the R key
+// windows, then the weight rows and first gradient rows of the positions that
+// turned out to be row heads) are issued together: the kernel lives on memory
+// latency, and the rows in flight per wave are what hides it.
+template <int NV, bool VEC, int R>
 __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
     const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
     float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
   const int lane = threadIdx.x & 63;
-  const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
-  if (i >= n) return;
-  // one coalesced look at this and the next 63 sorted positions
-  const int64_t p = i + lane;
-  const uint64_t kk = keys[p < n ? p : n - 1];
-  const uint32_t vv = vals[p < n ? p : n - 1];
-  const uint64_t row = lane_u64(kk, 0) >> kbits;
-  if (i > 0 && (keys[i - 1] >> kbits) == row) return;
-  if ((int64_t)row >= rows0 + rows1) return;  // out-of-range indices are parked past both tables
-
-  float* wrow;
-  float* gptr;
-  if ((int64_t)row < rows0) {
-    wrow = w0 + (int64_t)row * dim;
-    gptr = g0 + row;
-  } else {
-    wrow = w1 + ((int64_t)row - rows0) * dim;
-    gptr = g1 + ((int64_t)row - rows0);
-  }
+  const int64_t first = ((int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6)) * R;
+  if (first >= n) return;
   const int nv = VEC ? (dim >> 2) : dim;
   const float fdim = (float)dim;
-  RowRegs<NV, VEC> w;
-  w.load(wrow, nv, lane);
-  float gsum = *gptr;
-
-  const uint64_t in_row = __ballot(p < n && (kk >> kbits) == row);
-  if (~in_row != 0ull) {
-    // the row ends inside the window: its runs are known from the keys in registers
-    const int len = __ffsll((unsigned long long)~in_row) - 1;
-    const uint64_t up = __shfl_up(kk, 1, 64);
-    uint64_t heads = __ballot(lane < len && (lane == 0 || up != kk));  // first position of every run
-    RowRegs<NV, VEC> g;
-    g.load(grad_rows + (int64_t)lane_u32(vv, 0) * dim, nv, lane);  // each run's sum sits in its first row
-    heads &= heads - 1;
-    while (heads != 0ull) {  // the next run's row is in flight while this one is applied
-      const int a = __ffsll((unsigned long long)heads) - 1;
-      heads &= heads - 1;
-      RowRegs<NV, VEC> next;
-      next.load(grad_rows + (int64_t)lane_u32(vv, a) * dim, nv, lane);
-      gsum = adagrad_apply(w, g, gsum, fdim, lr);
-      g = next;
-    }
-    gsum = adagrad_apply(w, g, gsum, fdim, lr);
-  } else {
-    int64_t j = i;
-    while (j < n && (keys[j] >> kbits) == row) {
-      const uint64_t key = keys[j];
-      RowRegs<NV, VEC> g;
-      g.load(grad_rows + (int64_t)vals[j] * dim, nv, lane);
-      // a single-worker call has one run per row: no need to look for its end
-      j = (kbits == 0) ? n : scan_end(keys, j, n, key, 0, lane);
-      gsum = adagrad_apply(w, g, gsum, fdim, lr);
-    }
+  // one coalesced look at each position and the 63 sorted positions after it
+  uint64_t kk[R], before[R];
+  uint32_t vv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t i = first + r < n ? first + r : n - 1;
+    const int64_t p = i + lane < n ? i + lane : n - 1;
+    kk[r] = keys[p];
+    vv[r] = vals[p];
+    before[r] = keys[i > 0 ? i - 1 : 0];
   }
-  w.store(wrow, nv, lane);
-  if (lane == 0) *gptr = gsum;
+  bool head[R];
+  float* wrow[R];
+  float* gptr[R];
+  float gsum[R];
+  RowRegs<NV, VEC> w[R], g[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t i = first + r;
+    const uint64_t row = lane_u64(kk[r], 0) >> kbits;
+    // out-of-range indices are parked past both tables
+    head[r] = i < n && !(i > 0 && (before[r] >> kbits) == row) && (int64_t)row < rows0 + rows1;
+    if (!head[r]) continue;
+    if ((int64_t)row < rows0) {
+      wrow[r] = w0 + (int64_t)row * dim;
+      gptr[r] = g0 + row;
+    } else {
+      wrow[r] = w1 + ((int64_t)row - rows0) * dim;
+      gptr[r] = g1 + ((int64_t)row - rows0);
+    }
+    w[r].load(wrow[r], nv, lane);
+    gsum[r] = *gptr[r];
+    g[r].load(grad_rows + (int64_t)lane_u32(vv[r], 0) * dim, nv, lane);  // each run's sum sits in its first row
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (!head[r]) continue;
+    const int64_t i = first + r;
+    const uint64_t row = lane_u64(kk[r], 0) >> kbits;
+    const uint64_t in_row = __ballot(i + lane < n && (kk[r] >> kbits) == row);
+    if (~in_row != 0ull) {
+      // the row ends inside the window: its runs are known from the keys in registers
+      const int len = __ffsll((unsigned long long)~in_row) - 1;
+      const uint64_t up = __shfl_up(kk[r], 1, 64);
+      uint64_t heads = __ballot(lane < len && (lane == 0 || up != kk[r]));  // first position of every run
+      heads &= heads - 1;
+      while (heads != 0ull) {  // the next run's row is in flight while this one is applied
+        const int a = __ffsll((unsigned long long)heads) - 1;
+        heads &= heads - 1;
+        RowRegs<NV, VEC> next;
+        next.load(grad_rows + (int64_t)lane_u32(vv[r], a) * dim, nv, lane);
+        gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+        g[r] = next;
+      }
+      gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+    } else {
+      int64_t j = i;
+      while (true) {
+        // a single-worker call has one run per row: no need to look for its end
+        j = (kbits == 0) ? n : scan_end(keys, j, n, keys[j], 0, lane);
+        gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+        if (j >= n || (keys[j] >> kbits) != row) break;
+        g[r].load(grad_rows + (int64_t)vals[j] * dim, nv, lane);
+      }
+    }
+    w[r].store(wrow[r], nv, lane);
+    if (lane == 0) *gptr[r] = gsum[r];
+  }
 }
 
 // keys for the stand-alone sparse step: key = row index, value = position
@@ -333,7 +355,7 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
                   int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
                   hipStream_t stream) {
   const int wpb = kRowThreads / kWave;
-  const dim3 grid((unsigned)ceil_div(n, wpb)), block(kRowThreads);
+  const dim3 block(kRowThreads);
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
   const int64_t borders = ceil_div(n, kTile) - 1;
   const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
@@ -342,8 +364,12 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim);  \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
-    hipLaunchKernelGGL((row_update_kernel<NV, VEC>), grid, block, 0, stream, keys, vals, n, kbits, grad_rows, dim,  \
-                       w0, g0, rows0, w1, g1, rows1, lr);                                                          \
+    {                                                                                                              \
+      constexpr int R = NV <= 2 ? 4 : (NV <= 4 ? 2 : 1);                                                           \
+      const dim3 ugrid((unsigned)ceil_div(ceil_div(n, R), wpb));                                                   \
+      hipLaunchKernelGGL((row_update_kernel<NV, VEC, R>), ugrid, block, 0, stream, keys, vals, n, kbits, grad_rows, \
+                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+    }                                                                                                              \
   } while (0)
   if (nvec <= 1) PBG_LAUNCH(1);
   else if (nvec <= 2) PBG_LAUNCH(2);
