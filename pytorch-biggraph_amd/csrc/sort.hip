@@ -1,214 +1,221 @@
 // Stable radix sort of (uint64 key, uint32 value) pairs on a bit range of the key.
 //
 // The top (up to 9) bits of the range are sorted by ONE global pass: every block
-// owns a contiguous power-of-two tile of positions, a histogram kernel counts the
-// digit per tile, and the scatter kernel derives its digit offsets from the
-// per-tile counts of all tiles (at most 256 of them, stored digit-major so that a
-// thread reads its digit's counts with a few independent 128-bit loads), ranks
-// its keys slice by slice (ballot matching inside a wave, LDS counts across the
-// 4 waves, a running per-digit cursor across slices) and scatters them.  That
-// leaves one bucket per digit value, contiguous in memory; the remaining low bits
-// are sorted inside each bucket, one block per bucket, 8 bits per launch from the
-// lowest up: no counts to exchange between blocks, no atomics on global memory.
-// Every step is stable, so equal keys keep the order of the input, which keeps
-// segmented gradient sums deterministic and lets a caller whose input is already
-// ordered by the low bits leave those bits out.
+// owns a contiguous power-of-two tile of at least 4096 positions, a histogram
+// kernel counts the digit per tile, and the scatter kernel derives its digit
+// offsets from the per-tile counts of all tiles (at most 256 tiles, and few for
+// the sizes of a training step, so the table that every block reads stays
+// small), ranks its keys slice by slice (ballot matching inside a wave, LDS
+// counts across the 16 waves, a running per-digit cursor across slices) and
+// scatters them.  That leaves one bucket per digit value, contiguous in memory;
+// the remaining low bits are sorted inside each bucket, one block per bucket,
+// 8 bits per launch from the lowest up: no counts to exchange between blocks, no
+// atomics on global memory.  Every step is stable, so equal keys keep the order
+// of the input, which keeps segmented gradient sums deterministic and lets a
+// caller whose input is already ordered by the low bits leave those bits out.
 #include "pbg_internal.h"
 
 namespace pbg {
 namespace {
 
-constexpr int kSortThreads = 256;
+constexpr int kGlobalWaves = 16;  // global pass: 1024 threads per block
+constexpr int kBucketWaves = 4;   // bucket passes: 256 threads per block
 constexpr int kMaxDigitBits = 9;
+constexpr int kMaxDigits = 1 << kMaxDigitBits;
 constexpr int kMaxSortBlocks = 256;
+constexpr int kMinTileShift = 12;
 
 struct SortPlan {
   int tile_shift;  // keys per block = 1 << tile_shift
   int blocks;
-  int stride;      // blocks rounded up to a multiple of 4: row length of the digit-major counts
 };
 
 SortPlan plan_sort(int64_t n) {
   SortPlan p;
-  p.tile_shift = 9;
+  p.tile_shift = kMinTileShift;
   while (ceil_div(n, (int64_t)1 << p.tile_shift) > kMaxSortBlocks) ++p.tile_shift;
   p.blocks = (int)ceil_div(n > 0 ? n : 1, (int64_t)1 << p.tile_shift);
-  p.stride = (p.blocks + 3) / 4 * 4;
   return p;
 }
 
-// counts[digit][stride] of the global pass (padding columns cleared)
-__global__ __launch_bounds__(kSortThreads) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n,
-                                                                 int tile_shift, int shift, int digit_bits, int stride,
-                                                                 uint32_t* __restrict__ counts) {
-  __shared__ uint32_t hist[1 << kMaxDigitBits];
-  const int digits = 1 << digit_bits;
-  const uint32_t mask = (uint32_t)digits - 1u;
-  for (int d = threadIdx.x; d < digits; d += kSortThreads) hist[d] = 0;
-  if (blockIdx.x == 0)
-    for (int d = threadIdx.x; d < digits; d += kSortThreads)
-      for (int b = gridDim.x; b < stride; ++b) counts[(int64_t)d * stride + b] = 0;
+// counts[block][kMaxDigits] of the global pass
+__global__ __launch_bounds__(kGlobalWaves * 64) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n,
+                                                                      int tile_shift, int shift, int digit_bits,
+                                                                      uint32_t* __restrict__ counts) {
+  __shared__ uint32_t hist[kMaxDigits];
+  const uint32_t mask = (1u << digit_bits) - 1u;
+  if (threadIdx.x < kMaxDigits) hist[threadIdx.x] = 0;
   __syncthreads();
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kSortThreads)
+  for (int64_t i = begin + threadIdx.x; i < end; i += kGlobalWaves * 64)
     atomicAdd(&hist[(uint32_t)(keys[i] >> shift) & mask], 1u);
   __syncthreads();
-  for (int d = threadIdx.x; d < digits; d += kSortThreads) counts[(int64_t)d * stride + blockIdx.x] = hist[d];
+  if (threadIdx.x < kMaxDigits) counts[(int64_t)blockIdx.x * kMaxDigits + threadIdx.x] = hist[threadIdx.x];
 }
 
-// One slice of up to 256 keys: rank every key among the keys of the slice with
-// the same digit (earlier positions first), scatter it to cursor[digit] + rank,
-// advance the cursors.  wave_count must be zero on entry and is zero on exit.
-template <int DPT>
-__device__ __forceinline__ void scatter_slice(bool valid, uint64_t key, uint32_t val, uint32_t digit,
-                                              uint32_t* cursor, uint32_t (*wave_count)[DPT * kSortThreads],
-                                              uint64_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out) {
-  constexpr int kBits = DPT == 1 ? 8 : 9;
+// Exclusive scan over one value per thread of the first `waves` waves of the
+// block (all threads of the block must call it); *grand gets the sum.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t value, int waves, uint32_t* wave_total,
+                                                         uint32_t* grand) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  uint32_t incl = value;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63 && wave < waves) wave_total[wave] = incl;
+  __syncthreads();
+  uint32_t ahead = 0, all = 0;
+  for (int w = 0; w < waves; ++w) {
+    const uint32_t wt = wave_total[w];
+    if (w < wave) ahead += wt;
+    all += wt;
+  }
+  __syncthreads();
+  *grand = all;
+  return ahead + incl - value;
+}
+
+// Rank-and-scatter state of one block: NW waves, digits of up to BITS bits.
+template <int NW, int BITS>
+struct SliceState {
+  uint32_t cursor[1 << BITS];             // next output slot of each digit
+  uint32_t slot[1 << BITS];               // first output slot of each digit in the current slice
+  uint16_t wave_count[2][NW][1 << BITS];  // per-wave digit counts, one buffer per slice parity
+  uint32_t wave_total[NW];
+};
+
+// One slice of up to NW * 64 keys: rank every key among the keys of the slice
+// with the same digit (earlier positions first), scatter it to cursor[digit] +
+// rank, advance the cursors.  Both count buffers must be zero before the first
+// slice; each slice clears the buffer the previous one used.
+template <int NW, int BITS>
+__device__ __forceinline__ void scatter_slice(SliceState<NW, BITS>& st, int parity, bool valid, uint64_t key,
+                                              uint32_t val, uint32_t digit, uint64_t* __restrict__ keys_out,
+                                              uint32_t* __restrict__ vals_out) {
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   // lanes of this wave holding the same digit
   uint64_t peers = __ballot(valid);
 #pragma unroll
-  for (int b = 0; b < kBits; ++b) {
+  for (int b = 0; b < BITS; ++b) {
     const bool bit = (digit >> b) & 1u;
     const uint64_t m = __ballot(valid && bit);
     peers &= bit ? m : ~m;
   }
   const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   const int rank_in_wave = __popcll(peers & below);
-  if (valid && rank_in_wave == 0) wave_count[wave][digit] = (uint32_t)__popcll(peers);
+  if (valid && rank_in_wave == 0) st.wave_count[parity][wave][digit] = (uint16_t)__popcll(peers);
+  __syncthreads();
+  // per digit: the waves' counts become the waves' offsets from the digit's first slot
+  for (int d = t; d < (1 << BITS); d += NW * 64) {
+    uint32_t at = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const uint32_t c = st.wave_count[parity][w][d];
+      st.wave_count[parity][w][d] = (uint16_t)at;
+      at += c;
+      st.wave_count[parity ^ 1][w][d] = 0;
+    }
+    const uint32_t first = st.cursor[d];
+    st.slot[d] = first;
+    st.cursor[d] = first + at;
+  }
   __syncthreads();
   if (valid) {
-    uint32_t ahead = 0;
-    for (int w = 0; w < wave; ++w) ahead += wave_count[w][digit];
-    const uint32_t pos = cursor[digit] + ahead + (uint32_t)rank_in_wave;
+    const uint32_t pos = st.slot[digit] + st.wave_count[parity][wave][digit] + (uint32_t)rank_in_wave;
     keys_out[pos] = key;
     vals_out[pos] = val;
   }
-  __syncthreads();
-#pragma unroll
-  for (int d = 0; d < DPT; ++d) {
-    uint32_t slice_total = 0;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      slice_total += wave_count[w][t + d * kSortThreads];
-      wave_count[w][t + d * kSortThreads] = 0;
-    }
-    cursor[t + d * kSortThreads] += slice_total;
-  }
-  __syncthreads();
 }
 
-// Exclusive scan over the 256 * DPT digit totals (digit = t + d * 256), in place.
-template <int DPT>
-__device__ __forceinline__ void scan_digits(uint32_t* total, uint32_t* wave_total, uint32_t* grand) {
-  const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
-  uint32_t carry = 0;
-#pragma unroll
-  for (int d = 0; d < DPT; ++d) {
-    uint32_t incl = total[d];
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const uint32_t up = __shfl_up(incl, off, 64);
-      if (lane >= off) incl += up;
-    }
-    if (lane == 63) wave_total[wave] = incl;
-    __syncthreads();
-    uint32_t ahead = carry;
-    for (int w = 0; w < wave; ++w) ahead += wave_total[w];
-    carry += wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
-    total[d] = ahead + incl - total[d];
-    __syncthreads();
-  }
-  *grand = carry;
-}
-
-// The global pass.  DPT digits per thread: 1 (up to 8 digit bits) or 2 (9 digit
-// bits); digit d belongs to thread d % 256.  Block 0 also writes the bucket
-// offsets (digit d's keys end up in [bucket_off[d], bucket_off[d + 1])).
-template <int DPT>
-__global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(
-    const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
-    uint32_t* __restrict__ vals_out, int64_t n, int tile_shift, int shift, int digit_bits, int stride,
-    const uint32_t* __restrict__ counts, uint32_t* __restrict__ bucket_off) {
-  constexpr int kDigits = DPT * kSortThreads;
-  __shared__ uint32_t cursor[kDigits];         // next output slot of each digit for this block
-  __shared__ uint32_t wave_count[4][kDigits];  // per-wave digit counts of the current slice
-  __shared__ uint32_t wave_total[4];
+template <int NW, int BITS>
+__device__ __forceinline__ void scatter_range(SliceState<NW, BITS>& st, const uint64_t* __restrict__ keys_in,
+                                              const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
+                                              uint32_t* __restrict__ vals_out, int64_t begin, int64_t end, int shift,
+                                              uint32_t mask, uint64_t key_next, uint32_t val_next) {
   const int t = threadIdx.x;
-  const int me = blockIdx.x;
-  // offset of digit d for this block = keys with a smaller digit anywhere
-  //                                  + keys with digit d in earlier blocks
-  uint32_t total[DPT], before[DPT];
-#pragma unroll
-  for (int d = 0; d < DPT; ++d) total[d] = before[d] = 0;
-  const int quads = stride >> 2;
-  for (int q0 = 0; q0 < quads; q0 += 16) {  // 16 x DPT independent 128-bit loads in flight
-    uint4 cnt[DPT][16];
-#pragma unroll
-    for (int d = 0; d < DPT; ++d) {
-      const uint4* row = reinterpret_cast<const uint4*>(counts + (int64_t)(t + d * kSortThreads) * stride);
-      const bool has = ((t + d * kSortThreads) >> digit_bits) == 0;  // digits past the pass's width hold no keys
-#pragma unroll
-      for (int u = 0; u < 16; ++u) cnt[d][u] = (has && q0 + u < quads) ? row[q0 + u] : make_uint4(0u, 0u, 0u, 0u);
+  int parity = 0;
+  // the next slice's loads are issued before the current slice is ranked
+  for (int64_t base = begin; base < end; base += NW * 64) {
+    const int64_t i = base + t;
+    const uint64_t key = key_next;
+    const uint32_t val = val_next;
+    if (i + NW * 64 < end) {
+      key_next = keys_in[i + NW * 64];
+      val_next = vals_in[i + NW * 64];
     }
-#pragma unroll
-    for (int d = 0; d < DPT; ++d) {
-#pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int b = (q0 + u) * 4;
-        const uint4 c4 = cnt[d][u];
-        total[d] += c4.x + c4.y + c4.z + c4.w;
-        before[d] += (b < me ? c4.x : 0u) + (b + 1 < me ? c4.y : 0u) + (b + 2 < me ? c4.z : 0u) +
-                     (b + 3 < me ? c4.w : 0u);
-      }
-    }
+    scatter_slice<NW, BITS>(st, parity, i < end, key, val, (uint32_t)(key >> shift) & mask, keys_out, vals_out);
+    parity ^= 1;
   }
-  uint32_t grand;
-  scan_digits<DPT>(total, wave_total, &grand);
-#pragma unroll
-  for (int d = 0; d < DPT; ++d) {
-    const int digit = t + d * kSortThreads;
-    cursor[digit] = total[d] + before[d];
-    if (me == 0 && (digit >> digit_bits) == 0) bucket_off[digit] = total[d];
-    for (int w = 0; w < 4; ++w) wave_count[w][digit] = 0;
-  }
-  if (me == 0 && t == 0) bucket_off[1 << digit_bits] = grand;
-  __syncthreads();
+}
 
-  const uint32_t mask = (1u << digit_bits) - 1u;
+// The global pass.  Block 0 also writes the bucket offsets (digit d's keys end up
+// in [bucket_off[d], bucket_off[d + 1])).
+__global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
+    const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out, int64_t n, int tile_shift, int shift, int digit_bits,
+    const uint32_t* __restrict__ counts, uint32_t* __restrict__ bucket_off) {
+  __shared__ SliceState<kGlobalWaves, kMaxDigitBits> st;
+  __shared__ uint32_t part[2][2][kMaxDigits];  // [half][total, before][digit]
+  const int t = threadIdx.x;
+  const int me = blockIdx.x, blocks = gridDim.x;
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
-  // the next slice's loads are issued before the current slice is ranked
   uint64_t key_next = 0;
   uint32_t val_next = 0;
   if (begin + t < end) {
     key_next = keys_in[begin + t];
     val_next = vals_in[begin + t];
   }
-  for (int64_t base = begin; base < end; base += kSortThreads) {
-    const int64_t i = base + t;
-    const uint64_t key = key_next;
-    const uint32_t val = val_next;
-    if (i + kSortThreads < end) {
-      key_next = keys_in[i + kSortThreads];
-      val_next = vals_in[i + kSortThreads];
+  // offset of digit d for this block = keys with a smaller digit anywhere
+  //                                  + keys with digit d in earlier blocks;
+  // two threads per digit, each over every other block, 16 loads in flight
+  {
+    const int d = t & (kMaxDigits - 1), half = t >> kMaxDigitBits;
+    uint32_t total = 0, before = 0;
+    for (int b0 = half; b0 < blocks; b0 += 32) {
+      uint32_t c[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) c[u] = (b0 + 2 * u < blocks) ? counts[(int64_t)(b0 + 2 * u) * kMaxDigits + d] : 0u;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        total += c[u];
+        if (b0 + 2 * u < me) before += c[u];
+      }
     }
-    scatter_slice<DPT>(i < end, key, val, (uint32_t)(key >> shift) & mask, cursor, wave_count, keys_out, vals_out);
+    part[half][0][d] = total;
+    part[half][1][d] = before;
+    for (int w = 0; w < kGlobalWaves; ++w) st.wave_count[half][w][d] = 0;
   }
+  __syncthreads();
+  uint32_t total = 0, before = 0;
+  if (t < kMaxDigits) {
+    total = part[0][0][t] + part[1][0][t];
+    before = part[0][1][t] + part[1][1][t];
+  }
+  uint32_t grand;
+  const uint32_t excl = block_exclusive_scan(total, kMaxDigits / 64, st.wave_total, &grand);
+  if (t < kMaxDigits) {
+    st.cursor[t] = excl + before;
+    if (me == 0) bucket_off[t] = excl;  // digits past the pass's width hold no keys: their offset is n
+  }
+  if (me == 0 && t == 0) bucket_off[kMaxDigits] = grand;
+  __syncthreads();
+  scatter_range<kGlobalWaves, kMaxDigitBits>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift,
+                                             (1u << digit_bits) - 1u, key_next, val_next);
 }
 
 // A local pass: block b sorts bucket b (positions [bucket_off[b], bucket_off[b + 1]))
 // by one digit of up to 8 bits, reading from the "in" pair and writing the same
 // positions of the "out" pair.
-__global__ __launch_bounds__(kSortThreads) void sort_bucket_kernel(
+__global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out, const uint32_t* __restrict__ bucket_off, int shift, int digit_bits) {
-  __shared__ uint32_t cursor[kSortThreads];
-  __shared__ uint32_t wave_count[4][kSortThreads];
-  __shared__ uint32_t wave_total[4];
+  __shared__ SliceState<kBucketWaves, 8> st;
   const int t = threadIdx.x;
   const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
   if (begin >= end) return;
@@ -219,35 +226,26 @@ __global__ __launch_bounds__(kSortThreads) void sort_bucket_kernel(
     key_next = keys_in[begin + t];
     val_next = vals_in[begin + t];
   }
-  cursor[t] = 0;
-  for (int w = 0; w < 4; ++w) wave_count[w][t] = 0;
+  st.cursor[t] = 0;
+  for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
   __syncthreads();
-  if (begin + t < end) atomicAdd(&cursor[(uint32_t)(key_next >> shift) & mask], 1u);
-  for (int64_t i = begin + kSortThreads + t; i < end; i += kSortThreads)
-    atomicAdd(&cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
+  if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
+  for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
+    atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
   __syncthreads();
-  uint32_t total[1] = {cursor[t]};
   uint32_t grand;
-  scan_digits<1>(total, wave_total, &grand);
-  cursor[t] = (uint32_t)begin + total[0];
+  const uint32_t excl = block_exclusive_scan(st.cursor[t], kBucketWaves, st.wave_total, &grand);
+  st.cursor[t] = (uint32_t)begin + excl;
   __syncthreads();
-  for (int64_t base = begin; base < end; base += kSortThreads) {
-    const int64_t i = base + t;
-    const uint64_t key = key_next;
-    const uint32_t val = val_next;
-    if (i + kSortThreads < end) {
-      key_next = keys_in[i + kSortThreads];
-      val_next = vals_in[i + kSortThreads];
-    }
-    scatter_slice<1>(i < end, key, val, (uint32_t)(key >> shift) & mask, cursor, wave_count, keys_out, vals_out);
-  }
+  scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
+                                 val_next);
 }
 
 }  // namespace
 
 size_t sort_temp_bytes(int64_t n) {
   SortPlan p = plan_sort(n);
-  return align_up(((size_t)(1 << kMaxDigitBits) * p.stride + (1 << kMaxDigitBits) + 1) * sizeof(uint32_t), 256);
+  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 1) * sizeof(uint32_t), 256);
 }
 
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
@@ -260,22 +258,17 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   if (low_bit < 0 || key_bits > 64 || low_bit > key_bits) return fail(PBG_ERR_INVALID, "sort_pairs: bad bit range");
   SortPlan p = plan_sort(n);
   uint32_t* counts = (uint32_t*)temp;
-  uint32_t* bucket_off = counts + (size_t)(1 << kMaxDigitBits) * p.stride;
+  uint32_t* bucket_off = counts + (size_t)kMaxDigits * p.blocks;
   int bits = key_bits - low_bit;
   if (bits < 1) bits = 1;
   const int top = bits < kMaxDigitBits ? bits : kMaxDigitBits;  // width of the global pass
   const int rest = bits - top;                                  // bits left for the bucket passes
   const int local = (rest + 7) / 8;
   const int top_shift = low_bit + rest;
-  hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kSortThreads), 0, stream, keys_in, n, p.tile_shift,
-                     top_shift, top, p.stride, counts);
-  if (top <= 8) {
-    hipLaunchKernelGGL(sort_scatter_kernel<1>, dim3(p.blocks), dim3(kSortThreads), 0, stream, keys_in, vals_in,
-                       keys_out, vals_out, n, p.tile_shift, top_shift, top, p.stride, counts, bucket_off);
-  } else {
-    hipLaunchKernelGGL(sort_scatter_kernel<2>, dim3(p.blocks), dim3(kSortThreads), 0, stream, keys_in, vals_in,
-                       keys_out, vals_out, n, p.tile_shift, top_shift, top, p.stride, counts, bucket_off);
-  }
+  hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, n, p.tile_shift,
+                     top_shift, top, counts);
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, vals_in,
+                     keys_out, vals_out, n, p.tile_shift, top_shift, top, counts, bucket_off);
   uint64_t* ksrc = keys_out;
   uint32_t* vsrc = vals_out;
   uint64_t* kdst = keys_in;
@@ -283,7 +276,7 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   int shift = low_bit;
   for (int pass = 0; pass < local; ++pass) {  // lowest digit first; digits of (almost) equal width
     const int width = (rest - (shift - low_bit) + (local - pass) - 1) / (local - pass);
-    hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kSortThreads), 0, stream, ksrc, vsrc, kdst, vdst,
+    hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kBucketWaves * 64), 0, stream, ksrc, vsrc, kdst, vdst,
                        bucket_off, shift, width);
     shift += width;
     uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
