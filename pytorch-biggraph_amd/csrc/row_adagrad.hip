@@ -311,6 +311,126 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   }
 }
 
+// The same for rows of at most 128 floats (dim % 4 == 0): half a wave per sorted
+// position, one 128-bit word per lane, so a wave keeps twice as many rows in
+// flight for the same registers.  The two halves of a wave run the same code on
+// different positions; everything that is uniform per position is uniform per
+// half only, so values cross lanes through shuffles inside the half, never
+// through scalar registers.
+__device__ __forceinline__ uint64_t half_bcast_u64(uint64_t v, int src) {
+  const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)v, src, 64);
+  const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)(v >> 32), src, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ float half_sum(float v) {  // sum over the 32 lanes of a half, in every lane
+  v = row16_sum(v);
+  return v + __shfl_xor(v, 16, 64);
+}
+__device__ __forceinline__ float4 load_or_zero(const float* __restrict__ p, bool has) {
+  return has ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+__device__ __forceinline__ float adagrad_apply_half(float4& w, const float4& g, float gsum, float fdim, float lr) {
+  gsum += half_sum(g.x * g.x + g.y * g.y + g.z * g.z + g.w * g.w) / fdim;
+  const float stdv = sqrtf(gsum) + 1e-10f;
+  w.x += (-lr * g.x) / stdv;
+  w.y += (-lr * g.y) / stdv;
+  w.z += (-lr * g.z) / stdv;
+  w.w += (-lr * g.w) / stdv;
+  return gsum;
+}
+
+template <int R>
+__global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
+    const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
+    const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
+    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
+  const int lane = threadIdx.x & 63, gl = lane & 31, gbase = lane & 32;
+  const int64_t first = ((((int64_t)blockIdx.x * kRowThreads) + threadIdx.x) >> 5) * R;
+  const bool has = gl < (dim >> 2);
+  const int col = gl << 2;
+  const float fdim = (float)dim;
+  // one coalesced look at each position and the 31 sorted positions after it
+  uint64_t kk[R], before[R];
+  uint32_t vv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t i = first + r < n ? first + r : n - 1;
+    const int64_t p = i + gl < n ? i + gl : n - 1;
+    kk[r] = keys[p];
+    vv[r] = vals[p];
+    before[r] = keys[i > 0 ? i - 1 : 0];
+  }
+  bool head[R];
+  float* wrow[R];
+  float* gptr[R];
+  float gsum[R];
+  float4 w[R], g[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t i = first + r;
+    const uint64_t row = half_bcast_u64(kk[r], gbase) >> kbits;
+    // out-of-range indices are parked past both tables
+    head[r] = i < n && !(i > 0 && (before[r] >> kbits) == row) && (int64_t)row < rows0 + rows1;
+    if (!head[r]) continue;
+    if ((int64_t)row < rows0) {
+      wrow[r] = w0 + (int64_t)row * dim + col;
+      gptr[r] = g0 + row;
+    } else {
+      wrow[r] = w1 + ((int64_t)row - rows0) * dim + col;
+      gptr[r] = g1 + ((int64_t)row - rows0);
+    }
+    w[r] = load_or_zero(wrow[r], has);
+    gsum[r] = *gptr[r];
+    g[r] = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase, 64) * dim + col, has);
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (!head[r]) continue;
+    const int64_t i = first + r;
+    const uint64_t row = half_bcast_u64(kk[r], gbase) >> kbits;
+    const uint32_t in_row = (uint32_t)(__ballot(i + gl < n && (kk[r] >> kbits) == row) >> gbase);
+    if (in_row != 0xffffffffu) {
+      // the row ends inside the window: its runs are known from the keys in registers
+      const int len = __ffs((int)~in_row) - 1;
+      const uint64_t up = __shfl_up((unsigned long long)kk[r], 1, 64);
+      uint32_t heads = (uint32_t)(__ballot(gl < len && (gl == 0 || up != kk[r])) >> gbase);  // first position of every run
+      heads &= heads - 1;
+      while (heads != 0u) {  // the next run's row is in flight while this one is applied
+        const int a = __ffs((int)heads) - 1;
+        heads &= heads - 1;
+        const float4 next = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + a, 64) * dim + col, has);
+        gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+        g[r] = next;
+      }
+      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+    } else {
+      int64_t j = i;
+      while (true) {
+        if (kbits == 0) {  // a single-worker call has one run per row
+          j = n;
+        } else {
+          const uint64_t key = keys[j];
+          int64_t base = j + 1;
+          while (true) {  // first position after j with another key, 32 positions at a time
+            const int64_t q = base + gl;
+            const uint32_t same = (uint32_t)(__ballot(q < n && keys[q < n ? q : n - 1] == key) >> gbase);
+            if (same != 0xffffffffu) {
+              j = base + (__ffs((int)~same) - 1);
+              break;
+            }
+            base += 32;
+          }
+        }
+        gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+        if (j >= n || (keys[j] >> kbits) != row) break;
+        g[r] = load_or_zero(grad_rows + (int64_t)vals[j] * dim + col, has);
+      }
+    }
+    if (has) *reinterpret_cast<float4*>(wrow[r]) = w[r];
+    if (gl == 0) *gptr[r] = gsum[r];
+  }
+}
+
 // keys for the stand-alone sparse step: key = row index, value = position
 __global__ void make_keys_kernel(const int64_t* __restrict__ idx, int64_t n, int64_t num_rows,
                                  uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
@@ -364,7 +484,12 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim);  \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
-    {                                                                                                              \
+    if (VEC && dim <= 128) {                                                                                       \
+      constexpr int R = 4;                                                                                         \
+      const dim3 hgrid((unsigned)ceil_div(ceil_div(n, R) * 32, kRowThreads));                                      \
+      hipLaunchKernelGGL((row_update_half_kernel<R>), hgrid, block, 0, stream, keys, vals, n, kbits, grad_rows,    \
+                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+    } else {                                                                                                       \
       constexpr int R = NV <= 2 ? 4 : (NV <= 4 ? 2 : 1);                                                           \
       const dim3 ugrid((unsigned)ceil_div(ceil_div(n, R), wpb));                                                   \
       hipLaunchKernelGGL((row_update_kernel<NV, VEC, R>), ugrid, block, 0, stream, keys, vals, n, kbits, grad_rows, \
