@@ -19,7 +19,7 @@ namespace pbg {
 namespace {
 
 constexpr int kGlobalWaves = 16;  // global pass: 1024 threads per block
-constexpr int kBucketWaves = 4;   // bucket passes: 256 threads per block
+constexpr int kBucketWaves = 16;  // bucket passes: 1024 threads per block, for the sake of buckets swollen by hot keys
 constexpr int kMaxDigitBits = 9;
 constexpr int kMaxDigits = 1 << kMaxDigitBits;
 constexpr int kMaxSortBlocks = 256;
@@ -226,16 +226,18 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
     key_next = keys_in[begin + t];
     val_next = vals_in[begin + t];
   }
-  st.cursor[t] = 0;
-  for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
+  if (t < 256) {
+    st.cursor[t] = 0;
+    for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
+  }
   __syncthreads();
   if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
   for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
     atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
   __syncthreads();
   uint32_t grand;
-  const uint32_t excl = block_exclusive_scan(st.cursor[t], kBucketWaves, st.wave_total, &grand);
-  st.cursor[t] = (uint32_t)begin + excl;
+  const uint32_t excl = block_exclusive_scan(t < 256 ? st.cursor[t] : 0u, 4, st.wave_total, &grand);
+  if (t < 256) st.cursor[t] = (uint32_t)begin + excl;
   __syncthreads();
   scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
                                  val_next);

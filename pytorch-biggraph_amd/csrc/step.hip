@@ -708,14 +708,28 @@ __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at
   constexpr bool l2 = CMP == PBG_CMP_L2;
   float t[kQuadCols];
   uint32_t live = 0xffffffffu;  // bit e clear: column qd + 4e is a constant with no gradient
+  if (!l2) {
 #pragma unroll
-  for (int e = 0; e < kQuadCols; ++e) t[e] = lds[row_at + min(qd + 4 * e, N - 1)];
-  if (l2) {
+    for (int e = 0; e < kQuadCols; ++e) t[e] = lds[row_at + min(qd + 4 * e, N - 1)];
+  } else {
+    // eight columns at a time, fenced, so that the scheduler does not pull all 64
+    // loads to the front and run out of registers
 #pragma unroll
-    for (int e = 0; e < kQuadCols; ++e) {
-      const float q = fmaf(-2.0f, t[e], lds[bn_at + min(qd + 4 * e, N - 1)]) + a2;
-      if (!(q >= 1e-30f)) live &= ~(1u << e);
-      t[e] = -sqrtf(fmaxf(q, 1e-30f));
+    for (int e0 = 0; e0 < kQuadCols; e0 += 8) {
+      float raw[8], bn[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = min(qd + 4 * (e0 + u), N - 1);
+        raw[u] = lds[row_at + j];
+        bn[u] = lds[bn_at + j];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float q = fmaf(-2.0f, raw[u], bn[u]) + a2;
+        if (!(q >= 1e-30f)) live &= ~(1u << (e0 + u));
+        t[e0 + u] = -sqrtf(fmaxf(q, 1e-30f));
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 #pragma unroll
