@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
+# HBM bytes per launch of (workload, kernel) at the default --workers, from the
+# rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under profiles/ (not measured live).
+TRAFFIC = {}
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
@@ -140,6 +143,14 @@ def algorithmic(w, spec):
         op_rows = b + c * u
         out["operator"] = ("mfma", 2.0 * op_rows * d * d)
         out["params"] = ("mfma", 2.0 * 2 * op_rows * d * d)
+    # The LDS-resident chunk kernel does gather, operator, scores, loss, backward
+    # and the chain rule in one launch: forward + 2 x backward multiply-adds of the
+    # positive pairs and of both score matrices.  Its arithmetic intensity
+    # (flops / (rows read once + gradient rows written once)) is above the
+    # machine balance of 157.3 TFLOP/s : 8 TB/s = 20 flop/byte, so the matrix
+    # cores are the roofline that bounds it.
+    out["fused_chunk"] = ("mfma", 3 * 2.0 * (b * d + 2 * c * p * n * d))
+    out["fused_chunk_bytes"] = rows * (2 * 4 * d + 8) + 3 * b * 8
     return out
 
 
@@ -265,6 +276,10 @@ def main():
                 ms = one_call(warm_calls + calls + i, profiled=True)
                 acc = ms if acc is None else [a + m for a, m in zip(acc, ms)]
             stages = dict(zip(runner.STAGES, [a / profile_calls for a in acc]))
+            if runner.fused:
+                # one kernel covers stages "prep" .. "rowback"; "loss" holds the per-batch reduction of the statistics
+                stages = {"fused_chunk": stages["prep"], "loss_reduce": stages["loss"], "params": stages["params"],
+                          "sort": stages["sort"], "update": stages["update"]}
         loss = float(runner.loss_out.mean().item()) / b
         return spec, calls * per_call / dt, dt / (calls * workers) * 1e3, calls * workers, stages, loss
 
@@ -292,13 +307,16 @@ def main():
         achieved, peak, unit = units / seconds / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
-        "frac": achieved / peak, "traffic": None, "launches_in_stage": launches,
+        "frac": achieved / peak, "traffic": TRAFFIC.get((args.workload, dominant)), "launches_in_stage": launches,
         "avg_launch_ms": stages[dominant] / launches,
         "stages_ms": stages,
         "all": {k: {"bound": alg[k][0],
                     "achieved": (alg[k][1] * workers / (stages[k] * 1e-3) / (1e9 if alg[k][0] == "hbm" else 1e12)) if stages[k] > 0 else None}
                 for k in stages if k in alg},
     }
+    if dominant == "fused_chunk":
+        # the same launch against the other roofline: rows read once + gradient rows written once
+        roofline["algorithmic_hbm_gbs"] = alg["fused_chunk_bytes"] * workers / seconds / 1e9
 
     line = {
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X",

@@ -163,6 +163,11 @@ int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_
  * 8 key sort, 9 RowAdagrad update.  No counterpart in the reference (it logs wall-clock per bucket,
  * train_cpu.py:696-703). */
 int pbg_train_step_num_stages(void);
+/* 1 when pbg_train_step runs this configuration's chain from the gather to the
+ * raw-row gradients as ONE kernel with a chunk's operands resident in LDS (then
+ * stage 0 is that kernel and stages 1-6 are empty), 0 when it runs the staged
+ * kernels.  No counterpart in the reference. */
+int pbg_train_step_is_fused(const pbg_step_desc* desc);
 int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,
                            float* stage_ms);
 

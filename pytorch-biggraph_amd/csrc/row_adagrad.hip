@@ -38,6 +38,48 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const float* _
   }
 }
 
+// Rows of at most 4 * LPR floats (dim % 4 == 0): LPR lanes per row, one 128-bit
+// word per lane, and U rows per lane group, so that a wave has 64 / LPR * U row
+// reads in flight at once.  A short row is a single memory request; the kernel
+// is as fast as the number of requests the chip keeps outstanding.
+template <int LPR, int U>
+__global__ __launch_bounds__(kRowThreads) void gather_rows_multi_kernel(const float* __restrict__ table,
+                                                                        int64_t num_rows, int dim,
+                                                                        const int64_t* __restrict__ idx, int64_t n,
+                                                                        float* __restrict__ out,
+                                                                        int32_t* __restrict__ oob_flag) {
+  constexpr int kGroups = kWave / LPR;      // rows a wave moves per step
+  constexpr int kRowsPerWave = kGroups * U;
+  const int lane = threadIdx.x & 63;
+  const int q = lane / LPR, v = lane % LPR;
+  const int64_t wave = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  const int64_t base = wave * kRowsPerWave + q;
+  const bool col_ok = v < (dim >> 2);
+  int64_t r[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kGroups;
+    r[u] = i < n ? idx[i] : 0;
+  }
+  float4 x[U];
+  bool bad = false;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const bool in = base + u * kGroups < n;
+    const bool ok = r[u] >= 0 && r[u] < num_rows;
+    bad |= in && !ok;
+    x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (ok && col_ok && in)
+      x[u] = reinterpret_cast<const float4*>(table + r[u] * (int64_t)dim)[v];
+  }
+  if (bad && v == 0 && oob_flag) *oob_flag = 1;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kGroups;
+    if (col_ok && i < n) reinterpret_cast<float4*>(out + i * (int64_t)dim)[v] = x[u];
+  }
+}
+
 // ---- segmented RowAdagrad over sorted keys -----------------------------------
 // Keys are (row << kbits | worker), sorted.  Equal keys form a "run" (the
 // duplicates of one row inside one worker's batch, to be summed); the runs of
@@ -536,7 +578,20 @@ extern "C" int pbg_gather_rows(const float* table, int64_t num_rows, int32_t dim
   const dim3 grid((unsigned)ceil_div(n, kRowThreads / kWave)), block(kRowThreads);
   hipStream_t s = (hipStream_t)stream;
   const bool vec = dim % 4 == 0 && ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0);
-  if (vec) {
+  if (vec && dim <= 256) {
+    constexpr int kU = 8;
+    const int waves_per_block = kRowThreads / kWave;
+    if (dim <= 64) {
+      const dim3 g((unsigned)ceil_div(n, (int64_t)waves_per_block * 4 * kU));
+      hipLaunchKernelGGL((gather_rows_multi_kernel<16, kU>), g, block, 0, s, table, num_rows, dim, idx, n, out, oob_flag);
+    } else if (dim <= 128) {
+      const dim3 g((unsigned)ceil_div(n, (int64_t)waves_per_block * 2 * kU));
+      hipLaunchKernelGGL((gather_rows_multi_kernel<32, kU>), g, block, 0, s, table, num_rows, dim, idx, n, out, oob_flag);
+    } else {
+      const dim3 g((unsigned)ceil_div(n, (int64_t)waves_per_block * kU));
+      hipLaunchKernelGGL((gather_rows_multi_kernel<64, kU>), g, block, 0, s, table, num_rows, dim, idx, n, out, oob_flag);
+    }
+  } else if (vec) {
     hipLaunchKernelGGL(gather_rows_kernel<true>, grid, block, 0, s, table, num_rows, dim, idx, n, out, oob_flag);
   } else {
     hipLaunchKernelGGL(gather_rows_kernel<false>, grid, block, 0, s, table, num_rows, dim, idx, n, out, oob_flag);

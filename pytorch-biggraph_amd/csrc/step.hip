@@ -1974,6 +1974,13 @@ extern "C" int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers*
 
 extern "C" int pbg_train_step_num_stages(void) { return kStages; }
 
+extern "C" int pbg_train_step_is_fused(const pbg_step_desc* desc) {
+  if (validate(desc, true) != PBG_OK) return 0;
+  Plan plan;
+  make_plan(desc, nullptr, &plan);
+  return plan.fused ? 1 : 0;
+}
+
 extern "C" int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,
                                       float* stage_ms) {
   if (!stage_ms) return fail(PBG_ERR_INVALID, "pbg_train_step_profile: null output");

@@ -316,6 +316,11 @@ class StepRunner:
 
     STAGES = ("prep", "operator", "scores", "loss", "backward_dn", "backward_da", "rowback", "params", "sort", "update")
 
+    @property
+    def fused(self) -> bool:
+        """True when the step runs as the single LDS-resident chunk kernel."""
+        return bool(_lib.lib().pbg_train_step_is_fused(ctypes.byref(self.desc)))
+
     def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> List[float]:
         """train() with HIP events between the stages; synchronises and returns
         the stage durations in milliseconds (order: StepRunner.STAGES)."""
