@@ -17,6 +17,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kGemmThreads = 256;
 constexpr int BK = 16;
 constexpr int PAD = 16;
+constexpr int kFoldTiles = 8;  // depth-16 tiles per partial sum (128 values of k)
 
 struct Quad {
   float v[4];
@@ -86,7 +87,7 @@ struct TileLoader {
 };
 
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR>
-__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g, int a_vec, int b_vec) {
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g, int a_vec, int b_vec) {
   constexpr int TM = BM / 2 / 16;  // MFMA tiles per wave along m
   constexpr int TN = BN / 2 / 16;
   __shared__ __attribute__((aligned(16))) float lds_a[2][BK * (BM + PAD)];
@@ -106,11 +107,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g, int a_ve
         g.b + (int64_t)batch * g.stride_b + (g.b_index ? g.b_index[batch] * g.b_index_stride : 0);
     float* __restrict__ c = g.c + (int64_t)batch * g.stride_c;
 
-    float4v acc[TM][TN];
+    // Blocked summation: `acc` collects kFoldTiles depth-16 tiles, then is folded
+    // into `tot`.  A single accumulator over k = 1000 is a sequential fp32 sum of
+    // 250 partial products, whose rounding errors add up coherently when the terms
+    // are alike (a power-law batch repeats the same rows); two levels keep the
+    // error at that of a blocked CPU BLAS.
+    float4v acc[TM][TN], tot[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = (float4v){0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j] = (float4v){0.f, 0.f, 0.f, 0.f};
+        tot[i][j] = (float4v){0.f, 0.f, 0.f, 0.f};
+      }
 
     TileLoader<BM, A_KMAJOR> la;
     TileLoader<BN, B_KMAJOR> lb;
@@ -143,6 +152,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g, int a_ve
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
       }
+      if ((kt & (kFoldTiles - 1)) == kFoldTiles - 1) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            tot[i][j] += acc[i][j];
+            acc[i][j] = (float4v){0.f, 0.f, 0.f, 0.f};
+          }
+      }
       if (kt + 1 < nk) {
         la.stash(lds_a[cur ^ 1]);
         lb.stash(lds_b[cur ^ 1]);
@@ -161,7 +179,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g, int a_ve
           const int row = m0 + wm0 + i * 16 + 4 * (lane >> 4) + r;
           if (row < g.m && col < g.n) {
             float* dst = c + (int64_t)row * g.ldc + col;
-            float v = g.alpha * acc[i][j][r];
+            float v = g.alpha * (tot[i][j][r] + acc[i][j][r]);
             if (g.beta != 0.f) v += g.beta * *dst;
             *dst = v;
           }
