@@ -61,4 +61,22 @@ struct GemmArgs {
 };
 int gemm_f32(const GemmArgs& args, hipStream_t stream);
 
+// ---- `linear` operator with one relation per edge, over edges sorted by relation ----
+// keys[n] = (relation << kbits | batch), sorted ascending; vals[n] = edge number
+// e = batch * edges_per_batch + position.  Row of edge e in an array laid out
+// [batches, batch_stride rows, dim]: (e / edges_per_batch) * batch_stride + e % edges_per_batch.
+//   out[e] (+)= W[rel_e] in[e]     (transpose_w = false)
+//   out[e] (+)= W[rel_e]^T in[e]   (transpose_w = true)
+int seg_linear_apply(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, int edges_per_batch,
+                     const float* in, int64_t in_batch_stride, const float* w, int dim, bool transpose_w, float* out,
+                     int64_t out_batch_stride, bool accumulate, hipStream_t stream);
+// For every relation and batch present: dW = sum over the run's edges of dz[e] (x) x[e]
+// (dz, x: [n, dim] by edge number), then wsum += dW^2, w -= lr * dW / (sqrt(wsum) + 1e-10),
+// batch after batch in ascending order.
+// `temp` holds seg_linear_update_temp_bytes(num_relations) bytes.
+size_t seg_linear_update_temp_bytes(int num_relations);
+int seg_linear_update(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, const float* dz,
+                      const float* x, int dim, int num_relations, float* w, float* wsum, float lr, void* temp,
+                      hipStream_t stream);
+
 }  // namespace pbg

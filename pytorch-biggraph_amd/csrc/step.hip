@@ -1235,43 +1235,6 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
 // ---------------------------------------------------------------------------
 // operator parameters, dynamic relations (one relation per edge)
 // ---------------------------------------------------------------------------
-// `linear` with a relation per row: z_e = W[rel_e] x_e, one wave per positive
-// (operators.py:259-269).  Reads the raw rows staged by prep.
-__global__ __launch_bounds__(kRowThreads) void dyn_linear_forward_kernel(StepCtx c, int s) {
-  const SideCtx& sd = c.side[s];
-  const int lane = threadIdx.x & 63;
-  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (job >= (int64_t)c.K * c.B) return;
-  const int D = c.D;
-  const float* m = sd.p0 + clamp_index(c.rel[job], c.num_relations) * D * D;
-  const float* x = sd.xraw + job * D;
-  float* z = sd.z + job * D;
-  for (int o = 0; o < D; ++o) {
-    float acc = 0.f;
-    for (int d = lane; d < D; d += kWave) acc += m[(int64_t)o * D + d] * x[d];
-    acc = wave_sum(acc);
-    if (lane == 0) z[o] = acc;
-  }
-}
-
-// gr[row of e] += W[rel_e]^T dz_e
-__global__ __launch_bounds__(kRowThreads) void dyn_linear_backward_kernel(StepCtx c, int s) {
-  const SideCtx& sd = c.side[s];
-  const int lane = threadIdx.x & 63;
-  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (job >= (int64_t)c.K * c.B) return;
-  const int D = c.D;
-  const int k = (int)(job / c.B), q = (int)(job % c.B);
-  const float* m = sd.p0 + clamp_index(c.rel[job], c.num_relations) * D * D;
-  const float* g = sd.dz + job * D;
-  float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + q) * D;
-  for (int d = lane; d < D; d += kWave) {
-    float acc = 0.f;
-    for (int o = 0; o < D; ++o) acc += m[(int64_t)o * D + d] * g[o];
-    out[d] += acc;
-  }
-}
-
 // sort keys (relation << kbits | batch) of every positive, value = k * B + q
 __global__ void rel_keys_kernel(StepCtx c, uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1362,75 +1325,6 @@ __global__ __launch_bounds__(256) void dyn_param_kernel(StepCtx c, int s, const 
   }
 }
 
-// `linear`: one workgroup per (relation present, 64 x 64 tile of its matrix); thread
-// (ty, tx) owns a 4 x 4 block of dW[o, i] = sum over the run's edges of dz[o] x[i].
-__global__ __launch_bounds__(256) void dyn_linear_param_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
-                                                               const uint32_t* __restrict__ vals, float* w,
-                                                               float* wsum, float lr) {
-  constexpr int kRows = 16;
-  __shared__ float sh_dz[kRows][64];
-  __shared__ float sh_x[kRows][64];
-  __shared__ int64_t sh_end;
-  const SideCtx& sd = c.side[s];
-  const int64_t n = (int64_t)c.K * c.B;
-  const int64_t i = blockIdx.x;
-  const uint64_t rel = keys[i] >> c.kbits;
-  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;
-  const int D = c.D;
-  const int tiles = (D + 63) / 64;
-  const int o0 = (blockIdx.y / tiles) * 64, i0 = (blockIdx.y % tiles) * 64;
-  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
-  float* wr = w + (int64_t)rel * D * D;
-  float* sr = wsum + (int64_t)rel * D * D;
-  int64_t j = i;
-  while (j < n && (keys[j] >> c.kbits) == rel) {
-    const int64_t end = block_scan_end(keys, j, n, keys[j], 0, &sh_end);
-    float acc[4][4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
-    for (int64_t r0 = j; r0 < end; r0 += kRows) {
-      // stage up to kRows edges: 64 values of dz (rows of the tile) and of x (columns of the tile) each
-      for (int t = threadIdx.x; t < kRows * 64; t += 256) {
-        const int rr = t >> 6, col = t & 63;
-        float vdz = 0.f, vx = 0.f;
-        if (r0 + rr < end) {
-          const int64_t edge = vals[r0 + rr];
-          if (o0 + col < D) vdz = sd.dz[edge * D + o0 + col];
-          if (i0 + col < D) vx = sd.xraw[edge * D + i0 + col];
-        }
-        sh_dz[rr][col] = vdz;
-        sh_x[rr][col] = vx;
-      }
-      __syncthreads();
-#pragma unroll 4
-      for (int rr = 0; rr < kRows; ++rr) {
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-          for (int b = 0; b < 4; ++b) acc[a][b] += sh_dz[rr][ty * 4 + a] * sh_x[rr][tx * 4 + b];
-      }
-      __syncthreads();
-    }
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int o = o0 + ty * 4 + a, ii = i0 + tx * 4 + b;
-        if (o < D && ii < D) {
-          const int64_t at = (int64_t)o * D + ii;
-          const float g = acc[a][b];
-          const float sum = sr[at] + g * g;
-          sr[at] = sum;
-          wr[at] += -lr * (g / (sqrtf(sum) + 1e-10f));
-        }
-      }
-    }
-    j = end;
-  }
-}
-
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -1450,6 +1344,7 @@ struct Plan {
   uint64_t *rkeys_a, *rkeys_b;
   uint32_t *rvals_a, *rvals_b;
   void* rsort_temp;
+  void* rel_start;  // first sorted position of every relation (`linear` only)
   int nvh;
 };
 
@@ -1590,6 +1485,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     plan->rvals_a = (uint32_t*)take(ne, 4);
     plan->rvals_b = (uint32_t*)take(ne, 4);
     plan->rsort_temp = take(sort_temp_bytes(ne), 1);
+    if (c.op == PBG_OP_LINEAR) plan->rel_start = take(seg_linear_update_temp_bytes(c.num_relations), 1);
   }
   for (int s = 0; s < 2; ++s) {
     plan->pslices[s] = 1;
@@ -1683,15 +1579,38 @@ int run_prep(const Plan& plan, hipStream_t stream) {
   return check_launch("step prep");
 }
 
+// Dynamic relations: the call's edges ordered by (relation, batch).  Built once
+// per call, by the first stage that needs it.
+struct RelOrder {
+  uint64_t* keys = nullptr;
+  uint32_t* vals = nullptr;
+};
+
+int ensure_rel_order(const Plan& plan, hipStream_t stream, RelOrder* ro) {
+  if (ro->keys) return PBG_OK;
+  const StepCtx& c = plan.c;
+  const int64_t ne = (int64_t)c.K * c.B;
+  hipLaunchKernelGGL(rel_keys_kernel, dim3((unsigned)ceil_div(ne, 256)), dim3(256), 0, stream, c, plan.rkeys_a,
+                     plan.rvals_a);
+  // the edges arrive in batch order, so sorting on the relation bits orders by (relation, batch)
+  return sort_pairs(plan.rkeys_a, plan.rvals_a, plan.rkeys_b, plan.rvals_b, ne, c.kbits,
+                    bits_for((uint64_t)(c.num_relations - 1)) + c.kbits, plan.rsort_temp, stream, &ro->keys, &ro->vals);
+}
+
 // the `linear` operator: one GEMM per side that has it, then comparator.prepare
-int run_operator_forward(const Plan& plan, hipStream_t stream) {
+int run_operator_forward(const Plan& plan, hipStream_t stream, RelOrder* ro) {
   const StepCtx& c = plan.c;
   const int D = c.D, K = c.K;
   int rc;
   if (c.op == PBG_OP_LINEAR && c.dynamic) {
+    if ((rc = ensure_rel_order(plan, stream, ro)) != PBG_OK) return rc;
+    const int64_t ne = (int64_t)K * c.B;
     for (int s = 0; s < 2; ++s) {
-      hipLaunchKernelGGL(dyn_linear_forward_kernel, wave_grid((int64_t)K * c.B), dim3(kRowThreads), 0, stream, c, s);
-      PBG_DISPATCH_NVH(plan.nvh, prepare_staged_kernel, wave_grid((int64_t)K * c.B), stream, c, s);
+      const SideCtx& sd = c.side[s];  // z_e = W[rel_e] x_e (operators.py:259-269)
+      if ((rc = seg_linear_apply(ro->keys, ro->vals, ne, c.kbits, c.B, sd.xraw, sd.op_rows, sd.p0, D, false, sd.z,
+                                 sd.op_rows, false, stream)) != PBG_OK)
+        return rc;
+      PBG_DISPATCH_NVH(plan.nvh, prepare_staged_kernel, wave_grid(ne), stream, c, s);
     }
     return check_launch("step operator");
   }
@@ -1781,30 +1700,31 @@ int run_rowback(const Plan& plan, hipStream_t stream) {
   return check_launch("step rowback");
 }
 
-int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, hipStream_t stream) {
+int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, hipStream_t stream,
+               RelOrder* ro) {
   const StepCtx& c = plan.c;
   if (c.op == PBG_OP_NONE) return PBG_OK;
   const int D = c.D, K = c.K;
   int rc;
   if (c.dynamic) {
     const int64_t ne = (int64_t)K * c.B;
-    hipLaunchKernelGGL(rel_keys_kernel, dim3((unsigned)ceil_div(ne, 256)), dim3(256), 0, stream, c, plan.rkeys_a,
-                       plan.rvals_a);
-    uint64_t* rkeys;  // the edges arrive in batch order, so sorting on the relation bits orders by (relation, batch)
-    uint32_t* rvals;
-    rc = sort_pairs(plan.rkeys_a, plan.rvals_a, plan.rkeys_b, plan.rvals_b, ne, c.kbits,
-                    bits_for((uint64_t)(c.num_relations - 1)) + c.kbits, plan.rsort_temp, stream, &rkeys, &rvals);
-    if (rc != PBG_OK) return rc;
+    if ((rc = ensure_rel_order(plan, stream, ro)) != PBG_OK) return rc;
+    uint64_t* rkeys = ro->keys;
+    uint32_t* rvals = ro->vals;
     for (int s = 0; s < 2; ++s) {
+      const SideCtx& sd = c.side[s];
       float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
       float* p1 = s == 0 ? b->lhs_op_p1 : b->rhs_op_p1;
       float* s0 = s == 0 ? b->lhs_op_s0 : b->rhs_op_s0;
       float* s1 = s == 0 ? b->lhs_op_s1 : b->rhs_op_s1;
       if (c.op == PBG_OP_LINEAR) {
-        hipLaunchKernelGGL(dyn_linear_backward_kernel, wave_grid(ne), dim3(kRowThreads), 0, stream, c, s);
-        const int tiles = (D + 63) / 64;
-        hipLaunchKernelGGL(dyn_linear_param_kernel, dim3((unsigned)ne, (unsigned)(tiles * tiles)), dim3(256), 0, stream,
-                           c, s, rkeys, rvals, p0, s0, d->relation_lr);
+        // gr[row of e] += W[rel_e]^T dz_e, then the relation matrices' own step
+        if ((rc = seg_linear_apply(rkeys, rvals, ne, c.kbits, c.B, sd.dz, sd.op_rows, sd.p0, D, true,
+                                   c.gr + (int64_t)sd.slot_pos * D, c.rk, true, stream)) != PBG_OK)
+          return rc;
+        if ((rc = seg_linear_update(rkeys, rvals, ne, c.kbits, sd.dz, sd.xraw, D, c.num_relations, p0, s0,
+                                    d->relation_lr, plan.rel_start, stream)) != PBG_OK)
+          return rc;
       } else {
         hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
                            rkeys, rvals, p0, p1, s0, s1, d->relation_lr);
@@ -1912,6 +1832,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   make_plan(desc, bufs, &plan);
   if ((rc = check_buffers(desc, bufs, plan, true)) != PBG_OK) return rc;
   const StepCtx& c = plan.c;
+  RelOrder rel_order;
   auto mark = [&](int i) {
     if (ev) hipEventRecord(ev[i], s);
   };
@@ -1931,7 +1852,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   } else {
     if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
     mark(1);
-    if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
+    if ((rc = run_operator_forward(plan, s, &rel_order)) != PBG_OK) return rc;
     mark(2);
     if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
     mark(3);
@@ -1945,7 +1866,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
     mark(7);
   }
-  if ((rc = run_params(desc, bufs, plan, s)) != PBG_OK) return rc;
+  if ((rc = run_params(desc, bufs, plan, s, &rel_order)) != PBG_OK) return rc;
   mark(8);
   const int64_t npairs = (int64_t)c.K * c.rk;
   const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
@@ -2011,8 +1932,9 @@ extern "C" int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffe
   if (!lhs_pos || !rhs_pos || (c.side[0].nn > 0 && !lhs_neg) || (c.side[1].nn > 0 && !rhs_neg))
     return fail(PBG_ERR_INVALID, "pbg_model_forward: null output");
   hipStream_t s = (hipStream_t)stream;
+  RelOrder rel_order;
   if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
-  if ((rc = run_operator_forward(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_operator_forward(plan, s, &rel_order)) != PBG_OK) return rc;
   if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
   hipLaunchKernelGGL(scores_out_kernel, wave_grid((int64_t)c.K * c.B), dim3(kRowThreads), 0, s, c, lhs_pos, rhs_pos,
                      lhs_neg, rhs_neg);
