@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the PBG training step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1] [--workers 40]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1] [--workers 64]
 
 A "step" is one batch of `batch_size` edges through the whole hot path (gather,
 operator, scoring against batch + uniform negatives, loss, backward, RowAdagrad
@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of (workload, kernel) at the default --workers, from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under profiles/ (not measured live).
-TRAFFIC = {("cfg1", "fused_chunk"): 145.5e6, ("cfg1", "update"): 152.5e6}
+TRAFFIC = {("cfg1", "fused_chunk"): 232.7e6}  # 64 workers
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
@@ -160,7 +160,8 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed batches")
     ap.add_argument("--warmup", type=int, default=None, help="untimed batches")
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
-    ap.add_argument("--workers", type=int, default=40, help="batches in flight per call (HOGWILD workers)")
+    ap.add_argument("--workers", type=int, default=64,
+                    help="batches in flight per call (HOGWILD workers); 64 batches of cfg1 are 1280 chunks = 5 per compute unit")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="length of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-sequential", action="store_true", help="skip the workers=1 measurement")
     ap.add_argument("--calibrate-copy", action="store_true",
