@@ -684,7 +684,6 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
 typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kFusedThreads = 512;
 constexpr int kFusedIds = 256;  // slots of the row id array: 8 waves x 16 rounds x 2 half-waves
-constexpr int kQuadCols = 32;   // score columns per lane of a quad: N <= 128
 
 struct FusedLayout {
   int ldx, lds;                  // row strides (floats) of the operand rows and of the score rows
@@ -701,7 +700,7 @@ struct FusedLayout {
 // Columns at or past N act as scores of -inf: they add nothing to any loss and
 // are never written back.  Overwrites the row with dLoss/dscore (l2: -2 dLoss/d
 // squared distance); the outputs are quad-reduced.
-template <int CMP, int LOSS>
+template <int CMP, int LOSS, int kQuadCols>
 __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at, float a2, float margin, int N, int nb,
                                                int i, int masked_from, float pos, float w, int qd, float* loss_w,
                                                float* dpos_out, int* viol_out, float* rowsum_out) {
@@ -962,7 +961,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       __syncthreads();  // (a) operand rows of chunk kc in LDS
       if (kn < num_chunks) fused_load_ids(c, g, kn, t, ids);
       __syncthreads();  // (b)
-      __syncthreads();  // (c)
+      if (l2) __syncthreads();  // (c)
       __syncthreads();  // (d)
       __syncthreads();  // (e)
       __syncthreads();  // (f)
@@ -1015,6 +1014,12 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
               *reinterpret_cast<float4*>(&lds[at + ct * 16]) =
                   make_float4(acc[ct][0], col + 1 < N ? acc[ct][1] : 0.f, col + 2 < N ? acc[ct][2] : 0.f,
                               col + 3 < N ? acc[ct][3] : 0.f);
+            // dot: the i-th batch negative of the rhs side is the i-th positive's own rhs
+            // row, so the positive score is the diagonal of this block (model.py:177)
+            if (!l2 && s == 1 && row >= col && row < col + 4) {
+              const int r = row - col;
+              lds[f.pos + row] = r == 0 ? acc[ct][0] : (r == 1 ? acc[ct][1] : (r == 2 ? acc[ct][2] : acc[ct][3]));
+            }
           }
         }
       }
@@ -1023,7 +1028,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 
     // ---- phase 2: loss, dLoss/dS in place; one quad of lanes per (edge, side), columns interleaved ----
     const int qd = t & 3;
-    if (t < 4 * P) {  // positive scores (model.py:177,207,267-274)
+    if (l2 && t < 4 * P) {  // positive scores in the direct form (model.py:267-274)
       const int i = t >> 2;
       float acc = 0.f;
       for (int d0 = qd; d0 < D; d0 += 32) {  // eight columns of both rows in flight
@@ -1041,7 +1046,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       acc = quad_sum(acc);
       if (qd == 0) lds[f.pos + i] = l2 ? -sqrtf(fmaxf(acc, 1e-30f)) : acc;
     }
-    __syncthreads();  // (c)
+    if (l2) __syncthreads();  // (c)
     if (t < 8 * P) {
       const int pair = t >> 2;
       const int s = pair >= P, i = pair - s * P;
@@ -1053,7 +1058,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       } else {
         float w = c.rel_weights[rel];
         if (c.edge_weight) w *= c.edge_weight[(int64_t)k * c.B + cc * P + i];
-        quad_side_loss<CMP, LOSS>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f, c.margin, N, P,
+        quad_side_loss<CMP, LOSS, (l2 ? 32 : TN * 4)>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f, c.margin, N, P,
                                   i, valid, lds[f.pos + i], w, qd, &loss_w, &dpos_s, &viol, &rowsum);
       }
       if (qd == 0) {
