@@ -963,7 +963,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       __syncthreads();  // (b)
       if (l2) __syncthreads();  // (c)
       __syncthreads();  // (d)
-      __syncthreads();  // (e)
+      if (l2) __syncthreads();  // (e)
       __syncthreads();  // (f)
       // Issued here, the loads have the whole of phase 3 (no barriers inside) to
       // enter the memory pipeline; issued earlier, the loader waves would sit in
@@ -1075,15 +1075,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       c.lossrow[job] = lds[f.part + 1 * P + t] + lds[f.part + 4 * P + t];
       c.violrow[job * 2] = __float_as_int(lds[f.part + 2 * P + t]);
       c.violrow[job * 2 + 1] = __float_as_int(lds[f.part + 5 * P + t]);
-      if (l2) {
-        lds[f.dpos + t] = dpos;
-      } else {
-        // dot: dLoss/dpos_i goes onto the (masked, so far zero) diagonal of the
-        // scores against the rhs negatives, whose i-th batch negative is the i-th
-        // positive's own rhs row: the products of phase 3 then carry
-        // dpos_i * rhs_i into the lhs gradient and dpos_i * lhs_i into the rhs one.
-        lds[sc1 + t * lds_ + t] = dpos;
-      }
+      if (l2) lds[f.dpos + t] = dpos;
     }
     if (l2) {  // column sums of the stored -2 dLoss/dq
       for (int t2 = t; t2 < 2 * N; t2 += kFusedThreads) {
@@ -1094,7 +1086,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         lds[(s ? g.cs1 : g.cs0) + j] = acc;
       }
     }
-    __syncthreads();  // (e)
+    if (l2) __syncthreads();  // (e) the column sums read the blocks that the fold below rewrites
     // Both score blocks carry a P x P part against the batch negatives, and the
     // batch negatives of one side are the positives of that side: the gradient of
     // positive row i of the lhs is  sum_j dS_R[i][j] rhs_j + sum_j dS_L[j][i] rhs_j,
@@ -1102,7 +1094,12 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
     // rhs rows), kept in place, and phase 3 needs one product per row block.
     for (int e = t; e < P * P; e += kFusedThreads) {
       const int i = e / P, j = e - i * P;
-      const float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
+      float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
+      // dot: dLoss/dpos_i goes onto the (masked, so far zero) diagonal: the i-th batch
+      // negative of the rhs side is the i-th positive's own rhs row, so the products
+      // of phase 3 then carry dpos_i * rhs_i into the lhs gradient and dpos_i * lhs_i
+      // into the rhs one.
+      if (!l2 && i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
       lds[sc1 + i * lds_ + j] = sum;
       lds[sc0 + j * lds_ + i] = sum;
     }
