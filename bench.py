@@ -359,7 +359,7 @@ def main():
         full = n_edges // b * b
         rel_edges[:full] = rel_edges[:full].view(-1, b).sort(dim=1).values.reshape(-1)
 
-    def run(workers, batches, warm, profile_calls=0):
+    def run(workers, batches, warm, profile_calls=0, hip_graph=False):
         spec, runner = make_runner(workers)
         c, u = spec.num_chunks, w["uniform_negs"]
         per_call = workers * b
@@ -367,8 +367,22 @@ def main():
         warm_calls = max(1, warm // workers)
         n_r = tables[-1].shape[0]
 
+        static = None  # inputs of the captured step (hip_graph): the next call's edges and negatives are written into them
+
         def one_call(i, profiled=False):
             off = (i * per_call) % (n_edges - per_call + 1) // b * b
+            if static is not None:
+                s_lhs, s_rhs, s_rel, s_ul, s_ur, graph = static
+                s_lhs.copy_(lhs_all[off:off + per_call])
+                s_rhs.copy_(rhs_all[off:off + per_call])
+                if rel_edges is not None:
+                    s_rel.copy_(rel_edges[off:off + per_call])
+                else:
+                    s_rel.copy_(rel_pool[(i * workers) % (4096 - workers + 1):][:workers])
+                torch.randint(0, e, (workers, c, u), generator=gen, device=dev, out=s_ul)
+                torch.randint(0, n_r, (workers, c, u), generator=gen, device=dev, out=s_ur)
+                graph.replay()
+                return None
             lhs = lhs_all[off:off + per_call]
             rhs = rhs_all[off:off + per_call]
             if rel_edges is not None:
@@ -383,6 +397,12 @@ def main():
             runner.train(lhs, rhs, rel, ul, ur)
             return None
 
+        if hip_graph:
+            s_in = [torch.zeros(per_call, dtype=torch.int64, device=dev), torch.zeros(per_call, dtype=torch.int64, device=dev),
+                    torch.zeros(per_call if rel_edges is not None else workers, dtype=torch.int64, device=dev),
+                    torch.zeros((workers, c, u), dtype=torch.int64, device=dev),
+                    torch.zeros((workers, c, u), dtype=torch.int64, device=dev)]
+            static = (*s_in, runner.capture_train(*s_in))
         for i in range(warm_calls):
             one_call(i)
         torch.cuda.synchronize()
@@ -415,6 +435,10 @@ def main():
     if not args.no_sequential and workers > 1:
         _, seq_eps, seq_ms, seq_timed, _, _ = run(1, max(50, min(steps // 8, 1000)), 20)
         seq = {"value": seq_eps, "ms_per_step": seq_ms, "steps": seq_timed, "workers": 1}
+        # the same single-batch sequence with the step captured in a HIP graph (one launch per step
+        # instead of about ten) and the inputs written into the graph's static buffers
+        _, g_eps, g_ms, g_timed, _, _ = run(1, max(50, min(steps // 8, 1000)), 20, hip_graph=True)
+        seq["hip_graph"] = {"value": g_eps, "ms_per_step": g_ms, "steps": g_timed}
 
     # roofline of the dominant stage (HIP events around each stage of pbg_train_step, on its stream)
     alg = algorithmic(w, spec)

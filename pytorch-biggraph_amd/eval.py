@@ -1,0 +1,58 @@
+"""Ranking evaluation of a batch (reference: torchbiggraph/eval.py:43-86,
+util.py:420-428, stats.py:16-17).  The scores come from
+MultiRelationEmbedder.forward, i.e. from pbg_model_forward on the GPU; the
+metrics are a handful of reductions over [B] and [B, N] tensors."""
+from statistics import mean
+
+import torch
+
+from .batching import AbstractBatchProcessor
+from .edgelist import EdgeList
+from .model import MultiRelationEmbedder, Scores
+from .stats import Stats
+
+
+def average_of_sums(*tensors: torch.Tensor) -> float:
+    """stats.py:16-17."""
+    return mean(t.sum().item() for t in tensors)
+
+
+def compute_randomized_auc(pos_: torch.Tensor, neg_: torch.Tensor, num_samples: int) -> float:
+    """Probability that a randomly chosen positive scores higher than a randomly
+    chosen negative, from num_samples random pairs (util.py:420-428)."""
+    pos_, neg_ = pos_.reshape(-1), neg_.reshape(-1)
+    dev = pos_.device
+    diff = (pos_[torch.randint(len(pos_), (num_samples,), device=dev)]
+            > neg_[torch.randint(len(neg_), (num_samples,), device=dev)])
+    return float(diff.float().mean())
+
+
+class RankingEvaluator(AbstractBatchProcessor):
+    """eval.py:43-86: rank of each positive among its negatives (ties count
+    against the positive), MRR, hits@1/10/50 and a randomized AUC, averaged over
+    the sides that have negatives; sums over the batch, to be divided by count."""
+
+    def _process_one_batch(self, model: MultiRelationEmbedder, batch_edges: EdgeList) -> Stats:
+        with torch.no_grad():
+            scores, _ = model(batch_edges)
+        self._adjust_scores(scores, batch_edges)
+        batch_size = len(batch_edges)
+        loss = self.calc_loss(scores, batch_edges)
+        ranks, aucs = [], []
+        for pos, neg in ((scores.lhs_pos, scores.lhs_neg), (scores.rhs_pos, scores.rhs_neg)):
+            if neg.nelement() > 0:
+                ranks.append((neg >= pos.unsqueeze(1)).sum(1) + 1)
+                aucs.append(compute_randomized_auc(pos, neg, batch_size))
+        return Stats(
+            loss=float(loss),
+            pos_rank=average_of_sums(*ranks),
+            mrr=average_of_sums(*(rank.float().reciprocal() for rank in ranks)),
+            r1=average_of_sums(*(rank.le(1) for rank in ranks)),
+            r10=average_of_sums(*(rank.le(10) for rank in ranks)),
+            r50=average_of_sums(*(rank.le(50) for rank in ranks)),
+            auc=batch_size * sum(aucs) / len(aucs),  # averaged over count at the end
+            count=batch_size,
+        )
+
+    def _adjust_scores(self, scores: Scores, batch_edges: EdgeList) -> None:
+        """Hook for a filtered evaluator (eval.py:82-86)."""

@@ -314,6 +314,20 @@ class StepRunner:
         bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
         check(_lib.lib().pbg_train_step(ctypes.byref(self.desc), ctypes.byref(bufs), _stream()))
 
+    def capture_train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> "torch.cuda.CUDAGraph":
+        """Records one train() call into a HIP graph and returns it.  The tensors
+        passed here become the graph's static inputs: write the next step's edges
+        and negatives INTO them (copy_, randint(out=...)) and call replay().  The
+        launch-bound single-batch step (about ten dependent kernels of a few
+        microseconds each) is what this is for.  The step records kernels only (no
+        memset nodes, no allocation), so a replay does exactly what the call did."""
+        self.train(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)  # first-call set-up must not be captured
+        torch.cuda.current_stream(self.device).synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.train(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
+        return graph
+
     STAGES = ("prep", "operator", "scores", "loss", "backward_dn", "backward_da", "rowback", "params", "sort", "update")
 
     @property

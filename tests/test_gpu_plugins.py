@@ -300,3 +300,37 @@ def test_C_module_matches_the_reference_contract(pbg):
         assert np.array_equal(got[1].cpu().numpy(), ro[a:b])
         assert np.array_equal(got[2].cpu().numpy(), relo[a:b])
         assert got[0].data_ptr() == outs[0][a:b].data_ptr()  # views of the caller's storage
+
+
+def test_ranking_evaluator(pbg):
+    """RankingEvaluator (eval.py:43-86) on batch negatives only (nothing sampled):
+    loss, mean rank, MRR and hits@k equal the same formulas on the oracle's scores."""
+    say("ranking evaluator")
+    from tests.test_gpu_step import make_inputs
+
+    cfg = ostep.StepConfig(dim=16, operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=20,
+                           num_uniform_negs=0, num_relations=2, relation_weights=[1.0, 0.5])
+    num_pos = 57
+    st, batches = make_inputs(cfg, num_pos, 300, 1, seed=9)
+    model, w_l, w_r = build_model(pbg, cfg, st, 2)
+    EL, ED = pbg.entitylist.EntityList, pbg.edgelist.EdgeList
+    loss_fn = pbg.losses.LOSS_FUNCTIONS.get_class(cfg.loss)(margin=cfg.margin)
+    evaluator = pbg.eval.RankingEvaluator(loss_fn, list(cfg.relation_weights))
+    lhs, rhs, rel, ul, ur = batches[0]
+    before = w_l.detach().clone()
+    stats = evaluator.process_one_batch(model, ED(EL.from_tensor(lhs.to(DEV)), EL.from_tensor(rhs.to(DEV)), torch.tensor(rel)))
+    assert torch.equal(before, w_l.detach())  # evaluation does not train
+    want, _ = ostep.forward_backward(cfg, st, lhs, rhs, rel, None, None, keep_scores=True)
+    sc = want.scores
+    ranks = [(neg >= pos.unsqueeze(1)).sum(1) + 1 for pos, neg in ((sc.lhs_pos, sc.lhs_neg), (sc.rhs_pos, sc.rhs_neg))]
+    mean2 = lambda a, b: (float(a.sum()) + float(b.sum())) / 2
+    m = stats.metrics
+    assert stats.count == num_pos
+    assert m["loss"] == pytest.approx(want.loss, rel=1e-5)
+    assert m["pos_rank"] == pytest.approx(mean2(*ranks), abs=1.0)  # a score tie may move one rank
+    assert m["mrr"] == pytest.approx(mean2(*(r.float().reciprocal() for r in ranks)), abs=0.5)
+    for k in (1, 10, 50):
+        assert m[f"r{k}"] == pytest.approx(mean2(*(r.le(k) for r in ranks)), abs=1.0)
+    assert 0.0 <= m["auc"] <= num_pos
+    avg = pbg.stats.Stats.sum([stats]).average()
+    assert 0.0 <= avg.metrics["auc"] <= 1.0 and 1.0 <= avg.metrics["pos_rank"] <= 21.0

@@ -279,3 +279,34 @@ def test_hundred_steps(pbg, case):
     torch.cuda.synchronize()
     assert resyncs <= 10, resyncs
     compare_state(cfg, runner, st, 1e-4, "100 steps")
+
+
+def test_hip_graph_replays_match_eager(pbg):
+    """A captured step replayed with new inputs does what the eager call does:
+    two runners from the same state, one eager, one replaying its graph, with
+    eager work and synchronisations between the replays, stay bit-identical."""
+    say("hip graph")
+    cfg = ostep.StepConfig(dim=100, operator="translation", comparator="l2", loss="ranking", num_batch_negs=50,
+                           num_uniform_negs=50, lr=0.1, num_relations=3, relation_weights=[1.0, 0.5, 2.0])
+    num_pos, steps = 230, 4
+    st, batches = make_inputs(cfg, num_pos, 3000, steps + 1, seed=5)
+    eager = to_runner(pbg, cfg, st, num_pos, 1)
+    graphed = to_runner(pbg, cfg, st, num_pos, 1)
+    static = [t.clone() for t in pack(cfg, [batches[0]])]
+    graph = graphed.capture_train(*static)  # runs batch 0 twice (set-up call + capture is not a run) ...
+    copy_state(graphed, st)                 # ... so start again from the common state
+    graphed.loss_out.zero_()
+    for b in batches[1:]:
+        inputs = pack(cfg, [b])
+        eager.train(*inputs)
+        for dst, src in zip(static, inputs):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (eager.w_lhs.sum() + graphed.w_lhs.sum()).item()  # unrelated eager work between replays
+        assert torch.equal(eager.loss_out, graphed.loss_out)
+        assert torch.equal(eager.violators_out, graphed.violators_out)
+        assert torch.equal(eager.w_lhs, graphed.w_lhs) and torch.equal(eager.g_lhs, graphed.g_lhs)
+        for k in eager.rhs_op:
+            assert torch.equal(eager.rhs_op[k], graphed.rhs_op[k])
+            assert torch.equal(eager.rhs_op_sum[k], graphed.rhs_op_sum[k])
