@@ -359,6 +359,8 @@ def main():
         full = n_edges // b * b
         rel_edges[:full] = rel_edges[:full].view(-1, b).sort(dim=1).values.reshape(-1)
 
+    enqueue_s = [0.0]  # host time per call of the last run's timed loop (launches only, no wait)
+
     def run(workers, batches, warm, profile_calls=0, hip_graph=False):
         spec, runner = make_runner(workers)
         c, u = spec.num_chunks, w["uniform_negs"]
@@ -389,12 +391,10 @@ def main():
                 rel = rel_edges[off:off + per_call]
             else:
                 rel = rel_pool[(i * workers) % (4096 - workers + 1):][:workers]
-            # the uniform negatives of model.py:70-75, drawn on the device inside the timed loop
-            ul = torch.randint(0, e, (workers, c, u), generator=gen, device=dev)
-            ur = torch.randint(0, n_r, (workers, c, u), generator=gen, device=dev)
+            # the uniform negatives of model.py:70-75 are drawn inside the step, a fresh seed per call
             if profiled:
-                return runner.train_profiled(lhs, rhs, rel, ul, ur)
-            runner.train(lhs, rhs, rel, ul, ur)
+                return runner.train_profiled(lhs, rhs, rel, uniform_seed=0x5EED0000 + i)
+            runner.train(lhs, rhs, rel, uniform_seed=0x5EED0000 + i)
             return None
 
         if hip_graph:
@@ -409,6 +409,7 @@ def main():
         t0 = time.perf_counter()
         for i in range(calls):
             one_call(warm_calls + i)
+        enqueue_s[0] = (time.perf_counter() - t0) / calls
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         stages = None
@@ -425,11 +426,12 @@ def main():
         loss = float(runner.loss_out.mean().item()) / b
         return spec, calls * per_call / dt, dt / (calls * workers) * 1e3, calls * workers, stages, loss
 
-    default_steps = {"cfg1": 8000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 8000, "cfg5": 400, "cfg5s": 800}[args.workload]
+    default_steps = {"cfg1": 64000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
     steps = args.steps if args.steps is not None else default_steps
     warmup = args.warmup if args.warmup is not None else max(args.workers, steps // 10)
     workers = max(1, min(args.workers, steps))
     spec, eps, ms_per_step, timed, stages, loss = run(workers, steps, warmup, profile_calls=10)
+    host_enqueue_ms = enqueue_s[0] * 1e3
 
     seq = None
     if not args.no_sequential and workers > 1:
@@ -470,8 +472,8 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
-                   "hogwild_workers": workers, "uniform_negative_draw": "torch.randint on device, inside the timed loop",
-                   "mean_loss_per_edge_last_call": loss},
+                   "hogwild_workers": workers, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
+                   "mean_loss_per_edge_last_call": loss, "host_enqueue_ms_per_call": host_enqueue_ms},
         "sequential": seq,
         "roofline": roofline,
         "cpu_baseline": cpu,

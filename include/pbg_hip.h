@@ -137,7 +137,7 @@ typedef struct pbg_step_buffers {
   const int64_t* lhs;         /* [K, B] */
   const int64_t* rhs;         /* [K, B] */
   const int64_t* rel;         /* standard: [K]; dynamic: [K, B] */
-  const int64_t* uniform_lhs; /* [K, C, U] entity indices (model.py:70-75), null if unused */
+  const int64_t* uniform_lhs; /* [K, C, U] entity indices (model.py:70-75), null if unused or sample_uniform */
   const int64_t* uniform_rhs; /* [K, C, U] */
   const float* edge_weight;   /* [K, B] or null (EdgeList.weight, edgelist.py:51-95) */
   const float* relation_weights; /* [num_relations] (batching.py:144-148) */
@@ -150,7 +150,26 @@ typedef struct pbg_step_buffers {
   int64_t* violators_out;     /* [K, 2] violators_lhs, violators_rhs */
   void* workspace;
   size_t workspace_bytes;
+  /* sample_uniform != 0: uniform_lhs / uniform_rhs are null and the step draws the
+   * uniform negatives itself (SimpleEmbedding.sample_entities, model.py:70-75):
+   * negative (k, chunk, u) of side s is row
+   * pbg_sample_uniform_negatives(uniform_seed, s, num_rows)[(k * C + chunk) * U + u].
+   * Pass a fresh seed per call. */
+  int32_t sample_uniform;
+  uint64_t uniform_seed;
 } pbg_step_buffers;
+
+/* sizeof(pbg_step_desc) / sizeof(pbg_step_buffers) as this library was compiled:
+ * a binding checks its own struct layout against them. */
+size_t pbg_sizeof_step_desc(void);
+size_t pbg_sizeof_step_buffers(void);
+
+/* The rows the step draws for side `side` (0 lhs, 1 rhs) under `seed`:
+ * out[i] = Philox4x32-10(key = seed, counter = i, stream = side) mod num_rows, i < count.
+ * Replaces the torch.randint of sample_entities (model.py:72); lets a caller (or a
+ * test) see the negatives of a call that drew them itself. */
+int pbg_sample_uniform_negatives(uint64_t seed, int32_t side, int64_t num_rows, int64_t count, int64_t* out,
+                                 pbg_stream_t stream);
 
 size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc);
 int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream);

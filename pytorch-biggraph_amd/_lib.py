@@ -58,6 +58,7 @@ class StepBuffers(ctypes.Structure):
         ("lhs_op_p0", c_void_p), ("lhs_op_p1", c_void_p), ("lhs_op_s0", c_void_p), ("lhs_op_s1", c_void_p),
         ("loss_out", c_void_p), ("violators_out", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("sample_uniform", c_int32), ("uniform_seed", c_uint64),
     ]
 
 
@@ -73,6 +74,9 @@ SIGNATURES = {
     "pbg_async_adagrad_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p]),
     "pbg_gemm_f32": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_float, c_float, c_void_p]),
+    "pbg_sizeof_step_desc": (c_size_t, []),
+    "pbg_sizeof_step_buffers": (c_size_t, []),
+    "pbg_sample_uniform_negatives": (c_int32, [c_uint64, c_int32, c_int64, c_int64, c_void_p, c_void_p]),
     "pbg_train_step_workspace_bytes": (c_size_t, [POINTER(StepDesc)]),
     "pbg_train_step": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p]),
     "pbg_train_step_num_stages": (c_int32, []),
@@ -120,6 +124,9 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = restype
             fn.argtypes = argtypes
+        if handle.pbg_sizeof_step_desc() != ctypes.sizeof(StepDesc) or \
+                handle.pbg_sizeof_step_buffers() != ctypes.sizeof(StepBuffers):
+            raise RuntimeError(f"{LIB_PATH} was built from another include/pbg_hip.h than this binding: rebuild it")
         _lib = handle
     return _lib
 

@@ -10,6 +10,37 @@
 
 namespace pbg {
 
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"):
+// 64 random bits for (seed, counter, stream).  The uniform negatives of a step
+// are drawn with it, one counter per negative, so a draw depends on nothing but
+// its position and can be repeated anywhere (SimpleEmbedding.sample_entities,
+// model.py:70-75, only fixes the distribution: uniform over the table's rows).
+__host__ __device__ __forceinline__ uint64_t philox_u64(uint64_t seed, uint64_t counter, uint32_t stream) {
+  uint32_t c0 = (uint32_t)counter, c1 = (uint32_t)(counter >> 32), c2 = stream, c3 = 0u;
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return ((uint64_t)c1 << 32) | c0;
+}
+// id of uniform negative number `flat` of side `side`, in [0, num_rows): the high
+// word of (32 random bits x num_rows) for tables below 2^32 rows (no division;
+// the same 2^-32 * num_rows departure from uniformity as a 32-bit draw modulo
+// num_rows), a 64-bit remainder beyond.
+__host__ __device__ __forceinline__ int64_t sampled_row(uint64_t seed, uint64_t flat, uint32_t side, int64_t num_rows) {
+  const uint64_t r = philox_u64(seed, flat, side);
+  if ((uint64_t)num_rows <= 0xffffffffull) return (int64_t)(((r & 0xffffffffull) * (uint64_t)num_rows) >> 32);
+  return (int64_t)(r % (uint64_t)num_rows);
+}
+
 // Cross-lane reductions with DPP moves (ALU-rate) instead of LDS permutes: four
 // steps fold a row of 16 lanes onto itself (quad swaps, half-row mirror, row
 // mirror), two row broadcasts carry the row sums into lane 63, which is then

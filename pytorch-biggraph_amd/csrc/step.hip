@@ -34,7 +34,8 @@ constexpr int kWavesPerBlock = kRowThreads / kWave;
 struct SideCtx {
   const float* w;       // embedding table of this side
   const int64_t* idx;   // [K, B] positive entities
-  const int64_t* uidx;  // [K, C, U] uniform negatives (null if u == 0)
+  const int64_t* uidx;  // [K, C, U] uniform negatives (null if u == 0, or if they are drawn in the step)
+  uint64_t useed;       // seed of the in-step draw (uidx == null)
   int64_t key_base;     // offset of this table in the sort-key row space
   int64_t num_rows;
   int nb, u, nn;        // batch-negative / uniform / total negative columns of this side
@@ -73,6 +74,13 @@ struct StepCtx {
   unsigned long long* violators;  // [K, 2]
   float* loss_out;                // [K]
 };
+
+// Uniform negative number flat = (k * C + chunk) * U + u of side s: given by the
+// caller or drawn here (model.py:70-75).
+__device__ __forceinline__ int64_t uniform_negative(const SideCtx& sd, int s, int64_t flat) {
+  if (sd.uidx) return sd.uidx[flat];
+  return sampled_row(sd.useed, (uint64_t)flat, (uint32_t)s, sd.num_rows);
+}
 
 // ---------------------------------------------------------------------------
 // prep
@@ -137,7 +145,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     const int r2 = r - CP;
     const int cc = r2 / sd.u, uu = r2 % sd.u;
     const int64_t kc = (int64_t)k * c.C + cc;
-    const int64_t id = clamp_index(sd.uidx[kc * c.U + uu], sd.num_rows);
+    const int64_t id = clamp_index(uniform_negative(sd, s, kc * c.U + uu), sd.num_rows);
     const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
     if (lane == 0) {
       const int64_t slot = (int64_t)k * c.rk + sd.slot_uni + r2;
@@ -611,7 +619,7 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
         id = sd.idx[(int64_t)k * c.B + r];
       } else {
         const int r2 = r - c.B;
-        id = sd.uidx[((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u];
+        id = uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u);
       }
       const float* x = sd.w + clamp_index(id, sd.num_rows) * D;
       if (c.op == PBG_OP_DIAGONAL) {
@@ -854,7 +862,10 @@ __device__ __forceinline__ void fused_load_ids(const StepCtx& c, const FusedGeom
       }
     } else {
       const int u = j - g.P;
-      id = (s ? c.side[1].uidx : c.side[0].uidx)[kc * g.U + u];
+      const int64_t* given = s ? c.side[1].uidx : c.side[0].uidx;
+      id = given ? given[kc * g.U + u]
+                 : sampled_row(s ? c.side[1].useed : c.side[0].useed, (uint64_t)(kc * g.U + u), (uint32_t)s,
+                               s ? c.side[1].num_rows : c.side[0].num_rows);
       pair = (int64_t)k * c.rk + (s ? c.side[1].slot_uni : c.side[0].slot_uni) + cc * g.U + u;
     }
   }
@@ -1517,6 +1528,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     c.side[1].idx = b->rhs;
     c.side[0].uidx = b->uniform_lhs;
     c.side[1].uidx = b->uniform_rhs;
+    c.side[0].useed = c.side[1].useed = b->uniform_seed;
     c.side[0].p0 = b->lhs_op_p0;
     c.side[0].p1 = b->lhs_op_p1;
     c.side[1].p0 = b->rhs_op_p0;
@@ -1542,8 +1554,12 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
     return fail(PBG_ERR_INVALID, "step: w_lhs == w_rhs needs shared_table = 1");
   if ((uintptr_t)b->w_lhs % 16 != 0 || (uintptr_t)b->w_rhs % 16 != 0)
     return fail(PBG_ERR_INVALID, "step: tables must be 16-byte aligned");
-  if (plan.c.side[0].u > 0 && !b->uniform_lhs) return fail(PBG_ERR_INVALID, "step: uniform_lhs is null");
-  if (plan.c.side[1].u > 0 && !b->uniform_rhs) return fail(PBG_ERR_INVALID, "step: uniform_rhs is null");
+  if (!b->sample_uniform) {
+    if (plan.c.side[0].u > 0 && !b->uniform_lhs) return fail(PBG_ERR_INVALID, "step: uniform_lhs is null");
+    if (plan.c.side[1].u > 0 && !b->uniform_rhs) return fail(PBG_ERR_INVALID, "step: uniform_rhs is null");
+  } else if (b->uniform_lhs || b->uniform_rhs) {
+    return fail(PBG_ERR_INVALID, "step: sample_uniform is set but uniform negatives were passed");
+  }
   for (int s = 0; s < 2; ++s) {
     if (!plan.c.side[s].has_op || d->op == PBG_OP_NONE) continue;
     const float* p0 = s == 0 ? b->lhs_op_p0 : b->rhs_op_p0;
@@ -1769,6 +1785,28 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
 }  // namespace pbg
 
 using namespace pbg;
+
+namespace {
+__global__ void sample_uniform_kernel(uint64_t seed, uint32_t side, int64_t num_rows, int64_t count,
+                                      int64_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) out[i] = sampled_row(seed, (uint64_t)i, side, num_rows);
+}
+}  // namespace
+
+extern "C" size_t pbg_sizeof_step_desc(void) { return sizeof(pbg_step_desc); }
+extern "C" size_t pbg_sizeof_step_buffers(void) { return sizeof(pbg_step_buffers); }
+
+extern "C" int pbg_sample_uniform_negatives(uint64_t seed, int32_t side, int64_t num_rows, int64_t count, int64_t* out,
+                                            pbg_stream_t stream) {
+  if (count < 0 || num_rows < 1 || (side != 0 && side != 1))
+    return fail(PBG_ERR_INVALID, "pbg_sample_uniform_negatives: bad arguments");
+  if (count == 0) return PBG_OK;
+  if (!out) return fail(PBG_ERR_INVALID, "pbg_sample_uniform_negatives: null output");
+  hipLaunchKernelGGL(sample_uniform_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, (hipStream_t)stream, seed,
+                     (uint32_t)side, num_rows, count, out);
+  return check_launch("pbg_sample_uniform_negatives");
+}
 
 extern "C" size_t pbg_train_step_workspace_bytes(const pbg_step_desc* desc) {
   if (validate(desc, false) != PBG_OK) return 0;

@@ -108,6 +108,14 @@ def gemm(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, a
                                   stride_c, int(a_kmajor), int(b_kmajor), float(alpha), float(beta), _stream()))
 
 
+def sample_uniform_negatives(seed: int, side: int, num_rows: int, shape, device) -> torch.Tensor:
+    """The rows a step draws for `side` (0 lhs, 1 rhs) under `seed`, as
+    [num_workers, num_chunks, num_uniform_negs] = `shape`."""
+    out = torch.empty(tuple(shape), dtype=torch.int64, device=device)
+    check(_lib.lib().pbg_sample_uniform_negatives(seed & (2**64 - 1), side, num_rows, out.numel(), _ptr(out), _stream()))
+    return out
+
+
 # ---------------------------------------------------------------------------
 def reverse_permutation(perm: torch.Tensor) -> torch.Tensor:
     _need(perm, torch.int64, "perm")
@@ -273,7 +281,7 @@ class StepRunner:
         (only,) = params.values()
         return only, None
 
-    def _buffers(self, lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight) -> StepBuffers:
+    def _buffers(self, lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight, uniform_seed=None) -> StepBuffers:
         s = self.spec
         k, b = s.num_workers, s.batch_size
         _need(lhs, torch.int64, "lhs")
@@ -284,10 +292,12 @@ class StepRunner:
         if rel.numel() != (k * b if s.dynamic else k):
             raise ValueError("rel must hold one entry per edge (dynamic) or per batch (standard)")
         c, u = s.num_chunks, s.num_uniform_negs
+        if uniform_seed is not None and (uniform_lhs is not None or uniform_rhs is not None):
+            raise ValueError("pass uniform negatives or a seed to draw them with, not both")
         for name, t, off in (("uniform_lhs", uniform_lhs, s.disable_lhs_negs), ("uniform_rhs", uniform_rhs, s.disable_rhs_negs)):
-            if u > 0 and not off:
+            if u > 0 and not off and uniform_seed is None:
                 if t is None:
-                    raise ValueError(f"{name} is required")
+                    raise ValueError(f"{name} is required (or uniform_seed, to draw the negatives in the step)")
                 _need(t, torch.int64, name)
                 if t.numel() != k * c * u:
                     raise ValueError(f"{name} must be [num_workers, num_chunks, num_uniform_negs] = [{k}, {c}, {u}]")
@@ -306,12 +316,16 @@ class StepRunner:
         bufs.lhs_op_p0, bufs.lhs_op_p1, bufs.lhs_op_s0, bufs.lhs_op_s1 = _ptr(p0), _ptr(p1), _ptr(s0), _ptr(s1)
         bufs.loss_out, bufs.violators_out = _ptr(self.loss_out), _ptr(self.violators_out)
         bufs.workspace, bufs.workspace_bytes = _ptr(self.workspace), self.workspace.numel()
+        bufs.sample_uniform = int(uniform_seed is not None)
+        bufs.uniform_seed = (uniform_seed or 0) & (2**64 - 1)
         return bufs
 
-    def train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> None:
+    def train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None, uniform_seed=None) -> None:
         """One lock-step training step over num_workers batches; statistics land
-        in self.loss_out / self.violators_out (device, no sync)."""
-        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
+        in self.loss_out / self.violators_out (device, no sync).  The uniform
+        negatives are either given ([K, C, U] per side) or drawn inside the step
+        from `uniform_seed` (sample_uniform_negatives shows which)."""
+        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight, uniform_seed)
         check(_lib.lib().pbg_train_step(ctypes.byref(self.desc), ctypes.byref(bufs), _stream()))
 
     def capture_train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> "torch.cuda.CUDAGraph":
@@ -335,10 +349,11 @@ class StepRunner:
         """True when the step runs as the single LDS-resident chunk kernel."""
         return bool(_lib.lib().pbg_train_step_is_fused(ctypes.byref(self.desc)))
 
-    def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> List[float]:
+    def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None,
+                       uniform_seed=None) -> List[float]:
         """train() with HIP events between the stages; synchronises and returns
         the stage durations in milliseconds (order: StepRunner.STAGES)."""
-        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
+        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight, uniform_seed)
         n = _lib.lib().pbg_train_step_num_stages()
         out = (ctypes.c_float * n)()
         check(_lib.lib().pbg_train_step_profile(ctypes.byref(self.desc), ctypes.byref(bufs), _stream(), out))

@@ -310,3 +310,51 @@ def test_hip_graph_replays_match_eager(pbg):
         for k in eager.rhs_op:
             assert torch.equal(eager.rhs_op[k], graphed.rhs_op[k])
             assert torch.equal(eager.rhs_op_sum[k], graphed.rhs_op_sum[k])
+
+
+@pytest.mark.parametrize("case", [
+    dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50,
+         num_pos=230, dim=100),                                                  # fused chunk kernel
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=20,
+         num_uniform_negs=30, num_pos=70, dim=40),                               # staged kernels, parameter gradient
+    dict(operator="translation", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=0,
+         num_uniform_negs=9, num_pos=40, dim=10),                                # uniform negatives only
+], ids=ids)
+def test_negatives_drawn_in_the_step(pbg, case):
+    """A step that draws its uniform negatives from a seed is bit-identical to a
+    step that is handed pbg_sample_uniform_negatives(seed) and the draw is uniform
+    over the table."""
+    say("in-step negatives", case)
+    from pytorch_biggraph_amd import native
+
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, **case)
+    workers, n_ent, seed = 3, 700, 0x1234567890ABCDEF
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=3, shared=False)
+    lhs, rhs, rel, _, _ = pack(cfg, batches)
+    a = to_runner(pbg, cfg, st, num_pos, workers)
+    b = to_runner(pbg, cfg, st, num_pos, workers)
+    shape = (workers, a.spec.num_chunks, cfg.num_uniform_negs)
+    ul = native.sample_uniform_negatives(seed, 0, st.w_lhs.shape[0], shape, DEV)
+    ur = native.sample_uniform_negatives(seed, 1, st.w_rhs.shape[0], shape, DEV)
+    assert int(ul.min()) >= 0 and int(ul.max()) < st.w_lhs.shape[0]
+    assert int(ur.min()) >= 0 and int(ur.max()) < st.w_rhs.shape[0]
+    assert not torch.equal(ul, ur)
+    a.train(lhs, rhs, rel, ul, ur)
+    b.train(lhs, rhs, rel, uniform_seed=seed)
+    torch.cuda.synchronize()
+    assert torch.equal(a.loss_out, b.loss_out) and torch.equal(a.violators_out, b.violators_out)
+    for x, y in ((a.w_lhs, b.w_lhs), (a.g_lhs, b.g_lhs), (a.w_rhs, b.w_rhs), (a.g_rhs, b.g_rhs)):
+        assert torch.equal(x, y)
+    for k in a.rhs_op:
+        assert torch.equal(a.rhs_op[k], b.rhs_op[k])
+    with pytest.raises(ValueError):
+        b.train(lhs, rhs, rel, ul, ur, uniform_seed=seed)
+    # uniformity: 200 000 draws over 1000 rows, chi-square with 999 degrees of freedom (mean 999, sd 44.7)
+    draws = native.sample_uniform_negatives(seed + 1, 0, 1000, (200_000,), DEV)
+    counts = torch.bincount(draws, minlength=1000).double()
+    chi2 = float(((counts - 200.0) ** 2 / 200.0).sum())
+    assert 999 - 6 * 44.7 < chi2 < 999 + 6 * 44.7, chi2
+    other = native.sample_uniform_negatives(seed + 2, 0, 1000, (200_000,), DEV)
+    assert float((draws == other).double().mean()) < 0.01
