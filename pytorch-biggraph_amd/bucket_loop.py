@@ -226,12 +226,6 @@ class BucketStats:
     violators_rhs: int
 
 
-def _default_negatives(workers: int, chunks: int, num_uniform: int, num_rows: int, generator: torch.Generator,
-                       device: torch.device) -> torch.Tensor:
-    """SimpleEmbedding.sample_entities (model.py:70-75) for `workers` batches at once."""
-    return torch.randint(0, num_rows, (workers, chunks, num_uniform), generator=generator, device=device)
-
-
 class BucketLoop:
     """One pass over all buckets = ``train_epoch()``.
 
@@ -267,7 +261,11 @@ class BucketLoop:
         self.generator = torch.Generator(device=self.device).manual_seed(seed)
         self.seed = seed
         self.edge_order = edge_order
-        self.negatives = negatives or _default_negatives
+        # None: the step draws its uniform negatives itself (SimpleEmbedding.sample_entities,
+        # model.py:70-75), one seed per call; a callable(workers, chunks, num_uniform, num_rows,
+        # generator, device) -> [workers, chunks, num_uniform] supplies them instead
+        self.negatives = negatives
+        self.calls = 0
         self.epoch = 0
 
     def _keys(self, b: Bucket) -> List[PartitionKey]:
@@ -319,9 +317,14 @@ class BucketLoop:
             else:
                 r = rel[off:off + count:b_now].contiguous()  # one relation type per batch
             c = spec.num_chunks
-            ul = self.negatives(k, c, u, w_l.shape[0], self.generator, dev) if u else None
-            ur = self.negatives(k, c, u, w_r.shape[0], self.generator, dev) if u else None
-            runner.train(lhs[sl].contiguous(), rhs[sl].contiguous(), r, ul, ur)
+            if u and self.negatives is not None:
+                ul = self.negatives(k, c, u, w_l.shape[0], self.generator, dev)
+                ur = self.negatives(k, c, u, w_r.shape[0], self.generator, dev)
+                runner.train(lhs[sl].contiguous(), rhs[sl].contiguous(), r, ul, ur)
+            else:
+                self.calls += 1
+                call_seed = (self.seed * 0x9E3779B97F4A7C15 + self.calls) & (2**64 - 1) if u else None
+                runner.train(lhs[sl].contiguous(), rhs[sl].contiguous(), r, uniform_seed=call_seed)
             loss += runner.loss_out.double().sum()
             viol += runner.violators_out.sum(dim=0)
             off += count
