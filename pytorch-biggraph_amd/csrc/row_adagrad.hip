@@ -368,6 +368,17 @@ __device__ __forceinline__ float half_sum(float v) {  // sum over the 32 lanes o
   v = row16_sum(v);
   return v + __shfl_xor(v, 16, 64);
 }
+constexpr int kMaxBatchSlots = 8;  // batches per lane of a half wave: 256 batches per call at most
+// first position in [lo, hi) whose key is >= want (hi if none)
+__device__ __forceinline__ int64_t lower_bound_key(const uint64_t* __restrict__ keys, int64_t lo, int64_t hi,
+                                                   uint64_t want) {
+  while (lo < hi) {
+    const int64_t mid = lo + ((hi - lo) >> 1);
+    if (keys[mid] < want) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo;
+}
 __device__ __forceinline__ float4 load_or_zero(const float* __restrict__ p, bool has) {
   return has ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
 }
@@ -445,28 +456,40 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
         g[r] = next;
       }
       gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+    } else if (kbits == 0) {  // a single-worker call has one run per row
+      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
     } else {
-      int64_t j = i;
-      while (true) {
-        if (kbits == 0) {  // a single-worker call has one run per row
-          j = n;
-        } else {
-          const uint64_t key = keys[j];
-          int64_t base = j + 1;
-          while (true) {  // first position after j with another key, 32 positions at a time
-            const int64_t q = base + gl;
-            const uint32_t same = (uint32_t)(__ballot(q < n && keys[q < n ? q : n - 1] == key) >> gbase);
-            if (same != 0xffffffffu) {
-              j = base + (__ffs((int)~same) - 1);
-              break;
-            }
-            base += 32;
-          }
-        }
-        gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
-        if (j >= n || (keys[j] >> kbits) != row) break;
-        g[r] = load_or_zero(grad_rows + (int64_t)vals[j] * dim + col, has);
+      // A long row (a hot entity of a power-law graph): one run per batch that names
+      // it.  Lane l finds the first position of batches l, l + 32, ... by binary
+      // search in the sorted keys, all lanes at once, and fetches the number of the
+      // gradient row there; the runs are then applied in batch order with the next
+      // run's gradient in flight.  (Walking the runs one after the other costs two
+      // dependent memory round trips per 32 positions.)
+      const int nb = 1 << kbits;
+      const int64_t row_end = lower_bound_key(keys, i, n, (row + 1) << kbits);
+      uint32_t st[kMaxBatchSlots], sv[kMaxBatchSlots];  // run start (relative to i) and its gradient row, per batch of this lane
+#pragma unroll
+      for (int m = 0; m < kMaxBatchSlots; ++m) {
+        const int b = gl + 32 * m;
+        const int64_t at = b < nb ? lower_bound_key(keys, i, row_end, (row << kbits) | (uint64_t)b) : row_end;
+        st[m] = (uint32_t)(at - i);
+        sv[m] = vals[at < n ? at : n - 1];
       }
+      uint32_t run = 0;  // start of the run whose gradient g[r] holds (the row's first run starts at i)
+#pragma unroll
+      for (int m = 0; m < kMaxBatchSlots; ++m) {
+        if (32 * m >= nb) break;
+        for (int j = 0; j < 32 && 32 * m + j < nb; ++j) {
+          const uint32_t s_b = (uint32_t)__shfl((int)st[m], gbase + j, 64);
+          if (s_b == run || (int64_t)s_b >= row_end - i) continue;  // batch absent, or it is the run in hand
+          const uint32_t v_b = (uint32_t)__shfl((int)sv[m], gbase + j, 64);
+          const float4 next = load_or_zero(grad_rows + (int64_t)v_b * dim + col, has);
+          gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+          g[r] = next;
+          run = s_b;
+        }
+      }
+      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
     }
     if (has) *reinterpret_cast<float4*>(wrow[r]) = w[r];
     if (gl == 0) *gptr[r] = gsum[r];

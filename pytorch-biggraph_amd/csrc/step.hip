@@ -672,6 +672,56 @@ __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ 
   }
 }
 
+// The same for K <= 64 with one wave per parameter element: lane k sums batch k's
+// slices and fetches the parameter and its Adagrad sum of batch k's relation, all
+// lanes at once; the K updates then run in order on registers, an updated value
+// handed on to the later batches of the same relation, and the last batch of
+// every relation stores.  The chain of K dependent global read-modify-writes of
+// the kernel above becomes one round trip.
+__global__ __launch_bounds__(kRowThreads) void param_update_wave_kernel(StepCtx c, int s, const float* __restrict__ dth,
+                                                                        int slices, int64_t psize, float* p0,
+                                                                        float* p1, float* s0, float* s1, float lr) {
+  const int lane = threadIdx.x & 63;
+  const int64_t e = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (e >= psize) return;
+  const int H = c.D / 2, K = c.K;
+  const bool on = lane < K;
+  const int64_t r = on ? clamp_index(c.rel[lane], c.num_relations) : -1 - lane;  // idle lanes match nobody
+  float* p = nullptr;
+  float* st = nullptr;
+  if (on) {
+    if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+      p = e < H ? p0 + r * H + e : p1 + r * H + (e - H);
+      st = e < H ? s0 + r * H + e : s1 + r * H + (e - H);
+    } else {
+      p = p0 + r * psize + e;
+      st = s0 + r * psize + e;
+    }
+  }
+  float g = 0.f;
+  if (on)
+    for (int sl = 0; sl < slices; ++sl) g += dth[((int64_t)lane * slices + sl) * psize + e];
+  float pv = on ? *p : 0.f, sv = on ? *st : 0.f;
+  const int rlo = (int)(uint32_t)r, rhi = (int)(uint32_t)((uint64_t)r >> 32);
+  bool last = on;
+  for (int k = 0; k < K; ++k) {
+    const bool same = __builtin_amdgcn_readlane(rlo, k) == rlo && __builtin_amdgcn_readlane(rhi, k) == rhi;
+    // batch k's step, computed by every lane from lane k's registers
+    const float gk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(g), k));
+    const float sum = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sv), k)) + gk * gk;
+    const float pn = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pv), k)) + -lr * (gk / (sqrtf(sum) + 1e-10f));
+    if (same && lane >= k) {  // lane k itself and the later batches of the same relation
+      sv = sum;
+      pv = pn;
+    }
+    if (same && lane < k) last = false;
+  }
+  if (last) {
+    *st = sv;
+    *p = pv;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // fused chunk kernel: the whole chain from gather to raw-row gradients for one
 // chunk in one workgroup, operands resident in LDS
@@ -1775,8 +1825,13 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
       hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
                          dim3(kParamGroups * 64), 0, stream, c, s, plan.dth[s], plan.pslices[s]);
     }
-    hipLaunchKernelGGL(param_update_kernel, dim3((unsigned)ceil_div(plan.psize, 256)), dim3(256), 0, stream, c, s,
-                       plan.dth[s], plan.pslices[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
+    if (K <= kWave && c.op != PBG_OP_LINEAR) {  // (a matrix's elements are better served one per thread)
+      hipLaunchKernelGGL(param_update_wave_kernel, dim3((unsigned)ceil_div(plan.psize, kWavesPerBlock)), dim3(kRowThreads),
+                         0, stream, c, s, plan.dth[s], plan.pslices[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
+    } else {
+      hipLaunchKernelGGL(param_update_kernel, dim3((unsigned)ceil_div(plan.psize, 256)), dim3(256), 0, stream, c, s,
+                         plan.dth[s], plan.pslices[s], plan.psize, p0, p1, s0, s1, d->relation_lr);
+    }
   }
   return check_launch("step params");
 }
