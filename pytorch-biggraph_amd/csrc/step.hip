@@ -763,6 +763,67 @@ __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at
                                                int i, int masked_from, float pos, float w, int qd, float* loss_w,
                                                float* dpos_out, int* viol_out, float* rowsum_out) {
   constexpr bool l2 = CMP == PBG_CMP_L2;
+  if (l2 && LOSS != PBG_LOSS_SOFTMAX) {
+    // No pass over the whole row is needed before the gradient (no softmax
+    // denominator), so the distances are formed, used and dropped eight columns at
+    // a time: holding all of a lane's columns next to the l2 operands does not fit
+    // the 128 registers a lane of this 1024-thread kernel has.  v_sqrt_f32 and
+    // v_rcp_f32 (1 ulp) stand in for the correctly rounded sequences: the expansion
+    // ||a||^2 - 2ab + ||b||^2 itself carries 1e-7 * ||a||^2 of rounding noise.
+    float loss_acc = 0.f, dpos_part = 0.f, rowsum = 0.f;
+    int viol = 0;
+    const float inv_nn = 1.0f / (float)N;
+    if (LOSS == PBG_LOSS_LOGISTIC && qd == 0) {
+      loss_acc += softplusf(-pos);
+      dpos_part += (sigmoidf(pos) - 1.0f) * w;
+    }
+#pragma unroll
+    for (int e0 = 0; e0 < kQuadCols; e0 += 8) {
+      float raw[8], bn[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = min(qd + 4 * (e0 + u), N - 1);
+        raw[u] = lds[row_at + j];
+        bn[u] = lds[bn_at + j];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = qd + 4 * (e0 + u);
+        const float q = fmaf(-2.0f, raw[u], bn[u]) + a2;
+        bool lv = q >= 1e-30f;  // clamped distances are constants (model.py:236)
+        float te = -__builtin_amdgcn_sqrtf(fmaxf(q, 1e-30f));
+        if (j < nb && (j == i || j >= masked_from)) {
+          te = -1e9f;
+          lv = false;
+        }
+        if (j >= N) {
+          te = -INFINITY;
+          lv = false;
+        }
+        float g;
+        if (LOSS == PBG_LOSS_RANKING) {
+          const float x = (te - pos) + margin;
+          if (x > 0.f) loss_acc += x;
+          g = (x >= 0.f) ? w : 0.f;
+          dpos_part -= g;
+        } else {
+          loss_acc += softplusf(te) * inv_nn;
+          g = sigmoidf(te) * inv_nn * w;
+        }
+        if (te > pos) ++viol;
+        // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq
+        const float dq = lv ? g * 0.5f * __builtin_amdgcn_rcpf(te) : 0.f;
+        rowsum += dq;
+        if (j < N) lds[row_at + j] = -2.0f * dq;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    *loss_w = quad_sum(loss_acc) * w;
+    *dpos_out = quad_sum(dpos_part);
+    *rowsum_out = quad_sum(rowsum);
+    *viol_out = quad_sum_int(viol);
+    return;
+  }
   float t[kQuadCols];
   uint32_t live = 0xffffffffu;  // bit e clear: column qd + 4e is a constant with no gradient
   if (!l2) {
