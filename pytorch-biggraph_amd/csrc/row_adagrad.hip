@@ -436,6 +436,7 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     gsum[r] = *gptr[r];
     g[r] = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase, 64) * dim + col, has);
   }
+  int long_r = -1;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (!head[r]) continue;
@@ -459,41 +460,62 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     } else if (kbits == 0) {  // a single-worker call has one run per row
       gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
     } else {
-      // A long row (a hot entity of a power-law graph): one run per batch that names
-      // it.  Lane l finds the first position of batches l, l + 32, ... by binary
-      // search in the sorted keys, all lanes at once, and fetches the number of the
-      // gradient row there; the runs are then applied in batch order with the next
-      // run's gradient in flight.  (Walking the runs one after the other costs two
-      // dependent memory round trips per 32 positions.)
-      const int nb = 1 << kbits;
-      const int64_t row_end = lower_bound_key(keys, i, n, (row + 1) << kbits);
-      uint32_t st[kMaxBatchSlots], sv[kMaxBatchSlots];  // run start (relative to i) and its gradient row, per batch of this lane
-#pragma unroll
-      for (int m = 0; m < kMaxBatchSlots; ++m) {
-        const int b = gl + 32 * m;
-        const int64_t at = b < nb ? lower_bound_key(keys, i, row_end, (row << kbits) | (uint64_t)b) : row_end;
-        st[m] = (uint32_t)(at - i);
-        sv[m] = vals[at < n ? at : n - 1];
-      }
-      uint32_t run = 0;  // start of the run whose gradient g[r] holds (the row's first run starts at i)
-#pragma unroll
-      for (int m = 0; m < kMaxBatchSlots; ++m) {
-        if (32 * m >= nb) break;
-        for (int j = 0; j < 32 && 32 * m + j < nb; ++j) {
-          const uint32_t s_b = (uint32_t)__shfl((int)st[m], gbase + j, 64);
-          if (s_b == run || (int64_t)s_b >= row_end - i) continue;  // batch absent, or it is the run in hand
-          const uint32_t v_b = (uint32_t)__shfl((int)sv[m], gbase + j, 64);
-          const float4 next = load_or_zero(grad_rows + (int64_t)v_b * dim + col, has);
-          gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
-          g[r] = next;
-          run = s_b;
-        }
-      }
-      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+      // A long row: handled after this loop.  There is at most one per half wave (the
+      // positions after its head belong to it), so the code below exists once
+      // instead of once per position.
+      long_r = r;
+      continue;
     }
     if (has) *reinterpret_cast<float4*>(wrow[r]) = w[r];
     if (gl == 0) *gptr[r] = gsum[r];
   }
+  if (long_r < 0) return;
+  // (only the position is carried out of the loop above: the row's weights, sum
+  // and first gradient are fetched again rather than held in registers by every
+  // half wave that has no long row)
+  const int64_t long_i = first + long_r;
+  const uint64_t long_row = keys[long_i] >> kbits;
+  float* long_wrow;
+  float* long_gptr;
+  if ((int64_t)long_row < rows0) {
+    long_wrow = w0 + (int64_t)long_row * dim + col;
+    long_gptr = g0 + long_row;
+  } else {
+    long_wrow = w1 + ((int64_t)long_row - rows0) * dim + col;
+    long_gptr = g1 + ((int64_t)long_row - rows0);
+  }
+  float4 long_w = load_or_zero(long_wrow, has);
+  float long_gsum = *long_gptr;
+  float4 long_g = load_or_zero(grad_rows + (int64_t)vals[long_i] * dim + col, has);
+  // A long row (a hot entity of a power-law graph): one run per batch that names
+  // it.  Lane l finds the first position of batch b0 + l by binary search in the
+  // sorted keys, 32 batches at once, and fetches the number of the gradient row
+  // there; the runs are then applied in batch order with the next run's gradient
+  // in flight.  (Walking the runs one after the other costs two dependent memory
+  // round trips per 32 positions.)
+  const int nb = 1 << kbits;
+  const int64_t row_end = lower_bound_key(keys, long_i, n, (long_row + 1) << kbits);
+  uint32_t run = 0;  // start (relative to long_i) of the run whose gradient long_g holds
+#pragma unroll 1
+  for (int b0 = 0; b0 < nb; b0 += 32) {
+    const int b = b0 + gl;
+    const int64_t at = b < nb ? lower_bound_key(keys, long_i, row_end, (long_row << kbits) | (uint64_t)b) : row_end;
+    const uint32_t st = (uint32_t)(at - long_i);    // first position of batch b (of the next batch present, if absent)
+    const uint32_t sv = vals[at < n ? at : n - 1];  // and the gradient row there
+#pragma unroll 1
+    for (int j = 0; j < 32 && b0 + j < nb; ++j) {
+      const uint32_t s_b = (uint32_t)__shfl((int)st, gbase + j, 64);
+      if (s_b == run || (int64_t)s_b >= row_end - long_i) continue;  // batch absent, or it is the run in hand
+      const uint32_t v_b = (uint32_t)__shfl((int)sv, gbase + j, 64);
+      const float4 next = load_or_zero(grad_rows + (int64_t)v_b * dim + col, has);
+      long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
+      long_g = next;
+      run = s_b;
+    }
+  }
+  long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
+  if (has) *reinterpret_cast<float4*>(long_wrow) = long_w;
+  if (gl == 0) *long_gptr = long_gsum;
 }
 
 // keys for the stand-alone sparse step: key = row index, value = position
