@@ -949,6 +949,49 @@ __device__ __forceinline__ void mfma_sweep(const float* lds, int a_at, int a_ste
   }
 }
 
+// The same product for operands whose k runs along the LDS rows (both operands
+// of the score products): a lane reads FOUR consecutive k of its row as one
+// 128-bit word and feeds them to four MFMAs, so the k slots of step r hold
+// k = 16 g + 4 (lane >> 4) + r for group g -- any assignment of k to slots is
+// right as long as both operands use the same one.  A quarter of the LDS
+// instructions of mfma_sweep; `groups` groups of 16 k, then `rest` single steps.
+// a_at / b_at address element (row, 0).  Reads up to 15 floats past the last k of
+// a row (never used: the groups cover whole multiples of 16 only).
+template <int T>
+__device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b_at, int b_tile, int groups, int rest,
+                                               int kq, float4v* acc) {
+  a_at += 4 * kq;
+  b_at += 4 * kq;
+  for (int gk = 0; gk < groups; ++gk) {
+    const float4 a = *reinterpret_cast<const float4*>(&lds[a_at]);
+    float4 b[T];
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) b[ct] = *reinterpret_cast<const float4*>(&lds[b_at + ct * b_tile]);
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].x, a.x, acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].y, a.y, acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].z, a.z, acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].w, a.w, acc[ct], 0, 0, 0);
+    a_at += 16;
+    b_at += 16;
+  }
+  a_at -= 3 * kq;  // single steps: slot kq holds k = 16 groups + 4 step + kq
+  b_at -= 3 * kq;
+  for (int ks = 0; ks < rest; ++ks) {
+    const float a = lds[a_at];
+    float b[T];
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) b[ct] = lds[b_at + ct * b_tile];
+#pragma unroll
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct], a, acc[ct], 0, 0, 0);
+    a_at += 4;
+    b_at += 4;
+  }
+}
+
 // Geometry of one chunk, the same for both roles.
 struct FusedGeom {
   int D, P, U, N, ldx, lds, xn0, xn1, sc0, sc1, sq0, sq1, rs0, rs1, cs0, cs1;
@@ -1123,9 +1166,10 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 #pragma unroll
         for (int ct = 0; ct < TN; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int ar = min(rt * 16 + (lane_ & 15), P - 1);
-        const int a_at = (s ? xn0 : xn1) + ar * ldx + (lane_ >> 4);
-        const int b_at = (s ? xn1 : xn0) + (lane_ & 15) * ldx + (lane_ >> 4);  // column tile ct: 16 rows further down
-        mfma_sweep<TN>(lds, a_at, 4, b_at, 4, 16 * ldx, (D + 3) >> 2, acc);
+        const int a_at = (s ? xn0 : xn1) + ar * ldx;
+        const int b_at = (s ? xn1 : xn0) + (lane_ & 15) * ldx;  // column tile ct: 16 rows further down
+        const int ksteps = (D + 3) >> 2;
+        mfma_sweep_k16<TN>(lds, a_at, b_at, 16 * ldx, ksteps >> 2, ksteps & 3, lane_ >> 4, acc);
         const int row = rt * 16 + (lane_ & 15);
         if (row < P) {
           const int at = (s ? sc1 : sc0) + row * lds_ + 4 * (lane_ >> 4);

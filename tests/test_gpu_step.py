@@ -358,3 +358,49 @@ def test_negatives_drawn_in_the_step(pbg, case):
     assert 999 - 6 * 44.7 < chi2 < 999 + 6 * 44.7, chi2
     other = native.sample_uniform_negatives(seed + 2, 0, 1000, (200_000,), DEV)
     assert float((draws == other).double().mean()) < 0.01
+
+
+def _fused_shape_cases():
+    """A fixed pseudo-random sample of the shapes the LDS-resident chunk kernel
+    accepts (and a few just outside, which take the staged kernels)."""
+    import random
+
+    rng = random.Random(7)
+    cases = []
+    for _ in range(48):
+        p = rng.choice([1, 2, 3, 15, 16, 17, 31, 33, 48, 50, 63, 64])
+        u = rng.choice([1, 2, 5, 16, 17, 49, 50, 64])
+        d = rng.choice([4, 8, 12, 36, 60, 64, 100, 116, 124, 128])
+        chunks = rng.choice([1, 2, 3])
+        num_pos = max(1, p * chunks - rng.choice([0, 0, 1, p // 2]))
+        cases.append(dict(operator=rng.choice(["none", "translation", "diagonal"]), comparator=rng.choice(["dot", "l2"]),
+                          loss=rng.choice(["ranking", "logistic", "softmax"]), dynamic=False, num_batch_negs=p,
+                          num_uniform_negs=u, num_pos=num_pos, dim=d))
+    return cases
+
+
+@pytest.mark.parametrize("case", _fused_shape_cases(), ids=ids)
+def test_fused_kernel_shapes(pbg, case):
+    """Chunk sizes, negative counts, dims and partial last chunks around the
+    tile borders of the fused chunk kernel, two batches per call."""
+    say("fused shapes", case)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    cfg = ostep.StepConfig(dim=dim, num_relations=2, relation_weights=[1.0, 0.5], lr=0.1, relation_lr=0.01, margin=0.1,
+                           **case)
+    n_ent = max(300, num_pos * (60 if cfg.comparator == "l2" else 4))
+    st, batches = make_inputs(cfg, num_pos, n_ent, 2, seed=num_pos * 131 + dim, shared=(dim % 8 == 0))
+    runner = to_runner(pbg, cfg, st, num_pos, 2)
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, batches, keep_scores=True)
+    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        sc = out.scores
+        for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
+                                     (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
+            pp = pos.unsqueeze(1)
+            ties = int(((neg - pp).abs() <= 2e-5 * pp.abs().clamp_min(1e-6)).sum())
+            assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
+    compare_state(cfg, runner, st, rtol, "step")
