@@ -404,3 +404,59 @@ def test_fused_kernel_shapes(pbg, case):
             ties = int(((neg - pp).abs() <= 2e-5 * pp.abs().clamp_min(1e-6)).sum())
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
     compare_state(cfg, runner, st, rtol, "step")
+
+
+def test_lockstep_training_learns_like_sequential(pbg):
+    """End to end on a graph with planted structure (a ring with chords: i -> i+1,
+    i -> i+7): ten passes with 1 batch per call and with 16 batches per call both
+    drive the loss down by a factor of five and rank the true tail of held-out
+    edges far above chance.  At an equal number of passes the lock-step run lags
+    the sequential one a little (16 batches read the same tables: a larger
+    effective batch), as HOGWILD workers do."""
+    say("learns")
+    n_ent, dim, bsz = 2000, 32, 100
+    g = torch.Generator().manual_seed(0)
+    src = torch.arange(n_ent).repeat(2)
+    dst = torch.cat([(torch.arange(n_ent) + 1) % n_ent, (torch.arange(n_ent) + 7) % n_ent])
+    perm = torch.randperm(src.shape[0], generator=g)
+    src, dst = src[perm].to(DEV), dst[perm].to(DEV)
+    held = 400  # held-out edges for ranking
+    tr_src, tr_dst = src[held:], dst[held:]
+    n_train = tr_src.shape[0] // (16 * bsz) * (16 * bsz)
+
+    def train(workers, epochs):
+        w = (torch.randn(n_ent, dim, generator=torch.Generator().manual_seed(1)) * 0.1).to(DEV)
+        gs = torch.zeros(n_ent, device=DEV)
+        spec = pbg.StepSpec(dim=dim, batch_size=bsz, num_workers=workers, num_batch_negs=50, num_uniform_negs=50,
+                            operator="translation", comparator="dot", loss="softmax", lr=0.1)
+        op = {"translation": torch.zeros(1, dim, device=DEV)}
+        op_sum = {"translation": torch.zeros(1, dim, device=DEV)}
+        runner = pbg.StepRunner(spec, w, gs, None, None, op, op_sum)
+        rel = torch.zeros(workers, dtype=torch.int64, device=DEV)
+        losses, call = [], 0
+        for epoch in range(epochs):
+            order = torch.randperm(n_train, generator=torch.Generator().manual_seed(100 + epoch)).to(DEV)
+            total = 0.0
+            for off in range(0, n_train, workers * bsz):
+                idx = order[off:off + workers * bsz]
+                call += 1
+                runner.train(tr_src[idx].contiguous(), tr_dst[idx].contiguous(), rel, uniform_seed=call)
+                total += float(runner.loss_out.sum())
+            losses.append(total / n_train)
+        # rank of the true rhs among 1000 uniform negatives, held-out edges
+        ev = pbg.StepSpec(dim=dim, batch_size=held, num_workers=1, num_batch_negs=0, num_uniform_negs=1000,
+                          operator="translation", comparator="dot", loss="softmax")
+        er = pbg.StepRunner(ev, w, gs, None, None, op, op_sum)
+        negs = torch.randint(0, n_ent, (1, er.spec.num_chunks, 1000), generator=torch.Generator().manual_seed(5)).to(DEV)
+        _, rhs_pos, _, rhs_neg = er.forward(src[:held].contiguous(), dst[:held].contiguous(),
+                                            torch.zeros(1, dtype=torch.int64, device=DEV), negs, negs)
+        rank = (rhs_neg[0] >= rhs_pos[0].unsqueeze(1)).sum(1) + 1
+        return losses, float(rank.float().reciprocal().mean()), float((rank <= 10).float().mean())
+
+    seq_losses, seq_mrr, seq_h10 = train(1, 10)
+    par_losses, par_mrr, par_h10 = train(16, 10)
+    say("sequential", seq_losses, seq_mrr, seq_h10, "lock-step x16", par_losses, par_mrr, par_h10)
+    assert seq_losses[-1] < 0.2 * seq_losses[0] and par_losses[-1] < 0.2 * par_losses[0]
+    assert par_losses[-1] < 1.25 * seq_losses[-1]
+    assert seq_h10 > 0.1 and par_h10 > 0.1          # chance: 10 / 1001
+    assert par_mrr > 0.5 * seq_mrr
