@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of (workload, kernel) at the default --workers, from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under profiles/ (not measured live).
-TRAFFIC = {("cfg1", "fused_chunk"): 232.7e6}  # 64 workers
+TRAFFIC = {("cfg1", "fused_chunk"): 231.4e6}  # 64 workers
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
