@@ -10,6 +10,7 @@
 namespace pbg {
 namespace {
 
+typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kRowThreads = 256;  // 4 waves per block, one row per wave
 constexpr int kMaxV4 = 4;         // float4 per lane: covers dim <= 1024
 
@@ -30,7 +31,11 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const float* _
     const int nv = dim >> 2;
     const float4* src = reinterpret_cast<const float4*>(table + (ok ? r : 0) * (int64_t)dim);
     float4* dst = reinterpret_cast<float4*>(out + i * (int64_t)dim);
-    for (int v = lane; v < nv; v += kWave) dst[v] = ok ? src[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+    // the output is written once and read by somebody else later: streaming stores
+    for (int v = lane; v < nv; v += kWave) {
+      const float4 x = ok ? src[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+      __builtin_nontemporal_store((float4v){x.x, x.y, x.z, x.w}, reinterpret_cast<float4v*>(dst) + v);
+    }
   } else {
     const float* src = table + (ok ? r : 0) * (int64_t)dim;
     float* dst = out + i * (int64_t)dim;
@@ -76,7 +81,10 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_multi_kernel(const fl
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int64_t i = base + u * kGroups;
-    if (col_ok && i < n) reinterpret_cast<float4*>(out + i * (int64_t)dim)[v] = x[u];
+    if (col_ok && i < n) {
+      float4v* dst = reinterpret_cast<float4v*>(out + i * (int64_t)dim) + v;
+      __builtin_nontemporal_store((float4v){x[u].x, x[u].y, x[u].z, x[u].w}, dst);
+    }
   }
 }
 
