@@ -39,6 +39,10 @@ def test_gather_out_of_range(pbg):
     (50, 100, 100, 7, 0, 0), (100, 100, 50, 5, 1, 1), (50, 100, 100, 5, 0, 1),
     (130, 200, 33, 3, 0, 0), (1, 1, 1, 1, 0, 0), (200, 131, 257, 2, 1, 1), (17, 300, 64, 2, 0, 1),
     (256, 256, 300, 2, 1, 1), (64, 64, 16, 1, 0, 0),
+    # aligned operands: the tiles that go from global memory straight into LDS, with
+    # partial tiles along m, n and k in each of the four operand layouts
+    (1000, 1100, 1024, 2, 0, 0), (1100, 1024, 1000, 2, 1, 1), (1000, 1024, 1100, 2, 0, 1), (132, 200, 36, 3, 1, 0),
+    (128, 128, 16, 1, 0, 0), (200, 132, 20, 2, 0, 1), (97, 101, 64, 2, 0, 0), (130, 129, 16, 66000, 0, 0),
 ])
 def test_gemm_against_float64(pbg, m, n, k, batch, akm, bkm):
     say("gemm", m, n, k, batch, akm, bkm)
