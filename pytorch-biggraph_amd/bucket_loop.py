@@ -19,7 +19,11 @@ Edges of a bucket hold partition-local entity offsets, as the reference's edge
 files do.  A bucket is trained by `pbg_train_step` calls of `num_workers`
 batches each (native.StepRunner); the tail of a bucket runs as one call of the
 remaining full batches and one call of the final partial batch
-(batching.py:109-112).
+(batching.py:109-112).  With `eval_fraction` a random sample of each bucket's
+edges is held out of training and ranked before and after the bucket is trained
+(train_cpu.py:648-693).  Standard (non-dynamic) relations are trained in
+single-relation batches, the relation of the next batch drawn in proportion to
+the edges each relation has left (batching.py:60-79).
 """
 import random
 from dataclasses import dataclass
@@ -28,6 +32,10 @@ from typing import Callable, Dict, List, Optional, Sequence, Tuple
 import torch
 
 from . import native
+from .eval import ranking_stats
+from .losses import LOSS_FUNCTIONS
+from .stats import Stats
+from .util import round_up_to_nearest_multiple
 
 PartitionKey = Tuple[str, int]  # (entity type, partition)
 
@@ -86,6 +94,57 @@ def create_ordered_buckets(nparts_lhs: int, nparts_rhs: int, order: str, *, gene
     if order in ("inside_out", "outside_in"):
         return create_buckets_ordered_by_layer(nparts_lhs, nparts_rhs, order, generator=generator)
     raise NotImplementedError("Unknown bucket order: %s" % order)
+
+
+def holdout_indices(num_edges: int, eval_fraction: float, bucket: Bucket, edge_path_idx: int = 0,
+                    edge_chunk_idx: int = 0) -> Optional[torch.Tensor]:
+    """The edges of a bucket that are held out for evaluation: int(num_edges *
+    eval_fraction) draws WITH replacement from a generator seeded by what
+    identifies the edge set, so every epoch holds out the same ones
+    (train_cpu.py:648-672).  None when nothing is held out."""
+    num_eval = int(num_edges * eval_fraction)
+    if num_eval <= 0:
+        return None
+    g = torch.Generator()
+    g.manual_seed(hash((edge_path_idx, edge_chunk_idx, bucket.lhs, bucket.rhs)))
+    return torch.randint(num_edges, (num_eval,), dtype=torch.long, generator=g)
+
+
+def train_edge_indices(num_edges: int, eval_edge_idxs: Optional[torch.Tensor], device=None) -> torch.Tensor:
+    """The edges a bucket is trained on, before shuffling (train_cpu.py:852-856):
+    position e of [0, num_edges) holds e, except that held-out position
+    eval_edge_idxs[j] holds num_train + j; the first num_train positions are kept.
+    A held-out edge drawn more than once keeps its LAST j, which is what the
+    reference's sequential index assignment leaves (here: a scatter that keeps the
+    largest value, so that the result does not depend on the order in which a GPU
+    applies the writes).  As in the reference, a held-out edge whose own number is
+    num_train + j for a j that was swapped in (e.g. 10 edges, [2, 8] held out: slot
+    2 receives 8) is trained on all the same; the statement is kept as it is so
+    that the same edges are trained."""
+    if eval_edge_idxs is None:
+        return torch.arange(num_edges, device=device)
+    num_train = num_edges - eval_edge_idxs.shape[0]
+    idx = eval_edge_idxs.to(device)
+    out = torch.arange(num_edges, device=device)
+    out.scatter_reduce_(0, idx, torch.arange(num_train, num_edges, device=device), reduce="amax", include_self=False)
+    return out[:num_train]
+
+
+def plan_relation_batches(group_sizes: Sequence[int], batch_size: int,
+                          generator: Optional[torch.Generator] = None) -> List[Tuple[int, int, int]]:
+    """The batches batch_edges_group_by_relation_type yields (batching.py:60-79),
+    as (group, offset inside the group, length): the group of the next batch is
+    drawn with probability proportional to the edges the groups have left, and a
+    batch is the group's next batch_size edges (fewer at the group's end)."""
+    left = torch.tensor(list(group_sizes), dtype=torch.long)
+    plan: List[Tuple[int, int, int]] = []
+    while int(left.sum()) > 0:
+        idx = int(torch.multinomial(left.float(), 1, generator=generator))
+        offset = int(group_sizes[idx]) - int(left[idx])
+        length = min(batch_size, int(left[idx]))
+        plan.append((idx, offset, length))
+        left[idx] -= length
+    return plan
 
 
 class PartitionStore:
@@ -224,6 +283,9 @@ class BucketStats:
     loss: float
     violators_lhs: int
     violators_rhs: int
+    # sums over the held-out edges (divide by .count, or call .average()); None without a hold-out
+    eval_before: Optional[Stats] = None
+    eval_after: Optional[Stats] = None
 
 
 class BucketLoop:
@@ -231,8 +293,6 @@ class BucketLoop:
 
     edges: {Bucket: (lhs, rhs, rel)} int64 tensors of partition-local offsets and
     relation types, on the host (pinned or not) or already on the device.
-    Standard (non-dynamic) relations need single-relation batches: pass one
-    relation type overall or dynamic=True.
     """
 
     def __init__(self, store: PartitionStore, edges: Dict[Bucket, Tuple[torch.Tensor, torch.Tensor, torch.Tensor]],
@@ -244,8 +304,10 @@ class BucketLoop:
                  lhs_op: Optional[Dict[str, torch.Tensor]] = None, lhs_op_sum: Optional[Dict[str, torch.Tensor]] = None,
                  resident_partitions: int = 2, bucket_order: str = "inside_out", seed: int = 0,
                  device: str = "cuda:0",
+                 eval_fraction: float = 0.0, eval_num_batch_negs: int = 1000, eval_num_uniform_negs: int = 1000,
                  edge_order: Optional[Callable[[Bucket, int], torch.Tensor]] = None,
-                 negatives: Optional[Callable[..., torch.Tensor]] = None) -> None:
+                 negatives: Optional[Callable[..., torch.Tensor]] = None,
+                 record_calls: bool = False) -> None:
         self.store, self.edges = store, edges
         self.lhs_entity, self.rhs_entity = lhs_entity, rhs_entity
         self.nparts_lhs, self.nparts_rhs = nparts_lhs, nparts_rhs
@@ -259,12 +321,22 @@ class BucketLoop:
         self.bucket_order = bucket_order
         self.rng = random.Random(seed)
         self.generator = torch.Generator(device=self.device).manual_seed(seed)
+        self.host_generator = torch.Generator().manual_seed(seed)  # the relation of the next batch
         self.seed = seed
+        # edge_order(bucket, n) -> permutation of the bucket's n TRAINING edges, in place
+        # of the shuffle of _coordinate_train (train_cpu.py:857-859)
         self.edge_order = edge_order
         # None: the step draws its uniform negatives itself (SimpleEmbedding.sample_entities,
         # model.py:70-75), one seed per call; a callable(workers, chunks, num_uniform, num_rows,
         # generator, device) -> [workers, chunks, num_uniform] supplies them instead
         self.negatives = negatives
+        # held-out evaluation (config.py: eval_fraction, eval_num_batch_negs, eval_num_uniform_negs)
+        self.eval_fraction = eval_fraction
+        self.eval_negs = (eval_num_batch_negs, eval_num_uniform_negs)
+        self.loss_fn = LOSS_FUNCTIONS.get_class(loss)(margin=margin)
+        # record_calls: keep, on the host, the edges and relation types of every training
+        # call (`self.calls_log`), for a caller that wants to replay the epoch elsewhere
+        self.calls_log: Optional[List[dict]] = [] if record_calls else None
         self.calls = 0
         self.epoch = 0
 
@@ -274,62 +346,151 @@ class BucketLoop:
             keys.append((self.rhs_entity, b.rhs))
         return keys
 
+    def _call_plan(self, rel: torch.Tensor, batch_size: int, workers: int, draw: bool):
+        """Splits edges (already in training order) into calls of up to `workers`
+        equally sized batches.  Returns (order, starts, rels, calls): `order` (or
+        None) rearranges the edges so that every batch is a contiguous run,
+        batch i covers [starts[i], starts[i] + its length) and has relation
+        rels[i] (standard relations only), and calls = [(first batch, number of
+        batches, batch length)].
+
+        Dynamic relations, or a single relation type: consecutive batches in the
+        given order; the tail runs as one call of the remaining full batches and
+        one of the final partial batch.  Standard relations of several types:
+        single-relation batches (batching.py:60-79), in drawn order when `draw`,
+        else relation by relation."""
+        n = rel.shape[0]
+        dynamic = self.spec_args["dynamic"]
+        if dynamic or self.spec_args["num_relations"] == 1:
+            starts = list(range(0, n, batch_size))
+            lengths = [min(batch_size, n - s0) for s0 in starts]
+            order, rels = None, None
+        else:
+            sorted_rel, order = torch.sort(rel, stable=True)
+            sizes = torch.bincount(rel, minlength=self.spec_args["num_relations"]).tolist()
+            present = [r for r, c in enumerate(sizes) if c > 0]
+            begin, acc = {}, 0
+            for r in present:
+                begin[r] = acc
+                acc += sizes[r]
+            if draw:
+                plan = plan_relation_batches([sizes[r] for r in present], batch_size, self.host_generator)
+            else:
+                plan = [(gi, off, min(batch_size, sizes[r] - off)) for gi, r in enumerate(present)
+                        for off in range(0, sizes[r], batch_size)]
+            starts = [begin[present[gi]] + off for gi, off, _ in plan]
+            lengths = [ln for _, _, ln in plan]
+            rels = [present[gi] for gi, _, _ in plan]
+        calls, i = [], 0
+        while i < len(starts):
+            j = i + 1
+            if lengths[i] == batch_size:
+                while j < len(starts) and j - i < workers and lengths[j] == batch_size:
+                    j += 1
+            calls.append((i, j - i, lengths[i]))
+            i = j
+        return order, starts, rels, calls
+
+    def _call_edges(self, lhs, rhs, rel, starts, rels, first, k, b_now, starts_dev):
+        """The [k * b_now] edges of one call and its relation argument."""
+        dynamic = self.spec_args["dynamic"]
+        if rels is None:  # consecutive batches
+            sl = slice(starts[first], starts[first] + k * b_now)
+            r = rel[sl].contiguous() if dynamic else rel[sl][::b_now].contiguous()
+            return lhs[sl].contiguous(), rhs[sl].contiguous(), r
+        idx = (starts_dev[first:first + k, None] + torch.arange(b_now, device=lhs.device)).reshape(-1)
+        return lhs[idx], rhs[idx], torch.tensor(rels[first:first + k], dtype=torch.int64, device=lhs.device)
+
+    def _runner(self, runners, tables, k: int, b_now: int, **spec_overrides) -> native.StepRunner:
+        runner = runners.get((k, b_now))
+        if runner is None:
+            (w_l, g_l), (w_r, g_r) = tables[0], tables[-1]
+            shared = len(tables) == 1
+            spec = native.StepSpec(batch_size=b_now, num_workers=k, **{**self.spec_args, **spec_overrides})
+            runner = native.StepRunner(spec, w_l, g_l, None if shared else w_r, None if shared else g_r, *self.ops)
+            runners[(k, b_now)] = runner
+        return runner
+
+    def _uniform(self, k: int, chunks: int, u: int, rows: int, side: int) -> torch.Tensor:
+        if self.negatives is not None:
+            return self.negatives(k, chunks, u, rows, self.generator, self.device)
+        self.calls += 1
+        return native.sample_uniform_negatives((self.seed * 0x9E3779B97F4A7C15 + self.calls) & (2**64 - 1), side, rows,
+                                               (k, chunks, u), self.device)
+
+    def _evaluate(self, tables, lhs, rhs, rel, eval_idx: torch.Tensor) -> Stats:
+        """Ranks the held-out edges (train_cpu.py:886-911, eval.py:43-81) with the
+        evaluation-time numbers of negatives; sums, to be averaged by the caller."""
+        dev = self.device
+        idx = eval_idx.to(dev)
+        lhs, rhs, rel = lhs[idx], rhs[idx], rel[idx]
+        nb, nu = self.eval_negs
+        bsz = round_up_to_nearest_multiple(self.batch_size, nb) if nb > 0 else self.batch_size
+        order, starts, rels, calls = self._call_plan(rel, bsz, min(self.num_workers, 8), draw=False)
+        if order is not None:
+            lhs, rhs, rel = lhs[order], rhs[order], rel[order]
+        starts_dev = torch.tensor(starts, dtype=torch.int64, device=dev) if rels is not None else None
+        rows_l, rows_r = tables[0][0].shape[0], tables[-1][0].shape[0]
+        runners: Dict[Tuple[int, int], native.StepRunner] = {}
+        stats = []
+        for first, k, b_now in calls:
+            runner = self._runner(runners, tables, k, b_now, num_batch_negs=nb, num_uniform_negs=nu)
+            l, r, t = self._call_edges(lhs, rhs, rel, starts, rels, first, k, b_now, starts_dev)
+            c = runner.spec.num_chunks
+            ul = self._uniform(k, c, nu, rows_l, 0) if nu else None
+            ur = self._uniform(k, c, nu, rows_r, 1) if nu else None
+            lhs_pos, rhs_pos, lhs_neg, rhs_neg = runner.forward(l, r, t, ul, ur)
+            count = k * b_now
+            sides = [(lhs_pos.reshape(count), lhs_neg.reshape(count, -1)),
+                     (rhs_pos.reshape(count), rhs_neg.reshape(count, -1))]
+            # AbstractBatchProcessor.calc_loss (batching.py:139-150) with relation weights of 1
+            loss = sum(float(self.loss_fn(pos, neg, None)) for pos, neg in sides)
+            stats.append(ranking_stats(sides, loss, count))
+        return Stats.sum(stats)
+
     def _train_bucket(self, b: Bucket, tables) -> BucketStats:
         dev = self.device
         lhs, rhs, rel = (t.to(dev, non_blocking=True) for t in self.edges[b])
         n = lhs.shape[0]
         if n == 0:
             return BucketStats(b, 0, 0.0, 0, 0)
+        eval_idx = holdout_indices(n, self.eval_fraction, b)
+        eval_before = self._evaluate(tables, lhs, rhs, rel, eval_idx) if eval_idx is not None else None
+        num_train = n - (eval_idx.shape[0] if eval_idx is not None else 0)
         if self.edge_order is not None:
-            perm = self.edge_order(b, n).to(dev)
-        else:  # _coordinate_train shuffles the bucket's edges (train_cpu.py:857-859)
-            perm = native.randperm(n, hash((self.seed, self.epoch, b.lhs, b.rhs)) & 0x7FFFFFFF, dev)
-        lhs, rhs, rel = lhs[perm], rhs[perm], rel[perm]
-        (w_l, g_l) = tables[0]
-        (w_r, g_r) = tables[-1]
-        shared = len(tables) == 1
-        dynamic = self.spec_args["dynamic"]
-        bsz, kmax = self.batch_size, self.num_workers
+            perm = self.edge_order(b, num_train).to(dev)
+        else:  # _coordinate_train shuffles the bucket's training edges (train_cpu.py:857-859)
+            perm = native.randperm(num_train, hash((self.seed, self.epoch, b.lhs, b.rhs)) & 0x7FFFFFFF, dev)
+        if eval_idx is not None:
+            perm = train_edge_indices(n, eval_idx, dev)[perm]
+        lhs_t, rhs_t, rel_t = lhs[perm], rhs[perm], rel[perm]
+        order, starts, rels, calls = self._call_plan(rel_t, self.batch_size, self.num_workers, draw=True)
+        if order is not None:
+            lhs_t, rhs_t, rel_t = lhs_t[order], rhs_t[order], rel_t[order]
+        starts_dev = torch.tensor(starts, dtype=torch.int64, device=dev) if rels is not None else None
+        rows_l, rows_r = tables[0][0].shape[0], tables[-1][0].shape[0]
         u = self.spec_args["num_uniform_negs"]
-        if not dynamic and self.spec_args["num_relations"] != 1:
-            raise NotImplementedError("standard (non-dynamic) relations need single-relation batches: "
-                                      "use one relation type or dynamic=True")
         loss = torch.zeros((), dtype=torch.float64, device=dev)
         viol = torch.zeros(2, dtype=torch.int64, device=dev)
         runners: Dict[Tuple[int, int], native.StepRunner] = {}
-        off = 0
-        while off < n:
-            left = n - off
-            if left >= bsz:
-                k, b_now = min(kmax, left // bsz), bsz
-            else:
-                k, b_now = 1, left  # the final partial batch (batching.py:109-112)
-            runner = runners.get((k, b_now))
-            if runner is None:
-                spec = native.StepSpec(batch_size=b_now, num_workers=k, **self.spec_args)
-                runner = native.StepRunner(spec, w_l, g_l, None if shared else w_r, None if shared else g_r, *self.ops)
-                runners[(k, b_now)] = runner
-            spec = runner.spec
-            count = k * b_now
-            sl = slice(off, off + count)
-            if dynamic:
-                r = rel[sl].contiguous()
-            else:
-                r = rel[off:off + count:b_now].contiguous()  # one relation type per batch
-            c = spec.num_chunks
+        for first, k, b_now in calls:
+            runner = self._runner(runners, tables, k, b_now)
+            l, r, t = self._call_edges(lhs_t, rhs_t, rel_t, starts, rels, first, k, b_now, starts_dev)
+            if self.calls_log is not None:
+                self.calls_log.append(dict(bucket=b, epoch=self.epoch, workers=k, batch_size=b_now, lhs=l.cpu(),
+                                           rhs=r.cpu(), rel=t.cpu()))
+            c = runner.spec.num_chunks
             if u and self.negatives is not None:
-                ul = self.negatives(k, c, u, w_l.shape[0], self.generator, dev)
-                ur = self.negatives(k, c, u, w_r.shape[0], self.generator, dev)
-                runner.train(lhs[sl].contiguous(), rhs[sl].contiguous(), r, ul, ur)
+                runner.train(l, r, t, self._uniform(k, c, u, rows_l, 0), self._uniform(k, c, u, rows_r, 1))
             else:
                 self.calls += 1
                 call_seed = (self.seed * 0x9E3779B97F4A7C15 + self.calls) & (2**64 - 1) if u else None
-                runner.train(lhs[sl].contiguous(), rhs[sl].contiguous(), r, uniform_seed=call_seed)
+                runner.train(l, r, t, uniform_seed=call_seed)
             loss += runner.loss_out.double().sum()
             viol += runner.violators_out.sum(dim=0)
-            off += count
+        eval_after = self._evaluate(tables, lhs, rhs, rel, eval_idx) if eval_idx is not None else None
         v = viol.tolist()
-        return BucketStats(b, n, float(loss), int(v[0]), int(v[1]))
+        return BucketStats(b, num_train, float(loss), int(v[0]), int(v[1]), eval_before, eval_after)
 
     def train_epoch(self) -> List[BucketStats]:
         buckets = [b for b in create_ordered_buckets(self.nparts_lhs, self.nparts_rhs, self.bucket_order,

@@ -27,6 +27,27 @@ def compute_randomized_auc(pos_: torch.Tensor, neg_: torch.Tensor, num_samples: 
     return float(diff.float().mean())
 
 
+def ranking_stats(sides, loss: float, count: int) -> Stats:
+    """The sums RankingEvaluator reports for `count` edges (eval.py:57-81).
+    sides: (pos [n], neg [n, N]) per side; a side without negatives is skipped.
+    Rank = 1 + number of negatives scoring at least as high as the positive."""
+    ranks, aucs = [], []
+    for pos, neg in sides:
+        if neg.nelement() > 0:
+            ranks.append((neg >= pos.unsqueeze(1)).sum(1) + 1)
+            aucs.append(compute_randomized_auc(pos, neg, count))
+    return Stats(
+        loss=float(loss),
+        pos_rank=average_of_sums(*ranks),
+        mrr=average_of_sums(*(rank.float().reciprocal() for rank in ranks)),
+        r1=average_of_sums(*(rank.le(1) for rank in ranks)),
+        r10=average_of_sums(*(rank.le(10) for rank in ranks)),
+        r50=average_of_sums(*(rank.le(50) for rank in ranks)),
+        auc=count * sum(aucs) / len(aucs),  # averaged over count at the end
+        count=count,
+    )
+
+
 class RankingEvaluator(AbstractBatchProcessor):
     """eval.py:43-86: rank of each positive among its negatives (ties count
     against the positive), MRR, hits@1/10/50 and a randomized AUC, averaged over
@@ -36,23 +57,9 @@ class RankingEvaluator(AbstractBatchProcessor):
         with torch.no_grad():
             scores, _ = model(batch_edges)
         self._adjust_scores(scores, batch_edges)
-        batch_size = len(batch_edges)
         loss = self.calc_loss(scores, batch_edges)
-        ranks, aucs = [], []
-        for pos, neg in ((scores.lhs_pos, scores.lhs_neg), (scores.rhs_pos, scores.rhs_neg)):
-            if neg.nelement() > 0:
-                ranks.append((neg >= pos.unsqueeze(1)).sum(1) + 1)
-                aucs.append(compute_randomized_auc(pos, neg, batch_size))
-        return Stats(
-            loss=float(loss),
-            pos_rank=average_of_sums(*ranks),
-            mrr=average_of_sums(*(rank.float().reciprocal() for rank in ranks)),
-            r1=average_of_sums(*(rank.le(1) for rank in ranks)),
-            r10=average_of_sums(*(rank.le(10) for rank in ranks)),
-            r50=average_of_sums(*(rank.le(50) for rank in ranks)),
-            auc=batch_size * sum(aucs) / len(aucs),  # averaged over count at the end
-            count=batch_size,
-        )
+        return ranking_stats(((scores.lhs_pos, scores.lhs_neg), (scores.rhs_pos, scores.rhs_neg)), float(loss),
+                             len(batch_edges))
 
     def _adjust_scores(self, scores: Scores, batch_edges: EdgeList) -> None:
         """Hook for a filtered evaluator (eval.py:82-86)."""

@@ -119,3 +119,186 @@ def test_bucket_orders(pbg):
     assert [min(b.lhs, b.rhs) for b in in_out] == sorted(layers, reverse=True)
     with pytest.raises(NotImplementedError):
         bl.create_ordered_buckets(2, 2, "affinity", generator=random.Random(0))
+
+
+def _calls_of(n, bsz, workers):
+    """(offset, batches, batch length) of the calls that cut n consecutive edges."""
+    out, off = [], 0
+    while off < n:
+        left = n - off
+        k, b_now = (min(workers, left // bsz), bsz) if left >= bsz else (1, left)
+        out.append((off, k, b_now))
+        off += k * b_now
+    return out
+
+
+def _oracle_eval(cfg_eval, st, lhs, rhs, eval_idx, bsz, workers, draws):
+    """RankingEvaluator's sums (eval.py:57-81) over the held-out edges on the
+    oracle's scores, as (low, high) bounds: a negative that is the positive's own
+    entity scores the same as the positive up to rounding, and which way such a tie
+    falls differs between two fp32 implementations."""
+    lhs, rhs = lhs[eval_idx], rhs[eval_idx]
+    keys = ("pos_rank", "mrr", "r1", "r10")
+    lo, hi = dict.fromkeys(keys, 0.0), dict.fromkeys(keys, 0.0)
+    loss, count = 0.0, 0
+    for off, k, b_now in _calls_of(lhs.shape[0], bsz, workers):
+        ul, ur = next(draws), next(draws)
+        for i in range(k):
+            sl = slice(off + i * b_now, off + (i + 1) * b_now)
+            out, _ = ostep.forward_backward(cfg_eval, st, lhs[sl], rhs[sl], 0, ul[i], ur[i], keep_scores=True)
+            sc = out.scores
+            loss += out.loss
+            count += b_now
+            for bound, sign in ((lo, -1.0), (hi, 1.0)):
+                # low ranks: a near-tie does not count against the positive; high ranks: it does
+                ranks = []
+                for pos, neg in ((sc.lhs_pos, sc.lhs_neg), (sc.rhs_pos, sc.rhs_neg)):
+                    tol = 1e-5 * (1.0 + pos.abs().unsqueeze(1))
+                    ranks.append((neg >= pos.unsqueeze(1) - sign * tol).sum(1) + 1)
+                mean2 = lambda a, b: (float(a.sum()) + float(b.sum())) / 2
+                bound["pos_rank"] += mean2(*ranks)
+                bound["mrr"] += mean2(*(r.float().reciprocal() for r in ranks))
+                bound["r1"] += mean2(*(r.le(1) for r in ranks))
+                bound["r10"] += mean2(*(r.le(10) for r in ranks))
+    # low ranks give the high mrr / hits, and the other way round
+    low = dict(pos_rank=lo["pos_rank"], mrr=hi["mrr"], r1=hi["r1"], r10=hi["r10"])
+    high = dict(pos_rank=hi["pos_rank"], mrr=lo["mrr"], r1=lo["r1"], r10=lo["r10"])
+    return dict(loss=loss, count=count, low=low, high=high)
+
+
+@pytest.mark.gpu
+def test_holdout_evaluation_matches_oracle(pbg):
+    """eval_fraction: the held-out edges (train_cpu.py:661-672) are not trained on
+    (:852-856) and are ranked before and after each bucket (:675,690) with the
+    evaluation-time negatives; tables, losses and ranking sums against the oracle
+    driven through the same sequence."""
+    bl = pbg.bucket_loop
+    nparts, dim, bsz, workers, nb, nu, enb, enu, frac = 2, 12, 50, 2, 10, 5, 20, 7, 0.2
+    tables, edges = make_graph(nparts, 300, dim, 330, seed=5)
+    drawn, perms = [], {}
+
+    def negatives(k, c, u, rows, generator, device):
+        t = torch.randint(0, rows, (k, c, u), generator=generator, device=device)
+        drawn.append(t.cpu())
+        return t
+
+    def edge_order(bucket, n):
+        perms.setdefault((bucket.lhs, bucket.rhs), []).append(torch.randperm(n, generator=torch.Generator().manual_seed(n)))
+        return perms[(bucket.lhs, bucket.rhs)][-1]
+
+    store, stats, loop = run_loop(pbg, tables, edges, nparts, dim, 2, hooks=dict(negatives=negatives, edge_order=edge_order),
+                                  batch_size=bsz, num_workers=workers, num_batch_negs=nb, num_uniform_negs=nu,
+                                  loss="softmax", bucket_order="lexicographic", eval_fraction=frac,
+                                  eval_num_batch_negs=enb, eval_num_uniform_negs=enu)
+    cfg = ostep.StepConfig(dim=dim, loss="softmax", num_batch_negs=nb, num_uniform_negs=nu, lr=0.1)
+    cfg_eval = ostep.StepConfig(dim=dim, loss="softmax", num_batch_negs=enb, num_uniform_negs=enu, lr=0.1)
+    ebsz = 60  # batch_size rounded up to a multiple of eval_num_batch_negs (train_cpu.py:887-889)
+    w = {p: t.clone() for p, t in tables.items()}
+    g = {p: torch.zeros(t.shape[0]) for p, t in tables.items()}
+    it = iter(drawn)
+    flat = [s for e in stats for s in e]
+    pos = 0
+    for epoch in range(2):
+        for lhs_p in range(nparts):
+            for rhs_p in range(nparts):
+                got = flat[pos]
+                pos += 1
+                lhs, rhs, _ = edges[(lhs_p, rhs_p)]
+                n = lhs.shape[0]
+                eval_idx = bl.holdout_indices(n, frac, bl.Bucket(lhs_p, rhs_p))
+                assert eval_idx.shape[0] == int(n * frac)
+                st = ostep.make_state(cfg, w[lhs_p], None if lhs_p == rhs_p else w[rhs_p])
+                st.g_lhs = g[lhs_p]
+                st.g_rhs = g[lhs_p] if lhs_p == rhs_p else g[rhs_p]
+                want_before = _oracle_eval(cfg_eval, st, lhs, rhs, eval_idx, ebsz, workers, it)
+                # the training edges, by the reference's own statements
+                num_train = n - eval_idx.shape[0]
+                train_idx = torch.arange(n)
+                train_idx[eval_idx] = torch.arange(num_train, n)
+                order = train_idx[:num_train][perms[(lhs_p, rhs_p)][epoch]]
+                assert got.num_edges == num_train
+                tl, tr = lhs[order], rhs[order]
+                total = 0.0
+                for off, k, b_now in _calls_of(num_train, bsz, workers):
+                    ul, ur = next(it), next(it)
+                    batches = [(tl[off + i * b_now: off + (i + 1) * b_now], tr[off + i * b_now: off + (i + 1) * b_now],
+                                0, ul[i], ur[i]) for i in range(k)]
+                    total += sum(o.loss for o in ostep.train_lockstep(cfg, st, batches))
+                want_after = _oracle_eval(cfg_eval, st, lhs, rhs, eval_idx, ebsz, workers, it)
+                assert got.loss == pytest.approx(total, rel=1e-4)
+                for have, want in ((got.eval_before, want_before), (got.eval_after, want_after)):
+                    m = have.metrics
+                    assert have.count == want["count"] == eval_idx.shape[0]
+                    assert m["loss"] == pytest.approx(want["loss"], rel=1e-4)
+                    for key in ("pos_rank", "mrr", "r1", "r10"):
+                        assert want["low"][key] - 1e-3 <= m[key] <= want["high"][key] + 1e-3, key
+                    assert want["high"]["pos_rank"] - want["low"]["pos_rank"] <= 0.2 * have.count  # the bounds bind
+                    assert 0.0 <= have.average().metrics["auc"] <= 1.0
+    assert next(it, None) is None  # every draw was accounted for
+    for p in range(nparts):
+        assert torch.allclose(store.tables[("e", p)], w[p], rtol=1e-4, atol=1e-6)
+        assert torch.allclose(store.sums[("e", p)], g[p], rtol=1e-4, atol=1e-9)
+
+
+@pytest.mark.gpu
+def test_standard_relations_train_in_single_relation_batches(pbg):
+    """Several standard (non-dynamic) relation types: every batch holds one type
+    (batching.py:60-79), every training edge is used once, and the calls the loop
+    made, replayed on the oracle, give the same tables and operator parameters."""
+    bl = pbg.bucket_loop
+    nparts, dim, bsz, workers, nb, nu, nrel = 2, 8, 40, 3, 10, 5, 3
+    tables, edges = make_graph(nparts, 250, dim, 420, seed=7)
+    g0 = torch.Generator().manual_seed(11)
+    edges = {k: (l, r, torch.randint(0, nrel, l.shape, generator=g0) ** 2 % nrel) for k, (l, r, _) in edges.items()}
+    cfg = ostep.StepConfig(dim=dim, operator="translation", loss="ranking", margin=0.1, num_batch_negs=nb,
+                           num_uniform_negs=nu, num_relations=nrel, relation_weights=[1.0] * nrel, lr=0.1)
+    st0 = ostep.make_state(cfg, tables[0])
+    for k in st0.rhs_op:
+        st0.rhs_op[k] = st0.rhs_op[k] + 0.1 * torch.randn(st0.rhs_op[k].shape, generator=g0)
+    rhs_op = {k: v.clone().to(DEV) for k, v in st0.rhs_op.items()}
+    rhs_sum = {k: torch.zeros_like(v) for k, v in rhs_op.items()}
+    drawn = []
+
+    def negatives(k, c, u, rows, generator, device):
+        t = torch.randint(0, rows, (k, c, u), generator=generator, device=device)
+        drawn.append(t.cpu())
+        return t
+
+    store, stats, loop = run_loop(pbg, tables, edges, nparts, dim, 2, hooks=dict(negatives=negatives, record_calls=True),
+                                  batch_size=bsz, num_workers=workers, num_batch_negs=nb, num_uniform_negs=nu,
+                                  operator="translation", num_relations=nrel, rhs_op=rhs_op, rhs_op_sum=rhs_sum,
+                                  bucket_order="lexicographic")
+    w = {p: t.clone() for p, t in tables.items()}
+    g = {p: torch.zeros(t.shape[0]) for p, t in tables.items()}
+    op = {k: v.clone() for k, v in st0.rhs_op.items()}
+    op_sum = {k: torch.zeros_like(v) for k, v in op.items()}
+    it = iter(drawn)
+    seen = {}
+    for call in loop.calls_log:
+        b, k, b_now = call["bucket"], call["workers"], call["batch_size"]
+        lhs, rhs, rel = call["lhs"], call["rhs"], call["rel"]
+        assert lhs.shape == (k * b_now,) and rel.shape == (k,) and k <= workers
+        # a batch holds edges of its one relation type, taken from the bucket
+        el, er, erel = edges[(b.lhs, b.rhs)]
+        keys = set(zip(el.tolist(), er.tolist(), erel.tolist()))
+        for i in range(k):
+            for a, c in zip(lhs[i * b_now:(i + 1) * b_now].tolist(), rhs[i * b_now:(i + 1) * b_now].tolist()):
+                assert (a, c, int(rel[i])) in keys
+        seen[(call["epoch"], b.lhs, b.rhs)] = seen.get((call["epoch"], b.lhs, b.rhs), 0) + k * b_now
+        st = ostep.make_state(cfg, w[b.lhs], None if b.lhs == b.rhs else w[b.rhs])
+        st.g_lhs = g[b.lhs]
+        st.g_rhs = g[b.lhs] if b.lhs == b.rhs else g[b.rhs]
+        st.rhs_op, st.rhs_op_sum = op, op_sum
+        ul, ur = next(it), next(it)
+        batches = [(lhs[i * b_now:(i + 1) * b_now], rhs[i * b_now:(i + 1) * b_now], int(rel[i]), ul[i], ur[i])
+                   for i in range(k)]
+        ostep.train_lockstep(cfg, st, batches)
+    for (epoch, l, r), count in seen.items():
+        assert count == edges[(l, r)][0].shape[0]
+    assert len(seen) == 2 * nparts * nparts
+    for p in range(nparts):
+        assert torch.allclose(store.tables[("e", p)], w[p], rtol=1e-4, atol=1e-6)
+    for k in op:
+        assert not torch.equal(op[k], st0.rhs_op[k])
+        assert torch.allclose(rhs_op[k].cpu(), op[k], rtol=1e-4, atol=1e-6)
+        assert torch.allclose(rhs_sum[k].cpu(), op_sum[k], rtol=1e-4, atol=1e-9)
