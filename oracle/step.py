@@ -38,6 +38,9 @@ class StepConfig:
     lr: float = 0.1
     relation_lr: Optional[float] = None
     relation_weights: Sequence[float] = field(default_factory=lambda: [1.0])
+    # config.py:221-230: coefficient of the N3 regularizer (the only one registered,
+    # regularizers.py:51); 0 = none (model.py:905-909)
+    regularization_coef: float = 0.0
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
@@ -222,6 +225,55 @@ def loss_value(
 
 
 # --------------------------------------------------------------------------
+# N3 regularizer (regularizers.py:51-97) with the operators' hooks
+# (operators.py:39-43,55-56,69-70,83-84,151-157 static; :185-191,206-209,225-228,
+# 246-249,332-338 dynamic)
+# --------------------------------------------------------------------------
+
+def _embs_for_reg(operator: str, embs: torch.Tensor) -> torch.Tensor:
+    """prepare_embs_for_reg: the modulus of each complex coordinate for
+    complex_diagonal (operators.py:154-157), |x| otherwise (operators.py:42-43)."""
+    if operator == "complex_diagonal":
+        h = embs.shape[-1] // 2
+        real, imag = embs[..., :h], embs[..., h:]
+        return torch.sqrt(real ** 2 + imag ** 2)
+    return embs.abs()
+
+
+def _params_for_reg(operator: str, params: Optional[Dict[str, torch.Tensor]], rel) -> Optional[torch.Tensor]:
+    """get_operator_params_for_reg of the operator of relation `rel` (an int:
+    operators.py:55-56,69-70,83-84,151-152) or of the operators of the edges
+    (LongTensor[B]: operators.py:206-209,225-228,246-249,332-333)."""
+    if operator == "none":
+        return None
+    if operator == "diagonal":
+        return params["diagonal"][rel].abs()
+    if operator == "translation":
+        return params["translation"][rel].abs()
+    if operator == "complex_diagonal":
+        return torch.sqrt(params["real"][rel] ** 2 + params["imag"][rel] ** 2)
+    raise NotImplementedError("Regularizer not implemented for this operator")  # operators.py:40,188
+
+
+def n3_regularizer(cfg: StepConfig, src_pos: torch.Tensor, dst_pos: torch.Tensor, rel, op_params) -> torch.Tensor:
+    """N3Regularizer.forward (standard relations, regularizers.py:82-97) or
+    forward_dynamic (regularizers.py:66-80).  src_pos / dst_pos are the chunked
+    [C, P, D] positives after operator and comparator.prepare, as
+    forward_direction_agnostic passes them (model.py:784-785,800-801,846-854), so
+    `len(src_pos)` in the standard branch is the number of CHUNKS."""
+    total = 0
+    params = _params_for_reg(cfg.operator, op_params, rel)
+    if params is not None:
+        if isinstance(rel, int):
+            total = total + torch.sum(params ** 3) * len(src_pos)
+        else:
+            total = total + torch.sum(params ** 3)
+    for x in (src_pos, dst_pos):
+        total = total + torch.sum(_embs_for_reg(cfg.operator, x) ** 3)
+    return total * cfg.regularization_coef
+
+
+# --------------------------------------------------------------------------
 # the model forward (model.py:478-856)
 # --------------------------------------------------------------------------
 
@@ -231,6 +283,7 @@ class Scores:
     rhs_pos: torch.Tensor
     lhs_neg: torch.Tensor
     rhs_neg: torch.Tensor
+    reg: Optional[torch.Tensor] = None  # the second value MultiRelationEmbedder.forward returns
 
 
 def _adjust(cfg: StepConfig, embs, rel, op_params) -> torch.Tensor:
@@ -307,7 +360,10 @@ def _direction_agnostic(
     pos_scores = pos_scores.flatten(0, 1)[:num_pos]
     src_neg_scores = src_neg_scores.flatten(0, 1)[:num_pos]
     dst_neg_scores = dst_neg_scores.flatten(0, 1)[:num_pos]
-    return pos_scores, src_neg_scores, dst_neg_scores
+    reg = None
+    if cfg.regularization_coef != 0:  # model.py:845-854
+        reg = n3_regularizer(cfg, src_pos, dst_pos, rel, dst_op_params)
+    return pos_scores, src_neg_scores, dst_neg_scores, reg
 
 
 def model_forward(
@@ -335,27 +391,28 @@ def model_forward(
             )
         if not isinstance(rel, int):
             raise TypeError("All positive pairs must come from the same relation")
-        pos, lneg, rneg = _direction_agnostic(
+        pos, lneg, rneg, reg = _direction_agnostic(
             cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, rhs_uniform, rel,
             rhs_op_params if cfg.operator != "none" else None,
             chunk_size, lhs_method, rhs_method,
         )
-        return Scores(pos, pos, lneg, rneg)
+        return Scores(pos, pos, lneg, rneg, reg)
     if isinstance(rel, int):
         raise TypeError("Need relation for each positive pair")
     # model.py:721-754: forward edges (operator on rhs, negatives on lhs),
     # then reverse edges (operator on lhs, negatives on rhs).
-    lpos, lneg, _ = _direction_agnostic(
+    lpos, lneg, _, l_reg = _direction_agnostic(
         cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, None, rel,
         rhs_op_params if cfg.operator != "none" else None,
         chunk_size, lhs_method, "none",
     )
-    rpos, rneg, _ = _direction_agnostic(
+    rpos, rneg, _, r_reg = _direction_agnostic(
         cfg, num_pos, rhs_pos, lhs_pos, rhs_uniform, None, rel,
         lhs_op_params if cfg.operator != "none" else None,
         chunk_size, rhs_method, "none",
     )
-    return Scores(lpos, rpos, lneg, rneg)
+    reg = None if l_reg is None or r_reg is None else l_reg + r_reg  # model.py:755-758
+    return Scores(lpos, rpos, lneg, rneg, reg)
 
 
 # --------------------------------------------------------------------------
@@ -445,6 +502,7 @@ class StepOutput:
     violators_rhs: int
     count: int
     scores: Optional[Scores] = None
+    reg: float = 0.0
 
 
 @dataclass
@@ -504,8 +562,12 @@ def forward_backward(
             scores.lhs_pos.detach(), scores.rhs_pos.detach(),
             scores.lhs_neg.detach(), scores.rhs_neg.detach(),
         ) if keep_scores else None,
+        reg=float(scores.reg.detach()) if scores.reg is not None else 0.0,
     )
-    loss.backward()
+    if scores.reg is not None:  # train_cpu.py:102-105
+        (loss + scores.reg).backward()
+    else:
+        loss.backward()
     grads = StepGrads(
         sparse_lhs=w_l.grad,
         sparse_rhs=None if st.shared else w_r.grad,
