@@ -127,6 +127,12 @@ typedef struct pbg_step_desc {
   int32_t shared_table;     /* 1: lhs and rhs index the same table (w_rhs == w_lhs, g_rhs == g_lhs) */
   int64_t num_lhs_rows;     /* rows of w_lhs */
   int64_t num_rhs_rows;     /* rows of w_rhs */
+  /* config.regularization_coef with config.regularizer = "N3" (the one registered,
+   * regularizers.py:51-97, model.py:845-854): the step minimises loss + reg
+   * (train_cpu.py:102-103).  0 = no regularizer.  Not defined for `linear`
+   * (operators.py:40). */
+  float regularization_coef;
+  int32_t reserved0;        /* keep 0 */
 } pbg_step_desc;
 
 typedef struct pbg_step_buffers {
@@ -157,6 +163,7 @@ typedef struct pbg_step_buffers {
    * Pass a fresh seed per call. */
   int32_t sample_uniform;
   uint64_t uniform_seed;
+  float* reg_out;             /* [K] regularizer value of each batch (Stats.reg, train_cpu.py:97), or null */
 } pbg_step_buffers;
 
 /* sizeof(pbg_step_desc) / sizeof(pbg_step_buffers) as this library was compiled:

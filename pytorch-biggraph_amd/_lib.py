@@ -43,6 +43,8 @@ class StepDesc(ctypes.Structure):
         ("shared_table", c_int32),
         ("num_lhs_rows", c_int64),
         ("num_rhs_rows", c_int64),
+        ("regularization_coef", c_float),
+        ("reserved0", c_int32),
     ]
 
 
@@ -58,7 +60,7 @@ class StepBuffers(ctypes.Structure):
         ("lhs_op_p0", c_void_p), ("lhs_op_p1", c_void_p), ("lhs_op_s0", c_void_p), ("lhs_op_s1", c_void_p),
         ("loss_out", c_void_p), ("violators_out", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
-        ("sample_uniform", c_int32), ("uniform_seed", c_uint64),
+        ("sample_uniform", c_int32), ("uniform_seed", c_uint64), ("reg_out", c_void_p),
     ]
 
 

@@ -52,6 +52,10 @@ struct SideCtx {
   const float *p0, *p1; // operator parameters
   float *xraw, *z, *dz; // [K, op_rows, D] staging of operator inputs / outputs / output grads
   int op_rows;
+  // N3 regularizer, dynamic relations: per relation, the gradient of the parameter
+  // term per edge [num_relations, D] and the term itself [num_relations], both
+  // from the parameters as they are before the call's updates
+  float *reg_pgrad, *reg_pcube;
   int plain_written, opd_written;  // dxp / dxa were produced by a GEMM
 };
 
@@ -73,6 +77,9 @@ struct StepCtx {
   uint32_t* vals;
   unsigned long long* violators;  // [K, 2]
   float* loss_out;                // [K]
+  float reg_coef;  // N3 regularizer weight (0: none)
+  float* regrow;   // [K, 2, B] sum of cubed moduli of each positive's prepared row(s), per side
+  float* reg_out;  // [K] or null
 };
 
 // Uniform negative number flat = (k * C + chunk) * U + u of side s: given by the
@@ -477,6 +484,31 @@ __device__ __forceinline__ float column_sum(const float* __restrict__ s, int64_t
   return wave_sum(acc);
 }
 
+// N3 regularizer (regularizers.py:51-97) on one prepared row y: adds
+// d (coef * sum m^3) / dy = 3 coef m y to dy and returns this lane's share of
+// sum m^3, where m is the modulus of a complex coordinate (y[e], y[e + D/2]) for
+// complex_diagonal (operators.py:154-157) and |y[e]| otherwise (operators.py:42-43).
+template <int NVH>
+__device__ __forceinline__ float n3_term(int op, float coef, RowV<NVH>& dy, const RowV<NVH>& y) {
+  float cubes = 0.f;
+  const float c3 = 3.0f * coef;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    if (op == PBG_OP_COMPLEX_DIAGONAL) {
+      const float m = sqrtf(y.a[0][v] * y.a[0][v] + y.a[1][v] * y.a[1][v]);
+      dy.a[0][v] += c3 * m * y.a[0][v];
+      dy.a[1][v] += c3 * m * y.a[1][v];
+      cubes += m * m * m;
+    } else {
+      const float m0 = fabsf(y.a[0][v]), m1 = fabsf(y.a[1][v]);
+      dy.a[0][v] += c3 * m0 * y.a[0][v];
+      dy.a[1][v] += c3 * m1 * y.a[1][v];
+      cubes += m0 * m0 * m0 + m1 * m1 * m1;
+    }
+  }
+  return cubes;
+}
+
 // dy += dpos * d kappa(self, other) / d self
 template <int NVH>
 __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos, const RowV<NVH>& self,
@@ -533,6 +565,10 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       }
       const RowV<NVH> other = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
       add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq]);
+      if (c.reg_coef != 0.f) {  // src_pos / dst_pos of the regularizer are these prepared rows (model.py:784-785,854)
+        const float cubes = wave_sum(n3_term<NVH>(c.op, c.reg_coef, dy, y1));
+        if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
+      }
       const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
       if (sd.has_op) {
         if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz, D, H, lane);
@@ -551,6 +587,10 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       }
       const RowV<NVH> other = row_load<NVH>(so.xa + (kc * c.P + i) * D, D, H, lane);
       add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq]);
+      // the plain row is src_pos of one direction's regularizer, the operated row
+      // dst_pos of the other's (model.py:722-754)
+      float cubes = 0.f;
+      if (c.reg_coef != 0.f) cubes = n3_term<NVH>(c.op, c.reg_coef, dy, y1);
       RowV<NVH> dx = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
       // role 2: the operated row f(op(x)), scored against the other side's negatives
       const RowV<NVH> y2 = row_load<NVH>(sd.xa + (kc * c.P + i) * D, D, H, lane);
@@ -562,6 +602,10 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       }
       const RowV<NVH> other2 = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
       add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq]);
+      if (c.reg_coef != 0.f) {
+        cubes = wave_sum(cubes + n3_term<NVH>(c.op, c.reg_coef, dy2, y2));
+        if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
+      }
       const RowV<NVH> dz2 = prepare_backward<NVH>(c.cmp, dy2, y2, aux2);
       if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz2, D, H, lane);
       if (c.op != PBG_OP_LINEAR) {
@@ -638,6 +682,20 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
     float total = 0.f;
 #pragma unroll
     for (int g = 0; g < kParamGroups; ++g) total += sh[g][lane];
+    if (slice == 0 && c.reg_coef != 0.f) {
+      // N3 on the operator's parameters (regularizers.py:90-93): coef * C * sum m^3, with
+      // m = |p| (operators.py:69-70,83-84) or the modulus of (real, imag) (operators.py:151-152)
+      const int64_t r = clamp_index(c.rel[k], c.num_relations);
+      const float c3 = 3.0f * c.reg_coef * (float)c.C;
+      if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+        const int h = e < H ? e : e - H;
+        const float re = sd.p0[r * H + h], im = sd.p1[r * H + h];
+        total += c3 * sqrtf(re * re + im * im) * (e < H ? re : im);
+      } else {
+        const float pv = sd.p0[r * D + e];
+        total += c3 * fabsf(pv) * pv;
+      }
+    }
     dth[((int64_t)k * slices + slice) * D + e] = total;
   }
 }
@@ -1483,7 +1541,9 @@ __global__ __launch_bounds__(256) void dyn_param_kernel(StepCtx c, int s, const 
     sh[rg][lane] = acc;
     __syncthreads();
     if (rg == 0 && e < D) {
-      const float g = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+      float g = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+      // N3 on the parameters of the run's edges (regularizers.py:73-76), from the values before this call
+      if (c.reg_coef != 0.f) g += (float)(end - j) * sd.reg_pgrad[rel * D + e];
       const float sum = *st + g * g;
       *st = sum;
       *p += -lr * (g / (sqrtf(sum) + 1e-10f));
@@ -1491,6 +1551,79 @@ __global__ __launch_bounds__(256) void dyn_param_kernel(StepCtx c, int s, const 
     __syncthreads();
     j = end;
   }
+}
+
+// ---------------------------------------------------------------------------
+// N3 regularizer: parameter terms and the per-batch value
+// ---------------------------------------------------------------------------
+// Dynamic relations, one wave per relation: reg_pgrad[rel, e] = d (coef * sum m^3) / d p[rel, e]
+// for one edge of the relation, reg_pcube[rel] = sum m^3 (regularizers.py:73-76;
+// operators.py:225-228,246-249,332-333).
+__global__ __launch_bounds__(kRowThreads) void reg_factor_kernel(StepCtx c, int s) {
+  const SideCtx& sd = c.side[s];
+  const int lane = threadIdx.x & 63;
+  const int64_t rel = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (rel >= c.num_relations) return;
+  const int D = c.D, H = D / 2;
+  const float c3 = 3.0f * c.reg_coef;
+  float cubes = 0.f;
+  for (int e = lane; e < D; e += kWave) {
+    float m, pv;
+    if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+      const int h = e < H ? e : e - H;
+      const float re = sd.p0[rel * H + h], im = sd.p1[rel * H + h];
+      m = sqrtf(re * re + im * im);
+      pv = e < H ? re : im;
+      if (e < H) cubes += m * m * m;  // one modulus per complex coordinate
+    } else {
+      pv = sd.p0[rel * D + e];
+      m = fabsf(pv);
+      cubes += m * m * m;
+    }
+    sd.reg_pgrad[rel * D + e] = c3 * m * pv;
+  }
+  cubes = wave_sum(cubes);
+  if (lane == 0) sd.reg_pcube[rel] = cubes;
+}
+
+// One workgroup per batch: reg_out[k] = coef * (sum over the positives' prepared rows
+// of m^3 (written by rowback_kernel) + the parameter term), summed in a fixed order.
+__global__ __launch_bounds__(256) void reg_reduce_kernel(StepCtx c) {
+  __shared__ float sh[256];
+  const int k = blockIdx.x, t = threadIdx.x;
+  const int D = c.D, H = D / 2;
+  float acc = 0.f;
+  const float* rows = c.regrow + (int64_t)k * 2 * c.B;
+  for (int i = t; i < 2 * c.B; i += 256) acc += rows[i];
+  if (c.op != PBG_OP_NONE) {
+    if (c.dynamic) {  // once per edge and direction (regularizers.py:73-76, model.py:755-758)
+      for (int i = t; i < c.B; i += 256) {
+        const int64_t r = clamp_index(c.rel[(int64_t)k * c.B + i], c.num_relations);
+        acc += c.side[0].reg_pcube[r] + c.side[1].reg_pcube[r];
+      }
+    } else {  // once per chunk (regularizers.py:91-93)
+      const SideCtx& sd = c.side[1];
+      const int64_t r = clamp_index(c.rel[k], c.num_relations);
+      const int count = c.op == PBG_OP_COMPLEX_DIAGONAL ? H : D;
+      for (int e = t; e < count; e += 256) {
+        float m;
+        if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+          const float re = sd.p0[r * H + e], im = sd.p1[r * H + e];
+          m = sqrtf(re * re + im * im);
+        } else {
+          m = fabsf(sd.p0[r * D + e]);
+        }
+        acc += (float)c.C * m * m * m;
+      }
+    }
+  }
+  sh[t] = acc;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) sh[t] += sh[t + w];
+    __syncthreads();
+  }
+  if (t == 0 && c.reg_out) c.reg_out[k] = c.reg_coef * sh[0];
 }
 
 // ---------------------------------------------------------------------------
@@ -1531,6 +1664,8 @@ int validate(const pbg_step_desc* d, bool training) {
     return fail(PBG_ERR_INVALID,
                 "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");  // operators.py:132-136
   if (d->num_relations < 1) return fail(PBG_ERR_INVALID, "step: num_relations must be positive");
+  if (d->regularization_coef != 0.f && d->op == PBG_OP_LINEAR)
+    return fail(PBG_ERR_UNSUPPORTED, "Regularizer not implemented for this operator");  // operators.py:40,188
   if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
   return PBG_OK;
 }
@@ -1642,6 +1777,15 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   }
   c.lossrow = takef(K * CP);
   c.violrow = (int*)take(K * CP * 2, sizeof(int));
+  c.reg_coef = d->regularization_coef;
+  if (c.reg_coef != 0.f) {
+    c.regrow = takef((size_t)K * 2 * c.B);
+    if (c.dynamic && c.op != PBG_OP_NONE)
+      for (int s = 0; s < 2; ++s) {
+        c.side[s].reg_pgrad = takef((size_t)c.num_relations * D);
+        c.side[s].reg_pcube = takef((size_t)c.num_relations);
+      }
+  }
 
   plan->psize = 0;
   if (c.op == PBG_OP_LINEAR) plan->psize = (int64_t)D * D;
@@ -1674,7 +1818,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->sort_temp = take(sort_temp_bytes(npairs), 1);
   plan->bytes = off;
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
-  plan->fused = fused_layout(c, &plan->fl) && getenv("PBG_DISABLE_FUSED") == nullptr;
+  // (the regularizer's terms live in the staged kernels only)
+  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && getenv("PBG_DISABLE_FUSED") == nullptr;
 
   if (b) {
     c.side[0].w = b->w_lhs;
@@ -1693,6 +1838,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     c.rel_weights = b->relation_weights;
     c.violators = (unsigned long long*)b->violators_out;
     c.loss_out = b->loss_out;
+    c.reg_out = b->reg_out;
   }
   return PBG_OK;
 }
@@ -2064,6 +2210,12 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if ((rc = run_backward_da(plan, s)) != PBG_OK) return rc;
     mark(6);
     if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
+    if (c.reg_coef != 0.f) {  // reads the operator parameters: before run_params updates them
+      if (c.dynamic && c.op != PBG_OP_NONE)
+        for (int side = 0; side < 2; ++side)
+          hipLaunchKernelGGL(reg_factor_kernel, wave_grid(c.num_relations), dim3(kRowThreads), 0, s, c, side);
+      hipLaunchKernelGGL(reg_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+    }
     mark(7);
   }
   if ((rc = run_params(desc, bufs, plan, s, &rel_order)) != PBG_OK) return rc;

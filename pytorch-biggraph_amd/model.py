@@ -11,9 +11,12 @@ outside, so that two implementations can be fed the same negatives.  Training
 goes through ``train.Trainer`` (one pbg_train_step call per batch), not through
 autograd on these scores.
 
+``regularizer``: an ``N3Regularizer`` (the one the reference registers); the
+training step takes its weight, ``forward`` returns its value as the reference's
+does.
+
 Not provided (outside the accelerated path): FeaturizedEmbedding, squared_l2,
-BiasedComparator, all_negs, global embeddings, max_norm, half precision,
-regularizers.
+BiasedComparator, all_negs, global embeddings, max_norm, half precision.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -28,6 +31,7 @@ from .config import EntitySchema, RelationSchema
 from .edgelist import EdgeList
 from .entitylist import EntityList
 from .native import _need, _ptr, _stream
+from .regularizers import AbstractRegularizer, N3Regularizer
 from .operators import AbstractDynamicOperator, AbstractOperator
 from .plugin import PluginRegistry
 from .types import Bucket, FloatTensorType, LongTensorType, Side
@@ -240,8 +244,8 @@ class MultiRelationEmbedder(nn.Module):
         half_precision: bool = False,
     ) -> None:
         super().__init__()
-        if regularizer is not None:
-            raise NotImplementedError("Regularizers are not supported")
+        if regularizer is not None and not isinstance(regularizer, N3Regularizer):
+            raise NotImplementedError("Only the N3 regularizer is supported")
         if global_emb:
             raise NotImplementedError("Global embeddings are not supported")
         if max_norm is not None:
@@ -270,7 +274,7 @@ class MultiRelationEmbedder(nn.Module):
         self.global_embs = None
         self.max_norm = None
         self.half_precision = False
-        self.regularizer = None
+        self.regularizer: Optional[AbstractRegularizer] = regularizer
         self._runners: Dict[tuple, native.StepRunner] = {}
 
     # --- embeddings ---------------------------------------------------------
@@ -324,7 +328,8 @@ class MultiRelationEmbedder(nn.Module):
             disable_rhs_negs=bool(self.disable_rhs_negs),
             operator=rhs_op.op_name if rhs_op is not None else "none", dynamic=dynamic,
             num_relations=self.num_dynamic_rels if dynamic else 1,
-            comparator=self.comparator.comparator_name, **training)
+            comparator=self.comparator.comparator_name,
+            regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0, **training)
 
     def operator_tensors(self, relation_idx: int):
         """({name: tensor} of the rhs operator, of the lhs operator) in the
@@ -347,9 +352,32 @@ class MultiRelationEmbedder(nn.Module):
         ur = rhs_module.sample_indices(num_chunks, u) if (u > 0 and not self.disable_rhs_negs) else None
         return ul, ur
 
-    def forward(self, edges: EdgeList, uniform_negs=None) -> Tuple[Scores, None]:
-        """Scores of a batch (model.py:624-762).  `uniform_negs` = (lhs [C,U],
-        rhs [C,U]) entity indices; drawn with torch.randint when omitted."""
+    def _regularizer_value(self, relation_idx: int, lhs_module, rhs_module, lhs, rhs, rel, chunk_size: int):
+        """What forward_direction_agnostic hands the regularizer (model.py:784-801,
+        845-854), per direction: the positives after operator and
+        comparator.prepare, zero-padded to whole chunks, as [C, P, D]."""
+        def chunked(embs, operator):
+            if operator is not None:
+                embs = operator(embs, rel) if self.num_dynamic_rels > 0 else operator(embs)
+            embs = self.comparator.prepare(embs)
+            pad = -embs.shape[0] % chunk_size
+            if pad:
+                embs = torch.cat((embs, embs.new_zeros((pad, embs.shape[1]))), dim=0)
+            return embs.view(-1, chunk_size, embs.shape[1])
+
+        with torch.no_grad():
+            lhs_pos, rhs_pos = lhs_module.get(lhs), rhs_module.get(rhs)
+            if self.num_dynamic_rels == 0:
+                op = self.rhs_operators[relation_idx]
+                return self.regularizer.forward(chunked(lhs_pos, None), chunked(rhs_pos, op), op)
+            rhs_op, lhs_op = self.rhs_operators[relation_idx], self.lhs_operators[relation_idx]
+            return (self.regularizer.forward_dynamic(chunked(lhs_pos, None), chunked(rhs_pos, rhs_op), rhs_op, rel)
+                    + self.regularizer.forward_dynamic(chunked(rhs_pos, None), chunked(lhs_pos, lhs_op), lhs_op, rel))
+
+    def forward(self, edges: EdgeList, uniform_negs=None) -> Tuple[Scores, Optional[FloatTensorType]]:
+        """Scores of a batch and the regularizer's value, None without a
+        regularizer (model.py:624-762).  `uniform_negs` = (lhs [C,U], rhs [C,U])
+        entity indices; drawn with torch.randint when omitted."""
         num_pos = len(edges)
         relation_idx, lhs_module, rhs_module = self.resolve(edges)
         if self.num_batch_negs == 0 and self.num_uniform_negs == 0:
@@ -382,4 +410,7 @@ class MultiRelationEmbedder(nn.Module):
             rel = torch.zeros(1, dtype=torch.int64, device=dev)  # the runner holds this relation's operator only
         lp, rp, ln, rn = runner.forward(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
                                         ur.contiguous() if ur is not None else None)
-        return Scores(lp[0], rp[0], ln[0], rn[0]), None
+        reg = None
+        if self.regularizer is not None:
+            reg = self._regularizer_value(relation_idx, lhs_module, rhs_module, lhs, rhs, rel, spec.chunk_size)
+        return Scores(lp[0], rp[0], ln[0], rn[0]), reg

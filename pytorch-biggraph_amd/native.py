@@ -194,6 +194,7 @@ class StepSpec:
     margin: float = 0.1
     lr: float = 0.1
     relation_lr: Optional[float] = None
+    regularization_coef: float = 0.0  # config.regularization_coef of the N3 regularizer; 0 = none
 
     @property
     def chunk_size(self) -> int:
@@ -255,6 +256,7 @@ class StepRunner:
         d.shared_table = int(shared)
         d.num_lhs_rows = self.w_lhs.shape[0]
         d.num_rhs_rows = self.w_rhs.shape[0]
+        d.regularization_coef = spec.regularization_coef
         self.desc = d
         self.rhs_op = rhs_op or {}
         self.rhs_op_sum = rhs_op_sum or {}
@@ -271,6 +273,7 @@ class StepRunner:
         k = spec.num_workers
         self.loss_out = torch.zeros(k, dtype=torch.float32, device=dev)
         self.violators_out = torch.zeros((k, 2), dtype=torch.int64, device=dev)
+        self.reg_out = torch.zeros(k, dtype=torch.float32, device=dev)  # Stats.reg of each batch
 
     @staticmethod
     def _op_pair(params: Dict[str, torch.Tensor]) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
@@ -315,6 +318,7 @@ class StepRunner:
         s0, s1 = self._op_pair(self.lhs_op_sum)
         bufs.lhs_op_p0, bufs.lhs_op_p1, bufs.lhs_op_s0, bufs.lhs_op_s1 = _ptr(p0), _ptr(p1), _ptr(s0), _ptr(s1)
         bufs.loss_out, bufs.violators_out = _ptr(self.loss_out), _ptr(self.violators_out)
+        bufs.reg_out = _ptr(self.reg_out)
         bufs.workspace, bufs.workspace_bytes = _ptr(self.workspace), self.workspace.numel()
         bufs.sample_uniform = int(uniform_seed is not None)
         bufs.uniform_seed = (uniform_seed or 0) & (2**64 - 1)

@@ -110,5 +110,5 @@ class Trainer(AbstractBatchProcessor):
                      ur.contiguous() if ur is not None else None, weight)
         # the reference reads loss and both violator counts on the host for every batch (train_cpu.py:95-101)
         viol = runner.violators_out[0].tolist()
-        return Stats(loss=float(runner.loss_out[0]), reg=0.0, violators_lhs=int(viol[0]), violators_rhs=int(viol[1]),
+        return Stats(loss=float(runner.loss_out[0]), reg=float(runner.reg_out[0]), violators_lhs=int(viol[0]), violators_rhs=int(viol[1]),
                      count=num_pos)

@@ -61,6 +61,10 @@ FULL = {
     "cfg2-standard": dict(entities=14_951, relations=1345, dim=400, batch=1000, nb=50, nu=1000,
                           operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, zipf=1.1,
                           two_tables=False),
+    # ... with the N3 regularizer of the reference's FB15k example (fb15k_config_cpu.py:41)
+    "cfg2-standard-n3": dict(entities=14_951, relations=1345, dim=400, batch=1000, nb=50, nu=1000,
+                             operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, zipf=1.1,
+                             two_tables=False, reg=1e-3),
     "cfg2-dynamic": dict(entities=14_951, relations=1345, dim=400, batch=1000, nb=50, nu=1000,
                          operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=True, zipf=1.1,
                          two_tables=False),
@@ -86,7 +90,8 @@ def test_full_shape_step(pbg, name, workers):
     e, d, b, r = w["entities"], w["dim"], w["batch"], w["relations"]
     cfg = ostep.StepConfig(dim=d, operator=w["operator"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
                            num_batch_negs=w["nb"], num_uniform_negs=w["nu"], dynamic=w["dynamic"], num_relations=r,
-                           lr=0.1, relation_lr=0.01, relation_weights=[1.0] * r)
+                           lr=0.1, relation_lr=0.01, relation_weights=[1.0] * r,
+                           regularization_coef=w.get("reg", 0.0))
     _, c, _ = cfg.chunking(b)
     u = w["nu"]
     gen = torch.Generator().manual_seed(7)
@@ -152,7 +157,7 @@ def test_full_shape_step(pbg, name, workers):
 
     spec = pbg.StepSpec(dim=d, batch_size=b, num_workers=workers, num_batch_negs=w["nb"], num_uniform_negs=u,
                         operator=w["operator"], dynamic=w["dynamic"], num_relations=r, comparator=w["comparator"],
-                        loss=w["loss"], margin=0.1, lr=0.1, relation_lr=0.01)
+                        loss=w["loss"], margin=0.1, lr=0.1, relation_lr=0.01, regularization_coef=w.get("reg", 0.0))
     ops = [{k: v.clone().to(DEV) for k, v in dct.items()} for dct in (st.rhs_op, st.rhs_op_sum, st.lhs_op, st.lhs_op_sum)]
     runner = pbg.StepRunner(spec, tables[0], sums[0], tables[1] if w["two_tables"] else None,
                             sums[1] if w["two_tables"] else None, ops[0], ops[1], ops[2], ops[3])
@@ -183,6 +188,7 @@ def test_full_shape_step(pbg, name, workers):
     rtol = 1e-5 if w["comparator"] != "l2" else 1e-4
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
     want_w = [(st.w_lhs, st64.w_lhs)] + ([(st.w_rhs, st64.w_rhs)] if w["two_tables"] else [])
     want_g = [(st.g_lhs, st64.g_lhs)] + ([(st.g_rhs, st64.g_rhs)] if w["two_tables"] else [])
     for i in range(len(tables)):

@@ -157,9 +157,13 @@ def build_model(pbg, cfg, st, n_rel_schemas):
                     for i, op in enumerate(ops):
                         if op is not None:
                             getattr(op, k)[...] = v[i].to(DEV)
+    regularizer = None
+    if cfg.regularization_coef != 0:  # model.py:905-909
+        regularizer = pbg.regularizers.REGULARIZERS.get_class("N3")(cfg.regularization_coef)
     model = M.MultiRelationEmbedder(
         cfg.dim, rels, ent, cfg.num_batch_negs, cfg.num_uniform_negs, cfg.disable_lhs_negs, cfg.disable_rhs_negs,
-        lhs_ops, rhs_ops, M.COMPARATORS.get_class(cfg.comparator)(), num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
+        lhs_ops, rhs_ops, M.COMPARATORS.get_class(cfg.comparator)(), regularizer=regularizer,
+        num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
     model.set_embeddings("l", pbg.types.Side.LHS, w_l)
     model.set_embeddings("l" if st.shared else "r", pbg.types.Side.RHS, w_r)
     return model, w_l, w_r
@@ -172,6 +176,13 @@ MODEL_CASES = [
     dict(operator="linear", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=0, num_uniform_negs=7, num_pos=30, dim=9),
     dict(operator="none", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
+    # with the N3 regularizer (the reference's FB15k example uses 1e-3 on ComplEx)
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20,
+         num_pos=45, dim=16, regularization_coef=1e-2),
+    dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25,
+         dim=8, regularization_coef=5e-2),
+    dict(operator="translation", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=5,
+         num_pos=25, dim=9, regularization_coef=5e-2),
 ]
 
 
@@ -200,8 +211,11 @@ def test_model_forward_and_trainer_step(pbg, case):
         rel_t = rel.to(DEV) if cfg.dynamic else torch.tensor(rel)
         edges = ED(EL.from_tensor(lhs.to(DEV)), EL.from_tensor(rhs.to(DEV)), rel_t)
         scores, reg = model(edges, uniform_negs=(ul.to(DEV), ur.to(DEV)))
-        assert reg is None
         want, _ = ostep.forward_backward(cfg, st, lhs, rhs, rel, ul, ur, keep_scores=True)
+        if cfg.regularization_coef == 0:
+            assert reg is None
+        else:
+            assert float(reg) == pytest.approx(want.reg, rel=1e-5)
         compare_scores(cfg, tuple(scores), want.scores)
         trainer.next_uniform_negs = (ul.to(DEV), ur.to(DEV))
         stats = trainer.process_one_batch(model, edges)
@@ -209,6 +223,7 @@ def test_model_forward_and_trainer_step(pbg, case):
         rtol = 1e-4 if cfg.comparator == "l2" else 1e-5
         assert stats.count == num_pos
         assert stats.metrics["loss"] == pytest.approx(out.loss, rel=rtol, abs=1e-6)
+        assert stats.metrics["reg"] == pytest.approx(out.reg, rel=1e-5)
         for side, pos, neg, n_want in (("lhs", want.scores.lhs_pos, want.scores.lhs_neg, out.violators_lhs),
                                        ("rhs", want.scores.rhs_pos, want.scores.rhs_neg, out.violators_rhs)):
             pp = pos.unsqueeze(1)

@@ -47,7 +47,7 @@ def to_runner(pbg, cfg, st, num_pos, workers):
         num_uniform_negs=cfg.num_uniform_negs, disable_lhs_negs=cfg.disable_lhs_negs,
         disable_rhs_negs=cfg.disable_rhs_negs, operator=cfg.operator, dynamic=cfg.dynamic,
         num_relations=cfg.num_relations, comparator=cfg.comparator, loss=cfg.loss, margin=cfg.margin, lr=cfg.lr,
-        relation_lr=cfg.relation_lr)
+        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef)
     dev = lambda t: t.clone().to(DEV)
     w_l, g_l = dev(st.w_lhs), dev(st.g_lhs)
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))
@@ -246,6 +246,71 @@ def test_train_step(pbg, case, workers):
             ties = int(((neg - p).abs() <= 2e-5 * p.abs().clamp_min(1e-6)).sum())
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
     compare_state(cfg, runner, st, rtol, "step")
+
+
+REG_CASES = [
+    # the reference's FB15k example: ComplEx, softmax, N3 with coefficient 1e-3 (fb15k_config_cpu.py:33-41)
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=50,
+         num_uniform_negs=100, num_pos=130, dim=400, regularization_coef=1e-3),
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=20,
+         num_uniform_negs=10, num_pos=70, dim=32, regularization_coef=1e-2),
+    dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=8, num_uniform_negs=4,
+         num_pos=30, dim=9, regularization_coef=0.05),
+    dict(operator="diagonal", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=8, num_uniform_negs=4,
+         num_pos=30, dim=10, regularization_coef=0.05),
+    dict(operator="translation", comparator="l2", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=10,
+         num_pos=45, dim=12, regularization_coef=0.02),
+    dict(operator="translation", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=0,
+         num_pos=45, dim=12, regularization_coef=0.02, disable_rhs_negs=True),
+    # shapes the fused kernel would take without a regularizer
+    dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50,
+         num_pos=200, dim=100, regularization_coef=0.01),
+    dict(operator="none", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=6, num_uniform_negs=3,
+         num_pos=20, dim=8, regularization_coef=0.1),
+]
+
+
+@pytest.mark.parametrize("case", REG_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_n3_regularizer(pbg, case, workers):
+    """(loss + reg).backward() (train_cpu.py:102-103) with the N3 regularizer
+    (regularizers.py:51-97): loss, regularizer value, tables, Adagrad sums and
+    operator parameters against the oracle."""
+    say("train+N3", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, **case)
+    n_ent = max(200, num_pos * (40 if cfg.comparator == "l2" else 4))
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=(dim % 2 == 0))
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    assert not runner.fused
+    before = runner.w_lhs.clone()
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    plain = ostep.StepConfig(**{**cfg.__dict__, "regularization_coef": 0.0})
+    st_plain = ostep.TrainState(**{k: (v.clone() if torch.is_tensor(v) else {n: t.clone() for n, t in v.items()})
+                                   for k, v in st.__dict__.items()})
+    if st.shared:
+        st_plain.w_rhs, st_plain.g_rhs = st_plain.w_lhs, st_plain.g_lhs
+    outs = ostep.train_lockstep(cfg, st, batches)
+    ostep.train_lockstep(plain, st_plain, batches)
+    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert out.reg > 0.0
+        assert float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
+    compare_state(cfg, runner, st, rtol, "step+N3")
+    # the regularizer moved the result: the comparison above would not pass without it
+    assert (st.w_lhs - st_plain.w_lhs).abs().max() > 100 * rtol * (st.w_lhs - before.cpu()).abs().max()
+
+
+def test_regularizer_is_refused_for_linear(pbg):
+    spec = pbg.StepSpec(dim=8, batch_size=10, operator="linear", regularization_coef=1e-3)
+    w = torch.randn(20, 8, device=DEV)
+    with pytest.raises((RuntimeError, NotImplementedError), match="Regularizer not implemented"):
+        pbg.StepRunner(spec, w, torch.zeros(20, device=DEV), rhs_op={"linear_transformation": torch.eye(8, device=DEV)[None]},
+                       rhs_op_sum={"linear_transformation": torch.zeros(1, 8, 8, device=DEV)})
 
 
 @pytest.mark.parametrize("case", [
