@@ -46,7 +46,7 @@ typedef enum pbg_operator {
   PBG_OP_LINEAR = 3,
   PBG_OP_COMPLEX_DIAGONAL = 4
 } pbg_operator;
-typedef enum pbg_comparator { PBG_CMP_DOT = 0, PBG_CMP_COS = 1, PBG_CMP_L2 = 2 } pbg_comparator;
+typedef enum pbg_comparator { PBG_CMP_DOT = 0, PBG_CMP_COS = 1, PBG_CMP_L2 = 2, PBG_CMP_SQUARED_L2 = 3 } pbg_comparator;
 typedef enum pbg_loss { PBG_LOSS_RANKING = 0, PBG_LOSS_LOGISTIC = 1, PBG_LOSS_SOFTMAX = 2 } pbg_loss;
 
 int pbg_version(void);

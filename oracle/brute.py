@@ -50,6 +50,9 @@ def _kappa(comparator: str, a: np.ndarray, b: np.ndarray) -> float:
     if comparator == "l2":
         d = a - b
         return -math.sqrt(max(float(d @ d), 1e-30))
+    if comparator == "squared_l2":  # model.py:300-303
+        d = a - b
+        return -float(d @ d)
     raise NotImplementedError(comparator)
 
 

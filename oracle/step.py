@@ -13,7 +13,7 @@ import torch
 import torch.nn.functional as F
 
 OPERATOR_NAMES = ("none", "diagonal", "translation", "linear", "complex_diagonal")
-COMPARATOR_NAMES = ("dot", "cos", "l2")
+COMPARATOR_NAMES = ("dot", "cos", "l2", "squared_l2")
 LOSS_NAMES = ("ranking", "logistic", "softmax")
 
 
@@ -117,11 +117,11 @@ def apply_operator(
 # --------------------------------------------------------------------------
 
 def comparator_prepare(name: str, embs: torch.Tensor) -> torch.Tensor:
-    """model.py:161-162 (dot), :187-192 (cos), :251-252 (l2)."""
+    """model.py:161-162 (dot), :187-192 (cos), :251-252 (l2), :283-284 (squared_l2)."""
     if name == "cos":
         norm = embs.norm(2, dim=-1)
         return embs * norm.reciprocal().unsqueeze(-1)
-    if name in ("dot", "l2"):
+    if name in ("dot", "l2", "squared_l2"):
         return embs
     raise NotImplementedError(f"Unknown comparator {name}")
 
@@ -132,15 +132,18 @@ def _f32(x: torch.Tensor) -> torch.Tensor:
     return x if x.dtype == torch.float64 else x.float()
 
 
-def _all_pairs_l2(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """model.py:215-246: ||a||^2 - 2ab + ||b||^2 through baddbmm, clamped at
-    1e-30, square-rooted."""
+def _all_pairs_squared_l2(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """model.py:215-236: ||a||^2 - 2ab + ||b||^2 through baddbmm."""
     a_squared = a.norm(dim=-1).pow(2)
     b_squared = b.norm(dim=-1).pow(2)
-    res = torch.baddbmm(b_squared.unsqueeze(-2), a, b.transpose(-2, -1), alpha=-2).add_(
+    return torch.baddbmm(b_squared.unsqueeze(-2), a, b.transpose(-2, -1), alpha=-2).add_(
         a_squared.unsqueeze(-1)
     )
-    return res.clamp_min_(1e-30).sqrt_()
+
+
+def _all_pairs_l2(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """model.py:239-246: the above clamped at 1e-30, square-rooted."""
+    return _all_pairs_squared_l2(a, b).clamp_min_(1e-30).sqrt_()
 
 
 def comparator_scores(
@@ -152,7 +155,7 @@ def comparator_scores(
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(pos[C,P], lhs_neg_scores[C,P,Ln] = rhs_pos x lhs_neg,
     rhs_neg_scores[C,P,Rn] = lhs_pos x rhs_neg); model.py:164-182, 194-212,
-    254-278.  Note the cross pairing of the negative scores."""
+    254-278, 286-305.  Note the cross pairing of the negative scores."""
     if lhs_pos.dim() != 3 or rhs_pos.shape != lhs_pos.shape:
         raise TypeError("Shape doesn't match")
     c, p, d = lhs_pos.shape
@@ -169,6 +172,11 @@ def comparator_scores(
         pos = (_f32(lhs_pos) - _f32(rhs_pos)).pow(2).sum(dim=-1).clamp_min(1e-30).sqrt().neg()
         lneg = _all_pairs_l2(rhs_pos, lhs_neg).neg()
         rneg = _all_pairs_l2(lhs_pos, rhs_neg).neg()
+        return pos, lneg, rneg
+    if name == "squared_l2":
+        pos = (_f32(lhs_pos) - _f32(rhs_pos)).pow(2).sum(dim=-1).neg()
+        lneg = _all_pairs_squared_l2(rhs_pos, lhs_neg).neg()
+        rneg = _all_pairs_squared_l2(lhs_pos, rhs_neg).neg()
         return pos, lneg, rneg
     raise NotImplementedError(f"Unknown comparator {name}")
 

@@ -186,12 +186,13 @@ __global__ __launch_bounds__(kRowThreads) void pos_scores_kernel(int cmp, int D,
   float acc = 0.f;
   const float* a = lp + i * D;
   const float* b = rp + i * D;
-  if (cmp == PBG_CMP_L2) {
+  if (cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2) {
     for (int d = lane; d < D; d += kWave) {
       const float t = a[d] - b[d];
       acc += t * t;
     }
-    acc = -sqrtf(fmaxf(wave_sum(acc), 1e-30f));
+    acc = wave_sum(acc);
+    acc = cmp == PBG_CMP_L2 ? -sqrtf(fmaxf(acc, 1e-30f)) : -acc;  // model.py:267-274 | :300
   } else {
     for (int d = lane; d < D; d += kWave) acc += a[d] * b[d];
     acc = wave_sum(acc);
@@ -199,29 +200,31 @@ __global__ __launch_bounds__(kRowThreads) void pos_scores_kernel(int cmp, int D,
   if (lane == 0) pos[i] = acc;
 }
 
-// l2 epilogue (model.py:228-246): s[c,i,j] <- -sqrt(max(a2[c,i] - 2 s + b2[c,j], 1e-30))
-__global__ void l2_epilogue_kernel(float* __restrict__ s, const float* __restrict__ a2, const float* __restrict__ b2,
-                                   int64_t chunks, int P, int N) {
+// l2 epilogue (model.py:228-246): s[c,i,j] <- -sqrt(max(a2[c,i] - 2 s + b2[c,j], 1e-30));
+// squared_l2 (model.py:228-236,301-302): s[c,i,j] <- -(a2[c,i] - 2 s + b2[c,j])
+__global__ void l2_epilogue_kernel(int cmp, float* __restrict__ s, const float* __restrict__ a2,
+                                   const float* __restrict__ b2, int64_t chunks, int P, int N) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= chunks * P * N) return;
   const int64_t row = e / N;  // c * P + i
   const int j = (int)(e % N);
   const int64_t c = row / P;
   const float q = fmaf(-2.0f, s[e], b2[c * N + j]) + a2[row];
-  s[e] = -sqrtf(fmaxf(q, 1e-30f));
+  s[e] = cmp == PBG_CMP_L2 ? -sqrtf(fmaxf(q, 1e-30f)) : -q;
 }
 
 // l2 backward, step 1: g[c,i,j] (dLoss/dscore) -> -2 dLoss/dq in `out`; rowsum of dLoss/dq
-__global__ __launch_bounds__(kRowThreads) void l2_grad_kernel(const float* __restrict__ g, const float* __restrict__ score,
-                                                              int64_t rows, int N, float* __restrict__ out,
-                                                              float* __restrict__ rowsum) {
+__global__ __launch_bounds__(kRowThreads) void l2_grad_kernel(int cmp, const float* __restrict__ g,
+                                                              const float* __restrict__ score, int64_t rows, int N,
+                                                              float* __restrict__ out, float* __restrict__ rowsum) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
   float acc = 0.f;
   for (int j = lane; j < N; j += kWave) {
     const float t = score[row * N + j];
-    const float dq = (t * t > 1e-30f) ? g[row * N + j] * 0.5f / t : 0.f;
+    // score = -sqrt(q): dq = g / (2 score), none where the clamp is active; score = -q: dq = -g
+    const float dq = cmp == PBG_CMP_SQUARED_L2 ? -g[row * N + j] : ((t * t > 1e-30f) ? g[row * N + j] * 0.5f / t : 0.f);
     acc += dq;
     out[row * N + j] = -2.0f * dq;
   }
@@ -250,10 +253,10 @@ __global__ __launch_bounds__(kRowThreads) void comparator_terms_kernel(int cmp, 
   const RowV<NVH> s = row_load<NVH>(self + i * D, D, H, lane);
   if (role == 0) {
     const RowV<NVH> o = row_load<NVH>(other + i * D, D, H, lane);
-    if (cmp == PBG_CMP_L2) {
+    if (cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2) {
       const float p = pos[i];
-      if (p * p > 1e-30f) {
-        const float coef = dpos[i] / p;
+      if (cmp == PBG_CMP_SQUARED_L2 || p * p > 1e-30f) {
+        const float coef = cmp == PBG_CMP_L2 ? dpos[i] / p : -2.0f * dpos[i];
 #pragma unroll
         for (int v = 0; v < NVH; ++v) {
           d.a[0][v] += coef * (s.a[0][v] - o.a[0][v]);
@@ -364,7 +367,7 @@ __global__ __launch_bounds__(256) void sum_rows_kernel(const float* __restrict__
 }
 
 bool valid_op(int op) { return op >= PBG_OP_NONE && op <= PBG_OP_COMPLEX_DIAGONAL; }
-bool valid_cmp(int cmp) { return cmp >= PBG_CMP_DOT && cmp <= PBG_CMP_L2; }
+bool valid_cmp(int cmp) { return cmp >= PBG_CMP_DOT && cmp <= PBG_CMP_SQUARED_L2; }
 
 struct CmpWs {
   float *a2_l, *a2_r, *b2_l, *b2_r;  // squared norms: lhs_pos, rhs_pos rows [C*P]; lhs_neg [C*Ln]; rhs_neg [C*Rn]
@@ -491,7 +494,7 @@ extern "C" int pbg_comparator_forward(int32_t cmp, int32_t chunks, int32_t p, in
       (rn > 0 && (!rhs_neg || !rhs_neg_scores)))
     return fail(PBG_ERR_INVALID, "pbg_comparator_forward: null pointer");
   CmpWs ws = carve_cmp(workspace, chunks, p, ln, rn);
-  if (cmp == PBG_CMP_L2 && (!workspace || workspace_bytes < ws.total))
+  if ((cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2) && (!workspace || workspace_bytes < ws.total))
     return fail(PBG_ERR_WORKSPACE, "pbg_comparator_forward: workspace needs %zu bytes", ws.total);
   hipStream_t s = (hipStream_t)stream;
   const int64_t np = (int64_t)chunks * p;
@@ -510,14 +513,14 @@ extern "C" int pbg_comparator_forward(int32_t cmp, int32_t chunks, int32_t p, in
     g.c = out; g.stride_c = (int64_t)p * nn; g.ldc = nn;
     g.m = p; g.n = nn; g.k = dim; g.batch = chunks; g.alpha = 1.f; g.beta = 0.f;
     if ((rc = gemm_f32(g, s)) != PBG_OK) return rc;
-    if (cmp == PBG_CMP_L2) {
+    if (cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2) {
       float* a2 = side == 0 ? ws.a2_r : ws.a2_l;
       float* b2 = side == 0 ? ws.b2_l : ws.b2_r;
       PBG_DISPATCH_NVH(nvh, prepare_kernel, wave_grid(np), s, cmp, dim, np, a, (float*)nullptr, a2);
       PBG_DISPATCH_NVH(nvh, prepare_kernel, wave_grid((int64_t)chunks * nn), s, cmp, dim, (int64_t)chunks * nn, b,
                        (float*)nullptr, b2);
       const int64_t total = np * nn;
-      hipLaunchKernelGGL(l2_epilogue_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, s, out, a2, b2,
+      hipLaunchKernelGGL(l2_epilogue_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, s, cmp, out, a2, b2,
                          (int64_t)chunks, p, nn);
     }
   }
@@ -539,7 +542,7 @@ extern "C" int pbg_comparator_backward(int32_t cmp, int32_t chunks, int32_t p, i
   if ((ln > 0 && (!lhs_neg || !lhs_neg_scores || !dlhs_neg_scores || !dlhs_neg)) ||
       (rn > 0 && (!rhs_neg || !rhs_neg_scores || !drhs_neg_scores || !drhs_neg)))
     return fail(PBG_ERR_INVALID, "pbg_comparator_backward: null pointer");
-  const bool l2 = cmp == PBG_CMP_L2;
+  const bool l2 = cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2;
   CmpWs ws = carve_cmp(workspace, chunks, p, ln, rn);
   if (l2 && (!workspace || workspace_bytes < ws.total))
     return fail(PBG_ERR_WORKSPACE, "pbg_comparator_backward: workspace needs %zu bytes", ws.total);
@@ -565,7 +568,7 @@ extern "C" int pbg_comparator_backward(int32_t cmp, int32_t chunks, int32_t p, i
     float* dq = side == 0 ? ws.dq_l : ws.dq_r;
     float* rs = side == 0 ? ws.rs_l : ws.rs_r;
     if (l2) {
-      hipLaunchKernelGGL(l2_grad_kernel, wave_grid(np), dim3(kRowThreads), 0, s, g, sc, np, nn, dq, rs);
+      hipLaunchKernelGGL(l2_grad_kernel, wave_grid(np), dim3(kRowThreads), 0, s, cmp, g, sc, np, nn, dq, rs);
       gg = dq;
     }
     GemmArgs ga{};  // dA = G * B

@@ -208,16 +208,20 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
 // ---------------------------------------------------------------------------
 // loss
 // ---------------------------------------------------------------------------
-// comparator on a matched pair (model.py:177,207,267-274)
+// l2 and squared_l2 score a pair by ||a||^2 - 2ab + ||b||^2 (model.py:215-236)
+__host__ __device__ __forceinline__ bool is_distance(int cmp) { return cmp == PBG_CMP_L2 || cmp == PBG_CMP_SQUARED_L2; }
+
+// comparator on a matched pair (model.py:177,207,267-274,300)
 __device__ __forceinline__ float kappa(int cmp, const float* __restrict__ a, const float* __restrict__ b, int D,
                                        int lane) {
   float acc = 0.f;
-  if (cmp == PBG_CMP_L2) {
+  if (is_distance(cmp)) {
     for (int d = lane; d < D; d += kWave) {
       const float t = a[d] - b[d];
       acc += t * t;
     }
-    return -sqrtf(fmaxf(wave_sum(acc), 1e-30f));
+    const float q = wave_sum(acc);
+    return cmp == PBG_CMP_L2 ? -sqrtf(fmaxf(q, 1e-30f)) : -q;
   }
   for (int d = lane; d < D; d += kWave) acc += a[d] * b[d];
   return wave_sum(acc);
@@ -238,6 +242,8 @@ struct ScoreRow {
       const float qd = fmaf(-2.0f, t, bn[j]) + a2;
       ok = qd >= 1e-30f;
       t = -sqrtf(fmaxf(qd, 1e-30f));
+    } else if (cmp == PBG_CMP_SQUARED_L2) {
+      t = -(fmaf(-2.0f, t, bn[j]) + a2);
     }
     if (j < nb && (j == i || j >= masked_from)) {
       t = -1e9f;
@@ -268,7 +274,7 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   sr.cmp = c.cmp;
   sr.bn = nullptr;
   sr.a2 = 0.f;
-  if (c.cmp == PBG_CMP_L2) {
+  if (is_distance(c.cmp)) {
     sr.bn = sd.an + kc * sd.nn;
     sr.a2 = c.dynamic ? so.aa[kc * c.P + i] : so.ap[kc * so.stride_p + i];
   }
@@ -329,10 +335,11 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
     }
     if (t > pos) ++viol;
     if (!live) g = 0.f;
-    if (cmp == PBG_CMP_L2) {
-      // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq so that the
-      // backward GEMMs produce the cross terms of ||a||^2 - 2ab + ||b||^2
-      const float dq = live ? g * 0.5f / t : 0.f;
+    if (is_distance(cmp)) {
+      // t = -sqrt(q): dLoss/dq = g * 0.5 / t (squared_l2, t = -q: -g); stored as
+      // -2 dLoss/dq so that the backward GEMMs produce the cross terms of
+      // ||a||^2 - 2ab + ||b||^2
+      const float dq = !live ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / t : -g);
       rowsum += dq;
       out[j] = -2.0f * dq;
     } else {
@@ -513,10 +520,11 @@ __device__ __forceinline__ float n3_term(int op, float coef, RowV<NVH>& dy, cons
 template <int NVH>
 __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos, const RowV<NVH>& self,
                                              const RowV<NVH>& other, float pos) {
-  if (cmp == PBG_CMP_L2) {
-    // kappa = -sqrt(max(sum (a-b)^2, 1e-30)); no gradient where the clamp is active
-    if (pos * pos <= 1e-30f) return;
-    const float coef = dpos / pos;
+  if (is_distance(cmp)) {
+    // kappa = -sqrt(max(sum (a-b)^2, 1e-30)); no gradient where the clamp is active.
+    // squared_l2: kappa = -sum (a-b)^2
+    if (cmp == PBG_CMP_L2 && pos * pos <= 1e-30f) return;
+    const float coef = cmp == PBG_CMP_L2 ? dpos / pos : -2.0f * dpos;
 #pragma unroll
     for (int v = 0; v < NVH; ++v) {
       dy.a[0][v] += coef * (self.a[0][v] - other.a[0][v]);
@@ -542,7 +550,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
   const SideCtx& sd = c.side[s];
   const SideCtx& so = c.side[1 - s];
   const int D = c.D, H = (D + 1) / 2;
-  const bool l2 = c.cmp == PBG_CMP_L2;
+  const bool l2 = is_distance(c.cmp);
   const bool keep_dz = sd.dz != nullptr;
 
   if (r < c.B) {
@@ -1658,7 +1666,7 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->num_batch_negs == 0 && d->num_uniform_negs == 0)
     return fail(PBG_ERR_INVALID, "step: num_batch_negs and num_uniform_negs cannot both be 0");
   if (d->op < PBG_OP_NONE || d->op > PBG_OP_COMPLEX_DIAGONAL) return fail(PBG_ERR_INVALID, "step: unknown operator %d", d->op);
-  if (d->comparator < PBG_CMP_DOT || d->comparator > PBG_CMP_L2) return fail(PBG_ERR_INVALID, "step: unknown comparator %d", d->comparator);
+  if (d->comparator < PBG_CMP_DOT || d->comparator > PBG_CMP_SQUARED_L2) return fail(PBG_ERR_INVALID, "step: unknown comparator %d", d->comparator);
   if (d->loss < PBG_LOSS_RANKING || d->loss > PBG_LOSS_SOFTMAX) return fail(PBG_ERR_INVALID, "step: unknown loss %d", d->loss);
   if (d->op == PBG_OP_COMPLEX_DIAGONAL && d->dim % 2 != 0)
     return fail(PBG_ERR_INVALID,
@@ -1737,7 +1745,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
       sd.dxn = takef(KC * sd.nn * D);
       if (need_aux) sd.an = takef(KC * sd.nn);
       sd.s = takef(KC * P * sd.nn);
-      if (c.cmp == PBG_CMP_L2) sd.rs = takef(KC * P);
+      if (is_distance(c.cmp)) sd.rs = takef(KC * P);
     }
     if (sd.alias) {
       sd.xp = sd.xn;

@@ -1,7 +1,7 @@
 """Embeddings, comparators and the multi-relation model (reference:
 torchbiggraph/model.py).
 
-``COMPARATORS`` holds ``dot``, ``cos`` and ``l2`` with the reference's
+``COMPARATORS`` holds ``dot``, ``cos``, ``l2`` and ``squared_l2`` with the reference's
 ``prepare`` / ``forward`` contract (differentiable, computed by
 pbg_comparator_*).  ``MultiRelationEmbedder`` keeps the reference's constructor,
 ``set_embeddings`` / ``set_all_embeddings`` / ``clear_all_embeddings`` and
@@ -15,7 +15,7 @@ autograd on these scores.
 training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
-Not provided (outside the accelerated path): FeaturizedEmbedding, squared_l2,
+Not provided (outside the accelerated path): FeaturizedEmbedding,
 BiasedComparator, all_negs, global embeddings, max_norm, half precision.
 """
 from abc import ABC, abstractmethod
@@ -198,6 +198,13 @@ class CosComparator(AbstractComparator):
 @COMPARATORS.register_as("l2")
 class L2Comparator(AbstractComparator):
     comparator_name = "l2"
+
+
+@COMPARATORS.register_as("squared_l2")
+class SquaredL2Comparator(AbstractComparator):
+    """Negative squared distance (model.py:281-305)."""
+
+    comparator_name = "squared_l2"
 
 
 # ---------------------------------------------------------------------------

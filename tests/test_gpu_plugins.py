@@ -67,7 +67,7 @@ def test_reference_comparator_vectors(pbg, golden):
             assert (t.grad != 0).any()
 
 
-@pytest.mark.parametrize("name", ["dot", "cos", "l2"])
+@pytest.mark.parametrize("name", ["dot", "cos", "l2", "squared_l2"])
 @pytest.mark.parametrize("shape", [(3, 5, 7, 4, 6), (1, 50, 100, 100, 100), (2, 4, 0, 3, 8), (2, 100, 130, 70, 256)])
 def test_comparator_forward_backward_vs_oracle(pbg, name, shape):
     say("comparator grad", name, shape)

@@ -22,7 +22,7 @@ def test_plugin_registry(pbg):
         reg.get_class("b")
     assert sorted(pbg.operators.OPERATORS.registry) == ["complex_diagonal", "diagonal", "linear", "none", "translation"]
     assert sorted(pbg.operators.DYNAMIC_OPERATORS.registry) == sorted(pbg.operators.OPERATORS.registry)
-    assert sorted(pbg.model.COMPARATORS.registry) == ["cos", "dot", "l2"]
+    assert sorted(pbg.model.COMPARATORS.registry) == ["cos", "dot", "l2", "squared_l2"]
     assert sorted(pbg.losses.LOSS_FUNCTIONS.registry) == ["logistic", "ranking", "softmax"]
     with pytest.raises(TypeError):
         pbg.losses.LOSS_FUNCTIONS.get_class("ranking")()  # margin is keyword-required
