@@ -2,7 +2,8 @@
 
 The package keeps registries of its own under the reference's names: operators
 ``none | diagonal | translation | linear | complex_diagonal``, comparators
-``dot | cos | l2`` and loss functions ``ranking | logistic | softmax``.
+``dot | cos | l2 | squared_l2``, loss functions ``ranking | logistic | softmax``
+and the regularizer ``N3``.
 """
 from typing import Callable, Dict, Generic, Type, TypeVar
 

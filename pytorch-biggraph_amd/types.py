@@ -1,39 +1,41 @@
-"""Small shared types (reference: torchbiggraph/types.py:23-68)."""
-from enum import Enum
-from typing import NamedTuple, TypeVar
+"""Type aliases and the two small value types of the step's interface
+(reference: torchbiggraph/types.py:23-68): ``Side`` and ``Bucket``."""
+import enum
+import typing
 
 import torch
 
-FloatTensorType = torch.Tensor  # float32
-LongTensorType = torch.Tensor  # int64
-T = TypeVar("T")
+T = typing.TypeVar("T")
+
+# Annotations only: every tensor is a torch.Tensor, the alias states the dtype.
+LongTensorType = torch.Tensor   # int64 indices
+FloatTensorType = torch.Tensor  # float32 values
+
+Partition = int
+EntityName = str
+UNPARTITIONED: Partition = 0  # the partition number of an entity type that is not partitioned
 
 
-class Side(Enum):
+class Side(enum.Enum):
+    """Left- or right-hand side of an edge."""
+
     LHS = 0
     RHS = 1
 
     def pick(self, lhs: T, rhs: T) -> T:
-        if self is Side.LHS:
-            return lhs
-        if self is Side.RHS:
-            return rhs
-        raise NotImplementedError("Unknown side: %s" % self)
+        """`lhs` for Side.LHS, `rhs` for Side.RHS."""
+        return (lhs, rhs)[self.value]
 
 
-EntityName = str
-Partition = int
+class Bucket(typing.NamedTuple):
+    """The edges whose left entities lie in partition `lhs` and whose right
+    entities lie in partition `rhs`."""
 
-
-class Bucket(NamedTuple):
     lhs: Partition
     rhs: Partition
 
-    def get_partition(self, side: Side) -> Partition:
-        return side.pick(self.lhs, self.rhs)
-
     def __str__(self) -> str:
-        return "( %d , %d )" % (self.lhs, self.rhs)
+        return f"( {self.lhs:d} , {self.rhs:d} )"
 
-
-UNPARTITIONED: Partition = 0
+    def get_partition(self, side: Side) -> Partition:
+        return self[side.value]
