@@ -41,6 +41,9 @@ class StepConfig:
     # config.py:221-230: coefficient of the N3 regularizer (the only one registered,
     # regularizers.py:51); 0 = none (model.py:905-909)
     regularization_coef: float = 0.0
+    # config.py:181-188: a learned vector per entity type added to every embedding
+    # of the type (model.py:433-441,486-492); standard relations only
+    global_emb: bool = False
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
@@ -294,9 +297,14 @@ class Scores:
     reg: Optional[torch.Tensor] = None  # the second value MultiRelationEmbedder.forward returns
 
 
-def _adjust(cfg: StepConfig, embs, rel, op_params) -> torch.Tensor:
-    """model.py:478-506 without global_emb / half precision: operator then
-    comparator.prepare.  ``op_params is None`` means "no operator"."""
+def _adjust(cfg: StepConfig, embs, rel, op_params, glob=None) -> torch.Tensor:
+    """model.py:478-506 without half precision: global embedding of the entity
+    type (``glob``, None = disabled), operator, comparator.prepare.
+    ``op_params is None`` means "no operator"."""
+    if glob is not None:
+        if not isinstance(rel, int):
+            raise RuntimeError("Cannot have global embs with dynamic rels")  # model.py:488-489
+        embs = embs + glob
     if op_params is not None:
         embs = apply_operator(cfg.operator, embs, op_params, rel)
     return comparator_prepare(cfg.comparator, embs)
@@ -314,12 +322,14 @@ def _direction_agnostic(
     chunk_size: int,
     src_method: str,
     dst_method: str,
+    src_glob=None,
+    dst_glob=None,
 ):
     """model.py:764-856.  ``src_uniform`` / ``dst_uniform`` are the raw rows
     of the uniformly sampled entities, [C,U,D] (model.py:544,550)."""
     dim = src_pos.shape[-1]
-    src_pos = _adjust(cfg, src_pos, rel, None)
-    dst_pos = _adjust(cfg, dst_pos, rel, dst_op_params)
+    src_pos = _adjust(cfg, src_pos, rel, None, src_glob)
+    dst_pos = _adjust(cfg, dst_pos, rel, dst_op_params, dst_glob)
     num_chunks = (num_pos - 1) // chunk_size + 1
     pad = num_chunks * chunk_size - num_pos
     if pad > 0:
@@ -329,17 +339,17 @@ def _direction_agnostic(
     dst_pos = dst_pos.view(num_chunks, chunk_size, dim)
     last = num_pos - (num_chunks - 1) * chunk_size
 
-    def negatives(pos_embs, uniform, method, op_params):
+    def negatives(pos_embs, uniform, method, op_params, glob):
         # model.py:508-622 (NONE / UNIFORM / BATCH_UNIFORM branches)
         masked_batch = False
         if method == "none":
             neg = pos_embs.new_empty((num_chunks, 0, dim))
         elif method == "uniform":
-            neg = _adjust(cfg, uniform, rel_for_uniform, op_params)
+            neg = _adjust(cfg, uniform, rel_for_uniform, op_params, glob)
         elif method == "batch_uniform":
             neg = pos_embs
             if uniform is not None and uniform.shape[1] > 0:
-                neg = torch.cat([pos_embs, _adjust(cfg, uniform, rel_for_uniform, op_params)], dim=1)
+                neg = torch.cat([pos_embs, _adjust(cfg, uniform, rel_for_uniform, op_params, glob)], dim=1)
             masked_batch = True
         else:
             raise NotImplementedError(method)
@@ -348,8 +358,8 @@ def _direction_agnostic(
     # The operator is only ever applied to uniform negatives in standard mode,
     # where rel is an int; dynamic mode passes no operator for the negatives.
     rel_for_uniform = rel
-    src_neg, src_masked = negatives(src_pos, src_uniform, src_method, None)
-    dst_neg, dst_masked = negatives(dst_pos, dst_uniform, dst_method, dst_op_params)
+    src_neg, src_masked = negatives(src_pos, src_uniform, src_method, None, src_glob)
+    dst_neg, dst_masked = negatives(dst_pos, dst_uniform, dst_method, dst_op_params, dst_glob)
 
     pos_scores, src_neg_scores, dst_neg_scores = comparator_scores(
         cfg.comparator, src_pos, dst_pos, src_neg, dst_neg
@@ -383,6 +393,8 @@ def model_forward(
     rel,
     lhs_op_params: Optional[Dict[str, torch.Tensor]],
     rhs_op_params: Optional[Dict[str, torch.Tensor]],
+    glob_lhs: Optional[torch.Tensor] = None,
+    glob_rhs: Optional[torch.Tensor] = None,
 ) -> Scores:
     """MultiRelationEmbedder.forward (model.py:624-762) on already gathered
     rows.  lhs_pos/rhs_pos: [B,D] raw rows; *_uniform: [C,U,D] raw rows of the
@@ -402,11 +414,13 @@ def model_forward(
         pos, lneg, rneg, reg = _direction_agnostic(
             cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, rhs_uniform, rel,
             rhs_op_params if cfg.operator != "none" else None,
-            chunk_size, lhs_method, rhs_method,
+            chunk_size, lhs_method, rhs_method, glob_lhs, glob_rhs,
         )
         return Scores(pos, pos, lneg, rneg, reg)
     if isinstance(rel, int):
         raise TypeError("Need relation for each positive pair")
+    if glob_lhs is not None or glob_rhs is not None:
+        raise RuntimeError("Cannot have global embs with dynamic rels")  # model.py:488-489
     # model.py:721-754: forward edges (operator on rhs, negatives on lhs),
     # then reverse edges (operator on lhs, negatives on rhs).
     lpos, lneg, _, l_reg = _direction_agnostic(
@@ -480,6 +494,12 @@ class TrainState:
     rhs_op: Dict[str, torch.Tensor] = field(default_factory=dict)
     lhs_op_sum: Dict[str, torch.Tensor] = field(default_factory=dict)
     rhs_op_sum: Dict[str, torch.Tensor] = field(default_factory=dict)
+    # global embeddings of the two sides' entity types and their AsyncAdagrad sums
+    # (None = disabled); the same tensors on both sides when the sides share a type
+    glob_lhs: Optional[torch.Tensor] = None
+    glob_rhs: Optional[torch.Tensor] = None
+    glob_lhs_sum: Optional[torch.Tensor] = None
+    glob_rhs_sum: Optional[torch.Tensor] = None
 
     @property
     def shared(self) -> bool:
@@ -500,6 +520,12 @@ def make_state(cfg: StepConfig, w_lhs: torch.Tensor, w_rhs: Optional[torch.Tenso
     if cfg.dynamic:
         st.lhs_op = init_operator_params(cfg.operator, cfg.dim, cfg.num_relations)
         st.lhs_op_sum = {k: torch.zeros_like(v) for k, v in st.lhs_op.items()}
+    if cfg.global_emb:  # model.py:433-439: zeros, one vector per entity type
+        st.glob_lhs, st.glob_lhs_sum = torch.zeros(cfg.dim), torch.zeros(cfg.dim)
+        if shared:
+            st.glob_rhs, st.glob_rhs_sum = st.glob_lhs, st.glob_lhs_sum
+        else:
+            st.glob_rhs, st.glob_rhs_sum = torch.zeros(cfg.dim), torch.zeros(cfg.dim)
     return st
 
 
@@ -521,6 +547,8 @@ class StepGrads:
     sparse_rhs: Optional[torch.Tensor]
     lhs_op: Dict[str, torch.Tensor]
     rhs_op: Dict[str, torch.Tensor]
+    glob_lhs: Optional[torch.Tensor] = None  # also carries the rhs side's sum when the sides share a type
+    glob_rhs: Optional[torch.Tensor] = None
 
 
 def forward_backward(
@@ -553,7 +581,11 @@ def forward_backward(
         if uniform_rhs is not None and not cfg.disable_rhs_negs and uniform_rhs.numel() > 0
         else None
     )
-    scores = model_forward(cfg, lhs_pos, rhs_pos, lhs_u, rhs_u, rel, lhs_op or None, rhs_op or None)
+    glob_l = glob_r = None
+    if st.glob_lhs is not None:
+        glob_l = st.glob_lhs.detach().requires_grad_(True)
+        glob_r = glob_l if st.glob_rhs is st.glob_lhs else st.glob_rhs.detach().requires_grad_(True)
+    scores = model_forward(cfg, lhs_pos, rhs_pos, lhs_u, rhs_u, rel, lhs_op or None, rhs_op or None, glob_l, glob_r)
 
     # batching.py:139-150
     lhs_loss = loss_value(cfg.loss, scores.lhs_pos, scores.lhs_neg, weight, cfg.margin)
@@ -581,6 +613,9 @@ def forward_backward(
         sparse_rhs=None if st.shared else w_r.grad,
         lhs_op={k: (v.grad if v.grad is not None else torch.zeros_like(v)) for k, v in lhs_op.items()},
         rhs_op={k: (v.grad if v.grad is not None else torch.zeros_like(v)) for k, v in rhs_op.items()},
+        glob_lhs=None if glob_l is None else (glob_l.grad if glob_l.grad is not None else torch.zeros_like(glob_l)),
+        glob_rhs=None if glob_r is None or glob_r is glob_l else
+        (glob_r.grad if glob_r.grad is not None else torch.zeros_like(glob_r)),
     )
     return out, grads
 
@@ -596,6 +631,11 @@ def apply_grads(cfg: StepConfig, st: TrainState, grads: StepGrads) -> None:
         ):
             for name, p in params.items():
                 async_adagrad_dense(p, sums[name], g[name], rel_lr)
+        # the global embeddings are parameters of the model too (model.py:433-439)
+        if grads.glob_lhs is not None:
+            async_adagrad_dense(st.glob_lhs, st.glob_lhs_sum, grads.glob_lhs, rel_lr)
+        if grads.glob_rhs is not None:
+            async_adagrad_dense(st.glob_rhs, st.glob_rhs_sum, grads.glob_rhs, rel_lr)
         if grads.sparse_lhs is not None:
             row_adagrad_sparse(st.w_lhs, st.g_lhs, grads.sparse_lhs, cfg.lr)
         if grads.sparse_rhs is not None:
