@@ -164,6 +164,13 @@ typedef struct pbg_step_buffers {
   int32_t sample_uniform;
   uint64_t uniform_seed;
   float* reg_out;             /* [K] regularizer value of each batch (Stats.reg, train_cpu.py:97), or null */
+  /* config.global_emb (model.py:433-441,486-492): the learned vector [D] of each side's
+   * entity type, added to every gathered row of that side before the operator, and
+   * its AsyncAdagrad state["sum"] [D] (step size relation_lr: it is a parameter of the
+   * model optimizer).  Null = disabled.  When both sides have the same entity type
+   * pass the same pointers twice: the two sides' gradients are summed into one step.
+   * Standard relations only (model.py:488-489). */
+  float* lhs_global; float* rhs_global; float* lhs_global_sum; float* rhs_global_sum;
 } pbg_step_buffers;
 
 /* sizeof(pbg_step_desc) / sizeof(pbg_step_buffers) as this library was compiled:

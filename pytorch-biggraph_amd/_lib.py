@@ -61,6 +61,7 @@ class StepBuffers(ctypes.Structure):
         ("loss_out", c_void_p), ("violators_out", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("sample_uniform", c_int32), ("uniform_seed", c_uint64), ("reg_out", c_void_p),
+        ("lhs_global", c_void_p), ("rhs_global", c_void_p), ("lhs_global_sum", c_void_p), ("rhs_global_sum", c_void_p),
     ]
 
 

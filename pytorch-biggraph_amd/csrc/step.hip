@@ -33,6 +33,7 @@ constexpr int kWavesPerBlock = kRowThreads / kWave;
 
 struct SideCtx {
   const float* w;       // embedding table of this side
+  const float* glob;    // global embedding of this side's entity type [D], or null
   const int64_t* idx;   // [K, B] positive entities
   const int64_t* uidx;  // [K, C, U] uniform negatives (null if u == 0, or if they are drawn in the step)
   uint64_t useed;       // seed of the in-step draw (uidx == null)
@@ -89,6 +90,14 @@ __device__ __forceinline__ int64_t uniform_negative(const SideCtx& sd, int s, in
   return sampled_row(sd.useed, (uint64_t)flat, (uint32_t)s, sd.num_rows);
 }
 
+// x + the global embedding of the side's entity type (model.py:486-492)
+template <int NVH>
+__device__ __forceinline__ RowV<NVH> gathered_row(const SideCtx& sd, int64_t id, int D, int H, int lane) {
+  RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+  if (sd.glob) row_axpy<NVH>(x, 1.0f, row_load<NVH>(sd.glob, D, H, lane));
+  return x;
+}
+
 // ---------------------------------------------------------------------------
 // prep
 // ---------------------------------------------------------------------------
@@ -125,7 +134,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     const int64_t e = (int64_t)k * c.B + r;
     const int64_t id = clamp_index(sd.idx[e], sd.num_rows);
     const int64_t rel = clamp_index(c.dynamic ? c.rel[e] : c.rel[k], c.num_relations);
-    const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+    const RowV<NVH> x = gathered_row<NVH>(sd, id, D, H, lane);
     if (lane == 0) {
       const int64_t slot = (int64_t)k * c.rk + sd.slot_pos + r;
       c.keys[slot] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     const int cc = r2 / sd.u, uu = r2 % sd.u;
     const int64_t kc = (int64_t)k * c.C + cc;
     const int64_t id = clamp_index(uniform_negative(sd, s, kc * c.U + uu), sd.num_rows);
-    const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+    const RowV<NVH> x = gathered_row<NVH>(sd, id, D, H, lane);
     if (lane == 0) {
       const int64_t slot = (int64_t)k * c.rk + sd.slot_uni + r2;
       c.keys[slot] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
@@ -674,13 +683,14 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
         id = uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u);
       }
       const float* x = sd.w + clamp_index(id, sd.num_rows) * D;
+      const float* gl = sd.glob;  // the operator's input is the row plus the global embedding
       if (c.op == PBG_OP_DIAGONAL) {
-        acc += x[e] * dz[e];
+        acc += (x[e] + (gl ? gl[e] : 0.f)) * dz[e];
       } else if (e < H) {  // d/d real
-        acc += x[e] * dz[e] + x[e + H] * dz[e + H];
+        acc += (x[e] + (gl ? gl[e] : 0.f)) * dz[e] + (x[e + H] + (gl ? gl[e + H] : 0.f)) * dz[e + H];
       } else {             // d/d imag
         const int h = e - H;
-        acc += x[h] * dz[h + H] - x[h + H] * dz[h];
+        acc += (x[h] + (gl ? gl[h] : 0.f)) * dz[h + H] - (x[h + H] + (gl ? gl[h + H] : 0.f)) * dz[h];
       }
     }
   }
@@ -1124,6 +1134,9 @@ __device__ __forceinline__ void fused_store_rows(const StepCtx& c, const FusedGe
   const bool col_ok = c4 < g.D;
   float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
   if (c.op != PBG_OP_NONE && col_ok) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * g.D + c4);
+  float4 glob0 = make_float4(0.f, 0.f, 0.f, 0.f), glob1 = glob0;
+  if (c.side[0].glob && col_ok) glob0 = *reinterpret_cast<const float4*>(c.side[0].glob + c4);
+  if (c.side[1].glob && col_ok) glob1 = *reinterpret_cast<const float4*>(c.side[1].glob + c4);
   const int slot0 = half * 8 + lwave;
 #pragma unroll
   for (int u = 0; u < kFusedRounds; ++u) {
@@ -1131,6 +1144,10 @@ __device__ __forceinline__ void fused_store_rows(const StepCtx& c, const FusedGe
     if (slot >= 2 * g.N) break;  // uniform per half-wave; the reduction below stays inside a half
     const int s = slot >= g.N, j = slot - s * g.N;
     float4 y = v[u];
+    if (idv[u] >= 0) {  // the global embedding of the side's entity type (model.py:486-492)
+      const float4 gv = s ? glob1 : glob0;
+      y.x += gv.x; y.y += gv.y; y.z += gv.z; y.w += gv.w;
+    }
     if (s == 1 && idv[u] >= 0) {
       if (c.op == PBG_OP_DIAGONAL) {
         y.x *= par.x; y.y *= par.y; y.z *= par.z; y.w *= par.w;
@@ -1635,6 +1652,102 @@ __global__ __launch_bounds__(256) void reg_reduce_kernel(StepCtx c) {
 }
 
 // ---------------------------------------------------------------------------
+// global embeddings (model.py:433-441,486-492): gradient and AsyncAdagrad step
+// ---------------------------------------------------------------------------
+// The gradient of a side's global embedding is the sum of the raw-row gradients
+// of the side's gathered rows: gth[s, k, slice, :] = sum over the rows
+// r = slice (mod slices) of side s in batch k of gr[k, r, :].  Half a wave per
+// row, 128-bit loads; fixed order, no atomics.
+constexpr int kGlobalHalves = 8;  // half-waves per workgroup
+__global__ __launch_bounds__(kGlobalHalves * 32) void global_grad_kernel(StepCtx c, float* __restrict__ gth, int slices) {
+  __shared__ float4 sh[kGlobalHalves][32];
+  const int lane = threadIdx.x & 31, hw = threadIdx.x >> 5;
+  const int k = blockIdx.x, s = blockIdx.y / slices, slice = blockIdx.y % slices;
+  const int D = c.D;
+  const int begin = c.side[s].slot_pos;
+  const int end = s == 0 ? c.side[1].slot_pos : c.rk;  // a side's positives and uniform negatives are contiguous
+  const bool vec = (D & 3) == 0;
+  for (int c0 = 0; c0 < D; c0 += 128) {
+    const int col = c0 + lane * 4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int r = begin + slice * kGlobalHalves + hw; r < end; r += slices * kGlobalHalves) {
+      const float* row = c.gr + ((int64_t)k * c.rk + r) * D;
+      if (vec) {
+        if (col < D) {
+          const float4 v = *reinterpret_cast<const float4*>(row + col);
+          acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+      } else {
+        if (col < D) acc.x += row[col];
+        if (col + 1 < D) acc.y += row[col + 1];
+        if (col + 2 < D) acc.z += row[col + 2];
+        if (col + 3 < D) acc.w += row[col + 3];
+      }
+    }
+    sh[hw][lane] = acc;
+    __syncthreads();
+    if (hw == 0) {
+      float4 t = sh[0][lane];
+#pragma unroll
+      for (int h = 1; h < kGlobalHalves; ++h) {
+        t.x += sh[h][lane].x; t.y += sh[h][lane].y; t.z += sh[h][lane].z; t.w += sh[h][lane].w;
+      }
+      float* out = gth + (((int64_t)s * c.K + k) * slices + slice) * D;
+      if (col < D) out[col] = t.x;
+      if (col + 1 < D) out[col + 1] = t.y;
+      if (col + 2 < D) out[col + 2] = t.z;
+      if (col + 3 < D) out[col + 3] = t.w;
+    }
+    __syncthreads();
+  }
+}
+
+// AsyncAdagrad (async_adagrad.py:75-85) on the global embeddings, the K batches'
+// gradients applied in order.  `shared`: both sides have one entity type and one
+// vector, whose gradient is the sum of the two sides'.  One wave per element:
+// lane j sums the partial sums of batches j, j + 64, ...; the steps then run in
+// batch order on registers.
+__global__ __launch_bounds__(kRowThreads) void global_update_kernel(StepCtx c, const float* __restrict__ gth, int slices,
+                                                                    int shared, float* p_l, float* s_l, float* p_r,
+                                                                    float* s_r, float lr) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (e >= c.D) return;
+  const int D = c.D;
+  float p[2] = {p_l[e], shared ? 0.f : p_r[e]};
+  float st[2] = {s_l[e], shared ? 0.f : s_r[e]};
+  for (int k0 = 0; k0 < c.K; k0 += kWave) {
+    const int k = k0 + lane;
+    float g[2] = {0.f, 0.f};
+    if (k < c.K)
+      for (int s = 0; s < 2; ++s)
+        for (int sl = 0; sl < slices; ++sl) g[s] += gth[(((int64_t)s * c.K + k) * slices + sl) * D + e];
+    if (shared) {
+      g[0] += g[1];
+      g[1] = 0.f;
+    }
+    const int count = c.K - k0 < kWave ? c.K - k0 : kWave;
+    for (int j = 0; j < count; ++j) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        if (s == 1 && shared) continue;
+        const float gj = __shfl(g[s], j, 64);
+        st[s] += gj * gj;
+        p[s] += -lr * (gj / (sqrtf(st[s]) + 1e-10f));
+      }
+    }
+  }
+  if (lane == 0) {
+    p_l[e] = p[0];
+    s_l[e] = st[0];
+    if (!shared) {
+      p_r[e] = p[1];
+      s_r[e] = st[1];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 struct Plan {
@@ -1655,6 +1768,8 @@ struct Plan {
   void* rsort_temp;
   void* rel_start;  // first sorted position of every relation (`linear` only)
   int nvh;
+  float* gth;   // partial sums of the global embeddings' gradients [2, K, gslices, D]
+  int gslices;
 };
 
 int validate(const pbg_step_desc* d, bool training) {
@@ -1785,6 +1900,11 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   }
   c.lossrow = takef(K * CP);
   c.violrow = (int*)take(K * CP * 2, sizeof(int));
+  if (!c.dynamic) {  // room for the global embeddings' gradient (whether a call uses it is in its buffers)
+    int sl = (int)ceil_div(c.rk, 2 * 16 * kGlobalHalves);  // about 16 rows per half-wave
+    plan->gslices = sl < 1 ? 1 : (sl > 16 ? 16 : sl);
+    plan->gth = takef((size_t)2 * K * plan->gslices * D);
+  }
   c.reg_coef = d->regularization_coef;
   if (c.reg_coef != 0.f) {
     c.regrow = takef((size_t)K * 2 * c.B);
@@ -1837,6 +1957,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     c.side[0].uidx = b->uniform_lhs;
     c.side[1].uidx = b->uniform_rhs;
     c.side[0].useed = c.side[1].useed = b->uniform_seed;
+    c.side[0].glob = b->lhs_global;
+    c.side[1].glob = b->rhs_global;
     c.side[0].p0 = b->lhs_op_p0;
     c.side[0].p1 = b->lhs_op_p1;
     c.side[1].p0 = b->rhs_op_p0;
@@ -1878,6 +2000,17 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
     const bool two = d->op == PBG_OP_COMPLEX_DIAGONAL;
     if (!p0 || (two && !p1)) return fail(PBG_ERR_INVALID, "step: null operator parameter");
     if (training && (!s0 || (two && !s1))) return fail(PBG_ERR_INVALID, "step: null operator optimizer state");
+  }
+  if ((b->lhs_global == nullptr) != (b->rhs_global == nullptr))
+    return fail(PBG_ERR_INVALID, "step: global embeddings need both sides' vectors (the same pointer for one entity type)");
+  if (b->lhs_global) {
+    if (d->dynamic) return fail(PBG_ERR_INVALID, "Cannot have global embs with dynamic rels");  // model.py:488-489
+    if ((uintptr_t)b->lhs_global % 16 != 0 || (uintptr_t)b->rhs_global % 16 != 0)
+      return fail(PBG_ERR_INVALID, "step: global embeddings must be 16-byte aligned");
+    if (training && (!b->lhs_global_sum || !b->rhs_global_sum))
+      return fail(PBG_ERR_INVALID, "step: null optimizer state of the global embeddings");
+    if (training && (b->lhs_global == b->rhs_global) != (b->lhs_global_sum == b->rhs_global_sum))
+      return fail(PBG_ERR_INVALID, "step: one global embedding needs one optimizer state");
   }
   if (!b->workspace || b->workspace_bytes < plan.bytes)
     return fail(PBG_ERR_WORKSPACE, "step: workspace needs %zu bytes, got %zu", plan.bytes, b->workspace_bytes);
@@ -2227,6 +2360,14 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(7);
   }
   if ((rc = run_params(desc, bufs, plan, s, &rel_order)) != PBG_OK) return rc;
+  if (bufs->lhs_global) {  // the raw-row gradients are complete and still one per gathered row
+    hipLaunchKernelGGL(global_grad_kernel, dim3((unsigned)c.K, (unsigned)(2 * plan.gslices)), dim3(kGlobalHalves * 32), 0,
+                       s, c, plan.gth, plan.gslices);
+    hipLaunchKernelGGL(global_update_kernel, wave_grid(c.D), dim3(kRowThreads), 0, s, c, plan.gth, plan.gslices,
+                       bufs->lhs_global == bufs->rhs_global ? 1 : 0, bufs->lhs_global, bufs->lhs_global_sum,
+                       bufs->rhs_global, bufs->rhs_global_sum, desc->relation_lr);
+    if ((rc = check_launch("step global embeddings")) != PBG_OK) return rc;
+  }
   mark(8);
   const int64_t npairs = (int64_t)c.K * c.rk;
   const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);

@@ -16,7 +16,7 @@ training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
 Not provided (outside the accelerated path): FeaturizedEmbedding,
-BiasedComparator, all_negs, global embeddings, max_norm, half precision.
+BiasedComparator, all_negs, max_norm, half precision.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -253,8 +253,6 @@ class MultiRelationEmbedder(nn.Module):
         super().__init__()
         if regularizer is not None and not isinstance(regularizer, N3Regularizer):
             raise NotImplementedError("Only the N3 regularizer is supported")
-        if global_emb:
-            raise NotImplementedError("Global embeddings are not supported")
         if max_norm is not None:
             raise NotImplementedError("max_norm is not supported")
         if half_precision:
@@ -278,7 +276,12 @@ class MultiRelationEmbedder(nn.Module):
         self.comparator = comparator
         self.lhs_embs: nn.ModuleDict = nn.ModuleDict()
         self.rhs_embs: nn.ModuleDict = nn.ModuleDict()
-        self.global_embs = None
+        # model.py:433-441: one learned vector per entity type, zeros at first
+        self.global_embs: Optional[nn.ParameterDict] = None
+        if global_emb:
+            self.global_embs = nn.ParameterDict({
+                self.EMB_PREFIX + entity: nn.Parameter(torch.zeros((schema.dimension or default_dim,)))
+                for entity, schema in entities.items()})
         self.max_norm = None
         self.half_precision = False
         self.regularizer: Optional[AbstractRegularizer] = regularizer
@@ -325,6 +328,16 @@ class MultiRelationEmbedder(nn.Module):
         lhs_module = self.lhs_embs[self.EMB_PREFIX + relation.lhs]
         rhs_module = self.rhs_embs[self.EMB_PREFIX + relation.rhs]
         return relation_idx, lhs_module, rhs_module
+
+    def global_vectors(self, relation_idx: int):
+        """(lhs, rhs) global embedding Parameters of the relation's entity types,
+        or None when global embeddings are off (model.py:486-492)."""
+        if self.global_embs is None:
+            return None
+        if self.num_dynamic_rels > 0:
+            raise RuntimeError("Cannot have global embs with dynamic rels")
+        relation = self.relations[relation_idx]
+        return (self.global_embs[self.EMB_PREFIX + relation.lhs], self.global_embs[self.EMB_PREFIX + relation.rhs])
 
     def step_spec(self, relation_idx: int, num_pos: int, dim: int, **training) -> native.StepSpec:
         rhs_op = self.rhs_operators[relation_idx]
@@ -403,8 +416,10 @@ class MultiRelationEmbedder(nn.Module):
         runner = self._runners.get(key)
         if runner is None:
             rhs_op, lhs_op = self.operator_tensors(relation_idx)
+            glob = self.global_vectors(relation_idx)
             runner = native.StepRunner(spec, w_l.data, torch.empty(0, device=dev), w_r.data, torch.empty(0, device=dev),
-                                       rhs_op, None, lhs_op, None)
+                                       rhs_op, None, lhs_op, None,
+                                       global_embs=None if glob is None else (glob[0].data, glob[1].data))
             self._runners[key] = runner
         if uniform_negs is None:
             uniform_negs = self.sample_uniform(lhs_module, rhs_module, spec.num_chunks)

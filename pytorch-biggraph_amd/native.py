@@ -222,7 +222,11 @@ class StepRunner:
                  w_rhs: Optional[torch.Tensor] = None, g_rhs: Optional[torch.Tensor] = None,
                  rhs_op: Optional[Dict[str, torch.Tensor]] = None, rhs_op_sum: Optional[Dict[str, torch.Tensor]] = None,
                  lhs_op: Optional[Dict[str, torch.Tensor]] = None, lhs_op_sum: Optional[Dict[str, torch.Tensor]] = None,
-                 relation_weights: Optional[torch.Tensor] = None):
+                 relation_weights: Optional[torch.Tensor] = None,
+                 global_embs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 global_sums: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+        """global_embs / global_sums: (lhs, rhs) global embedding [D] of each side's entity
+        type and its AsyncAdagrad sum; the same tensor twice when the sides share a type."""
         self.spec = spec
         shared = w_rhs is None or w_rhs.data_ptr() == w_lhs.data_ptr()
         self.w_lhs = _need(w_lhs, torch.float32, "w_lhs")
@@ -262,6 +266,10 @@ class StepRunner:
         self.rhs_op_sum = rhs_op_sum or {}
         self.lhs_op = lhs_op or {}
         self.lhs_op_sum = lhs_op_sum or {}
+        if global_embs is not None and spec.dynamic:
+            raise RuntimeError("Cannot have global embs with dynamic rels")  # model.py:488-489
+        self.global_embs = global_embs
+        self.global_sums = global_sums
         self.relation_weights = (
             relation_weights if relation_weights is not None
             else torch.ones(spec.num_relations, dtype=torch.float32, device=dev)
@@ -319,6 +327,11 @@ class StepRunner:
         bufs.lhs_op_p0, bufs.lhs_op_p1, bufs.lhs_op_s0, bufs.lhs_op_s1 = _ptr(p0), _ptr(p1), _ptr(s0), _ptr(s1)
         bufs.loss_out, bufs.violators_out = _ptr(self.loss_out), _ptr(self.violators_out)
         bufs.reg_out = _ptr(self.reg_out)
+        if self.global_embs is not None:
+            bufs.lhs_global, bufs.rhs_global = (_ptr(_need(t, torch.float32, "global embedding")) for t in self.global_embs)
+            if self.global_sums is not None:
+                bufs.lhs_global_sum, bufs.rhs_global_sum = (_ptr(_need(t, torch.float32, "global embedding sum"))
+                                                            for t in self.global_sums)
         bufs.workspace, bufs.workspace_bytes = _ptr(self.workspace), self.workspace.numel()
         bufs.sample_uniform = int(uniform_seed is not None)
         bufs.uniform_seed = (uniform_seed or 0) & (2**64 - 1)

@@ -89,8 +89,14 @@ class Trainer(AbstractBatchProcessor):
             if dynamic:
                 weights = (weights + [1.0] * model.num_dynamic_rels)[:model.num_dynamic_rels]
             rw = torch.tensor(weights, dtype=torch.float32, device=dev)
+            glob = model.global_vectors(relation_idx)
+            glob_sums = None
+            if glob is not None:  # parameters of the model optimizer, like the operators'
+                glob_sums = tuple(self._operator_state({}, {"g": p})["g"] for p in glob)
             runner = native.StepRunner(spec, w_l.data, opt_l.state[w_l]["sum"], w_r.data, opt_r.state[w_r]["sum"],
-                                       rhs_op, rhs_sum, lhs_op, lhs_sum, relation_weights=rw)
+                                       rhs_op, rhs_sum, lhs_op, lhs_sum, relation_weights=rw,
+                                       global_embs=None if glob is None else (glob[0].data, glob[1].data),
+                                       global_sums=glob_sums)
             self._runners[key] = runner
         negs = self.next_uniform_negs
         self.next_uniform_negs = None

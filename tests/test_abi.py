@@ -28,7 +28,7 @@ def test_struct_sizes_match_the_header(pbg):
     # 15 x 4-byte fields + one 4-byte field, then two int64: 16 * 4 + 16
     assert ctypes.sizeof(pbg._lib.StepDesc) == 88
     # 22 pointers + workspace_bytes, then sample_uniform (4 + 4 padding) and uniform_seed
-    assert ctypes.sizeof(pbg._lib.StepBuffers) == 26 * 8
+    assert ctypes.sizeof(pbg._lib.StepBuffers) == 30 * 8
     lib = pbg._lib.lib()
     assert lib.pbg_sizeof_step_desc() == ctypes.sizeof(pbg._lib.StepDesc)
     assert lib.pbg_sizeof_step_buffers() == ctypes.sizeof(pbg._lib.StepBuffers)

@@ -163,7 +163,13 @@ def build_model(pbg, cfg, st, n_rel_schemas):
     model = M.MultiRelationEmbedder(
         cfg.dim, rels, ent, cfg.num_batch_negs, cfg.num_uniform_negs, cfg.disable_lhs_negs, cfg.disable_rhs_negs,
         lhs_ops, rhs_ops, M.COMPARATORS.get_class(cfg.comparator)(), regularizer=regularizer,
-        num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
+        global_emb=cfg.global_emb, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
+    if cfg.global_emb:
+        model.global_embs.to(DEV)
+        with torch.no_grad():
+            model.global_embs[M.MultiRelationEmbedder.EMB_PREFIX + "l"][...] = st.glob_lhs.to(DEV)
+            if not st.shared:
+                model.global_embs[M.MultiRelationEmbedder.EMB_PREFIX + "r"][...] = st.glob_rhs.to(DEV)
     model.set_embeddings("l", pbg.types.Side.LHS, w_l)
     model.set_embeddings("l" if st.shared else "r", pbg.types.Side.RHS, w_r)
     return model, w_l, w_r
@@ -183,6 +189,11 @@ MODEL_CASES = [
          dim=8, regularization_coef=5e-2),
     dict(operator="translation", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=5,
          num_pos=25, dim=9, regularization_coef=5e-2),
+    # with global embeddings (the reference's default), one entity type (even dim) and two
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20,
+         num_pos=45, dim=16, global_emb=True),
+    dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=10, num_uniform_negs=5,
+         num_pos=25, dim=9, global_emb=True),
 ]
 
 
@@ -234,6 +245,13 @@ def test_model_forward_and_trainer_step(pbg, case):
         assert_close(opt_l.state[w_l]["sum"], st.g_lhs, rtol, "g_lhs")
         if not st.shared:
             assert_close(w_r.data, st.w_rhs, rtol, "w_rhs")
+        if cfg.global_emb:
+            g_l = model.global_embs[pbg.model.MultiRelationEmbedder.EMB_PREFIX + "l"]
+            assert_close(g_l.data, st.glob_lhs, rtol, "glob_lhs")
+            assert_close(trainer.model_optimizer.state[g_l]["sum"], st.glob_lhs_sum, rtol, "glob_lhs.sum")
+            if not st.shared:
+                g_r = model.global_embs[pbg.model.MultiRelationEmbedder.EMB_PREFIX + "r"]
+                assert_close(g_r.data, st.glob_rhs, rtol, "glob_rhs")
         if not cfg.dynamic and st.rhs_op:
             op = model.rhs_operators[rel]
             for k, v in st.rhs_op.items():

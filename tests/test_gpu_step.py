@@ -38,6 +38,10 @@ def make_inputs(cfg, num_pos, n_ent, workers, seed, shared=True, scale=0.3):
     for d in (st.lhs_op, st.rhs_op):
         for k in d:
             d[k] = d[k] + 0.2 * torch.randn(d[k].shape, generator=g)
+    if st.glob_lhs is not None:
+        st.glob_lhs += 0.3 * scale * torch.randn(cfg.dim, generator=g)
+        if st.glob_rhs is not st.glob_lhs:
+            st.glob_rhs += 0.3 * scale * torch.randn(cfg.dim, generator=g)
     return st, batches
 
 
@@ -53,7 +57,13 @@ def to_runner(pbg, cfg, st, num_pos, workers):
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))
     ops = [{k: dev(v) for k, v in d.items()} for d in (st.rhs_op, st.rhs_op_sum, st.lhs_op, st.lhs_op_sum)]
     rw = torch.tensor(list(cfg.relation_weights), dtype=torch.float32, device=DEV)
-    runner = pbg.StepRunner(spec, w_l, g_l, w_r, g_r, ops[0], ops[1], ops[2], ops[3], relation_weights=rw)
+    glob = sums = None
+    if st.glob_lhs is not None:
+        gl, sl = dev(st.glob_lhs), dev(st.glob_lhs_sum)
+        one = st.glob_rhs is st.glob_lhs
+        glob, sums = (gl, gl if one else dev(st.glob_rhs)), (sl, sl if one else dev(st.glob_rhs_sum))
+    runner = pbg.StepRunner(spec, w_l, g_l, w_r, g_r, ops[0], ops[1], ops[2], ops[3], relation_weights=rw,
+                            global_embs=glob, global_sums=sums)
     return runner
 
 
@@ -194,6 +204,11 @@ def compare_state(cfg, runner, st, rtol, tag):
                             ("lhs_op", runner.lhs_op, st.lhs_op), ("lhs_op_sum", runner.lhs_op_sum, st.lhs_op_sum)):
         for k in want:
             assert_close(got[k], want[k], rtol, f"{tag} {name}.{k}")
+    if st.glob_lhs is not None:
+        assert_close(runner.global_embs[0], st.glob_lhs, rtol, tag + " glob_lhs")
+        assert_close(runner.global_sums[0], st.glob_lhs_sum, rtol, tag + " glob_lhs_sum")
+        assert_close(runner.global_embs[1], st.glob_rhs, rtol, tag + " glob_rhs")
+        assert_close(runner.global_sums[1], st.glob_rhs_sum, rtol, tag + " glob_rhs_sum")
 
 
 def hinge_ties(cfg, scores, eps=2e-6):
@@ -248,6 +263,61 @@ def test_train_step(pbg, case, workers):
     compare_state(cfg, runner, st, rtol, "step")
 
 
+GLOBAL_CASES = [
+    # fused route
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=200, dim=100),
+    # (a distance between two rows of ONE type does not depend on the type's vector: its gradient would be
+    # rounding noise, which Adagrad turns into full steps; two types here)
+    dict(operator="translation", comparator="l2", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=100,
+         shared=False),
+    dict(operator="diagonal", comparator="dot", loss="softmax", num_batch_negs=20, num_uniform_negs=10, num_pos=45, dim=32),
+    # staged route
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=100,
+         num_pos=130, dim=400),
+    dict(operator="linear", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=10, num_pos=45, dim=24),
+    dict(operator="diagonal", comparator="squared_l2", loss="ranking", num_batch_negs=0, num_uniform_negs=7, num_pos=30,
+         dim=9, disable_lhs_negs=True),
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=10, num_uniform_negs=5, num_pos=33,
+         dim=16, regularization_coef=1e-2),
+    dict(operator="none", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
+         shared=False),
+]
+
+
+@pytest.mark.parametrize("case", GLOBAL_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_global_embeddings(pbg, case, workers):
+    """config.global_emb (model.py:433-441,486-492): every gathered row is shifted by
+    its entity type's vector, which is trained by the model optimizer; one vector
+    when the sides share the type (even dim here), two otherwise."""
+    say("train+global", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", dim % 2 == 0)
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, global_emb=True, **case)
+    n_ent = max(200, num_pos * (40 if cfg.comparator == "l2" else 4))
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=shared)
+    zero_glob = (st.glob_lhs.clone(), st.glob_rhs.clone())
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, batches)
+    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+    compare_state(cfg, runner, st, rtol, "step+global")
+    assert not torch.equal(st.glob_lhs, zero_glob[0])  # it was trained
+
+
+def test_global_embeddings_are_refused_for_dynamic_relations(pbg):
+    spec = pbg.StepSpec(dim=8, batch_size=10, dynamic=True, num_relations=2)
+    w = torch.randn(20, 8, device=DEV)
+    g = torch.zeros(8, device=DEV)
+    with pytest.raises(RuntimeError, match="Cannot have global embs with dynamic rels"):
+        pbg.StepRunner(spec, w, torch.zeros(20, device=DEV), global_embs=(g, g), global_sums=(g.clone(), g.clone()))
+
+
 REG_CASES = [
     # the reference's FB15k example: ComplEx, softmax, N3 with coefficient 1e-3 (fb15k_config_cpu.py:33-41)
     dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=50,
@@ -290,7 +360,7 @@ def test_train_step_with_n3_regularizer(pbg, case, workers):
     torch.cuda.synchronize()
     plain = ostep.StepConfig(**{**cfg.__dict__, "regularization_coef": 0.0})
     st_plain = ostep.TrainState(**{k: (v.clone() if torch.is_tensor(v) else {n: t.clone() for n, t in v.items()})
-                                   for k, v in st.__dict__.items()})
+                                   for k, v in st.__dict__.items() if v is not None})
     if st.shared:
         st_plain.w_rhs, st_plain.g_rhs = st_plain.w_lhs, st_plain.g_lhs
     outs = ostep.train_lockstep(cfg, st, batches)
