@@ -304,6 +304,8 @@ class BucketLoop:
                  lhs_op: Optional[Dict[str, torch.Tensor]] = None, lhs_op_sum: Optional[Dict[str, torch.Tensor]] = None,
                  resident_partitions: int = 2, bucket_order: str = "inside_out", seed: int = 0,
                  device: str = "cuda:0",
+                 regularization_coef: float = 0.0,
+                 global_embs: Optional[Dict[str, Tuple[torch.Tensor, torch.Tensor]]] = None,
                  eval_fraction: float = 0.0, eval_num_batch_negs: int = 1000, eval_num_uniform_negs: int = 1000,
                  edge_order: Optional[Callable[[Bucket, int], torch.Tensor]] = None,
                  negatives: Optional[Callable[..., torch.Tensor]] = None,
@@ -315,7 +317,13 @@ class BucketLoop:
         self.batch_size, self.num_workers = batch_size, num_workers
         self.spec_args = dict(dim=dim, num_batch_negs=num_batch_negs, num_uniform_negs=num_uniform_negs,
                               operator=operator, dynamic=dynamic, num_relations=num_relations, comparator=comparator,
-                              loss=loss, margin=margin, lr=lr, relation_lr=relation_lr)
+                              loss=loss, margin=margin, lr=lr, relation_lr=relation_lr,
+                              regularization_coef=regularization_coef)
+        # config.global_emb: {entity type: (vector [D], its AsyncAdagrad sum [D])} on the device
+        self.global_embs = None
+        if global_embs is not None:
+            (gl, sl), (gr, sr) = global_embs[lhs_entity], global_embs[rhs_entity]
+            self.global_embs = ((gl, gr), (sl, sr))
         self.ops = (rhs_op or {}, rhs_op_sum or {}, lhs_op or {}, lhs_op_sum or {})
         self.cache = PartitionCache(store, self.device, resident_partitions)
         self.bucket_order = bucket_order
@@ -407,7 +415,9 @@ class BucketLoop:
             (w_l, g_l), (w_r, g_r) = tables[0], tables[-1]
             shared = len(tables) == 1
             spec = native.StepSpec(batch_size=b_now, num_workers=k, **{**self.spec_args, **spec_overrides})
-            runner = native.StepRunner(spec, w_l, g_l, None if shared else w_r, None if shared else g_r, *self.ops)
+            glob, sums = self.global_embs if self.global_embs is not None else (None, None)
+            runner = native.StepRunner(spec, w_l, g_l, None if shared else w_r, None if shared else g_r, *self.ops,
+                                       global_embs=glob, global_sums=sums)
             runners[(k, b_now)] = runner
         return runner
 

@@ -251,12 +251,15 @@ def test_standard_relations_train_in_single_relation_batches(pbg):
     g0 = torch.Generator().manual_seed(11)
     edges = {k: (l, r, torch.randint(0, nrel, l.shape, generator=g0) ** 2 % nrel) for k, (l, r, _) in edges.items()}
     cfg = ostep.StepConfig(dim=dim, operator="translation", loss="ranking", margin=0.1, num_batch_negs=nb,
-                           num_uniform_negs=nu, num_relations=nrel, relation_weights=[1.0] * nrel, lr=0.1)
+                           num_uniform_negs=nu, num_relations=nrel, relation_weights=[1.0] * nrel, lr=0.1,
+                           regularization_coef=0.01, global_emb=True)
     st0 = ostep.make_state(cfg, tables[0])
     for k in st0.rhs_op:
         st0.rhs_op[k] = st0.rhs_op[k] + 0.1 * torch.randn(st0.rhs_op[k].shape, generator=g0)
     rhs_op = {k: v.clone().to(DEV) for k, v in st0.rhs_op.items()}
     rhs_sum = {k: torch.zeros_like(v) for k, v in rhs_op.items()}
+    glob0 = 0.05 * torch.randn(dim, generator=g0)
+    glob_dev, glob_sum_dev = glob0.clone().to(DEV), torch.zeros(dim, device=DEV)
     drawn = []
 
     def negatives(k, c, u, rows, generator, device):
@@ -267,11 +270,13 @@ def test_standard_relations_train_in_single_relation_batches(pbg):
     store, stats, loop = run_loop(pbg, tables, edges, nparts, dim, 2, hooks=dict(negatives=negatives, record_calls=True),
                                   batch_size=bsz, num_workers=workers, num_batch_negs=nb, num_uniform_negs=nu,
                                   operator="translation", num_relations=nrel, rhs_op=rhs_op, rhs_op_sum=rhs_sum,
-                                  bucket_order="lexicographic")
+                                  bucket_order="lexicographic", regularization_coef=0.01,
+                                  global_embs={"e": (glob_dev, glob_sum_dev)})
     w = {p: t.clone() for p, t in tables.items()}
     g = {p: torch.zeros(t.shape[0]) for p, t in tables.items()}
     op = {k: v.clone() for k, v in st0.rhs_op.items()}
     op_sum = {k: torch.zeros_like(v) for k, v in op.items()}
+    glob, glob_sum = glob0.clone(), torch.zeros(dim)
     it = iter(drawn)
     seen = {}
     for call in loop.calls_log:
@@ -289,6 +294,8 @@ def test_standard_relations_train_in_single_relation_batches(pbg):
         st.g_lhs = g[b.lhs]
         st.g_rhs = g[b.lhs] if b.lhs == b.rhs else g[b.rhs]
         st.rhs_op, st.rhs_op_sum = op, op_sum
+        st.glob_lhs = st.glob_rhs = glob  # one entity type: one vector, whatever the partitions
+        st.glob_lhs_sum = st.glob_rhs_sum = glob_sum
         ul, ur = next(it), next(it)
         batches = [(lhs[i * b_now:(i + 1) * b_now], rhs[i * b_now:(i + 1) * b_now], int(rel[i]), ul[i], ur[i])
                    for i in range(k)]
@@ -298,6 +305,9 @@ def test_standard_relations_train_in_single_relation_batches(pbg):
     assert len(seen) == 2 * nparts * nparts
     for p in range(nparts):
         assert torch.allclose(store.tables[("e", p)], w[p], rtol=1e-4, atol=1e-6)
+    assert not torch.equal(glob, glob0)
+    assert torch.allclose(glob_dev.cpu(), glob, rtol=1e-4, atol=1e-6)
+    assert torch.allclose(glob_sum_dev.cpu(), glob_sum, rtol=1e-4, atol=1e-9)
     for k in op:
         assert not torch.equal(op[k], st0.rhs_op[k])
         assert torch.allclose(rhs_op[k].cpu(), op[k], rtol=1e-4, atol=1e-6)
