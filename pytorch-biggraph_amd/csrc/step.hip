@@ -268,7 +268,15 @@ __device__ __forceinline__ void positive_scores(const StepCtx& c, int64_t kc, in
   const float* lp = c.side[0].xp + (kc * c.side[0].stride_p + i) * D;
   const float* rp = c.side[1].xp + (kc * c.side[1].stride_p + i) * D;
   if (!c.dynamic) {
-    posv[0] = posv[1] = kappa(c.cmp, lp, rp, D, lane);
+    // With batch negatives the score block already holds the pair: column i of row i
+    // is (rhs positive i) . (lhs positive i), before masking.  (Distances are
+    // recomputed from the rows: the block's ||a||^2 - 2ab + ||b||^2 cancels for a close pair.)
+    if (!is_distance(c.cmp) && c.side[0].nb > 0)
+      posv[0] = posv[1] = c.side[0].s[(kc * c.P + i) * c.side[0].nn + i];
+    else if (!is_distance(c.cmp) && c.side[1].nb > 0)
+      posv[0] = posv[1] = c.side[1].s[(kc * c.P + i) * c.side[1].nn + i];
+    else
+      posv[0] = posv[1] = kappa(c.cmp, lp, rp, D, lane);
   } else {
     posv[0] = kappa(c.cmp, lp, c.side[1].xa + (kc * c.P + i) * D, D, lane);
     posv[1] = kappa(c.cmp, rp, c.side[0].xa + (kc * c.P + i) * D, D, lane);
@@ -307,17 +315,65 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
   int viol = 0;
   float mx = pos, inv_z = 0.f;
   const float inv_nn = 1.0f / (float)nn;
+  // softmax makes three passes over the row; a wave keeps a row of up to
+  // kWave * kSoftmaxCache scores in registers after the first
+  constexpr int kSoftmaxCache = 20;
+  const bool cached = loss == PBG_LOSS_SOFTMAX && R::kStep == kWave && nn <= kWave * kSoftmaxCache;
+  float held[kSoftmaxCache];
+  unsigned held_live = 0u;
   if (loss == PBG_LOSS_SOFTMAX) {
     bool live;
-    for (int j = first; j < nn; j += R::kStep) mx = fmaxf(mx, sr.at(j, &live));
+    if (cached) {
+#pragma unroll
+      for (int u = 0; u < kSoftmaxCache; ++u) {
+        const int j = first + u * kWave;
+        held[u] = -INFINITY;
+        if (j < nn) {
+          held[u] = sr.at(j, &live);
+          held_live |= live ? 1u << u : 0u;
+          mx = fmaxf(mx, held[u]);
+        }
+      }
+    } else {
+      for (int j = first; j < nn; j += R::kStep) mx = fmaxf(mx, sr.at(j, &live));
+    }
     mx = R::max(mx);
     float z = 0.f;
-    for (int j = first; j < nn; j += R::kStep) z += expf(sr.at(j, &live) - mx);
+    if (cached) {
+#pragma unroll
+      for (int u = 0; u < kSoftmaxCache; ++u)
+        if (first + u * kWave < nn) z += expf(held[u] - mx);
+    } else {
+      for (int j = first; j < nn; j += R::kStep) z += expf(sr.at(j, &live) - mx);
+    }
     z = R::sum(z) + expf(pos - mx);
     inv_z = 1.0f / z;
     if (first == 0) {
       *loss_acc += (mx + logf(z)) - pos;
       dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+    }
+    if (cached) {  // third pass from the registers
+#pragma unroll
+      for (int u = 0; u < kSoftmaxCache; ++u) {
+        const int j = first + u * kWave;
+        if (j >= nn) continue;
+        const float t = held[u];
+        const bool live_u = (held_live >> u) & 1u;
+        float g = expf(t - mx) * inv_z * w;
+        if (t > pos) ++viol;
+        if (!live_u) g = 0.f;
+        if (is_distance(cmp)) {
+          const float dq = !live_u ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / t : -g);
+          rowsum += dq;
+          out[j] = -2.0f * dq;
+        } else {
+          out[j] = g;
+        }
+      }
+      *dpos_out = R::sum(dpos_part);
+      *rowsum_out = R::sum(rowsum);
+      *viol_out = R::sum_int(viol);
+      return;
     }
   } else if (loss == PBG_LOSS_LOGISTIC) {
     if (first == 0) {
