@@ -693,7 +693,8 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
     const int64_t kc = (int64_t)k * c.C + cc;
     const int col = sd.nb + uu;
     float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + r2) * D;
-    const RowV<NVH> y = row_load<NVH>(sd.xn + (kc * sd.nn + col) * D, D, H, lane);
+    // the prepared row itself only enters through the norm terms (l2, squared_l2) and cos's normalisation
+    const RowV<NVH> y = c.cmp != PBG_CMP_DOT ? row_load<NVH>(sd.xn + (kc * sd.nn + col) * D, D, H, lane) : row_zero<NVH>();
     RowV<NVH> dy = row_load<NVH>(sd.dxn + (kc * sd.nn + col) * D, D, H, lane);
     if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, col, lane), y);
     const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y, sd.an ? sd.an[kc * sd.nn + col] : 0.f);
