@@ -73,10 +73,11 @@ int seg_linear_apply(const uint64_t* keys, const uint32_t* vals, int64_t n, int 
 // For every relation and batch present: dW = sum over the run's edges of dz[e] (x) x[e]
 // (dz, x: [n, dim] by edge number), then wsum += dW^2, w -= lr * dW / (sqrt(wsum) + 1e-10),
 // batch after batch in ascending order.
-// `temp` holds seg_linear_update_temp_bytes(num_relations) bytes.
-size_t seg_linear_update_temp_bytes(int num_relations);
-int seg_linear_update(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, const float* dz,
-                      const float* x, int dim, int num_relations, float* w, float* wsum, float lr, void* temp,
-                      hipStream_t stream);
+// `num_batches`: batch numbers in the keys are below it.
+// `temp` holds seg_linear_update_temp_bytes(num_relations, n, dim, num_batches) bytes.
+size_t seg_linear_update_temp_bytes(int num_relations, int64_t n, int dim, int num_batches);
+int seg_linear_update(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, int num_batches,
+                      const float* dz, const float* x, int dim, int num_relations, float* w, float* wsum, float lr,
+                      void* temp, hipStream_t stream);
 
 }  // namespace pbg

@@ -17,10 +17,18 @@
 //                      after run in batch order.  A workgroup owns one 64 x 64
 //                      tile of one relation's matrix and keeps it (and its
 //                      Adagrad sum) in registers over all the relation's runs.
+//                      A relation with many edges in the call would make that
+//                      one long chain of dependent steps: the gradients of its
+//                      runs do not depend on one another, so other workgroups
+//                      compute them first (one per run, or per part of a run)
+//                      and the relation's workgroup only adds them up and takes
+//                      the Adagrad steps.
 //
 // Both use v_mfma_f32_16x16x4_f32 with depth-16 tiles staged through LDS
 // (k-major, row stride 80 floats), double buffered.
 #include "pbg_internal.h"
+
+#include <algorithm>
 
 namespace pbg {
 namespace {
@@ -193,6 +201,61 @@ __global__ void rel_start_kernel(const uint64_t* __restrict__ keys, int64_t n, i
 
 constexpr uint32_t kNone = 0xffffffffu;
 
+// rel_order: the relations by decreasing power of two of their edge count, so that
+// the workgroups with the longest chains of steps are dispatched first (any order
+// gives the same result; which of two relations of one size class comes first is
+// left to the atomics).  A relation with at least hot_min edges is "hot": it gets
+// a slot (hot_slot[r], hot_list[slot] = r, *hot_count slots in all; which slot is
+// left to the atomics too, the set of hot relations is not).  One workgroup.
+__global__ __launch_bounds__(1024) void rel_plan_kernel(const uint32_t* __restrict__ rel_start, int num_relations,
+                                                        uint32_t hot_min, uint32_t* __restrict__ rel_order,
+                                                        uint32_t* __restrict__ hot_slot,
+                                                        uint32_t* __restrict__ hot_count,
+                                                        uint32_t* __restrict__ hot_list) {
+  __shared__ unsigned count[34], base[34], nhot;
+  const int t = threadIdx.x;
+  if (t < 34) count[t] = 0u;
+  if (t == 0) nhot = 0u;
+  __syncthreads();
+  auto size_class = [&](uint32_t c) { return c == 0u ? 33 : __clz((int)c); };  // 0 for the largest counts
+  for (int r = t; r < num_relations; r += 1024) {
+    const uint32_t c = rel_start[r + 1] - rel_start[r];
+    atomicAdd(&count[size_class(c)], 1u);
+    uint32_t slot = kNone;
+    if (c >= hot_min) {
+      slot = atomicAdd(&nhot, 1u);
+      hot_list[slot] = (uint32_t)r;
+    }
+    hot_slot[r] = slot;
+  }
+  __syncthreads();
+  if (t == 0) {
+    unsigned run = 0u;
+    for (int b = 0; b < 34; ++b) {
+      base[b] = run;
+      run += count[b];
+    }
+    *hot_count = nhot;
+  }
+  __syncthreads();
+  for (int r = t; r < num_relations; r += 1024)
+    rel_order[atomicAdd(&base[size_class(rel_start[r + 1] - rel_start[r])], 1u)] = (uint32_t)r;
+}
+
+// run_start[slot * (num_batches + 1) + b]: first sorted position of the run (hot_list[slot], batch b);
+// entry num_batches is the end of the relation.
+__global__ void run_start_kernel(const uint64_t* __restrict__ keys, const uint32_t* __restrict__ rel_start, int kbits,
+                                 int num_batches, const uint32_t* __restrict__ hot_count,
+                                 const uint32_t* __restrict__ hot_list, uint32_t* __restrict__ run_start) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t slot = i / (num_batches + 1);
+  const int b = (int)(i % (num_batches + 1));
+  if (slot >= (int64_t)*hot_count) return;
+  const uint64_t rel = hot_list[slot];
+  const int64_t lo = rel_start[rel], hi = rel_start[rel + 1];
+  run_start[i] = (uint32_t)(b == num_batches ? hi : lower_bound(keys, lo, hi, (rel << kbits) | (uint64_t)b));
+}
+
 // A workgroup streams ALL edges of its relation, kStage sorted positions per
 // step, whatever batch they belong to; the rows of step s + 1 are requested
 // before the products of step s and written to LDS after them.  A step that
@@ -204,38 +267,91 @@ constexpr uint32_t kNone = 0xffffffffu;
 // not stay in the instruction cache is paid for by each of them.
 constexpr int kStage = 32;  // edges per step
 
-template <bool VEC>
+//
+// RUNS = false, grid (relation in rel_order, tile): as above; for a hot relation
+// the gradient tiles of its runs are read from `part` instead of being computed.
+// RUNS = true, grid ((slot * num_batches + batch) * splits + split, tile): the
+// gradient tile of one part of one run of a hot relation, written to
+// part[(blockIdx.x * tiles^2 + tile) * 256 + thread][16] in the MFMA result layout.
+struct HotRuns {
+  const uint32_t* rel_order;  // [num_relations]
+  const uint32_t* hot_slot;   // [num_relations], kNone: not hot
+  const uint32_t* hot_count;  // [1]
+  const uint32_t* hot_list;   // [*hot_count]
+  const uint32_t* run_start;  // [*hot_count][num_batches + 1]
+  float* part;                // null: no relation is hot
+  int num_batches, splits;
+};
+
+template <bool VEC, bool RUNS>
 __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, const uint32_t* __restrict__ rel_start,
     int kbits, const float* __restrict__ dz, const float* __restrict__ x, int dim, float* __restrict__ w,
-    float* __restrict__ wsum, float lr) {
+    float* __restrict__ wsum, float lr, HotRuns hot) {
   __shared__ __attribute__((aligned(16))) float lds_a[2][kStage * LD];
   __shared__ __attribute__((aligned(16))) float lds_b[2][kStage * LD];
   __shared__ uint32_t lds_batch[2][kStage];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
-  const uint64_t rel = blockIdx.x;
-  const int64_t lo = rel_start[rel], hi = rel_start[rel + 1];
-  if (lo == hi) return;  // the relation does not occur in this call: zero gradient, no change
   const int tiles = (dim + BN - 1) / BN;
   const int o0 = (blockIdx.y / tiles) * BM, i0 = (blockIdx.y % tiles) * BN;
+  uint64_t rel;
+  int64_t lo, hi;
+  float4v* part_out = nullptr;
+  if (RUNS) {
+    const int per_slot = hot.num_batches * hot.splits;
+    const uint32_t slot = blockIdx.x / per_slot;
+    if (slot >= *hot.hot_count) return;
+    const int batch = (blockIdx.x % per_slot) / hot.splits, split = blockIdx.x % hot.splits;
+    rel = hot.hot_list[slot];
+    const uint32_t* rs = hot.run_start + (int64_t)slot * (hot.num_batches + 1) + batch;
+    const int64_t run_lo = rs[0], len = (int64_t)rs[1] - run_lo;
+    lo = run_lo + len * split / hot.splits;
+    hi = run_lo + len * (split + 1) / hot.splits;
+    part_out = reinterpret_cast<float4v*>(hot.part + (((int64_t)blockIdx.x * tiles * tiles + blockIdx.y) * kThreads + tid) * 16);
+    if (lo == hi) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part_out[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+      return;
+    }
+  } else {
+    rel = hot.rel_order[blockIdx.x];  // busiest relations first
+    lo = rel_start[rel], hi = rel_start[rel + 1];
+    if (lo == hi) return;  // the relation does not occur in this call: zero gradient, no change
+  }
   float* wr = w + (int64_t)rel * dim * dim;
   float* sr = wsum + (int64_t)rel * dim * dim;
   const uint32_t batch_mask = (1u << kbits) - 1u;
 
   // this lane's 16 cells of the tile, in the MFMA result layout
   float wt[2][2][4], ht[2][2][4];
+  if (!RUNS) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int o = o0 + wm0 + i * 16 + 4 * (lane >> 4) + r, c = i0 + wn0 + j * 16 + (lane & 15);
-        const bool ok = o < dim && c < dim;
-        wt[i][j][r] = ok ? wr[(int64_t)o * dim + c] : 0.f;
-        ht[i][j][r] = ok ? sr[(int64_t)o * dim + c] : 0.f;
-      }
+        for (int r = 0; r < 4; ++r) {
+          const int o = o0 + wm0 + i * 16 + 4 * (lane >> 4) + r, c = i0 + wn0 + j * 16 + (lane & 15);
+          const bool ok = o < dim && c < dim;
+          wt[i][j][r] = ok ? wr[(int64_t)o * dim + c] : 0.f;
+          ht[i][j][r] = ok ? sr[(int64_t)o * dim + c] : 0.f;
+        }
+  }
+  auto write_back = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int o = o0 + wm0 + i * 16 + 4 * (lane >> 4) + r, c = i0 + wn0 + j * 16 + (lane & 15);
+          if (o < dim && c < dim) {
+            wr[(int64_t)o * dim + c] = wt[i][j][r];
+            sr[(int64_t)o * dim + c] = ht[i][j][r];
+          }
+        }
+  };
 
   // staging: thread -> edges kk and kk + 16 of the step, 4 consecutive columns.
   // Loads are issued unconditionally from addresses clamped into bounds and
@@ -284,13 +400,39 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
+          // One such step per run and matrix cell is most of this kernel's arithmetic when the
+          // runs are short: the hardware's square root and reciprocal (1 ulp each) in place
+          // of the correctly rounded sequences.
           const float g = tot[i][j][r] + acc[i][j][r];
           const float sum = ht[i][j][r] + g * g;
           ht[i][j][r] = sum;
-          wt[i][j][r] += -lr * (g / (sqrtf(sum) + 1e-10f));
+          wt[i][j][r] += -lr * g * __builtin_amdgcn_rcpf(__builtin_amdgcn_sqrtf(sum) + 1e-10f);
         }
   };
   reset();
+
+  if (!RUNS && hot.part != nullptr) {
+    const uint32_t slot = hot.hot_slot[rel];
+    if (slot != kNone) {
+      // the runs' gradient tiles are there already: add up the parts of each, one Adagrad step per batch
+      const int64_t stride = (int64_t)tiles * tiles * kThreads * 4;  // float4v per part
+      const float4v* src = reinterpret_cast<const float4v*>(hot.part) +
+                           ((int64_t)slot * hot.num_batches * hot.splits * tiles * tiles + blockIdx.y) * kThreads * 4 + tid * 4;
+#pragma unroll 2
+      for (int b = 0; b < hot.num_batches; ++b) {
+        for (int sp = 0; sp < hot.splits; ++sp, src += stride) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) tot[i][j] += src[i * 2 + j];
+        }
+        adagrad();
+        reset();
+      }
+      write_back();
+      return;
+    }
+  }
 
   const int nk = (int)((hi - lo + kStage - 1) / kStage);
   // edge numbers run two steps ahead of the products, rows one step ahead
@@ -343,7 +485,7 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
       heads &= heads - 1;
       const int b = heads != 0u ? __ffs((int)heads) - 1 : count;
       const uint32_t bt = (uint32_t)__builtin_amdgcn_readlane((int)mine, a);
-      if (bt != cur) {
+      if (!RUNS && bt != cur) {  // (a part of a run is of one batch)
         if (cur != kNone) adagrad();
         reset();
         steps = 0;
@@ -382,20 +524,15 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
     }
     __syncthreads();
   }
+  if (RUNS) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) part_out[i * 2 + j] = tot[i][j] + acc[i][j];
+    return;
+  }
   if (cur != kNone) adagrad();
-
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int o = o0 + wm0 + i * 16 + 4 * (lane >> 4) + r, c = i0 + wn0 + j * 16 + (lane & 15);
-        if (o < dim && c < dim) {
-          wr[(int64_t)o * dim + c] = wt[i][j][r];
-          sr[(int64_t)o * dim + c] = ht[i][j][r];
-        }
-      }
+  write_back();
 }
 
 bool aligned16(const void* p) { return (uintptr_t)p % 16 == 0; }
@@ -418,25 +555,114 @@ int seg_linear_apply(const uint64_t* keys, const uint32_t* vals, int64_t n, int 
   return check_launch("seg_linear_apply");
 }
 
-size_t seg_linear_update_temp_bytes(int num_relations) { return ((size_t)num_relations + 1) * sizeof(uint32_t); }
+namespace {
 
-int seg_linear_update(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, const float* dz,
-                      const float* x, int dim, int num_relations, float* w, float* wsum, float lr, void* temp,
-                      hipStream_t stream) {
+constexpr size_t kPartBudget = (size_t)1 << 30;  // bytes of run gradients at most
+
+// How the gradients of hot relations' runs are laid out for a call of n edges.
+struct HotPlan {
+  int splits;        // parts per run
+  int64_t slots;     // hot relations at most (0: none)
+  uint32_t hot_min;  // edges from which a relation is hot
+  size_t part_bytes_per_slot;
+};
+
+HotPlan hot_plan(int64_t n, int dim, int num_batches) {
+  const int tiles = (int)ceil_div(dim, BN);
+  HotPlan p;
+  // a chain of about 64 additions per hot relation: runs of few batches are cut into parts
+  p.splits = num_batches >= 64 ? 1 : (64 + num_batches - 1) / num_batches;
+  p.part_bytes_per_slot = (size_t)num_batches * p.splits * tiles * tiles * kThreads * 16 * sizeof(float);
+  // Below about 16 steps of kStage edges the chain is as short as the additions would be.
+  const int64_t least = 16 * kStage;
+  int64_t slots = n / least;
+  if ((size_t)slots * p.part_bytes_per_slot > kPartBudget) slots = (int64_t)(kPartBudget / p.part_bytes_per_slot);
+  // the grid of the run kernel is slots * num_batches * splits workgroups in x
+  const int64_t grid_cap = ((int64_t)1 << 31) - 1;
+  if (slots * num_batches * p.splits > grid_cap) slots = grid_cap / ((int64_t)num_batches * p.splits);
+  p.slots = slots;
+  // at most n / hot_min relations have hot_min edges: never more than `slots`
+  p.hot_min = slots > 0 ? (uint32_t)std::max<int64_t>(least, n / slots + 1) : 0xffffffffu;
+  return p;
+}
+
+struct HotLayout {
+  size_t rel_order, hot_slot, hot_count, hot_list, run_start, part, total;
+};
+
+HotLayout hot_layout(int num_relations, const HotPlan& p, int num_batches) {
+  HotLayout l;
+  size_t at = align_up(((size_t)num_relations + 1) * sizeof(uint32_t), 256);  // rel_start comes first
+  auto take = [&](size_t count, size_t size) {
+    const size_t here = at;
+    at = align_up(at + count * size, 256);
+    return here;
+  };
+  l.rel_order = take(num_relations, 4);
+  l.hot_slot = take(num_relations, 4);
+  l.hot_count = take(1, 4);
+  l.hot_list = take(std::max<int64_t>(p.slots, 1), 4);
+  l.run_start = take((size_t)p.slots * (num_batches + 1), 4);
+  l.part = take((size_t)p.slots, p.part_bytes_per_slot);
+  l.total = at;
+  return l;
+}
+
+}  // namespace
+
+size_t seg_linear_update_temp_bytes(int num_relations, int64_t n, int dim, int num_batches) {
+  return hot_layout(num_relations, hot_plan(n, dim, num_batches), num_batches).total;
+}
+
+int seg_linear_update(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, int num_batches,
+                      const float* dz, const float* x, int dim, int num_relations, float* w, float* wsum, float lr,
+                      void* temp, hipStream_t stream) {
   if (n <= 0 || num_relations <= 0) return PBG_OK;
   if (n >= ((int64_t)1 << 32) - 1) return fail(PBG_ERR_UNSUPPORTED, "seg_linear_update: too many edges");
-  uint32_t* rel_start = (uint32_t*)temp;
+  if (num_batches < 1 || ((int64_t)num_batches - 1) >> kbits != 0)
+    return fail(PBG_ERR_INVALID, "seg_linear_update: num_batches does not fit the key's batch bits");
+  const HotPlan hp = hot_plan(n, dim, num_batches);
+  const HotLayout hl = hot_layout(num_relations, hp, num_batches);
+  char* base = (char*)temp;
+  uint32_t* rel_start = (uint32_t*)base;
+  uint32_t* hot_count = (uint32_t*)(base + hl.hot_count);
+  uint32_t* hot_list = (uint32_t*)(base + hl.hot_list);
+  uint32_t* run_start = (uint32_t*)(base + hl.run_start);
   hipLaunchKernelGGL(rel_start_kernel, dim3((unsigned)ceil_div(num_relations + 1, 256)), dim3(256), 0, stream, keys, n,
                      kbits, num_relations, rel_start);
+  hipLaunchKernelGGL(rel_plan_kernel, dim3(1), dim3(1024), 0, stream, rel_start, num_relations, hp.hot_min,
+                     (uint32_t*)(base + hl.rel_order), (uint32_t*)(base + hl.hot_slot), hot_count, hot_list);
+  HotRuns hot;
+  hot.rel_order = (const uint32_t*)(base + hl.rel_order);
+  hot.hot_slot = (const uint32_t*)(base + hl.hot_slot);
+  hot.hot_count = hot_count;
+  hot.hot_list = hot_list;
+  hot.run_start = run_start;
+  hot.part = hp.slots > 0 ? (float*)(base + hl.part) : nullptr;
+  hot.num_batches = num_batches;
+  hot.splits = hp.splits;
   const int vec_ok = dim % 4 == 0 && aligned16(dz) && aligned16(x);
   const int tiles = (int)ceil_div(dim, BN);
-  const dim3 grid((unsigned)num_relations, (unsigned)(tiles * tiles)), block(kThreads);
+  const dim3 block(kThreads);
+  if (hp.slots > 0) {
+    hipLaunchKernelGGL(run_start_kernel, dim3((unsigned)ceil_div(hp.slots * (num_batches + 1), 256)), dim3(256), 0, stream,
+                       keys, rel_start, kbits, num_batches, hot_count, hot_list, run_start);
+    const dim3 grid((unsigned)(hp.slots * num_batches * hp.splits), (unsigned)(tiles * tiles));
+    if (vec_ok) {
+      hipLaunchKernelGGL((seg_linear_update_kernel<true, true>), grid, block, 0, stream, keys, vals, rel_start, kbits, dz,
+                         x, dim, w, wsum, lr, hot);
+    } else {
+      hipLaunchKernelGGL((seg_linear_update_kernel<false, true>), grid, block, 0, stream, keys, vals, rel_start, kbits,
+                         dz, x, dim, w, wsum, lr, hot);
+    }
+  }
+  const dim3 grid((unsigned)num_relations, (unsigned)(tiles * tiles));
   if (vec_ok) {
-    hipLaunchKernelGGL(seg_linear_update_kernel<true>, grid, block, 0, stream, keys, vals, rel_start, kbits, dz, x, dim,
-                       w, wsum, lr);
+    hipLaunchKernelGGL((seg_linear_update_kernel<true, false>), grid, block, 0, stream, keys, vals, rel_start, kbits, dz,
+                       x, dim, w, wsum, lr, hot);
   } else {
-    hipLaunchKernelGGL(seg_linear_update_kernel<false>, grid, block, 0, stream, keys, vals, rel_start, kbits, dz, x, dim,
-                       w, wsum, lr);
+    hipLaunchKernelGGL((seg_linear_update_kernel<false, false>), grid, block, 0, stream, keys, vals, rel_start, kbits, dz,
+                       x, dim, w, wsum, lr, hot);
   }
   return check_launch("seg_linear_update");
 }

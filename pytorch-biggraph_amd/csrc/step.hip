@@ -1982,7 +1982,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     plan->rvals_a = (uint32_t*)take(ne, 4);
     plan->rvals_b = (uint32_t*)take(ne, 4);
     plan->rsort_temp = take(sort_temp_bytes(ne), 1);
-    if (c.op == PBG_OP_LINEAR) plan->rel_start = take(seg_linear_update_temp_bytes(c.num_relations), 1);
+    if (c.op == PBG_OP_LINEAR) plan->rel_start = take(seg_linear_update_temp_bytes(c.num_relations, ne, D, K), 1);
   }
   for (int s = 0; s < 2; ++s) {
     plan->pslices[s] = 1;
@@ -2239,7 +2239,7 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
         if ((rc = seg_linear_apply(rkeys, rvals, ne, c.kbits, c.B, sd.dz, sd.op_rows, sd.p0, D, true,
                                    c.gr + (int64_t)sd.slot_pos * D, c.rk, true, stream)) != PBG_OK)
           return rc;
-        if ((rc = seg_linear_update(rkeys, rvals, ne, c.kbits, sd.dz, sd.xraw, D, c.num_relations, p0, s0,
+        if ((rc = seg_linear_update(rkeys, rvals, ne, c.kbits, c.K, sd.dz, sd.xraw, D, c.num_relations, p0, s0,
                                     d->relation_lr, plan.rel_start, stream)) != PBG_OK)
           return rc;
       } else {
