@@ -44,7 +44,8 @@ typedef enum pbg_operator {
   PBG_OP_DIAGONAL = 1,
   PBG_OP_TRANSLATION = 2,
   PBG_OP_LINEAR = 3,
-  PBG_OP_COMPLEX_DIAGONAL = 4
+  PBG_OP_COMPLEX_DIAGONAL = 4,
+  PBG_OP_AFFINE = 5 /* linear_transformation, then translation (operators.py:102-115, 272-293) */
 } pbg_operator;
 typedef enum pbg_comparator { PBG_CMP_DOT = 0, PBG_CMP_COS = 1, PBG_CMP_L2 = 2, PBG_CMP_SQUARED_L2 = 3 } pbg_comparator;
 typedef enum pbg_loss { PBG_LOSS_RANKING = 0, PBG_LOSS_LOGISTIC = 1, PBG_LOSS_SOFTMAX = 2 } pbg_loss;
@@ -148,7 +149,8 @@ typedef struct pbg_step_buffers {
   const float* edge_weight;   /* [K, B] or null (EdgeList.weight, edgelist.py:51-95) */
   const float* relation_weights; /* [num_relations] (batching.py:144-148) */
   /* Operator parameters, leading axis [num_relations]; p0 = diagonal |
-   * translation | linear_transformation | real, p1 = imag; s0/s1 = AsyncAdagrad
+   * translation | linear_transformation | real, p1 = imag | translation of
+   * `affine`; s0/s1 = AsyncAdagrad
    * state["sum"] of the same shape.  lhs_* only in dynamic mode. */
   float* rhs_op_p0; float* rhs_op_p1; float* rhs_op_s0; float* rhs_op_s1;
   float* lhs_op_p0; float* lhs_op_p1; float* lhs_op_s0; float* lhs_op_s1;
@@ -218,7 +220,8 @@ int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, f
  * ---------------------------------------------------------------------- */
 /* AbstractOperator.forward / AbstractDynamicOperator.forward (operators.py:49-157,
  * 197-338): y[i] = op(x[i]).  rel == NULL: one operator, parameters p0 (diagonal
- * | translation | linear_transformation | real) and p1 (imag).  rel != NULL:
+ * | translation | linear_transformation | real) and p1 (imag | translation of
+ * `affine`).  rel != NULL:
  * rel[n_rows] selects one of num_ops parameter rows per input row. */
 int pbg_operator_forward(int32_t op, int32_t dim, int64_t n_rows, const float* x, const float* p0,
                          const float* p1, const int64_t* rel, int64_t num_ops, float* y, pbg_stream_t stream);

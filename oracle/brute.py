@@ -29,6 +29,8 @@ def _op(name: str, x: np.ndarray, params: Optional[Dict[str, np.ndarray]], r: in
         return x + params["translation"][r]
     if name == "linear":
         return params["linear_transformation"][r] @ x
+    if name == "affine":
+        return params["linear_transformation"][r] @ x + params["translation"][r]
     if name == "complex_diagonal":
         h = x.shape[0] // 2
         a = x[:h] + 1j * x[h:]

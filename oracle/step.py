@@ -12,7 +12,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 import torch.nn.functional as F
 
-OPERATOR_NAMES = ("none", "diagonal", "translation", "linear", "complex_diagonal")
+OPERATOR_NAMES = ("none", "diagonal", "translation", "linear", "affine", "complex_diagonal")
 COMPARATOR_NAMES = ("dot", "cos", "l2", "squared_l2")
 LOSS_NAMES = ("ranking", "logistic", "softmax")
 
@@ -75,6 +75,8 @@ def init_operator_params(name: str, dim: int, num_ops: int) -> Dict[str, torch.T
         return {"translation": torch.zeros(num_ops, dim)}
     if name == "linear":
         return {"linear_transformation": torch.eye(dim).repeat(num_ops, 1, 1)}
+    if name == "affine":  # operators.py:106-107, 276-279
+        return {"linear_transformation": torch.eye(dim).repeat(num_ops, 1, 1), "translation": torch.zeros(num_ops, dim)}
     if name == "complex_diagonal":
         if dim % 2 != 0:
             raise ValueError(
@@ -104,6 +106,9 @@ def apply_operator(
     if name == "linear":
         mat = pick(params["linear_transformation"])
         return torch.matmul(mat, embs.unsqueeze(-1)).squeeze(-1)
+    if name == "affine":  # operators.py:109-115, 283-293
+        mat = pick(params["linear_transformation"])
+        return torch.matmul(mat, embs.unsqueeze(-1)).squeeze(-1) + pick(params["translation"])
     if name == "complex_diagonal":
         half = dim // 2
         real_a, imag_a = embs[..., :half], embs[..., half:]

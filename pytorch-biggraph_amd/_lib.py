@@ -10,7 +10,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_size_t, c_uin
 _HERE = pathlib.Path(__file__).resolve().parent
 LIB_PATH = _HERE / "libpbg_hip.so"
 
-OPERATOR_CODES = {"none": 0, "diagonal": 1, "translation": 2, "linear": 3, "complex_diagonal": 4}
+OPERATOR_CODES = {"none": 0, "diagonal": 1, "translation": 2, "linear": 3, "complex_diagonal": 4, "affine": 5}
 COMPARATOR_CODES = {"dot": 0, "cos": 1, "l2": 2, "squared_l2": 3}
 LOSS_CODES = {"ranking": 0, "logistic": 1, "softmax": 2}
 

@@ -366,7 +366,7 @@ __global__ __launch_bounds__(256) void sum_rows_kernel(const float* __restrict__
   if (threadIdx.x == 0) *out = sh[0];
 }
 
-bool valid_op(int op) { return op >= PBG_OP_NONE && op <= PBG_OP_COMPLEX_DIAGONAL; }
+bool valid_op(int op) { return op >= PBG_OP_NONE && op <= PBG_OP_AFFINE; }
 bool valid_cmp(int cmp) { return cmp >= PBG_CMP_DOT && cmp <= PBG_CMP_SQUARED_L2; }
 
 struct CmpWs {
@@ -403,9 +403,14 @@ extern "C" int pbg_operator_forward(int32_t op, int32_t dim, int64_t n_rows, con
   if (op == PBG_OP_COMPLEX_DIAGONAL && dim % 2 != 0)
     return fail(PBG_ERR_INVALID, "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");
   if (n_rows == 0) return PBG_OK;
-  if (!x || !y || (op != PBG_OP_NONE && !p0) || (op == PBG_OP_COMPLEX_DIAGONAL && !p1))
+  if (!x || !y || (op != PBG_OP_NONE && !p0) || ((op == PBG_OP_COMPLEX_DIAGONAL || op == PBG_OP_AFFINE) && !p1))
     return fail(PBG_ERR_INVALID, "pbg_operator_forward: null pointer");
   hipStream_t s = (hipStream_t)stream;
+  if (op == PBG_OP_AFFINE) {  // the matrix product, then the translation in place (operators.py:109-115, 283-293)
+    const int rc = pbg_operator_forward(PBG_OP_LINEAR, dim, n_rows, x, p0, nullptr, rel, num_ops, y, stream);
+    if (rc != PBG_OK) return rc;
+    return pbg_operator_forward(PBG_OP_TRANSLATION, dim, n_rows, y, p1, nullptr, rel, num_ops, y, stream);
+  }
   if (op == PBG_OP_LINEAR) {
     if (!rel) {
       GemmArgs g{};
@@ -429,9 +434,17 @@ extern "C" int pbg_operator_backward(int32_t op, int32_t dim, int64_t n_rows, co
   if (!valid_op(op)) return fail(PBG_ERR_INVALID, "pbg_operator_backward: unknown operator %d", op);
   if (dim <= 0 || dim > 1024 || n_rows < 0) return fail(PBG_ERR_INVALID, "pbg_operator_backward: bad sizes");
   if (n_rows == 0) return PBG_OK;
-  if (!x || !dy || !dx || (op != PBG_OP_NONE && (!p0 || !dp0)) || (op == PBG_OP_COMPLEX_DIAGONAL && (!p1 || !dp1)))
+  if (!x || !dy || !dx || (op != PBG_OP_NONE && (!p0 || !dp0)) ||
+      ((op == PBG_OP_COMPLEX_DIAGONAL || op == PBG_OP_AFFINE) && (!p1 || !dp1)))
     return fail(PBG_ERR_INVALID, "pbg_operator_backward: null pointer");
   hipStream_t s = (hipStream_t)stream;
+  if (op == PBG_OP_AFFINE) {
+    // the translation's gradient first (it leaves a copy of dy in dx), then the matrix's, which writes dx
+    const int rc = pbg_operator_backward(PBG_OP_TRANSLATION, dim, n_rows, x, dy, p1, nullptr, rel, num_ops, dx, dp1,
+                                         nullptr, stream);
+    if (rc != PBG_OK) return rc;
+    return pbg_operator_backward(PBG_OP_LINEAR, dim, n_rows, x, dy, p0, nullptr, rel, num_ops, dx, dp0, nullptr, stream);
+  }
   if (op == PBG_OP_LINEAR) {
     if (!rel) {
       if (n_rows > INT32_MAX) return fail(PBG_ERR_UNSUPPORTED, "pbg_operator_backward: too many rows");

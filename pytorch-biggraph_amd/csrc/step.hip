@@ -62,6 +62,7 @@ struct SideCtx {
 
 struct StepCtx {
   int D, K, B, P, C, U, last, dynamic, op, cmp, loss, num_relations;
+  int affine;  // op == PBG_OP_LINEAR with a translation added to the product (operators.py:103-115, 272-293)
   float margin;
   SideCtx side[2];
   const int64_t* rel;
@@ -194,6 +195,10 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
   const int k = (int)(job / sd.op_rows), r = (int)(job % sd.op_rows);
   const int D = c.D, H = (D + 1) / 2;
   RowV<NVH> y = row_load<NVH>(sd.z + job * D, D, H, lane);
+  if (c.affine) {
+    const int64_t rel = clamp_index((c.dynamic && r < c.B) ? c.rel[(int64_t)k * c.B + r] : c.rel[k], c.num_relations);
+    y = op_forward<NVH>(PBG_OP_TRANSLATION, y, sd.p1, nullptr, rel, D, H, lane);
+  }
   const float aux = prepare_row<NVH>(c.cmp, y);
   if (r < c.B) {
     const int cc = r / c.P, i = r % c.P;
@@ -1812,6 +1817,8 @@ struct Plan {
   size_t bytes;
   // buffers that only the host-side orchestration touches
   float* dth[2];
+  float* dth_t[2];   // `affine`: the translations' gradients, [K, pslices_t, D]
+  int pslices_t[2];
   uint64_t* keys_b;
   uint32_t* vals_b;
   void* sort_temp;
@@ -1837,14 +1844,14 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->num_batch_negs < 0 || d->num_uniform_negs < 0) return fail(PBG_ERR_INVALID, "step: negative negatives count");
   if (d->num_batch_negs == 0 && d->num_uniform_negs == 0)
     return fail(PBG_ERR_INVALID, "step: num_batch_negs and num_uniform_negs cannot both be 0");
-  if (d->op < PBG_OP_NONE || d->op > PBG_OP_COMPLEX_DIAGONAL) return fail(PBG_ERR_INVALID, "step: unknown operator %d", d->op);
+  if (d->op < PBG_OP_NONE || d->op > PBG_OP_AFFINE) return fail(PBG_ERR_INVALID, "step: unknown operator %d", d->op);
   if (d->comparator < PBG_CMP_DOT || d->comparator > PBG_CMP_SQUARED_L2) return fail(PBG_ERR_INVALID, "step: unknown comparator %d", d->comparator);
   if (d->loss < PBG_LOSS_RANKING || d->loss > PBG_LOSS_SOFTMAX) return fail(PBG_ERR_INVALID, "step: unknown loss %d", d->loss);
   if (d->op == PBG_OP_COMPLEX_DIAGONAL && d->dim % 2 != 0)
     return fail(PBG_ERR_INVALID,
                 "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");  // operators.py:132-136
   if (d->num_relations < 1) return fail(PBG_ERR_INVALID, "step: num_relations must be positive");
-  if (d->regularization_coef != 0.f && d->op == PBG_OP_LINEAR)
+  if (d->regularization_coef != 0.f && (d->op == PBG_OP_LINEAR || d->op == PBG_OP_AFFINE))
     return fail(PBG_ERR_UNSUPPORTED, "Regularizer not implemented for this operator");  // operators.py:40,188
   if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
   return PBG_OK;
@@ -1872,7 +1879,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.C = (c.B - 1) / c.P + 1;
   c.last = c.B - (c.C - 1) * c.P;
   c.dynamic = d->dynamic;
-  c.op = d->op;
+  c.op = d->op == PBG_OP_AFFINE ? PBG_OP_LINEAR : d->op;
+  c.affine = d->op == PBG_OP_AFFINE;
   c.cmp = d->comparator;
   c.loss = d->loss;
   c.margin = d->margin;
@@ -1992,6 +2000,11 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
       plan->pslices[s] = sl < 1 ? 1 : (sl > 16 ? 16 : sl);
     }
     plan->dth[s] = takef((size_t)K * plan->pslices[s] * plan->psize);
+    if (c.affine) {
+      int sl = (int)ceil_div(c.side[s].op_rows, 32 * kParamGroups);
+      plan->pslices_t[s] = sl < 1 ? 1 : (sl > 16 ? 16 : sl);
+      plan->dth_t[s] = takef((size_t)K * plan->pslices_t[s] * D);
+    }
   }
 
   const int64_t npairs = (int64_t)K * c.rk;
@@ -2054,7 +2067,7 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
     const float* p1 = s == 0 ? b->lhs_op_p1 : b->rhs_op_p1;
     const float* s0 = s == 0 ? b->lhs_op_s0 : b->rhs_op_s0;
     const float* s1 = s == 0 ? b->lhs_op_s1 : b->rhs_op_s1;
-    const bool two = d->op == PBG_OP_COMPLEX_DIAGONAL;
+    const bool two = d->op == PBG_OP_COMPLEX_DIAGONAL || d->op == PBG_OP_AFFINE;
     if (!p0 || (two && !p1)) return fail(PBG_ERR_INVALID, "step: null operator parameter");
     if (training && (!s0 || (two && !s1))) return fail(PBG_ERR_INVALID, "step: null operator optimizer state");
   }
@@ -2242,6 +2255,12 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
         if ((rc = seg_linear_update(rkeys, rvals, ne, c.kbits, c.K, sd.dz, sd.xraw, D, c.num_relations, p0, s0,
                                     d->relation_lr, plan.rel_start, stream)) != PBG_OK)
           return rc;
+        if (c.affine) {  // the translations: the element-wise kernel on dz, parameters in the second slot
+          StepCtx ct = c;
+          ct.op = PBG_OP_TRANSLATION;
+          hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, ct,
+                             s, rkeys, rvals, p1, nullptr, s1, nullptr, d->relation_lr);
+        }
       } else {
         hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
                            rkeys, rvals, p0, p1, s0, s1, d->relation_lr);
@@ -2273,6 +2292,20 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
     } else {
       hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
                          dim3(kParamGroups * 64), 0, stream, c, s, plan.dth[s], plan.pslices[s]);
+    }
+    if (c.affine) {  // the translation: column sums of dz, then its own Adagrad steps (parameters in the second slot)
+      StepCtx ct = c;
+      ct.op = PBG_OP_TRANSLATION;
+      const int sl = plan.pslices_t[s];
+      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)sl),
+                         dim3(kParamGroups * 64), 0, stream, ct, s, plan.dth_t[s], sl);
+      if (K <= kWave) {
+        hipLaunchKernelGGL(param_update_wave_kernel, dim3((unsigned)ceil_div(D, kWavesPerBlock)), dim3(kRowThreads), 0,
+                           stream, ct, s, plan.dth_t[s], sl, (int64_t)D, p1, nullptr, s1, nullptr, d->relation_lr);
+      } else {
+        hipLaunchKernelGGL(param_update_kernel, dim3((unsigned)ceil_div(D, 256)), dim3(256), 0, stream, ct, s,
+                           plan.dth_t[s], sl, (int64_t)D, p1, nullptr, s1, nullptr, d->relation_lr);
+      }
     }
     if (K <= kWave && c.op != PBG_OP_LINEAR) {  // (a matrix's elements are better served one per thread)
       hipLaunchKernelGGL(param_update_wave_kernel, dim3((unsigned)ceil_div(plan.psize, kWavesPerBlock)), dim3(kRowThreads),

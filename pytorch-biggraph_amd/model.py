@@ -360,7 +360,7 @@ class MultiRelationEmbedder(nn.Module):
             p0, p1 = op.fused_params()
             if p0 is None:
                 return {}
-            return {"real": p0.data, "imag": p1.data} if p1 is not None else {"p0": p0.data}
+            return {"p0": p0.data, "p1": p1.data} if p1 is not None else {"p0": p0.data}
         lhs = pack(self.lhs_operators[relation_idx]) if self.num_dynamic_rels > 0 else {}
         return pack(self.rhs_operators[relation_idx]), lhs
 

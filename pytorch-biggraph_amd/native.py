@@ -287,8 +287,10 @@ class StepRunner:
     def _op_pair(params: Dict[str, torch.Tensor]) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
         if not params:
             return None, None
-        if "real" in params:
-            return params["real"], params["imag"]
+        # two-parameter operators: (first slot, second slot) of pbg_step_buffers
+        for first, second in (("p0", "p1"), ("real", "imag"), ("linear_transformation", "translation")):
+            if first in params and second in params:
+                return params[first], params[second]
         (only,) = params.values()
         return only, None
 

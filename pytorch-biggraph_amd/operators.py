@@ -160,6 +160,24 @@ class LinearOperator(AbstractOperator):
         return self._run(embeddings)
 
 
+@OPERATORS.register_as("affine")
+class AffineOperator(AbstractOperator):
+    """y = A x + t (operators.py:102-115)."""
+
+    op_name = "affine"
+
+    def __init__(self, dim: int):
+        super().__init__(dim)
+        self.linear_transformation = nn.Parameter(torch.eye(self.dim))
+        self.translation = nn.Parameter(torch.zeros((self.dim,)))
+
+    def fused_params(self):
+        return self.linear_transformation, self.translation
+
+    def forward(self, embeddings: FloatTensorType) -> FloatTensorType:
+        return self._run(embeddings)
+
+
 @OPERATORS.register_as("complex_diagonal")
 class ComplexDiagonalOperator(AbstractOperator):
     op_name = "complex_diagonal"
@@ -284,6 +302,24 @@ class LinearDynamicOperator(AbstractDynamicOperator):
 
     def fused_params(self):
         return self.linear_transformations, None
+
+    def forward(self, embeddings: FloatTensorType, operator_idxs: LongTensorType) -> FloatTensorType:
+        return self._run(embeddings, operator_idxs)
+
+
+@DYNAMIC_OPERATORS.register_as("affine")
+class AffineDynamicOperator(AbstractDynamicOperator):
+    """y_i = A[idx_i] x_i + t[idx_i] (operators.py:272-293)."""
+
+    op_name = "affine"
+
+    def __init__(self, dim: int, num_operations: int):
+        super().__init__(dim, num_operations)
+        self.linear_transformations = nn.Parameter(torch.diag_embed(torch.ones(()).expand(num_operations, dim)))
+        self.translations = nn.Parameter(torch.zeros((self.num_operations, self.dim)))
+
+    def fused_params(self):
+        return self.linear_transformations, self.translations
 
     def forward(self, embeddings: FloatTensorType, operator_idxs: LongTensorType) -> FloatTensorType:
         return self._run(embeddings, operator_idxs)

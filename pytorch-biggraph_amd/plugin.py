@@ -1,7 +1,7 @@
 """Name-keyed plugin registries (reference: torchbiggraph/plugin.py:16-40).
 
 The package keeps registries of its own under the reference's names: operators
-``none | diagonal | translation | linear | complex_diagonal``, comparators
+``none | diagonal | translation | linear | affine | complex_diagonal``, comparators
 ``dot | cos | l2 | squared_l2``, loss functions ``ranking | logistic | softmax``
 and the regularizer ``N3``.
 """

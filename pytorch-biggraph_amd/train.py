@@ -79,7 +79,7 @@ class Trainer(AbstractBatchProcessor):
                 if not tensors:
                     return {}
                 p0, p1 = op_module.fused_params()
-                owners = {"real": p0, "imag": p1} if p1 is not None else {"p0": p0}
+                owners = {"p0": p0, "p1": p1} if p1 is not None else {"p0": p0}
                 return self._operator_state(tensors, owners)
 
             rhs_sum = sums(model.rhs_operators[relation_idx], rhs_op)

@@ -181,6 +181,8 @@ MODEL_CASES = [
     dict(operator="translation", comparator="l2", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=10, num_pos=33, dim=12),
     dict(operator="linear", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=0, num_uniform_negs=7, num_pos=30, dim=9),
+    dict(operator="affine", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
+    dict(operator="affine", comparator="l2", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
     dict(operator="none", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
     # with the N3 regularizer (the reference's FB15k example uses 1e-3 on ComplEx)
     dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20,

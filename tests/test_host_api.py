@@ -20,7 +20,7 @@ def test_plugin_registry(pbg):
         reg.register("a", int)
     with pytest.raises(NotImplementedError, match="known names: a"):
         reg.get_class("b")
-    assert sorted(pbg.operators.OPERATORS.registry) == ["complex_diagonal", "diagonal", "linear", "none", "translation"]
+    assert sorted(pbg.operators.OPERATORS.registry) == ["affine", "complex_diagonal", "diagonal", "linear", "none", "translation"]
     assert sorted(pbg.operators.DYNAMIC_OPERATORS.registry) == sorted(pbg.operators.OPERATORS.registry)
     assert sorted(pbg.model.COMPARATORS.registry) == ["cos", "dot", "l2", "squared_l2"]
     assert sorted(pbg.losses.LOSS_FUNCTIONS.registry) == ["logistic", "ranking", "softmax"]
@@ -167,7 +167,11 @@ def test_argument_validation_without_gpu(pbg):
     with pytest.raises(ValueError, match="even dimension"):
         pbg.operators.ComplexDiagonalDynamicOperator(5, 2)
     with pytest.raises(NotImplementedError):
-        pbg.operators.instantiate_operator("affine", pbg.types.Side.RHS, 0, 4)
+        pbg.operators.instantiate_operator("rotation", pbg.types.Side.RHS, 0, 4)
+    aff = pbg.operators.instantiate_operator("affine", pbg.types.Side.RHS, 0, 4)
+    assert torch.equal(aff.linear_transformation, torch.eye(4)) and torch.equal(aff.translation, torch.zeros(4))
+    aff = pbg.operators.instantiate_operator("affine", pbg.types.Side.LHS, 3, 4)
+    assert tuple(aff.linear_transformations.shape) == (3, 4, 4) and tuple(aff.translations.shape) == (3, 4)
     assert pbg.operators.instantiate_operator("linear", pbg.types.Side.LHS, 0, 4) is None
     op = pbg.operators.instantiate_operator("linear", pbg.types.Side.LHS, 7, 4)
     assert tuple(op.linear_transformations.shape) == (7, 4, 4)
