@@ -62,6 +62,15 @@ const char* pbg_last_error(void);
 int pbg_gather_rows(const float* table, int64_t num_rows, int32_t dim, const int64_t* idx, int64_t n,
                     float* out, int32_t* oob_flag, pbg_stream_t stream);
 
+/* What F.embedding(max_norm=...) does to the table before it reads it
+ * (SimpleEmbedding with max_norm, model.py:52-61; torch.embedding_renorm_): every
+ * row named in idx whose 2-norm exceeds max_norm is scaled, in the table, by
+ * max_norm / (norm + 1e-7).  Indices outside [0, num_rows) are skipped.  The
+ * workspace holds pbg_embedding_renorm_workspace_bytes(n, dim) bytes. */
+size_t pbg_embedding_renorm_workspace_bytes(int64_t n, int32_t dim);
+int pbg_embedding_renorm(float* table, int64_t num_rows, int32_t dim, const int64_t* idx, int64_t n,
+                         float max_norm, void* workspace, size_t workspace_bytes, pbg_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * RowAdagrad.  Replaces RowAdagrad.step (row_adagrad.py:48-109).
  * Sparse branch (:80-96): `idx[n]` / `grad_rows[n, dim]` are the uncoalesced
@@ -133,7 +142,9 @@ typedef struct pbg_step_desc {
    * (train_cpu.py:102-103).  0 = no regularizer.  Not defined for `linear`
    * (operators.py:40). */
   float regularization_coef;
-  int32_t reserved0;        /* keep 0 */
+  float max_norm;           /* > 0: F.embedding(max_norm=...) (model.py:61,90-96): the rows a call looks up are
+                             * first renormalised IN THE TABLE to at most this 2-norm (pbg_model_forward
+                             * included, as in the reference); 0 = off */
 } pbg_step_desc;
 
 typedef struct pbg_step_buffers {

@@ -44,6 +44,9 @@ class StepConfig:
     # config.py:181-188: a learned vector per entity type added to every embedding
     # of the type (model.py:433-441,486-492); standard relations only
     global_emb: bool = False
+    # config.py:173-180: rows are looked up with F.embedding(max_norm=...), which first
+    # renormalises them in the table (model.py:61); None = off
+    max_norm: Optional[float] = None
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
@@ -574,15 +577,16 @@ def forward_backward(
     lhs_op = {k: v.detach().requires_grad_(True) for k, v in st.lhs_op.items()}
     rhs_op = {k: v.detach().requires_grad_(True) for k, v in st.rhs_op.items()}
 
-    lhs_pos = F.embedding(lhs, w_l, sparse=True)
-    rhs_pos = F.embedding(rhs, w_r, sparse=True)
+    # (with max_norm the tables themselves change here, before anything is computed: model.py:61)
+    lhs_pos = F.embedding(lhs, w_l, max_norm=cfg.max_norm, sparse=True)
+    rhs_pos = F.embedding(rhs, w_r, max_norm=cfg.max_norm, sparse=True)
     lhs_u = (
-        F.embedding(uniform_lhs, w_l, sparse=True)
+        F.embedding(uniform_lhs, w_l, max_norm=cfg.max_norm, sparse=True)
         if uniform_lhs is not None and not cfg.disable_lhs_negs and uniform_lhs.numel() > 0
         else None
     )
     rhs_u = (
-        F.embedding(uniform_rhs, w_r, sparse=True)
+        F.embedding(uniform_rhs, w_r, max_norm=cfg.max_norm, sparse=True)
         if uniform_rhs is not None and not cfg.disable_rhs_negs and uniform_rhs.numel() > 0
         else None
     )

@@ -44,7 +44,7 @@ class StepDesc(ctypes.Structure):
         ("num_lhs_rows", c_int64),
         ("num_rhs_rows", c_int64),
         ("regularization_coef", c_float),
-        ("reserved0", c_int32),
+        ("max_norm", c_float),
     ]
 
 
@@ -70,6 +70,8 @@ SIGNATURES = {
     "pbg_version": (c_int32, []),
     "pbg_last_error": (c_char_p, []),
     "pbg_gather_rows": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "pbg_embedding_renorm_workspace_bytes": (c_size_t, [c_int64, c_int32]),
+    "pbg_embedding_renorm": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_int64, c_float, c_void_p, c_size_t, c_void_p]),
     "pbg_row_adagrad_sparse_workspace_bytes": (c_size_t, [c_int64]),
     "pbg_row_adagrad_sparse": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64,
                                          c_float, c_void_p, c_size_t, c_void_p]),

@@ -653,6 +653,70 @@ extern "C" int pbg_gather_rows(const float* table, int64_t num_rows, int32_t dim
 }
 
 namespace {
+// torch.embedding_renorm_ (what F.embedding(max_norm=...) runs first, model.py:61,90-96) in two
+// passes, so that no wave reads a row that another is rewriting: the first only reads the
+// table and keeps a too-long row and its scale per index, the second writes row * scale.
+// Equal indices keep the same row and scale and write the same bytes.  One wave per index.
+__global__ __launch_bounds__(kRowThreads) void renorm_scan_kernel(const float* __restrict__ table, int64_t num_rows,
+                                                                  int dim, const int64_t* __restrict__ idx, int64_t n,
+                                                                  float max_norm, float* __restrict__ kept,
+                                                                  float* __restrict__ scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int64_t id = idx[i];
+  float sc = 0.f;
+  if (id >= 0 && id < num_rows) {
+    const float* row = table + id * dim;
+    float sq = 0.f;
+    for (int d = lane; d < dim; d += kWave) sq += row[d] * row[d];
+    const float norm = sqrtf(wave_sum(sq));
+    if (norm > max_norm) {
+      sc = max_norm / (norm + 1e-7f);
+      for (int d = lane; d < dim; d += kWave) kept[i * dim + d] = row[d];
+    }
+  }
+  if (lane == 0) scale[i] = sc;
+}
+
+__global__ __launch_bounds__(kRowThreads) void renorm_apply_kernel(float* __restrict__ table, int dim,
+                                                                   const int64_t* __restrict__ idx, int64_t n,
+                                                                   const float* __restrict__ kept,
+                                                                   const float* __restrict__ scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t i = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const float sc = scale[i];
+  if (sc == 0.f) return;
+  float* row = table + idx[i] * dim;
+  for (int d = lane; d < dim; d += kWave) row[d] = kept[i * dim + d] * sc;
+}
+}  // namespace
+
+extern "C" size_t pbg_embedding_renorm_workspace_bytes(int64_t n, int32_t dim) {
+  const size_t nn = (size_t)(n > 0 ? n : 1);
+  return align_up(nn * (size_t)(dim > 0 ? dim : 1) * sizeof(float), 256) + align_up(nn * sizeof(float), 256);
+}
+
+extern "C" int pbg_embedding_renorm(float* table, int64_t num_rows, int32_t dim, const int64_t* idx, int64_t n,
+                                    float max_norm, void* workspace, size_t workspace_bytes, pbg_stream_t stream) {
+  if (n < 0 || dim <= 0 || num_rows < 0) return fail(PBG_ERR_INVALID, "pbg_embedding_renorm: bad sizes");
+  if (!(max_norm > 0.f)) return fail(PBG_ERR_INVALID, "pbg_embedding_renorm: max_norm must be positive");
+  if (n == 0) return PBG_OK;
+  if (!table || !idx) return fail(PBG_ERR_INVALID, "pbg_embedding_renorm: null pointer");
+  if (!workspace || workspace_bytes < pbg_embedding_renorm_workspace_bytes(n, dim))
+    return fail(PBG_ERR_WORKSPACE, "pbg_embedding_renorm: workspace needs %zu bytes, got %zu",
+                pbg_embedding_renorm_workspace_bytes(n, dim), workspace_bytes);
+  float* kept = (float*)workspace;
+  float* scale = (float*)((char*)workspace + align_up((size_t)n * dim * sizeof(float), 256));
+  const dim3 grid((unsigned)ceil_div(n, kRowThreads / kWave)), block(kRowThreads);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(renorm_scan_kernel, grid, block, 0, s, table, num_rows, dim, idx, n, max_norm, kept, scale);
+  hipLaunchKernelGGL(renorm_apply_kernel, grid, block, 0, s, table, dim, idx, n, kept, scale);
+  return check_launch("pbg_embedding_renorm");
+}
+
+namespace {
 struct SparseWs {
   uint64_t* keys_a; uint64_t* keys_b; uint32_t* vals_a; uint32_t* vals_b; void* temp;
   size_t total;

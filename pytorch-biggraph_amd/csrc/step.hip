@@ -100,6 +100,66 @@ __device__ __forceinline__ RowV<NVH> gathered_row(const SideCtx& sd, int64_t id,
 }
 
 // ---------------------------------------------------------------------------
+// max_norm
+// ---------------------------------------------------------------------------
+// The reference looks rows up with F.embedding(max_norm=...) (model.py:61,90-96):
+// before they are read, the rows a batch names are renormalised in the table
+// itself -- a row whose 2-norm exceeds max_norm is scaled by max_norm / (norm +
+// 1e-7).  Two kernels, so that no wave reads a row that another is rewriting:
+// `scan` only reads the table and keeps, per gathered slot, a too-long row and
+// its scale; `apply` writes row * scale back for those slots.  Slots that name
+// the same row hold the same row and the same scale, so their writes carry the
+// same bytes.  The K batches of a call are renormalised together, then read.
+__device__ __forceinline__ const SideCtx& slot_row(const StepCtx& c, int k, int slot, int64_t* id) {
+  const int s = slot >= c.side[1].slot_pos;
+  const SideCtx& sd = c.side[s];
+  const int r = slot - sd.slot_pos;
+  if (r < c.B) {
+    *id = clamp_index(sd.idx[(int64_t)k * c.B + r], sd.num_rows);
+  } else {
+    const int r2 = r - c.B;
+    *id = clamp_index(uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u), sd.num_rows);
+  }
+  return sd;
+}
+
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void renorm_scan_kernel(StepCtx c, float max_norm, float* __restrict__ scale) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.rk) return;
+  const int D = c.D, H = (D + 1) / 2;
+  int64_t id;
+  const SideCtx& sd = slot_row(c, (int)(job / c.rk), (int)(job % c.rk), &id);
+  const RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
+  const float norm = sqrtf(wave_sum(row_dot(x, x)));
+  const bool renorm = norm > max_norm;
+  if (renorm) row_store<NVH>(c.gr + job * D, x, D, H, lane);
+  if (lane == 0) scale[job] = renorm ? max_norm / (norm + 1e-7f) : 0.f;
+}
+
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void renorm_apply_kernel(StepCtx c, const float* __restrict__ scale,
+                                                                    float* w_lhs, float* w_rhs) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.rk) return;
+  const float sc = scale[job];
+  if (sc == 0.f) return;
+  const int D = c.D, H = (D + 1) / 2;
+  int64_t id;
+  const int slot = (int)(job % c.rk);
+  slot_row(c, (int)(job / c.rk), slot, &id);
+  RowV<NVH> x = row_load<NVH>(c.gr + job * D, D, H, lane);
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    x.a[0][v] *= sc;
+    x.a[1][v] *= sc;
+  }
+  row_store<NVH>((slot >= c.side[1].slot_pos ? w_rhs : w_lhs) + id * D, x, D, H, lane);
+}
+
+// ---------------------------------------------------------------------------
 // prep
 // ---------------------------------------------------------------------------
 template <int NVH>
@@ -1817,6 +1877,8 @@ struct Plan {
   size_t bytes;
   // buffers that only the host-side orchestration touches
   float* dth[2];
+  float max_norm;      // 0: rows are read as they are
+  float* renorm_scale; // [K * rk]
   float* dth_t[2];   // `affine`: the translations' gradients, [K, pslices_t, D]
   int pslices_t[2];
   uint64_t* keys_b;
@@ -2008,6 +2070,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   }
 
   const int64_t npairs = (int64_t)K * c.rk;
+  plan->max_norm = d->max_norm > 0.f ? d->max_norm : 0.f;
+  if (plan->max_norm > 0.f) plan->renorm_scale = takef((size_t)npairs);
   c.gr = takef((size_t)npairs * D);
   c.keys = (uint64_t*)take(npairs, 8);
   plan->keys_b = (uint64_t*)take(npairs, 8);
@@ -2101,6 +2165,16 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
   } while (0)
 
 dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 1, kWavesPerBlock)); }
+
+int run_renorm(const Plan& plan, const pbg_step_buffers* b, hipStream_t stream) {
+  if (plan.max_norm <= 0.f) return PBG_OK;
+  const StepCtx& c = plan.c;
+  const dim3 grid = wave_grid((int64_t)c.K * c.rk);
+  PBG_DISPATCH_NVH(plan.nvh, renorm_scan_kernel, grid, stream, c, plan.max_norm, plan.renorm_scale);
+  PBG_DISPATCH_NVH(plan.nvh, renorm_apply_kernel, grid, stream, c, plan.renorm_scale, b->w_lhs,
+                   b->w_rhs ? b->w_rhs : b->w_lhs);
+  return check_launch("step max_norm");
+}
 
 int run_prep(const Plan& plan, hipStream_t stream) {
   const StepCtx& c = plan.c;
@@ -2414,6 +2488,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if (ev) hipEventRecord(ev[i], s);
   };
   mark(0);
+  if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
   if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
     const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
@@ -2524,6 +2599,7 @@ extern "C" int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffe
     return fail(PBG_ERR_INVALID, "pbg_model_forward: null output");
   hipStream_t s = (hipStream_t)stream;
   RelOrder rel_order;
+  if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
   if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
   if ((rc = run_operator_forward(plan, s, &rel_order)) != PBG_OK) return rc;
   if ((rc = run_scores(plan, s)) != PBG_OK) return rc;

@@ -16,7 +16,7 @@ training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
 Not provided (outside the accelerated path): FeaturizedEmbedding,
-BiasedComparator, all_negs, max_norm, half precision.
+BiasedComparator, all_negs, half precision.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -73,10 +73,8 @@ class SimpleEmbedding(AbstractEmbedding):
 
     def __init__(self, weight: nn.Parameter, max_norm: Optional[float] = None):
         super().__init__()
-        if max_norm is not None:
-            raise NotImplementedError("max_norm is not supported")
         self.weight: nn.Parameter = weight
-        self.max_norm = None
+        self.max_norm: Optional[float] = max_norm
 
     def forward(self, input_: EntityList) -> FloatTensorType:
         return self.get(input_.to_tensor())
@@ -84,6 +82,8 @@ class SimpleEmbedding(AbstractEmbedding):
     def get(self, input_: LongTensorType) -> FloatTensorType:
         if input_.numel() == 0:
             return self.weight.new_empty((*input_.shape, self.weight.shape[1]))
+        if self.max_norm is not None:  # F.embedding(max_norm=...): the table itself is renormalised first
+            native.embedding_renorm_(self.weight.data, input_, self.max_norm)
         return _GatherFunction.apply(self.weight, input_)
 
     def get_all_entities(self) -> FloatTensorType:
@@ -253,8 +253,6 @@ class MultiRelationEmbedder(nn.Module):
         super().__init__()
         if regularizer is not None and not isinstance(regularizer, N3Regularizer):
             raise NotImplementedError("Only the N3 regularizer is supported")
-        if max_norm is not None:
-            raise NotImplementedError("max_norm is not supported")
         if half_precision:
             raise NotImplementedError("Half precision is not supported")
         if any(e.featurized for e in entities.values()):
@@ -282,14 +280,14 @@ class MultiRelationEmbedder(nn.Module):
             self.global_embs = nn.ParameterDict({
                 self.EMB_PREFIX + entity: nn.Parameter(torch.zeros((schema.dimension or default_dim,)))
                 for entity, schema in entities.items()})
-        self.max_norm = None
+        self.max_norm: Optional[float] = max_norm
         self.half_precision = False
         self.regularizer: Optional[AbstractRegularizer] = regularizer
         self._runners: Dict[tuple, native.StepRunner] = {}
 
     # --- embeddings ---------------------------------------------------------
     def set_embeddings(self, entity: str, side: Side, weights: nn.Parameter) -> None:
-        emb = SimpleEmbedding(weights)
+        emb = SimpleEmbedding(weights, max_norm=self.max_norm)
         side.pick(self.lhs_embs, self.rhs_embs)[self.EMB_PREFIX + entity] = emb
         self._runners.clear()
 
@@ -349,7 +347,8 @@ class MultiRelationEmbedder(nn.Module):
             operator=rhs_op.op_name if rhs_op is not None else "none", dynamic=dynamic,
             num_relations=self.num_dynamic_rels if dynamic else 1,
             comparator=self.comparator.comparator_name,
-            regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0, **training)
+            regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0,
+            max_norm=self.max_norm, **training)
 
     def operator_tensors(self, relation_idx: int):
         """({name: tensor} of the rhs operator, of the lhs operator) in the

@@ -54,6 +54,22 @@ def gather_rows(table: torch.Tensor, idx: torch.Tensor, check_bounds: bool = Tru
     return out.view(*idx.shape, table.shape[1])
 
 
+def embedding_renorm_(table: torch.Tensor, idx: torch.Tensor, max_norm: float) -> None:
+    """In the table: every row named in idx with a 2-norm above max_norm is
+    scaled to max_norm (torch.embedding_renorm_, the first half of
+    F.embedding(max_norm=...), model.py:61)."""
+    _need(table, torch.float32, "table")
+    _need(idx, torch.int64, "idx")
+    flat = idx.reshape(-1).contiguous()
+    n, dim = flat.shape[0], table.shape[1]
+    if n == 0:
+        return
+    nbytes = _lib.lib().pbg_embedding_renorm_workspace_bytes(n, dim)
+    ws = _workspace(nbytes, table.device)
+    check(_lib.lib().pbg_embedding_renorm(_ptr(table), table.shape[0], dim, _ptr(flat), n, float(max_norm), _ptr(ws),
+                                          nbytes, _stream()))
+
+
 def row_adagrad_sparse(weight: torch.Tensor, state_sum: torch.Tensor, idx: torch.Tensor,
                        grad_rows: torch.Tensor, lr: float, workspace: Optional[torch.Tensor] = None) -> None:
     _need(weight, torch.float32, "weight")
@@ -195,6 +211,7 @@ class StepSpec:
     lr: float = 0.1
     relation_lr: Optional[float] = None
     regularization_coef: float = 0.0  # config.regularization_coef of the N3 regularizer; 0 = none
+    max_norm: Optional[float] = None  # config.max_norm: looked-up rows are first renormalised in the table
 
     @property
     def chunk_size(self) -> int:
@@ -261,6 +278,7 @@ class StepRunner:
         d.num_lhs_rows = self.w_lhs.shape[0]
         d.num_rhs_rows = self.w_rhs.shape[0]
         d.regularization_coef = spec.regularization_coef
+        d.max_norm = float(spec.max_norm) if spec.max_norm else 0.0
         self.desc = d
         self.rhs_op = rhs_op or {}
         self.rhs_op_sum = rhs_op_sum or {}

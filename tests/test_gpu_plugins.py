@@ -131,6 +131,16 @@ def test_gather_and_sampling(pbg, golden):
     assert tuple(s.shape) == (2, 2, 3)
     empty = emb(pbg.entitylist.EntityList.from_tensor(torch.empty((0,), dtype=torch.long, device=DEV)))
     assert tuple(empty.shape) == (0, 3)
+    # max_norm (test/test_model.py:72-84,102-116): looked-up rows are renormalised in the table first
+    m = g["max_norm"]
+    w = torch.nn.Parameter(torch.tensor(g["table"], device=DEV))
+    emb = pbg.model.SimpleEmbedding(w, max_norm=m["max_norm"])
+    out = emb(pbg.entitylist.EntityList.from_tensor(torch.tensor(m["index"], device=DEV)))
+    assert close(out, m["expected"], golden["tolerance"])
+    assert torch.equal(w.data[1].cpu(), torch.tensor(g["table"][1]))
+    assert close(emb.get_all_entities(), m["all_entities_expected"], golden["tolerance"])
+    assert close(w.data, m["all_entities_expected"], golden["tolerance"])
+    assert float(emb.sample_entities(2, 2).detach().norm(dim=-1).max()) <= 2.0 * (1 + 1e-6)
 
 
 def build_model(pbg, cfg, st, n_rel_schemas):
@@ -163,7 +173,7 @@ def build_model(pbg, cfg, st, n_rel_schemas):
     model = M.MultiRelationEmbedder(
         cfg.dim, rels, ent, cfg.num_batch_negs, cfg.num_uniform_negs, cfg.disable_lhs_negs, cfg.disable_rhs_negs,
         lhs_ops, rhs_ops, M.COMPARATORS.get_class(cfg.comparator)(), regularizer=regularizer,
-        global_emb=cfg.global_emb, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
+        global_emb=cfg.global_emb, max_norm=cfg.max_norm, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
     if cfg.global_emb:
         model.global_embs.to(DEV)
         with torch.no_grad():
@@ -181,6 +191,9 @@ MODEL_CASES = [
     dict(operator="translation", comparator="l2", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=10, num_pos=33, dim=12),
     dict(operator="linear", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=0, num_uniform_negs=7, num_pos=30, dim=9),
+    # max_norm: about half of the rows (0.3 * randn, dim 16) are longer than 1.2
+    dict(operator="diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20, num_pos=40,
+         dim=16, max_norm=1.2),
     dict(operator="affine", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="affine", comparator="l2", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
     dict(operator="none", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),

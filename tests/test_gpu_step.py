@@ -51,7 +51,7 @@ def to_runner(pbg, cfg, st, num_pos, workers):
         num_uniform_negs=cfg.num_uniform_negs, disable_lhs_negs=cfg.disable_lhs_negs,
         disable_rhs_negs=cfg.disable_rhs_negs, operator=cfg.operator, dynamic=cfg.dynamic,
         num_relations=cfg.num_relations, comparator=cfg.comparator, loss=cfg.loss, margin=cfg.margin, lr=cfg.lr,
-        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef)
+        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm)
     dev = lambda t: t.clone().to(DEV)
     w_l, g_l = dev(st.w_lhs), dev(st.g_lhs)
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))
@@ -308,6 +308,60 @@ def test_train_step_with_global_embeddings(pbg, case, workers):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
     compare_state(cfg, runner, st, rtol, "step+global")
     assert not torch.equal(st.glob_lhs, zero_glob[0])  # it was trained
+
+
+MAX_NORM_CASES = [
+    # fused route, one table and two
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=200, dim=100),
+    dict(operator="translation", comparator="l2", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=100,
+         shared=False),
+    # staged route
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=100,
+         num_pos=130, dim=400),
+    dict(operator="linear", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=10,
+         num_pos=45, dim=24),
+    dict(operator="diagonal", comparator="squared_l2", loss="ranking", num_batch_negs=0, num_uniform_negs=7, num_pos=30,
+         dim=9, disable_lhs_negs=True, shared=False),
+    dict(operator="none", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
+         global_emb=True),
+]
+
+
+@pytest.mark.parametrize("case", MAX_NORM_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_max_norm(pbg, case, workers):
+    """config.max_norm (model.py:61,90-96): rows are looked up with
+    F.embedding(max_norm=...), which first scales, IN THE TABLE, every looked-up
+    row whose 2-norm exceeds max_norm; about half of the rows here do."""
+    say("train+max_norm", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", True)
+    scale = 0.1
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, max_norm=scale * dim ** 0.5, **case)
+    n_ent = max(300, num_pos * (40 if cfg.comparator == "l2" else 6))
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=shared, scale=scale)
+    before = st.w_lhs.clone()
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    # the forward alone renormalises too, as the reference's does
+    got = runner.forward(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    for k, b in enumerate(batches):
+        want, _ = ostep.forward_backward(cfg, st, *b, keep_scores=True)
+        compare_scores(cfg, tuple(t[k] for t in got), want.scores)
+    touched = torch.cat([b[0] for b in batches])
+    norms = runner.w_lhs[touched.to(DEV)].norm(dim=1).cpu()
+    assert float(norms.max()) <= cfg.max_norm * (1 + 1e-6)
+    assert int((before[touched].norm(dim=1) > cfg.max_norm).sum()) > 0  # some rows were too long
+    assert_close(runner.w_lhs, st.w_lhs, 1e-6, "renormalised table")
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, batches)
+    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+    compare_state(cfg, runner, st, rtol, "step+max_norm")
 
 
 def test_global_embeddings_are_refused_for_dynamic_relations(pbg):

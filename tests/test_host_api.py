@@ -217,9 +217,12 @@ def test_model_argument_errors(pbg):
     ent = {"e": C.EntitySchema()}
     mk = lambda **kw: M.MultiRelationEmbedder(4, rel, ent, 2, 2, False, False, [None],
                                               [pbg.operators.TranslationOperator(4)], M.DotComparator(), **kw)
-    for kw in (dict(max_norm=1.0), dict(half_precision=True), dict(regularizer=object())):
+    for kw in (dict(half_precision=True), dict(regularizer=object())):
         with pytest.raises(NotImplementedError):
             mk(**kw)
+    capped = mk(max_norm=1.0)  # model.py:443-451: handed on to every embedding module
+    capped.set_embeddings("e", pbg.types.Side.LHS, torch.nn.Parameter(torch.zeros(5, 4)))
+    assert capped.lhs_embs["emb_e"].max_norm == 1.0 and capped.step_spec(0, 3, 4).max_norm == 1.0
     with_global = mk(global_emb=True)  # model.py:433-439: a zero vector per entity type
     assert list(with_global.global_embs) == ["emb_e"] and float(with_global.global_embs["emb_e"].abs().sum()) == 0.0
     assert mk().global_embs is None

@@ -75,6 +75,24 @@ def test_gather(golden):
     assert torch.equal(w.detach()[idx], torch.tensor(g["sample_expected"]))
 
 
+def test_gather_max_norm(golden):
+    """The oracle's lookup with max_norm (F.embedding(max_norm=...) inside
+    step.forward_backward) against the reference's vectors: the looked-up rows
+    come back renormalised and the table keeps them."""
+    g, m = golden["gather"], golden["gather"]["max_norm"]
+    tol = golden["tolerance"]
+    cfg = step.StepConfig(dim=3, num_batch_negs=3, num_uniform_negs=0, max_norm=m["max_norm"], lr=0.0)
+    st = step.make_state(cfg, torch.tensor(g["table"]))
+    idx = torch.tensor(m["index"])
+    step.forward_backward(cfg, st, idx, idx, 0, None, None)
+    assert close(st.w_lhs[idx], m["expected"], tol)
+    assert close(st.w_lhs[1], g["table"][1], 0.0)  # not looked up: left alone
+    st = step.make_state(cfg, torch.tensor(g["table"]))
+    every = torch.arange(3)
+    step.forward_backward(cfg, st, every, every, 0, None, None)
+    assert close(st.w_lhs, m["all_entities_expected"], tol)
+
+
 def test_operator_errors():
     with pytest.raises(ValueError):
         step.init_operator_params("complex_diagonal", 3, 1)
