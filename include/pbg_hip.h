@@ -145,6 +145,10 @@ typedef struct pbg_step_desc {
   float max_norm;           /* > 0: F.embedding(max_norm=...) (model.py:61,90-96): the rows a call looks up are
                              * first renormalised IN THE TABLE to at most this 2-norm (pbg_model_forward
                              * included, as in the reference); 0 = off */
+  int32_t bias;             /* config.bias: BiasedComparator around `comparator` (model.py:306-344,902-903): a
+                             * row's first coordinate stays out of the comparator and is added to its scores.
+                             * Not implemented for l2 or with a regularizer (PBG_ERR_UNSUPPORTED) */
+  int32_t reserved0;        /* keep 0 */
 } pbg_step_desc;
 
 typedef struct pbg_step_buffers {

@@ -40,13 +40,17 @@ def _op(name: str, x: np.ndarray, params: Optional[Dict[str, np.ndarray]], r: in
     raise NotImplementedError(name)
 
 
-def _prep(comparator: str, x: np.ndarray) -> np.ndarray:
+def _prep(comparator: str, x: np.ndarray, bias: bool = False) -> np.ndarray:
+    if bias:  # the first coordinate is the row's bias and stays as it is (model.py:311-314)
+        return np.concatenate([x[:1], _prep(comparator, x[1:])])
     if comparator == "cos":
         return x / math.sqrt(float(x @ x))
     return x
 
 
-def _kappa(comparator: str, a: np.ndarray, b: np.ndarray) -> float:
+def _kappa(comparator: str, a: np.ndarray, b: np.ndarray, bias: bool = False) -> float:
+    if bias:  # score of the remaining coordinates plus both rows' biases (model.py:328-342)
+        return _kappa(comparator, a[1:], b[1:]) + float(a[0]) + float(b[0])
     if comparator in ("dot", "cos"):
         return float(a @ b)
     if comparator == "l2":
@@ -76,20 +80,21 @@ def scores(cfg, w_lhs, w_rhs, lhs, rhs, rel, uniform_lhs, uniform_rhs, lhs_op, r
     lneg = np.zeros((num_pos, n_l))
     rneg = np.zeros((num_pos, n_r))
     cmp_ = cfg.comparator
+    bias = bool(getattr(cfg, "bias", False))
     name = cfg.operator
     for e in range(num_pos):
         c, i = divmod(e, chunk)
         r = int(rel) if np.ndim(rel) == 0 else int(rel[e])
         u_raw, v_raw = w_lhs[lhs[e]], w_rhs[rhs[e]]
         if not cfg.dynamic:
-            a_for_rneg = _prep(cmp_, u_raw)                      # f(u)
-            a_for_lneg = _prep(cmp_, _op(name, v_raw, rhs_op, r))  # f(op_r(v))
-            lpos[e] = rpos[e] = _kappa(cmp_, a_for_rneg, a_for_lneg)
+            a_for_rneg = _prep(cmp_, u_raw, bias)                      # f(u)
+            a_for_lneg = _prep(cmp_, _op(name, v_raw, rhs_op, r), bias)  # f(op_r(v))
+            lpos[e] = rpos[e] = _kappa(cmp_, a_for_rneg, a_for_lneg, bias)
         else:
-            a_for_lneg = _prep(cmp_, _op(name, v_raw, rhs_op, r))  # f(op^rhs_r(v))
-            a_for_rneg = _prep(cmp_, _op(name, u_raw, lhs_op, r))  # f(op^lhs_r(u))
-            lpos[e] = _kappa(cmp_, _prep(cmp_, u_raw), a_for_lneg)
-            rpos[e] = _kappa(cmp_, _prep(cmp_, v_raw), a_for_rneg)
+            a_for_lneg = _prep(cmp_, _op(name, v_raw, rhs_op, r), bias)  # f(op^rhs_r(v))
+            a_for_rneg = _prep(cmp_, _op(name, u_raw, lhs_op, r), bias)  # f(op^lhs_r(u))
+            lpos[e] = _kappa(cmp_, _prep(cmp_, u_raw, bias), a_for_lneg, bias)
+            rpos[e] = _kappa(cmp_, _prep(cmp_, v_raw, bias), a_for_rneg, bias)
         for side, n_cols, out, a_vec in (("l", n_l, lneg, a_for_lneg), ("r", n_r, rneg, a_for_rneg)):
             if n_cols == 0:
                 continue
@@ -102,11 +107,11 @@ def scores(cfg, w_lhs, w_rhs, lhs, rhs, rel, uniform_lhs, uniform_rhs, lhs_op, r
                 if other >= num_pos or j == i:
                     out[e, j] = -1e9
                     continue
-                b_vec = _prep(cmp_, _op(name, table[ids[other]], neg_op, r))
-                out[e, j] = _kappa(cmp_, a_vec, b_vec)
+                b_vec = _prep(cmp_, _op(name, table[ids[other]], neg_op, r), bias)
+                out[e, j] = _kappa(cmp_, a_vec, b_vec, bias)
             for j in range(n_uni):
-                b_vec = _prep(cmp_, _op(name, table[uni[c][j]], neg_op, r))
-                out[e, n_batch + j] = _kappa(cmp_, a_vec, b_vec)
+                b_vec = _prep(cmp_, _op(name, table[uni[c][j]], neg_op, r), bias)
+                out[e, n_batch + j] = _kappa(cmp_, a_vec, b_vec, bias)
     return lpos, rpos, lneg, rneg
 
 

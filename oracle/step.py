@@ -47,6 +47,9 @@ class StepConfig:
     # config.py:173-180: rows are looked up with F.embedding(max_norm=...), which first
     # renormalises them in the table (model.py:61); None = off
     max_norm: Optional[float] = None
+    # config.py:197-207: the first coordinate of every embedding is a bias: it is kept out of
+    # the comparator and added to the score (BiasedComparator, model.py:306-344,902-903)
+    bias: bool = False
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
@@ -137,6 +140,11 @@ def comparator_prepare(name: str, embs: torch.Tensor) -> torch.Tensor:
     raise NotImplementedError(f"Unknown comparator {name}")
 
 
+def biased_prepare(name: str, embs: torch.Tensor) -> torch.Tensor:
+    """BiasedComparator.prepare (model.py:311-314)."""
+    return torch.cat([embs[..., :1], comparator_prepare(name, embs[..., 1:])], dim=-1)
+
+
 def _f32(x: torch.Tensor) -> torch.Tensor:
     """The reference's ``.float()`` casts (model.py:177,268,827-829); float64
     inputs are let through so that tests can take finite differences."""
@@ -190,6 +198,18 @@ def comparator_scores(
         rneg = _all_pairs_squared_l2(lhs_pos, rhs_neg).neg()
         return pos, lneg, rneg
     raise NotImplementedError(f"Unknown comparator {name}")
+
+
+def biased_scores(name, lhs_pos, rhs_pos, lhs_neg, rhs_neg):
+    """BiasedComparator.forward (model.py:316-344): the base comparator on the
+    coordinates after the first, plus the biases of the two rows of a pair."""
+    pos, lneg, rneg = comparator_scores(name, lhs_pos[..., 1:], rhs_pos[..., 1:], lhs_neg[..., 1:], rhs_neg[..., 1:])
+    lhs_pos_bias = lhs_pos[..., 0]
+    rhs_pos_bias = rhs_pos[..., 0]
+    pos = pos + lhs_pos_bias + rhs_pos_bias
+    lneg = lneg + rhs_pos_bias.unsqueeze(-1) + lhs_neg[..., 0].unsqueeze(-2)
+    rneg = rneg + lhs_pos_bias.unsqueeze(-1) + rhs_neg[..., 0].unsqueeze(-2)
+    return pos, lneg, rneg
 
 
 # --------------------------------------------------------------------------
@@ -315,7 +335,7 @@ def _adjust(cfg: StepConfig, embs, rel, op_params, glob=None) -> torch.Tensor:
         embs = embs + glob
     if op_params is not None:
         embs = apply_operator(cfg.operator, embs, op_params, rel)
-    return comparator_prepare(cfg.comparator, embs)
+    return (biased_prepare if cfg.bias else comparator_prepare)(cfg.comparator, embs)
 
 
 def _direction_agnostic(
@@ -369,7 +389,7 @@ def _direction_agnostic(
     src_neg, src_masked = negatives(src_pos, src_uniform, src_method, None, src_glob)
     dst_neg, dst_masked = negatives(dst_pos, dst_uniform, dst_method, dst_op_params, dst_glob)
 
-    pos_scores, src_neg_scores, dst_neg_scores = comparator_scores(
+    pos_scores, src_neg_scores, dst_neg_scores = (biased_scores if cfg.bias else comparator_scores)(
         cfg.comparator, src_pos, dst_pos, src_neg, dst_neg
     )
     pos_scores = _f32(pos_scores)

@@ -45,6 +45,8 @@ class StepDesc(ctypes.Structure):
         ("num_rhs_rows", c_int64),
         ("regularization_coef", c_float),
         ("max_norm", c_float),
+        ("bias", c_int32),
+        ("reserved0", c_int32),
     ]
 
 

@@ -44,6 +44,8 @@ struct SideCtx {
   int alias;            // positives are the first P rows of the negatives matrix
   float *xn, *xp, *xa;  // prepared negatives matrix, positives, operated positives (dynamic)
   float *an, *ap, *aa;  // per-row aux of the above: 1/norm (cos) or squared norm (l2)
+  float *bn, *bp, *ba;  // with config.bias: the rows' biases (their first coordinates; the rows hold 0 there)
+  float* bs;            // with config.bias: [K*C*P] row sums of dLoss/dscore of this side's score matrix
   float *dxn, *dxp, *dxa;
   float* s;             // [K*C, P, nn] scores against this side's negatives, then dLoss/dS
   float* rs;            // [K*C*P] row sums of dLoss/d(squared distance) (l2)
@@ -62,6 +64,7 @@ struct SideCtx {
 
 struct StepCtx {
   int D, K, B, P, C, U, last, dynamic, op, cmp, loss, num_relations;
+  int bias;    // config.bias: BiasedComparator around the comparator (model.py:306-344,902-903)
   int affine;  // op == PBG_OP_LINEAR with a translation added to the product (operators.py:103-115, 272-293)
   float margin;
   SideCtx side[2];
@@ -97,6 +100,22 @@ __device__ __forceinline__ RowV<NVH> gathered_row(const SideCtx& sd, int64_t id,
   RowV<NVH> x = row_load<NVH>(sd.w + id * D, D, H, lane);
   if (sd.glob) row_axpy<NVH>(x, 1.0f, row_load<NVH>(sd.glob, D, H, lane));
   return x;
+}
+
+// BiasedComparator.prepare (model.py:311-314) keeps a row's first coordinate, its
+// bias, out of the comparator.  Here the bias is set aside and the row carries 0
+// in its place, so every product, norm and distance that follows runs over the
+// other coordinates only; the scores get the two biases of a pair added where
+// they are read (ScoreRow::at, positive_scores).  Element 0 of a row is lane 0's.
+template <int NVH>
+__device__ __forceinline__ float take_bias(RowV<NVH>& y, int lane) {
+  const float b = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(y.a[0][0])));
+  if (lane == 0) y.a[0][0] = 0.f;
+  return b;
+}
+template <int NVH>
+__device__ __forceinline__ void add_to_first(RowV<NVH>& y, float v, int lane) {
+  if (lane == 0) y.a[0][0] += v;
 }
 
 // ---------------------------------------------------------------------------
@@ -184,12 +203,16 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     float* ap = sd.ap ? sd.ap + kc * sd.stride_p + i : nullptr;
     float* xa_row = c.dynamic ? sd.xa + (kc * c.P + i) * D : nullptr;
     float* aa = (c.dynamic && sd.aa) ? sd.aa + kc * c.P + i : nullptr;
+    float* bp = c.bias ? sd.bp + kc * sd.stride_p + i : nullptr;
+    float* ba = (c.bias && c.dynamic) ? sd.ba + kc * c.P + i : nullptr;
     if (r >= c.B) {  // padding of an incomplete last chunk (model.py:790-798)
       const RowV<NVH> zero = row_zero<NVH>();
       row_store<NVH>(xp_row, zero, D, H, lane);
       if (ap && lane == 0) *ap = 0.f;
+      if (bp && lane == 0) *bp = 0.f;
       if (xa_row) row_store<NVH>(xa_row, zero, D, H, lane);
       if (aa && lane == 0) *aa = 0.f;
+      if (ba && lane == 0) *ba = 0.f;
       return;
     }
     const int64_t e = (int64_t)k * c.B + r;
@@ -203,19 +226,24 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     }
     if (c.dynamic || !sd.has_op) {
       RowV<NVH> y = x;
+      const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
       const float aux = prepare_row<NVH>(c.cmp, y);
       row_store<NVH>(xp_row, y, D, H, lane);
       if (ap && lane == 0) *ap = aux;
+      if (bp && lane == 0) *bp = b;
     }
     if (sd.has_op) {
       if (c.op == PBG_OP_LINEAR) {
         row_store<NVH>(sd.xraw + ((int64_t)k * sd.op_rows + r) * D, x, D, H, lane);
       } else {
         RowV<NVH> y = op_forward<NVH>(c.op, x, sd.p0, sd.p1, rel, D, H, lane);
+        const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
         const float aux = prepare_row<NVH>(c.cmp, y);
         row_store<NVH>(c.dynamic ? xa_row : xp_row, y, D, H, lane);
         float* auxdst = c.dynamic ? aa : ap;
         if (auxdst && lane == 0) *auxdst = aux;
+        float* bdst = c.dynamic ? ba : bp;
+        if (bdst && lane == 0) *bdst = b;
       }
     }
   } else {
@@ -238,9 +266,11 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
       const int64_t rel = clamp_index(c.rel[k], c.num_relations);
       y = op_forward<NVH>(c.op, x, sd.p0, sd.p1, rel, D, H, lane);
     }
+    const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
     const float aux = prepare_row<NVH>(c.cmp, y);
     row_store<NVH>(sd.xn + (kc * sd.nn + sd.nb + uu) * D, y, D, H, lane);
     if (sd.an && lane == 0) sd.an[kc * sd.nn + sd.nb + uu] = aux;
+    if (c.bias && lane == 0) sd.bn[kc * sd.nn + sd.nb + uu] = b;
   }
 }
 
@@ -259,6 +289,7 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
     const int64_t rel = clamp_index((c.dynamic && r < c.B) ? c.rel[(int64_t)k * c.B + r] : c.rel[k], c.num_relations);
     y = op_forward<NVH>(PBG_OP_TRANSLATION, y, sd.p1, nullptr, rel, D, H, lane);
   }
+  const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
   const float aux = prepare_row<NVH>(c.cmp, y);
   if (r < c.B) {
     const int cc = r / c.P, i = r % c.P;
@@ -266,9 +297,11 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
     if (c.dynamic) {
       row_store<NVH>(sd.xa + (kc * c.P + i) * D, y, D, H, lane);
       if (sd.aa && lane == 0) sd.aa[kc * c.P + i] = aux;
+      if (c.bias && lane == 0) sd.ba[kc * c.P + i] = b;
     } else {
       row_store<NVH>(sd.xp + (kc * sd.stride_p + i) * D, y, D, H, lane);
       if (sd.ap && lane == 0) sd.ap[kc * sd.stride_p + i] = aux;
+      if (c.bias && lane == 0) sd.bp[kc * sd.stride_p + i] = b;
     }
   } else {
     const int r2 = r - c.B;
@@ -276,6 +309,7 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
     const int64_t kc = (int64_t)k * c.C + cc;
     row_store<NVH>(sd.xn + (kc * sd.nn + sd.nb + uu) * D, y, D, H, lane);
     if (sd.an && lane == 0) sd.an[kc * sd.nn + sd.nb + uu] = aux;
+    if (c.bias && lane == 0) sd.bn[kc * sd.nn + sd.nb + uu] = b;
   }
 }
 
@@ -305,6 +339,8 @@ struct ScoreRow {
   const float* raw;  // chunk score row, a.b for every comparator
   const float* bn;   // squared norms of the negatives (l2)
   float a2;          // squared norm of the positive operand (l2)
+  const float* cb;   // biases of the negatives (config.bias), or null
+  float rb;          // bias of the positive operand
   int cmp, nb, i, masked_from;  // batch-negative columns; own column; first padded column
 
   // score of column j as the model returns it (model.py:234-246,836-839); `live`
@@ -319,6 +355,7 @@ struct ScoreRow {
     } else if (cmp == PBG_CMP_SQUARED_L2) {
       t = -(fmaf(-2.0f, t, bn[j]) + a2);
     }
+    if (cb) t += rb + cb[j];  // model.py:338-342
     if (j < nb && (j == i || j >= masked_from)) {
       t = -1e9f;
       ok = false;
@@ -346,6 +383,16 @@ __device__ __forceinline__ void positive_scores(const StepCtx& c, int64_t kc, in
     posv[0] = kappa(c.cmp, lp, c.side[1].xa + (kc * c.P + i) * D, D, lane);
     posv[1] = kappa(c.cmp, rp, c.side[0].xa + (kc * c.P + i) * D, D, lane);
   }
+  if (c.bias) {  // model.py:332-336: both rows' biases
+    const float bl = c.side[0].bp[kc * c.side[0].stride_p + i], br = c.side[1].bp[kc * c.side[1].stride_p + i];
+    if (!c.dynamic) {
+      posv[0] += bl + br;
+      posv[1] = posv[0];
+    } else {
+      posv[0] += bl + c.side[1].ba[kc * c.P + i];
+      posv[1] += br + c.side[0].ba[kc * c.P + i];
+    }
+  }
 }
 
 __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t kc, int cc, int i) {
@@ -359,6 +406,12 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   if (is_distance(c.cmp)) {
     sr.bn = sd.an + kc * sd.nn;
     sr.a2 = c.dynamic ? so.aa[kc * c.P + i] : so.ap[kc * so.stride_p + i];
+  }
+  sr.cb = nullptr;
+  sr.rb = 0.f;
+  if (c.bias) {
+    sr.cb = sd.bn + kc * sd.nn;
+    sr.rb = c.dynamic ? so.ba[kc * c.P + i] : so.bp[kc * so.stride_p + i];
   }
   sr.nb = sd.nb;
   sr.i = i;
@@ -375,8 +428,9 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
 template <class R>
 __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
                                           float pos, float w, int first, float* loss_acc, float* dpos_out,
-                                          int* viol_out, float* rowsum_out) {
+                                          int* viol_out, float* rowsum_out, float* gsum_out) {
   float dpos_part = 0.f, rowsum = 0.f;
+  float gsum = 0.f;  // row sum of dLoss/dscore: the gradient of the positive operand's bias (config.bias)
   int viol = 0;
   float mx = pos, inv_z = 0.f;
   const float inv_nn = 1.0f / (float)nn;
@@ -427,6 +481,7 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
         float g = expf(t - mx) * inv_z * w;
         if (t > pos) ++viol;
         if (!live_u) g = 0.f;
+        gsum += g;
         if (is_distance(cmp)) {
           const float dq = !live_u ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / t : -g);
           rowsum += dq;
@@ -437,6 +492,7 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
       }
       *dpos_out = R::sum(dpos_part);
       *rowsum_out = R::sum(rowsum);
+      *gsum_out = R::sum(gsum);
       *viol_out = R::sum_int(viol);
       return;
     }
@@ -465,6 +521,7 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
     }
     if (t > pos) ++viol;
     if (!live) g = 0.f;
+    gsum += g;
     if (is_distance(cmp)) {
       // t = -sqrt(q): dLoss/dq = g * 0.5 / t (squared_l2, t = -q: -g); stored as
       // -2 dLoss/dq so that the backward GEMMs produce the cross terms of
@@ -478,6 +535,7 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
   }
   *dpos_out = R::sum(dpos_part);
   *rowsum_out = R::sum(rowsum);
+  *gsum_out = R::sum(gsum);
   *viol_out = R::sum_int(viol);
 }
 
@@ -495,6 +553,7 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
       float* row = sd.s + (kc * c.P + i) * sd.nn;
       for (int j = lane; j < sd.nn; j += kWave) row[j] = 0.f;
       if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = 0.f;
+      if (sd.bs && lane == 0) sd.bs[kc * c.P + i] = 0.f;
     }
     if (lane == 0) {
       c.lossrow[job] = 0.f;
@@ -530,9 +589,11 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     }
     ScoreRow sr = score_row(c, s, kc, cc, i);
     float* out = sd.s + (kc * c.P + i) * nn;
-    float rowsum;
-    side_loss<WaveReduce>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum);
+    float rowsum, gsum;
+    side_loss<WaveReduce>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum,
+                          &gsum);
     if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = rowsum;
+    if (sd.bs && lane == 0) sd.bs[kc * c.P + i] = gsum;
   }
   const float loss_row = wave_sum(loss_acc) * w;
   if (lane == 0) {
@@ -682,6 +743,11 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
   const int D = c.D, H = (D + 1) / 2;
   const bool l2 = is_distance(c.cmp);
   const bool keep_dz = sd.dz != nullptr;
+  // config.bias: a row's bias enters every score of the row (model.py:332-342), so its gradient is
+  // the sum of dLoss/dscore over them: a row sum where the row is the positive operand, a column sum
+  // where it is a negative, plus the positive pair's.  It joins the gradient after comparator.prepare,
+  // which passes the first coordinate through.  (squared_l2 stores 2 dLoss/dscore in the matrix.)
+  const float stored = c.cmp == PBG_CMP_SQUARED_L2 ? 0.5f : 1.0f;
 
   if (r < c.B) {
     const int cc = r / c.P, i = r % c.P;
@@ -707,7 +773,13 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
         const float cubes = wave_sum(n3_term<NVH>(c.op, c.reg_coef, dy, y1));
         if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
       }
-      const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
+      RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
+      if (c.bias) {
+        float db = c.dpos[0][pq];
+        if (sd.nb > 0) db += stored * column_sum(sd.s, kc, c.P, sd.nn, i, lane);
+        if (so.nn > 0) db += so.bs[kc * c.P + i];
+        add_to_first<NVH>(dz, db, lane);
+      }
       if (sd.has_op) {
         if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz, D, H, lane);
         if (c.op != PBG_OP_LINEAR)
@@ -730,6 +802,11 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       float cubes = 0.f;
       if (c.reg_coef != 0.f) cubes = n3_term<NVH>(c.op, c.reg_coef, dy, y1);
       RowV<NVH> dx = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
+      if (c.bias) {
+        float db = c.dpos[s][pq];
+        if (sd.alias) db += stored * column_sum(sd.s, kc, c.P, sd.nn, i, lane);
+        add_to_first<NVH>(dx, db, lane);
+      }
       // role 2: the operated row f(op(x)), scored against the other side's negatives
       const RowV<NVH> y2 = row_load<NVH>(sd.xa + (kc * c.P + i) * D, D, H, lane);
       const float aux2 = sd.aa ? sd.aa[kc * c.P + i] : 0.f;
@@ -744,7 +821,8 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
         cubes = wave_sum(cubes + n3_term<NVH>(c.op, c.reg_coef, dy2, y2));
         if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
       }
-      const RowV<NVH> dz2 = prepare_backward<NVH>(c.cmp, dy2, y2, aux2);
+      RowV<NVH> dz2 = prepare_backward<NVH>(c.cmp, dy2, y2, aux2);
+      if (c.bias) add_to_first<NVH>(dz2, c.dpos[1 - s][pq] + (sd.opd_written ? so.bs[kc * c.P + i] : 0.f), lane);
       if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz2, D, H, lane);
       if (c.op != PBG_OP_LINEAR) {
         const RowV<NVH> dx2 = op_backward<NVH>(c.op, dz2, sd.p0, sd.p1, rel, D, H, lane);
@@ -762,7 +840,8 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
     const RowV<NVH> y = c.cmp != PBG_CMP_DOT ? row_load<NVH>(sd.xn + (kc * sd.nn + col) * D, D, H, lane) : row_zero<NVH>();
     RowV<NVH> dy = row_load<NVH>(sd.dxn + (kc * sd.nn + col) * D, D, H, lane);
     if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, col, lane), y);
-    const RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y, sd.an ? sd.an[kc * sd.nn + col] : 0.f);
+    RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y, sd.an ? sd.an[kc * sd.nn + col] : 0.f);
+    if (c.bias) add_to_first<NVH>(dz, stored * column_sum(sd.s, kc, c.P, sd.nn, col, lane), lane);
     if (sd.op_uniform) {
       const int64_t rel = clamp_index(c.rel[k], c.num_relations);
       if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D, dz, D, H, lane);
@@ -1916,6 +1995,13 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->regularization_coef != 0.f && (d->op == PBG_OP_LINEAR || d->op == PBG_OP_AFFINE))
     return fail(PBG_ERR_UNSUPPORTED, "Regularizer not implemented for this operator");  // operators.py:40,188
   if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
+  if (d->bias) {
+    if (d->dim < 2) return fail(PBG_ERR_INVALID, "step: bias needs at least two coordinates");
+    // -sqrt(q) stores dLoss/dq in the score matrix, from which the sums of dLoss/dscore cannot be read back
+    if (d->comparator == PBG_CMP_L2) return fail(PBG_ERR_UNSUPPORTED, "step: bias is not implemented for the l2 comparator");
+    // (the regularizer would need the bias coordinate of the prepared rows, which is kept aside)
+    if (d->regularization_coef != 0.f) return fail(PBG_ERR_UNSUPPORTED, "step: bias is not implemented with a regularizer");
+  }
   return PBG_OK;
 }
 
@@ -1943,6 +2029,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.dynamic = d->dynamic;
   c.op = d->op == PBG_OP_AFFINE ? PBG_OP_LINEAR : d->op;
   c.affine = d->op == PBG_OP_AFFINE;
+  c.bias = d->bias != 0;
   c.cmp = d->comparator;
   c.loss = d->loss;
   c.margin = d->margin;
@@ -1988,20 +2075,27 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
       if (need_aux) sd.an = takef(KC * sd.nn);
       sd.s = takef(KC * P * sd.nn);
       if (is_distance(c.cmp)) sd.rs = takef(KC * P);
+      if (c.bias) {
+        sd.bn = takef(KC * sd.nn);
+        sd.bs = takef(KC * P);
+      }
     }
     if (sd.alias) {
       sd.xp = sd.xn;
       sd.dxp = sd.dxn;
       sd.ap = sd.an;
+      sd.bp = sd.bn;
     } else {
       sd.xp = takef(KC * P * D);
       sd.dxp = takef(KC * P * D);
       if (need_aux) sd.ap = takef(KC * P);
+      if (c.bias) sd.bp = takef(KC * P);
     }
     if (c.dynamic) {
       sd.xa = takef(KC * P * D);
       sd.dxa = takef(KC * P * D);
       if (need_aux) sd.aa = takef(KC * P);
+      if (c.bias) sd.ba = takef(KC * P);
     }
     // which gradient buffers a GEMM fills (see run_backward)
     sd.plain_written = sd.alias || (!c.dynamic && (s == 0 ? (d->disable_rhs_negs == 0) : (d->disable_lhs_negs == 0)));
@@ -2081,7 +2175,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->bytes = off;
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
   // (the regularizer's terms live in the staged kernels only)
-  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && getenv("PBG_DISABLE_FUSED") == nullptr;
+  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && getenv("PBG_DISABLE_FUSED") == nullptr;
 
   if (b) {
     c.side[0].w = b->w_lhs;

@@ -16,7 +16,7 @@ training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
 Not provided (outside the accelerated path): FeaturizedEmbedding,
-BiasedComparator, all_negs, half precision.
+all_negs, half precision.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -207,6 +207,38 @@ class SquaredL2Comparator(AbstractComparator):
     comparator_name = "squared_l2"
 
 
+class BiasedComparator(AbstractComparator):
+    """config.bias (model.py:306-344,902-903): the first coordinate of every
+    embedding is a bias -- it stays out of the wrapped comparator and is added
+    to the scores of its row.  Inside the training step the same thing is the
+    ``bias`` field of the step description."""
+
+    def __init__(self, base_comparator: AbstractComparator):
+        super().__init__()
+        self.base_comparator = base_comparator
+
+    @property
+    def comparator_name(self) -> str:
+        return self.base_comparator.comparator_name
+
+    def prepare(self, embs: FloatTensorType) -> FloatTensorType:
+        return torch.cat([embs[..., :1], self.base_comparator.prepare(embs[..., 1:])], dim=-1)
+
+    def forward(self, lhs_pos, rhs_pos, lhs_neg, rhs_neg) -> Tuple[FloatTensorType, FloatTensorType, FloatTensorType]:
+        num_chunks, num_pos_per_chunk, dim = match_shape(lhs_pos, -1, -1, -1)
+        match_shape(rhs_pos, num_chunks, num_pos_per_chunk, dim)
+        match_shape(lhs_neg, num_chunks, -1, dim)
+        match_shape(rhs_neg, num_chunks, -1, dim)
+        pos_scores, lhs_neg_scores, rhs_neg_scores = self.base_comparator(
+            lhs_pos[..., 1:], rhs_pos[..., 1:], lhs_neg[..., 1:], rhs_neg[..., 1:])
+        lhs_pos_bias = lhs_pos[..., 0]
+        rhs_pos_bias = rhs_pos[..., 0]
+        pos_scores = pos_scores + lhs_pos_bias + rhs_pos_bias
+        lhs_neg_scores = lhs_neg_scores + rhs_pos_bias.unsqueeze(-1) + lhs_neg[..., 0].unsqueeze(-2)
+        rhs_neg_scores = rhs_neg_scores + lhs_pos_bias.unsqueeze(-1) + rhs_neg[..., 0].unsqueeze(-2)
+        return pos_scores, lhs_neg_scores, rhs_neg_scores
+
+
 # ---------------------------------------------------------------------------
 def ceil_of_ratio(num: int, den: int) -> int:
     return (num - 1) // den + 1
@@ -348,7 +380,7 @@ class MultiRelationEmbedder(nn.Module):
             num_relations=self.num_dynamic_rels if dynamic else 1,
             comparator=self.comparator.comparator_name,
             regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0,
-            max_norm=self.max_norm, **training)
+            max_norm=self.max_norm, bias=isinstance(self.comparator, BiasedComparator), **training)
 
     def operator_tensors(self, relation_idx: int):
         """({name: tensor} of the rhs operator, of the lhs operator) in the

@@ -212,6 +212,7 @@ class StepSpec:
     relation_lr: Optional[float] = None
     regularization_coef: float = 0.0  # config.regularization_coef of the N3 regularizer; 0 = none
     max_norm: Optional[float] = None  # config.max_norm: looked-up rows are first renormalised in the table
+    bias: bool = False  # config.bias: BiasedComparator around the comparator (not with l2 or a regularizer)
 
     @property
     def chunk_size(self) -> int:
@@ -279,6 +280,7 @@ class StepRunner:
         d.num_rhs_rows = self.w_rhs.shape[0]
         d.regularization_coef = spec.regularization_coef
         d.max_norm = float(spec.max_norm) if spec.max_norm else 0.0
+        d.bias = int(bool(spec.bias))
         self.desc = d
         self.rhs_op = rhs_op or {}
         self.rhs_op_sum = rhs_op_sum or {}

@@ -26,7 +26,7 @@ def test_struct_sizes_match_the_header(pbg):
     import ctypes
 
     # 15 x 4-byte fields + one 4-byte field, then two int64: 16 * 4 + 16
-    assert ctypes.sizeof(pbg._lib.StepDesc) == 88
+    assert ctypes.sizeof(pbg._lib.StepDesc) == 96
     # 22 pointers + workspace_bytes, then sample_uniform (4 + 4 padding) and uniform_seed
     assert ctypes.sizeof(pbg._lib.StepBuffers) == 30 * 8
     lib = pbg._lib.lib()

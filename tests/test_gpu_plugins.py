@@ -94,6 +94,28 @@ def test_comparator_forward_backward_vs_oracle(pbg, name, shape):
         assert torch.allclose(got.grad.cpu(), want.grad, rtol=1e-4, atol=2e-5 * max(scale, 1.0)), name
 
 
+@pytest.mark.parametrize("name", ["dot", "cos", "squared_l2"])
+def test_biased_comparator_forward_backward_vs_oracle(pbg, name):
+    """BiasedComparator (model.py:306-344) around the package's comparators against
+    the oracle's restatement, values and gradients."""
+    say("biased comparator", name)
+    c, p, ln, rn, d = 3, 5, 7, 4, 6
+    g = torch.Generator().manual_seed(11)
+    raw = [torch.randn(c, n, d, generator=g) for n in (p, p, ln, rn)]
+    weights = [torch.randn(c, p, generator=g), torch.randn(c, p, ln, generator=g), torch.randn(c, p, rn, generator=g)]
+    cmp_ = pbg.model.BiasedComparator(pbg.model.COMPARATORS.get_class(name)())
+    ts = [t.clone().to(DEV).requires_grad_(True) for t in raw]
+    outs = cmp_(*[cmp_.prepare(t) for t in ts])
+    sum((o * w.to(DEV)).sum() for o, w in zip(outs, weights)).backward()
+    to = [t.clone().requires_grad_(True) for t in raw]
+    oo = ostep.biased_scores(name, *[ostep.biased_prepare(name, t) for t in to])
+    sum((o * w).sum() for o, w in zip(oo, weights)).backward()
+    for got, want in zip(outs, oo):
+        assert torch.allclose(got.detach().cpu(), want.detach(), rtol=1e-5, atol=1e-5 * d ** 0.5)
+    for got, want in zip(ts, to):
+        assert torch.allclose(got.grad.cpu(), want.grad, rtol=1e-4, atol=2e-5 * max(want.grad.abs().max().item(), 1.0)), name
+
+
 def test_reference_loss_vectors(pbg, golden):
     tol = golden["tolerance"]
     for case in golden["losses"]:
@@ -170,9 +192,12 @@ def build_model(pbg, cfg, st, n_rel_schemas):
     regularizer = None
     if cfg.regularization_coef != 0:  # model.py:905-909
         regularizer = pbg.regularizers.REGULARIZERS.get_class("N3")(cfg.regularization_coef)
+    comparator = M.COMPARATORS.get_class(cfg.comparator)()
+    if cfg.bias:  # model.py:902-903
+        comparator = M.BiasedComparator(comparator)
     model = M.MultiRelationEmbedder(
         cfg.dim, rels, ent, cfg.num_batch_negs, cfg.num_uniform_negs, cfg.disable_lhs_negs, cfg.disable_rhs_negs,
-        lhs_ops, rhs_ops, M.COMPARATORS.get_class(cfg.comparator)(), regularizer=regularizer,
+        lhs_ops, rhs_ops, comparator, regularizer=regularizer,
         global_emb=cfg.global_emb, max_norm=cfg.max_norm, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
     if cfg.global_emb:
         model.global_embs.to(DEV)
@@ -191,6 +216,13 @@ MODEL_CASES = [
     dict(operator="translation", comparator="l2", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=10, num_pos=33, dim=12),
     dict(operator="linear", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=0, num_uniform_negs=7, num_pos=30, dim=9),
+    # config.bias: BiasedComparator around the comparator
+    dict(operator="diagonal", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=20, num_pos=40,
+         dim=16, bias=True),
+    # (with one relation per edge the operated row's bias shifts every score of its row alike: under softmax the
+    # operator's first element has a zero gradient, rounding noise for Adagrad -- logistic here)
+    dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25,
+         dim=9, bias=True),
     # max_norm: about half of the rows (0.3 * randn, dim 16) are longer than 1.2
     dict(operator="diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20, num_pos=40,
          dim=16, max_norm=1.2),

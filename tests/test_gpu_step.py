@@ -51,7 +51,7 @@ def to_runner(pbg, cfg, st, num_pos, workers):
         num_uniform_negs=cfg.num_uniform_negs, disable_lhs_negs=cfg.disable_lhs_negs,
         disable_rhs_negs=cfg.disable_rhs_negs, operator=cfg.operator, dynamic=cfg.dynamic,
         num_relations=cfg.num_relations, comparator=cfg.comparator, loss=cfg.loss, margin=cfg.margin, lr=cfg.lr,
-        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm)
+        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm, bias=cfg.bias)
     dev = lambda t: t.clone().to(DEV)
     w_l, g_l = dev(st.w_lhs), dev(st.g_lhs)
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))
@@ -362,6 +362,77 @@ def test_train_step_with_max_norm(pbg, case, workers):
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
     compare_state(cfg, runner, st, rtol, "step+max_norm")
+
+
+# (A translation moves the bias of every row of its side by the same amount, which ranking and softmax do
+# not see: its first element then has a zero gradient, rounding noise that Adagrad would turn into full
+# steps -- in the reference too.  Translations are paired with the logistic loss here.)
+BIAS_CASES = [
+    # shapes the fused kernel would take without the bias
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=100),
+    dict(operator="translation", comparator="squared_l2", loss="logistic", num_batch_negs=20, num_uniform_negs=10, num_pos=45,
+         dim=32),
+    dict(operator="diagonal", comparator="squared_l2", loss="softmax", num_batch_negs=20, num_uniform_negs=10, num_pos=45,
+         dim=32),
+    dict(operator="diagonal", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
+         shared=False),
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=100,
+         num_pos=130, dim=400),
+    dict(operator="linear", comparator="cos", loss="ranking", num_batch_negs=10, num_uniform_negs=10, num_pos=45, dim=24),
+    dict(operator="affine", comparator="dot", loss="logistic", num_batch_negs=8, num_uniform_negs=0, num_pos=30, dim=12),
+    dict(operator="diagonal", comparator="squared_l2", loss="ranking", num_batch_negs=0, num_uniform_negs=7, num_pos=30,
+         dim=9, disable_lhs_negs=True),
+    dict(operator="none", comparator="dot", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
+         global_emb=True),  # (a global embedding's first element is such a common shift too)
+    # one relation per edge
+    dict(operator="translation", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=5,
+         num_pos=33, dim=16),
+    dict(operator="diagonal", comparator="dot", loss="ranking", dynamic=True, num_batch_negs=10, num_uniform_negs=5,
+         num_pos=33, dim=16),
+    dict(operator="complex_diagonal", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=20, num_uniform_negs=10,
+         num_pos=70, dim=32),
+    dict(operator="linear", comparator="squared_l2", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=10,
+         num_pos=45, dim=24),
+    dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=8, num_uniform_negs=4,
+         num_pos=30, dim=9, disable_rhs_negs=True),
+    dict(operator="affine", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=6,
+         num_pos=21, dim=10),
+]
+
+
+@pytest.mark.parametrize("case", BIAS_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_bias(pbg, case, workers):
+    """config.bias (BiasedComparator, model.py:306-344): a row's first coordinate
+    stays out of the comparator and is added to every score of the row."""
+    say("train+bias", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", True)
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, bias=True, **case)
+    st, batches = make_inputs(cfg, num_pos, max(200, num_pos * 4), workers, seed=num_pos + dim, shared=shared)
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    assert not runner.fused
+    got = runner.forward(*pack(cfg, batches))
+    for k, b in enumerate(batches):
+        want, _ = ostep.forward_backward(cfg, st, *b, keep_scores=True)
+        compare_scores(cfg, tuple(t[k] for t in got), want.scores)
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, batches)
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=1e-5, abs=1e-6), ("loss", k)
+    compare_state(cfg, runner, st, 1e-5, "step+bias")
+
+
+def test_bias_is_refused_where_it_is_not_implemented(pbg):
+    w = torch.randn(20, 8, device=DEV)
+    for kw in (dict(comparator="l2"), dict(regularization_coef=0.1, operator="diagonal")):
+        spec = pbg.StepSpec(dim=8, batch_size=10, bias=True, **kw)
+        op = {"diagonal": torch.ones(1, 8, device=DEV)} if "operator" in kw else {}
+        with pytest.raises(NotImplementedError, match="bias is not implemented"):
+            pbg.StepRunner(spec, w, torch.zeros(20, device=DEV), rhs_op=op, rhs_op_sum={k: torch.zeros_like(v) for k, v in op.items()})
 
 
 def test_global_embeddings_are_refused_for_dynamic_relations(pbg):

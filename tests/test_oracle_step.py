@@ -52,6 +52,10 @@ CASES += [
     dict(operator="linear", comparator="cos", dynamic=False, num_batch_negs=3, num_uniform_negs=2, num_pos=7,
          shared=False),
 ]
+# config.bias (BiasedComparator, model.py:306-344) around every comparator, standard and dynamic
+for cmp_, dyn in itertools.product(step.COMPARATOR_NAMES, (False, True)):
+    CASES.append(dict(operator="diagonal" if dyn else "translation", comparator=cmp_, dynamic=dyn, num_batch_negs=4,
+                      num_uniform_negs=3, num_pos=10, bias=True))
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(str(v) for v in c.values()))
@@ -85,6 +89,44 @@ def test_forward_matches_brute_force(case):
             got = float(step.loss_value(name, pos, neg, None, margin=0.1))
             want = brute.loss(name, pos.double().numpy(), neg.double().numpy(), 0.1)
             assert got == pytest.approx(want, rel=1e-5, abs=1e-5)
+
+
+@pytest.mark.parametrize("comparator", step.COMPARATOR_NAMES)
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_bias_reduces_to_the_base_comparator_and_shifts_scores(comparator, dynamic):
+    """What the definition of BiasedComparator fixes (model.py:306-344), without
+    the brute force: (1) with a zero first coordinate everywhere, and an operator
+    that keeps it zero, the scores are the base comparator's on the remaining
+    D - 1 coordinates -- which the reference's own vectors pin; (2) adding c to
+    every row's first coordinate adds 2c to every score that is not masked."""
+    kw = dict(operator="diagonal", comparator=comparator, dynamic=dynamic, num_batch_negs=4, num_uniform_negs=3,
+              num_relations=3, relation_weights=[1.0, 1.0, 1.0])
+    cfg_b = step.StepConfig(dim=6, bias=True, **kw)
+    cfg_0 = step.StepConfig(dim=5, **kw)
+    st, lhs, rhs, rel, ul, ur = make_case(cfg_b, 10, 11, seed=5)
+    st.w_lhs[:, 0] = 0.0
+    st.w_rhs[:, 0] = 0.0
+    s_b = run_forward(cfg_b, st, lhs, rhs, rel, ul, ur)
+    st0 = step.make_state(cfg_0, st.w_lhs[:, 1:].clone(), None if st.shared else st.w_rhs[:, 1:].clone())
+    st0.lhs_op = {k: v[:, 1:].clone() for k, v in st.lhs_op.items()}
+    st0.rhs_op = {k: v[:, 1:].clone() for k, v in st.rhs_op.items()}
+    s_0 = run_forward(cfg_0, st0, lhs, rhs, rel, ul, ur)
+    for a, b in zip((s_b.lhs_pos, s_b.rhs_pos, s_b.lhs_neg, s_b.rhs_neg), (s_0.lhs_pos, s_0.rhs_pos, s_0.lhs_neg, s_0.rhs_neg)):
+        assert torch.allclose(a, b, rtol=1e-6, atol=1e-6)
+    # (2): the diagonal operator scales the first coordinate of the operated rows; with 1 there the shift is c + c
+    for d in (st.lhs_op, st.rhs_op):
+        for v in d.values():
+            v[:, 0] = 1.0
+    base = run_forward(cfg_b, st, lhs, rhs, rel, ul, ur)
+    st.w_lhs[:, 0] += 0.25
+    if not st.shared:
+        st.w_rhs[:, 0] += 0.25
+    moved = run_forward(cfg_b, st, lhs, rhs, rel, ul, ur)
+    for a, b in zip((base.lhs_pos, base.rhs_pos, base.lhs_neg, base.rhs_neg),
+                    (moved.lhs_pos, moved.rhs_pos, moved.lhs_neg, moved.rhs_neg)):
+        live = a != -1e9
+        assert torch.equal(b == -1e9, ~live)
+        assert torch.allclose(b[live], a[live] + 0.5, rtol=1e-5, atol=1e-5)
 
 
 def test_invariants_single_chunk_no_uniform():
