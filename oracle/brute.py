@@ -75,6 +75,9 @@ def scores(cfg, w_lhs, w_rhs, lhs, rhs, rel, uniform_lhs, uniform_rhs, lhs_op, r
     n_uni = cfg.num_uniform_negs
     n_l = 0 if cfg.disable_lhs_negs else n_batch + n_uni
     n_r = 0 if cfg.disable_rhs_negs else n_batch + n_uni
+    if mode == "all":  # every entity of the side's type, the edge's own entity masked (model.py:582-618)
+        n_l = 0 if cfg.disable_lhs_negs else len(w_lhs)
+        n_r = 0 if cfg.disable_rhs_negs else len(w_rhs)
     lpos = np.zeros(num_pos)
     rpos = np.zeros(num_pos)
     lneg = np.zeros((num_pos, n_l))
@@ -109,6 +112,13 @@ def scores(cfg, w_lhs, w_rhs, lhs, rhs, rel, uniform_lhs, uniform_rhs, lhs_op, r
                     continue
                 b_vec = _prep(cmp_, _op(name, table[ids[other]], neg_op, r), bias)
                 out[e, j] = _kappa(cmp_, a_vec, b_vec, bias)
+            if mode == "all":
+                for j in range(n_cols):
+                    if j == ids[e]:
+                        out[e, j] = -1e9
+                        continue
+                    out[e, j] = _kappa(cmp_, a_vec, _prep(cmp_, _op(name, table[j], neg_op, r), bias), bias)
+                continue
             for j in range(n_uni):
                 b_vec = _prep(cmp_, _op(name, table[uni[c][j]], neg_op, r), bias)
                 out[e, n_batch + j] = _kappa(cmp_, a_vec, b_vec, bias)

@@ -50,9 +50,14 @@ class StepConfig:
     # config.py:197-207: the first coordinate of every embedding is a bias: it is kept out of
     # the comparator and added to the score (BiasedComparator, model.py:306-344,902-903)
     bias: bool = False
+    # RelationSchema.all_negs (config.py:123-131): the negatives of an edge are ALL entities of the
+    # side's type, in one chunk (model.py:648-650,582-618)
+    all_negs: bool = False
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
+        if self.all_negs:
+            return num_pos, (1 if num_pos > 0 else 0), "all"
         if self.num_batch_negs == 0:
             chunk = min(self.num_uniform_negs, num_pos)
             mode = "uniform"
@@ -352,9 +357,13 @@ def _direction_agnostic(
     dst_method: str,
     src_glob=None,
     dst_glob=None,
+    src_ids=None,
+    dst_ids=None,
 ):
     """model.py:764-856.  ``src_uniform`` / ``dst_uniform`` are the raw rows
-    of the uniformly sampled entities, [C,U,D] (model.py:544,550)."""
+    of the uniformly sampled entities, [C,U,D] (model.py:544,550); in mode
+    "all" they are the side's whole table as [1,E,D] and ``src_ids`` /
+    ``dst_ids`` the positives' entities, whose own columns are masked."""
     dim = src_pos.shape[-1]
     src_pos = _adjust(cfg, src_pos, rel, None, src_glob)
     dst_pos = _adjust(cfg, dst_pos, rel, dst_op_params, dst_glob)
@@ -379,6 +388,8 @@ def _direction_agnostic(
             if uniform is not None and uniform.shape[1] > 0:
                 neg = torch.cat([pos_embs, _adjust(cfg, uniform, rel_for_uniform, op_params, glob)], dim=1)
             masked_batch = True
+        elif method == "all":  # model.py:582-618: get_all_entities().expand(num_chunks, -1, dim)
+            neg = _adjust(cfg, uniform.expand(num_chunks, -1, dim), rel_for_uniform, op_params, glob)
         else:
             raise NotImplementedError(method)
         return neg, masked_batch
@@ -402,6 +413,9 @@ def _direction_agnostic(
             scores[: num_chunks - 1, idx, idx] = -1e9
             scores[-1, idx[:last], idx[:last]] = -1e9
             scores[-1, :last, last:chunk_size] = -1e9
+    for scores, method, ids in ((src_neg_scores, src_method, src_ids), (dst_neg_scores, dst_method, dst_ids)):
+        if method == "all":  # model.py:596-618: ignore_mask[i, pos_input[i]] (one chunk of num_pos rows)
+            scores[0, torch.arange(num_pos), ids] = -1e9
 
     pos_scores = pos_scores.flatten(0, 1)[:num_pos]
     src_neg_scores = src_neg_scores.flatten(0, 1)[:num_pos]
@@ -423,11 +437,15 @@ def model_forward(
     rhs_op_params: Optional[Dict[str, torch.Tensor]],
     glob_lhs: Optional[torch.Tensor] = None,
     glob_rhs: Optional[torch.Tensor] = None,
+    lhs_ids: Optional[torch.Tensor] = None,
+    rhs_ids: Optional[torch.Tensor] = None,
 ) -> Scores:
     """MultiRelationEmbedder.forward (model.py:624-762) on already gathered
     rows.  lhs_pos/rhs_pos: [B,D] raw rows; *_uniform: [C,U,D] raw rows of the
     uniform negatives (None when U == 0 or the side is disabled); rel: int in
-    standard mode, LongTensor[B] in dynamic mode."""
+    standard mode, LongTensor[B] in dynamic mode.  With cfg.all_negs the
+    *_uniform are the whole tables as [1,E,D] and lhs_ids / rhs_ids the edges'
+    entities."""
     num_pos = lhs_pos.shape[0]
     chunk_size, _, mode = cfg.chunking(num_pos)
     lhs_method = "none" if cfg.disable_lhs_negs else mode
@@ -442,7 +460,7 @@ def model_forward(
         pos, lneg, rneg, reg = _direction_agnostic(
             cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, rhs_uniform, rel,
             rhs_op_params if cfg.operator != "none" else None,
-            chunk_size, lhs_method, rhs_method, glob_lhs, glob_rhs,
+            chunk_size, lhs_method, rhs_method, glob_lhs, glob_rhs, lhs_ids, rhs_ids,
         )
         return Scores(pos, pos, lneg, rneg, reg)
     if isinstance(rel, int):
@@ -454,12 +472,12 @@ def model_forward(
     lpos, lneg, _, l_reg = _direction_agnostic(
         cfg, num_pos, lhs_pos, rhs_pos, lhs_uniform, None, rel,
         rhs_op_params if cfg.operator != "none" else None,
-        chunk_size, lhs_method, "none",
+        chunk_size, lhs_method, "none", src_ids=lhs_ids,
     )
     rpos, rneg, _, r_reg = _direction_agnostic(
         cfg, num_pos, rhs_pos, lhs_pos, rhs_uniform, None, rel,
         lhs_op_params if cfg.operator != "none" else None,
-        chunk_size, rhs_method, "none",
+        chunk_size, rhs_method, "none", src_ids=rhs_ids,
     )
     reg = None if l_reg is None or r_reg is None else l_reg + r_reg  # model.py:755-758
     return Scores(lpos, rpos, lneg, rneg, reg)
@@ -610,11 +628,17 @@ def forward_backward(
         if uniform_rhs is not None and not cfg.disable_rhs_negs and uniform_rhs.numel() > 0
         else None
     )
+    if cfg.all_negs:  # module.get_all_entities() (model.py:66-68,584): every row, looked up like the others
+        lhs_u = None if cfg.disable_lhs_negs else F.embedding(
+            torch.arange(w_l.shape[0]).unsqueeze(0), w_l, max_norm=cfg.max_norm, sparse=True)
+        rhs_u = None if cfg.disable_rhs_negs else F.embedding(
+            torch.arange(w_r.shape[0]).unsqueeze(0), w_r, max_norm=cfg.max_norm, sparse=True)
     glob_l = glob_r = None
     if st.glob_lhs is not None:
         glob_l = st.glob_lhs.detach().requires_grad_(True)
         glob_r = glob_l if st.glob_rhs is st.glob_lhs else st.glob_rhs.detach().requires_grad_(True)
-    scores = model_forward(cfg, lhs_pos, rhs_pos, lhs_u, rhs_u, rel, lhs_op or None, rhs_op or None, glob_l, glob_r)
+    scores = model_forward(cfg, lhs_pos, rhs_pos, lhs_u, rhs_u, rel, lhs_op or None, rhs_op or None, glob_l, glob_r,
+                           lhs, rhs)
 
     # batching.py:139-150
     lhs_loss = loss_value(cfg.loss, scores.lhs_pos, scores.lhs_neg, weight, cfg.margin)

@@ -46,7 +46,7 @@ class StepDesc(ctypes.Structure):
         ("regularization_coef", c_float),
         ("max_norm", c_float),
         ("bias", c_int32),
-        ("reserved0", c_int32),
+        ("all_negs", c_int32),
     ]
 
 

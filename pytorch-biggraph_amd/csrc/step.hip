@@ -39,6 +39,7 @@ struct SideCtx {
   uint64_t useed;       // seed of the in-step draw (uidx == null)
   int64_t key_base;     // offset of this table in the sort-key row space
   int64_t num_rows;
+  int all;              // RelationSchema.all_negs: the negatives are the table's rows 0 .. num_rows - 1 (u == num_rows)
   int nb, u, nn;        // batch-negative / uniform / total negative columns of this side
   int stride_p;         // rows per chunk of the buffer that holds the positives
   int alias;            // positives are the first P rows of the negatives matrix
@@ -90,6 +91,7 @@ struct StepCtx {
 // Uniform negative number flat = (k * C + chunk) * U + u of side s: given by the
 // caller or drawn here (model.py:70-75).
 __device__ __forceinline__ int64_t uniform_negative(const SideCtx& sd, int s, int64_t flat) {
+  if (sd.all) return flat % sd.u;  // (one chunk: flat = batch * u + entity)
   if (sd.uidx) return sd.uidx[flat];
   return sampled_row(sd.useed, (uint64_t)flat, (uint32_t)s, sd.num_rows);
 }
@@ -137,7 +139,7 @@ __device__ __forceinline__ const SideCtx& slot_row(const StepCtx& c, int k, int 
     *id = clamp_index(sd.idx[(int64_t)k * c.B + r], sd.num_rows);
   } else {
     const int r2 = r - c.B;
-    *id = clamp_index(uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u), sd.num_rows);
+    *id = clamp_index(uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * sd.u + r2 % sd.u), sd.num_rows);
   }
   return sd;
 }
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     const int r2 = r - CP;
     const int cc = r2 / sd.u, uu = r2 % sd.u;
     const int64_t kc = (int64_t)k * c.C + cc;
-    const int64_t id = clamp_index(uniform_negative(sd, s, kc * c.U + uu), sd.num_rows);
+    const int64_t id = clamp_index(uniform_negative(sd, s, kc * sd.u + uu), sd.num_rows);
     const RowV<NVH> x = gathered_row<NVH>(sd, id, D, H, lane);
     if (lane == 0) {
       const int64_t slot = (int64_t)k * c.rk + sd.slot_uni + r2;
@@ -341,6 +343,7 @@ struct ScoreRow {
   float a2;          // squared norm of the positive operand (l2)
   const float* cb;   // biases of the negatives (config.bias), or null
   float rb;          // bias of the positive operand
+  int64_t own;       // all_negs: the column of the edge's own entity on this side (masked, model.py:596-618); else -1
   int cmp, nb, i, masked_from;  // batch-negative columns; own column; first padded column
 
   // score of column j as the model returns it (model.py:234-246,836-839); `live`
@@ -356,7 +359,7 @@ struct ScoreRow {
       t = -(fmaf(-2.0f, t, bn[j]) + a2);
     }
     if (cb) t += rb + cb[j];  // model.py:338-342
-    if (j < nb && (j == i || j >= masked_from)) {
+    if ((j < nb && (j == i || j >= masked_from)) || j == own) {
       t = -1e9f;
       ok = false;
     }
@@ -406,6 +409,11 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   if (is_distance(c.cmp)) {
     sr.bn = sd.an + kc * sd.nn;
     sr.a2 = c.dynamic ? so.aa[kc * c.P + i] : so.ap[kc * so.stride_p + i];
+  }
+  sr.own = -1;
+  if (sd.all) {
+    const int64_t e = (kc / c.C) * c.B + (int64_t)cc * c.P + i;
+    sr.own = clamp_index(sd.idx[e], sd.num_rows);
   }
   sr.cb = nullptr;
   sr.rb = 0.f;
@@ -881,7 +889,7 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
         id = sd.idx[(int64_t)k * c.B + r];
       } else {
         const int r2 = r - c.B;
-        id = uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * c.U + r2 % sd.u);
+        id = uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * sd.u + r2 % sd.u);
       }
       const float* x = sd.w + clamp_index(id, sd.num_rows) * D;
       const float* gl = sd.glob;  // the operator's input is the row plus the global embedding
@@ -1983,8 +1991,11 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->num_workers < 1 || d->num_workers > 256) return fail(PBG_ERR_INVALID, "step: num_workers must be in [1, 256]");
   if (d->batch_size < 1) return fail(PBG_ERR_INVALID, "step: batch_size must be positive");
   if (d->num_batch_negs < 0 || d->num_uniform_negs < 0) return fail(PBG_ERR_INVALID, "step: negative negatives count");
-  if (d->num_batch_negs == 0 && d->num_uniform_negs == 0)
+  if (d->num_batch_negs == 0 && d->num_uniform_negs == 0 && !d->all_negs)
     return fail(PBG_ERR_INVALID, "step: num_batch_negs and num_uniform_negs cannot both be 0");
+  if (d->all_negs && (d->num_lhs_rows > (1 << 24) || d->num_rhs_rows > (1 << 24) ||
+                      (int64_t)d->batch_size * (d->num_lhs_rows > d->num_rhs_rows ? d->num_lhs_rows : d->num_rhs_rows) > ((int64_t)1 << 31)))
+    return fail(PBG_ERR_UNSUPPORTED, "step: all_negs needs batch_size x entities of a type within 2^31 scores");
   if (d->op < PBG_OP_NONE || d->op > PBG_OP_AFFINE) return fail(PBG_ERR_INVALID, "step: unknown operator %d", d->op);
   if (d->comparator < PBG_CMP_DOT || d->comparator > PBG_CMP_SQUARED_L2) return fail(PBG_ERR_INVALID, "step: unknown comparator %d", d->comparator);
   if (d->loss < PBG_LOSS_RANKING || d->loss > PBG_LOSS_SOFTMAX) return fail(PBG_ERR_INVALID, "step: unknown loss %d", d->loss);
@@ -2022,8 +2033,11 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.K = d->num_workers;
   c.B = d->batch_size;
   c.U = d->num_uniform_negs;
-  const bool batch_mode = d->num_batch_negs > 0;
+  // all_negs (model.py:648-650,582-618): one chunk of all the positives, every entity of a side's type as negative
+  const bool all_negs = d->all_negs != 0;
+  const bool batch_mode = d->num_batch_negs > 0 && !all_negs;
   c.P = batch_mode ? (d->num_batch_negs < c.B ? d->num_batch_negs : c.B) : (c.U < c.B ? c.U : c.B);
+  if (all_negs) c.P = c.B;
   c.C = (c.B - 1) / c.P + 1;
   c.last = c.B - (c.C - 1) * c.P;
   c.dynamic = d->dynamic;
@@ -2043,11 +2057,12 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     SideCtx& sd = c.side[s];
     const bool enabled = s == 0 ? !d->disable_lhs_negs : !d->disable_rhs_negs;
     sd.nb = (enabled && batch_mode) ? P : 0;
-    sd.u = enabled ? c.U : 0;
+    sd.num_rows = s == 0 ? d->num_lhs_rows : d->num_rhs_rows;
+    sd.all = all_negs;
+    sd.u = enabled ? (all_negs ? (int)sd.num_rows : c.U) : 0;
     sd.nn = sd.nb + sd.u;
     sd.alias = sd.nb > 0;
     sd.stride_p = sd.alias ? sd.nn : P;
-    sd.num_rows = s == 0 ? d->num_lhs_rows : d->num_rhs_rows;
     sd.key_base = (s == 1 && !d->shared_table) ? d->num_lhs_rows : 0;
     sd.slot_pos = slot;
     slot += c.B;
@@ -2213,7 +2228,9 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
     return fail(PBG_ERR_INVALID, "step: w_lhs == w_rhs needs shared_table = 1");
   if ((uintptr_t)b->w_lhs % 16 != 0 || (uintptr_t)b->w_rhs % 16 != 0)
     return fail(PBG_ERR_INVALID, "step: tables must be 16-byte aligned");
-  if (!b->sample_uniform) {
+  if (d->all_negs) {
+    // the negatives are the tables' rows in order: nothing to pass and nothing to draw
+  } else if (!b->sample_uniform) {
     if (plan.c.side[0].u > 0 && !b->uniform_lhs) return fail(PBG_ERR_INVALID, "step: uniform_lhs is null");
     if (plan.c.side[1].u > 0 && !b->uniform_rhs) return fail(PBG_ERR_INVALID, "step: uniform_rhs is null");
   } else if (b->uniform_lhs || b->uniform_rhs) {

@@ -16,7 +16,7 @@ training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
 Not provided (outside the accelerated path): FeaturizedEmbedding,
-all_negs, half precision.
+half precision.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -289,8 +289,6 @@ class MultiRelationEmbedder(nn.Module):
             raise NotImplementedError("Half precision is not supported")
         if any(e.featurized for e in entities.values()):
             raise NotImplementedError("Featurized entities are not supported")
-        if any(r.all_negs for r in relations):
-            raise NotImplementedError("all_negs is not supported")
         self.default_dim = default_dim
         self.relations: List[RelationSchema] = relations
         self.entities: Dict[str, EntitySchema] = entities
@@ -380,7 +378,8 @@ class MultiRelationEmbedder(nn.Module):
             num_relations=self.num_dynamic_rels if dynamic else 1,
             comparator=self.comparator.comparator_name,
             regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0,
-            max_norm=self.max_norm, bias=isinstance(self.comparator, BiasedComparator), **training)
+            max_norm=self.max_norm, bias=isinstance(self.comparator, BiasedComparator),
+            all_negs=bool(self.relations[relation_idx].all_negs), **training)
 
     def operator_tensors(self, relation_idx: int):
         """({name: tensor} of the rhs operator, of the lhs operator) in the
@@ -431,7 +430,7 @@ class MultiRelationEmbedder(nn.Module):
         entity indices; drawn with torch.randint when omitted."""
         num_pos = len(edges)
         relation_idx, lhs_module, rhs_module = self.resolve(edges)
-        if self.num_batch_negs == 0 and self.num_uniform_negs == 0:
+        if self.num_batch_negs == 0 and self.num_uniform_negs == 0 and not self.relations[relation_idx].all_negs:
             raise ValueError("num_batch_negs and num_uniform_negs cannot both be 0")
         w_l, w_r = lhs_module.weight, rhs_module.weight
         dim = w_l.shape[1]
@@ -440,8 +439,8 @@ class MultiRelationEmbedder(nn.Module):
         if num_pos == 0:
             spec = self.step_spec(relation_idx, 1, dim)
             z = torch.empty((0,), dtype=torch.float32, device=dev)
-            return Scores(z, z.clone(), z.new_empty((0, spec.num_negs(self.disable_lhs_negs))),
-                          z.new_empty((0, spec.num_negs(self.disable_rhs_negs)))), None
+            return Scores(z, z.clone(), z.new_empty((0, spec.num_negs(self.disable_lhs_negs, w_l.shape[0]))),
+                          z.new_empty((0, spec.num_negs(self.disable_rhs_negs, w_r.shape[0])))), None
         spec = self.step_spec(relation_idx, num_pos, dim)
         key = ("fwd", relation_idx, num_pos, w_l.data_ptr(), w_r.data_ptr())
         runner = self._runners.get(key)

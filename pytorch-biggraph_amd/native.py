@@ -213,9 +213,13 @@ class StepSpec:
     regularization_coef: float = 0.0  # config.regularization_coef of the N3 regularizer; 0 = none
     max_norm: Optional[float] = None  # config.max_norm: looked-up rows are first renormalised in the table
     bias: bool = False  # config.bias: BiasedComparator around the comparator (not with l2 or a regularizer)
+    # RelationSchema.all_negs: one chunk, every entity of a side's type is a negative (model.py:648-650,582-618)
+    all_negs: bool = False
 
     @property
     def chunk_size(self) -> int:
+        if self.all_negs:
+            return self.batch_size
         if self.num_batch_negs > 0:
             return min(self.num_batch_negs, self.batch_size)
         return min(self.num_uniform_negs, self.batch_size)
@@ -224,9 +228,12 @@ class StepSpec:
     def num_chunks(self) -> int:
         return (self.batch_size - 1) // self.chunk_size + 1
 
-    def num_negs(self, side_disabled: bool) -> int:
+    def num_negs(self, side_disabled: bool, num_rows: int = 0) -> int:
+        """Negative columns of one side; with all_negs that is `num_rows`, the side's table size."""
         if side_disabled:
             return 0
+        if self.all_negs:
+            return num_rows
         return (self.chunk_size if self.num_batch_negs > 0 else 0) + self.num_uniform_negs
 
 
@@ -281,6 +288,7 @@ class StepRunner:
         d.regularization_coef = spec.regularization_coef
         d.max_norm = float(spec.max_norm) if spec.max_norm else 0.0
         d.bias = int(bool(spec.bias))
+        d.all_negs = int(bool(spec.all_negs))
         self.desc = d
         self.rhs_op = rhs_op or {}
         self.rhs_op_sum = rhs_op_sum or {}
@@ -324,7 +332,9 @@ class StepRunner:
             raise ValueError(f"lhs / rhs must hold num_workers * batch_size = {k * b} entries")
         if rel.numel() != (k * b if s.dynamic else k):
             raise ValueError("rel must hold one entry per edge (dynamic) or per batch (standard)")
-        c, u = s.num_chunks, s.num_uniform_negs
+        c, u = s.num_chunks, (0 if s.all_negs else s.num_uniform_negs)
+        if s.all_negs:
+            uniform_lhs = uniform_rhs = uniform_seed = None  # the negatives are the tables' rows in order
         if uniform_seed is not None and (uniform_lhs is not None or uniform_rhs is not None):
             raise ValueError("pass uniform negatives or a seed to draw them with, not both")
         for name, t, off in (("uniform_lhs", uniform_lhs, s.disable_lhs_negs), ("uniform_rhs", uniform_rhs, s.disable_rhs_negs)):
@@ -404,7 +414,8 @@ class StepRunner:
         k, b = s.num_workers, s.batch_size
         bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, None)
         dev = self.device
-        nl, nr = s.num_negs(s.disable_lhs_negs), s.num_negs(s.disable_rhs_negs)
+        nl = s.num_negs(s.disable_lhs_negs, self.w_lhs.shape[0])
+        nr = s.num_negs(s.disable_rhs_negs, self.w_rhs.shape[0])
         lhs_pos = torch.empty((k, b), dtype=torch.float32, device=dev)
         rhs_pos = torch.empty((k, b), dtype=torch.float32, device=dev)
         lhs_neg = torch.empty((k, b, nl), dtype=torch.float32, device=dev)

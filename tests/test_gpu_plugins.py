@@ -67,6 +67,19 @@ def test_reference_comparator_vectors(pbg, golden):
             assert (t.grad != 0).any()
 
 
+def test_reference_biased_comparator_vectors(pbg, golden):
+    tol = golden["tolerance"]
+    for case in golden["biased_comparators"]:
+        say("biased comparator", case["name"], case["ref"])
+        cmp_ = pbg.model.BiasedComparator(pbg.model.COMPARATORS.get_class(case["name"])())
+        ts = [torch.tensor(case[k], device=DEV, requires_grad=True) for k in ("lhs_pos", "rhs_pos", "lhs_neg", "rhs_neg")]
+        pos, lneg, rneg = cmp_(*[cmp_.prepare(t) for t in ts])
+        assert close(pos, case["pos"], tol) and close(lneg, case["lhs_neg_scores"], tol) and close(rneg, case["rhs_neg_scores"], tol)
+        (pos.sum() + lneg.sum() + rneg.sum()).backward()
+        for t in ts:
+            assert (t.grad != 0).any()
+
+
 @pytest.mark.parametrize("name", ["dot", "cos", "l2", "squared_l2"])
 @pytest.mark.parametrize("shape", [(3, 5, 7, 4, 6), (1, 50, 100, 100, 100), (2, 4, 0, 3, 8), (2, 100, 130, 70, 256)])
 def test_comparator_forward_backward_vs_oracle(pbg, name, shape):
@@ -172,7 +185,7 @@ def build_model(pbg, cfg, st, n_rel_schemas):
     w_r = w_l if st.shared else dev(st.w_rhs)
     ent = {"l": C.EntitySchema(), "r": C.EntitySchema()}
     rels = [C.RelationSchema(name=f"r{i}", lhs="l", rhs="l" if st.shared else "r", operator=cfg.operator,
-                             weight=cfg.relation_weights[i]) for i in range(n_rel_schemas)]
+                             weight=cfg.relation_weights[i], all_negs=cfg.all_negs) for i in range(n_rel_schemas)]
     if cfg.dynamic:
         lhs_ops = [O.instantiate_operator(cfg.operator, pbg.types.Side.LHS, cfg.num_relations, cfg.dim).to(DEV)]
         rhs_ops = [O.instantiate_operator(cfg.operator, pbg.types.Side.RHS, cfg.num_relations, cfg.dim).to(DEV)]
@@ -216,6 +229,11 @@ MODEL_CASES = [
     dict(operator="translation", comparator="l2", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=10, num_pos=33, dim=12),
     dict(operator="linear", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
     dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=0, num_uniform_negs=7, num_pos=30, dim=9),
+    # RelationSchema.all_negs: every entity of a side's type is a negative
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20,
+         num_pos=40, dim=16, all_negs=True),
+    dict(operator="diagonal", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=0, num_pos=25,
+         dim=9, all_negs=True),
     # config.bias: BiasedComparator around the comparator
     dict(operator="diagonal", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=10, num_uniform_negs=20, num_pos=40,
          dim=16, bias=True),

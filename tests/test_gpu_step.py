@@ -51,7 +51,7 @@ def to_runner(pbg, cfg, st, num_pos, workers):
         num_uniform_negs=cfg.num_uniform_negs, disable_lhs_negs=cfg.disable_lhs_negs,
         disable_rhs_negs=cfg.disable_rhs_negs, operator=cfg.operator, dynamic=cfg.dynamic,
         num_relations=cfg.num_relations, comparator=cfg.comparator, loss=cfg.loss, margin=cfg.margin, lr=cfg.lr,
-        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm, bias=cfg.bias)
+        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm, bias=cfg.bias, all_negs=cfg.all_negs)
     dev = lambda t: t.clone().to(DEV)
     w_l, g_l = dev(st.w_lhs), dev(st.g_lhs)
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))
@@ -424,6 +424,47 @@ def test_train_step_with_bias(pbg, case, workers):
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=1e-5, abs=1e-6), ("loss", k)
     compare_state(cfg, runner, st, 1e-5, "step+bias")
+
+
+ALL_NEGS_CASES = [
+    dict(operator="none", comparator="dot", loss="softmax", num_pos=64, dim=100),
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_pos=130, dim=64, shared=False),
+    dict(operator="translation", comparator="l2", loss="ranking", num_pos=45, dim=32),
+    dict(operator="diagonal", comparator="cos", loss="logistic", num_pos=33, dim=16, disable_lhs_negs=True, shared=False),
+    dict(operator="linear", comparator="squared_l2", loss="ranking", num_pos=30, dim=24),
+    dict(operator="diagonal", comparator="dot", loss="logistic", num_pos=40, dim=16, bias=True),
+    dict(operator="translation", comparator="dot", loss="softmax", num_pos=33, dim=16, dynamic=True, shared=False),
+    dict(operator="linear", comparator="cos", loss="ranking", num_pos=45, dim=24, dynamic=True),
+    dict(operator="none", comparator="cos", loss="logistic", num_pos=50, dim=16, global_emb=True, max_norm=1.1),
+]
+
+
+@pytest.mark.parametrize("case", ALL_NEGS_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_all_negs(pbg, case, workers):
+    """RelationSchema.all_negs (model.py:648-650,582-618): one chunk, every entity
+    of a side's type is a negative, the edge's own entity masked."""
+    say("train+all_negs", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", True)
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, all_negs=True, num_batch_negs=7, num_uniform_negs=0, **case)
+    n_ent = 150 if cfg.comparator != "l2" else 1500
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=shared)
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    got = runner.forward(*pack(cfg, batches))
+    assert got[2].shape[-1] == (0 if cfg.disable_lhs_negs else st.w_lhs.shape[0]) and got[3].shape[-1] == st.w_rhs.shape[0]
+    for k, b in enumerate(batches):
+        want, _ = ostep.forward_backward(cfg, st, *b, keep_scores=True)
+        compare_scores(cfg, tuple(t[k] for t in got), want.scores)
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, batches)
+    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+    compare_state(cfg, runner, st, rtol, "step+all_negs")
 
 
 def test_bias_is_refused_where_it_is_not_implemented(pbg):

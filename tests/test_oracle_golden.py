@@ -64,6 +64,21 @@ def test_losses(golden):
         loss.backward()
 
 
+def test_biased_comparators(golden):
+    """BiasedComparator (model.py:306-344) against the reference's own vectors."""
+    tol = golden["tolerance"]
+    for case in golden["biased_comparators"]:
+        ts = [torch.tensor(case[k], requires_grad=True) for k in ("lhs_pos", "rhs_pos", "lhs_neg", "rhs_neg")]
+        prep = [step.biased_prepare(case["name"], t) for t in ts]
+        pos, lneg, rneg = step.biased_scores(case["name"], *prep)
+        assert close(pos, case["pos"], tol), case["ref"]
+        assert close(lneg, case["lhs_neg_scores"], tol), case["ref"]
+        assert close(rneg, case["rhs_neg_scores"], tol), case["ref"]
+        (pos.sum() + lneg.sum() + rneg.sum()).backward()
+        for t in ts:
+            assert (t.grad != 0).any()
+
+
 def test_gather(golden):
     g = golden["gather"]
     w = torch.tensor(g["table"], requires_grad=True)

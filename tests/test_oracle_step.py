@@ -32,6 +32,10 @@ def make_case(cfg, num_pos, n_ent, seed, shared=True, scale=0.5):
 
 def run_forward(cfg, st, lhs, rhs, rel, ul, ur):
     lp, rp = st.w_lhs[lhs], st.w_rhs[rhs]
+    if cfg.all_negs:
+        lu = None if cfg.disable_lhs_negs else st.w_lhs.unsqueeze(0)
+        ru = None if cfg.disable_rhs_negs else st.w_rhs.unsqueeze(0)
+        return step.model_forward(cfg, lp, rp, lu, ru, rel, st.lhs_op or None, st.rhs_op or None, lhs_ids=lhs, rhs_ids=rhs)
     lu = st.w_lhs[ul] if (cfg.num_uniform_negs > 0 and not cfg.disable_lhs_negs) else None
     ru = st.w_rhs[ur] if (cfg.num_uniform_negs > 0 and not cfg.disable_rhs_negs) else None
     return step.model_forward(cfg, lp, rp, lu, ru, rel, st.lhs_op or None, st.rhs_op or None)
@@ -52,6 +56,12 @@ CASES += [
     dict(operator="linear", comparator="cos", dynamic=False, num_batch_negs=3, num_uniform_negs=2, num_pos=7,
          shared=False),
 ]
+# RelationSchema.all_negs (model.py:648-650,582-618), standard and dynamic, one table and two
+for cmp_, dyn, sh in itertools.product(("dot", "l2"), (False, True), (True, False)):
+    CASES.append(dict(operator="diagonal", comparator=cmp_, dynamic=dyn, num_batch_negs=4, num_uniform_negs=3, num_pos=10,
+                      all_negs=True, shared=sh))
+CASES.append(dict(operator="translation", comparator="cos", dynamic=False, num_batch_negs=0, num_uniform_negs=0, num_pos=7,
+                  all_negs=True, disable_lhs_negs=True))
 # config.bias (BiasedComparator, model.py:306-344) around every comparator, standard and dynamic
 for cmp_, dyn in itertools.product(step.COMPARATOR_NAMES, (False, True)):
     CASES.append(dict(operator="diagonal" if dyn else "translation", comparator=cmp_, dynamic=dyn, num_batch_negs=4,
@@ -127,6 +137,27 @@ def test_bias_reduces_to_the_base_comparator_and_shifts_scores(comparator, dynam
         live = a != -1e9
         assert torch.equal(b == -1e9, ~live)
         assert torch.allclose(b[live], a[live] + 0.5, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_all_negs_is_uniform_mode_over_every_entity_with_the_own_entity_masked(dynamic):
+    """all_negs reduces to a path the other tests pin: uniform-only negatives
+    (model.py:651-653) with U = E "samples" 0 .. E-1 in one chunk give the same
+    scores, except that all_negs masks column lhs[i] (rhs[i]) of row i."""
+    kw = dict(dim=6, operator="diagonal", comparator="cos", dynamic=dynamic, num_relations=3, relation_weights=[1.0] * 3)
+    n_ent, num_pos = 13, 9
+    cfg_all = step.StepConfig(all_negs=True, num_batch_negs=5, num_uniform_negs=2, **kw)
+    cfg_uni = step.StepConfig(num_batch_negs=0, num_uniform_negs=n_ent, **kw)  # chunk = min(U, B) = B: one chunk
+    st, lhs, rhs, rel, _, _ = make_case(cfg_all, num_pos, n_ent, seed=2)
+    every = torch.arange(n_ent).unsqueeze(0)
+    a = run_forward(cfg_all, st, lhs, rhs, rel, None, None)
+    u = run_forward(cfg_uni, st, lhs, rhs, rel, every, every)
+    assert torch.equal(a.lhs_pos, u.lhs_pos) and torch.equal(a.rhs_pos, u.rhs_pos)
+    for got, want, ids in ((a.lhs_neg, u.lhs_neg, lhs), (a.rhs_neg, u.rhs_neg, rhs)):
+        own = torch.zeros_like(got, dtype=torch.bool)
+        own[torch.arange(num_pos), ids] = True
+        assert torch.equal(got == -1e9, own)
+        assert torch.equal(got[~own], want[~own])
 
 
 def test_invariants_single_chunk_no_uniform():
