@@ -104,7 +104,20 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_multi_kernel(const fl
 //   row_update    a wave per few sorted positions; at each position that starts
 //                 a row it walks the row's runs (one gradient row each), the
 //                 keys of the next 64 positions held in registers.
+// In a single-worker call (kbits == 0: a row has ONE run, all its duplicates) most
+// runs are two or three positions long.  Sending those through tile_reduce costs
+// a read of every row of the run, a write of the sum and another read of it;
+// instead a run of at most kShort positions that lies inside one tile is left
+// alone by tile_reduce (and never concerns run_combine) and summed, in position
+// order, by the update kernel as it reads it, with the loads of the same phase.
+// (With several workers a row has a run per worker and the update kernels' loop
+// over them is latency bound: the extra loads cost more there than they save.)
 constexpr int kTile = 32;
+constexpr int kShort = 4;
+// [s, s + len) in sorted positions: summed by the update kernels themselves (single-worker calls)
+__device__ __forceinline__ bool folded_run(int64_t s, int64_t len) {
+  return len >= 2 && len <= kShort && (s / kTile) == ((s + len - 1) / kTile);
+}
 
 template <int NV, bool VEC>
 struct RowRegs {
@@ -138,6 +151,19 @@ struct RowRegs {
         } else {
           v[i] += p[e];
         }
+      }
+    }
+  }
+  // the same with the whole row switched off by `on` (the load is still an ordinary, hoistable one)
+  __device__ __forceinline__ void add_if(const float* __restrict__ p, int nv, int lane, bool on) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = i * kWave + lane;
+      if (VEC) {
+        const float4 x = (on && e < nv) ? reinterpret_cast<const float4*>(p)[e] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[i * W + 0] += x.x; v[i * W + 1] += x.y; v[i * W + 2] += x.z; v[i * W + 3] += x.w;
+      } else {
+        v[i] += (on && e < nv) ? p[e] : 0.f;
       }
     }
   }
@@ -186,7 +212,8 @@ __device__ __forceinline__ uint64_t lane_u64(uint64_t v, int l) {
 template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
-                                                                  float* __restrict__ grad_rows, int dim) {
+                                                                  float* __restrict__ grad_rows, int dim,
+                                                                  int leave_short) {
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
   const int64_t begin = tile * kTile;
@@ -200,11 +227,20 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
   const uint64_t prev = __shfl_up(key, 1, 64);
   const bool starts = (mine < end) && (lane == 0 || prev != key);
   uint64_t heads = __ballot(starts);  // bit l set: a piece starts at begin + l
+  // the keys next to the tile tell whether a piece at its edge is a whole run
+  const bool has_before = begin > 0, has_after = end < n;
+  const uint64_t key_before = (leave_short && has_before) ? keys[begin - 1] : 0ull;
+  const uint64_t key_after = (leave_short && has_after) ? keys[end] : 0ull;
   while (heads != 0ull) {
     const int a = __ffsll((unsigned long long)heads) - 1;
     heads &= heads - 1;
     const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
     if (b - a < 2) continue;
+    if (leave_short && b - a <= kShort) {  // a short run inside the tile is the update kernel's (folded_run)
+      const uint64_t kp = lane_u64(key, a);
+      const bool whole = (a > 0 || !has_before || key_before != kp) && (b < (int)(end - begin) || !has_after || key_after != kp);
+      if (whole) continue;
+    }
     RowRegs<NV, VEC> acc;
     float* head = grad_rows + (int64_t)lane_u32(val, a) * dim;
     acc.load(head, nv, lane);
@@ -323,7 +359,15 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     }
     w[r].load(wrow[r], nv, lane);
     gsum[r] = *gptr[r];
-    g[r].load(grad_rows + (int64_t)lane_u32(vv[r], 0) * dim, nv, lane);  // each run's sum sits in its first row
+    g[r].load(grad_rows + (int64_t)lane_u32(vv[r], 0) * dim, nv, lane);  // each run's sum sits in its first row ...
+    if (kbits == 0) {  // ... unless it is a short run left to this kernel (folded_run)
+      const uint64_t same = __ballot(i + lane < n && kk[r] == lane_u64(kk[r], 0));
+      const int run_len = ~same != 0ull ? __ffsll((unsigned long long)~same) - 1 : kWave;
+      const bool fold = folded_run(i, run_len);
+#pragma unroll
+      for (int t = 1; t < kShort; ++t)
+        g[r].add_if(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane, fold && t < run_len);
+    }
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -390,6 +434,9 @@ __device__ __forceinline__ int64_t lower_bound_key(const uint64_t* __restrict__ 
 __device__ __forceinline__ float4 load_or_zero(const float* __restrict__ p, bool has) {
   return has ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
 }
+__device__ __forceinline__ void add4(float4& a, const float4& b) {
+  a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+}
 __device__ __forceinline__ float adagrad_apply_half(float4& w, const float4& g, float gsum, float fdim, float lr) {
   gsum += half_sum(g.x * g.x + g.y * g.y + g.z * g.z + g.w * g.w) / fdim;
   const float stdv = sqrtf(gsum) + 1e-10f;
@@ -443,6 +490,14 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     w[r] = load_or_zero(wrow[r], has);
     gsum[r] = *gptr[r];
     g[r] = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase, 64) * dim + col, has);
+    if (kbits == 0) {  // the row's one run, if it is a short one left to this kernel (folded_run)
+      const uint32_t same = (uint32_t)(__ballot(i + gl < n && kk[r] == half_bcast_u64(kk[r], gbase)) >> gbase);
+      const int run_len = same != 0xffffffffu ? __ffs((int)~same) - 1 : 32;
+      const bool fold = folded_run(i, run_len);
+#pragma unroll
+      for (int t = 1; t < kShort; ++t)
+        add4(g[r], load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + t, 64) * dim + col, has && fold && t < run_len));
+    }
   }
   int long_r = -1;
 #pragma unroll
@@ -576,7 +631,8 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
-    hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim);  \
+    hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim,       \
+                       (int)(kbits == 0));                                                                      \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
     if (VEC && dim <= 128) {                                                                                       \
