@@ -152,6 +152,87 @@ __device__ __forceinline__ void scatter_range(SliceState<NW, BITS>& st, const ui
   }
 }
 
+// The same for a bucket swollen by hot keys (a power-law graph puts tens of
+// thousands of equal row numbers into one bucket, which one block walks slice by
+// slice): KPT keys per thread and slice.  A wave owns KPT * 64 CONSECUTIVE
+// positions of the slice, 64 at a time, so that (wave, round, lane) is the order
+// of the positions and the ranks stay stable; its digit counts accumulate over
+// the rounds in its own row of wave_count (no other wave touches it, so the
+// rounds need no barrier), and the two barriers and the walk over the waves'
+// counts are paid once per KPT * NW * 64 keys instead of once per NW * 64.
+template <int NW, int BITS, int KPT>
+__device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, const uint64_t* __restrict__ keys_in,
+                                                   const uint32_t* __restrict__ vals_in,
+                                                   uint64_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
+                                                   int64_t begin, int64_t end, int shift, uint32_t mask) {
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+  constexpr int kSlice = NW * 64 * KPT;
+  const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  int parity = 0;
+  uint64_t key[KPT], key_next[KPT];
+  uint32_t val[KPT], val_next[KPT];
+  auto fetch = [&](int64_t base) {
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+      const int64_t i = base + (int64_t)wave * (64 * KPT) + q * 64 + lane;
+      key_next[q] = i < end ? keys_in[i] : 0ull;
+      val_next[q] = i < end ? vals_in[i] : 0u;
+    }
+  };
+  fetch(begin);
+  for (int64_t base = begin; base < end; base += kSlice) {
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+      key[q] = key_next[q];
+      val[q] = val_next[q];
+    }
+    if (base + kSlice < end) fetch(base + kSlice);  // the next slice's loads are issued before this one is ranked
+    uint32_t rank[KPT], digit[KPT];
+    bool valid[KPT];
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+      const int64_t i = base + (int64_t)wave * (64 * KPT) + q * 64 + lane;
+      valid[q] = i < end;
+      digit[q] = (uint32_t)(key[q] >> shift) & mask;
+      uint64_t peers = __ballot(valid[q]);
+#pragma unroll
+      for (int b = 0; b < BITS; ++b) {
+        const bool bit = (digit[q] >> b) & 1u;
+        const uint64_t m = __ballot(valid[q] && bit);
+        peers &= bit ? m : ~m;
+      }
+      const int rank_in_round = __popcll(peers & below);
+      const uint32_t prior = valid[q] ? st.wave_count[parity][wave][digit[q]] : 0u;  // this wave's earlier rounds
+      rank[q] = prior + (uint32_t)rank_in_round;
+      if (valid[q] && rank_in_round == 0) st.wave_count[parity][wave][digit[q]] = (uint16_t)(prior + __popcll(peers));
+    }
+    __syncthreads();
+    for (int d = t; d < (1 << BITS); d += NW * 64) {
+      uint32_t at = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const uint32_t c = st.wave_count[parity][w][d];
+        st.wave_count[parity][w][d] = (uint16_t)at;
+        at += c;
+        st.wave_count[parity ^ 1][w][d] = 0;
+      }
+      const uint32_t first = st.cursor[d];
+      st.slot[d] = first;
+      st.cursor[d] = first + at;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+      if (valid[q]) {
+        const uint32_t pos = st.slot[digit[q]] + st.wave_count[parity][wave][digit[q]] + rank[q];
+        keys_out[pos] = key[q];
+        vals_out[pos] = val[q];
+      }
+    }
+    parity ^= 1;
+  }
+}
+
 // The global pass.  Block 0 also writes the bucket offsets (digit d's keys end up
 // in [bucket_off[d], bucket_off[d + 1])).
 __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
@@ -220,6 +301,7 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
   const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
   if (begin >= end) return;
   const uint32_t mask = (1u << digit_bits) - 1u;
+  const bool wide = end - begin > 2 * kBucketWaves * 64;  // a swollen bucket
   uint64_t key_next = 0;
   uint32_t val_next = 0;
   if (begin + t < end) {
@@ -231,16 +313,48 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
     for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
   }
   __syncthreads();
-  if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
-  for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
-    atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
+  if (!wide) {
+    if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
+    for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
+      atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
+  } else {
+    // equal keys would queue up on one counter: one addition per wave and digit value present.
+    // Eight loads per thread in flight (the ballots would otherwise wait for each load in turn).
+    const int lane = t & 63;
+    const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    constexpr int kInFlight = 8;
+    for (int64_t base = begin; base < end; base += (int64_t)kInFlight * kBucketWaves * 64) {
+      uint64_t kq[kInFlight];
+#pragma unroll
+      for (int q = 0; q < kInFlight; ++q) {
+        const int64_t i = base + (int64_t)q * kBucketWaves * 64 + t;
+        kq[q] = i < end ? keys_in[i] : 0ull;
+      }
+#pragma unroll
+      for (int q = 0; q < kInFlight; ++q) {
+        const bool valid = base + (int64_t)q * kBucketWaves * 64 + t < end;
+        const uint32_t digit = (uint32_t)(kq[q] >> shift) & mask;
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+          const bool bit = (digit >> b) & 1u;
+          const uint64_t m = __ballot(valid && bit);
+          peers &= bit ? m : ~m;
+        }
+        if (valid && (peers & below) == 0ull) atomicAdd(&st.cursor[digit], (uint32_t)__popcll(peers));
+      }
+    }
+  }
   __syncthreads();
   uint32_t grand;
   const uint32_t excl = block_exclusive_scan(t < 256 ? st.cursor[t] : 0u, 4, st.wave_total, &grand);
   if (t < 256) st.cursor[t] = (uint32_t)begin + excl;
   __syncthreads();
-  scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
-                                 val_next);
+  if (wide)
+    scatter_range_wide<kBucketWaves, 8, 4>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask);
+  else
+    scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
+                                   val_next);
 }
 
 }  // namespace
