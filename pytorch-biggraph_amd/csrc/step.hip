@@ -51,6 +51,11 @@ struct SideCtx {
   float* s;             // [K*C, P, nn] scores against this side's negatives, then dLoss/dS
   float* rs;            // [K*C*P] row sums of dLoss/d(squared distance) (l2)
   int slot_pos, slot_uni;
+  // The gradient rows of this side's uniform negatives are read where the backward GEMM wrote them
+  // (dxn, which then lies behind gr in one block; uni_row0 = row number of dxn's first row counted from gr):
+  // with the dot comparator and no operator on them the raw-row gradient IS that row.
+  int uni_direct;
+  int64_t uni_row0;
   int has_op;           // an operator acts on this side's positives
   int op_uniform;       // ... and on its uniform negatives (standard mode)
   const float *p0, *p1; // operator parameters
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     if (lane == 0) {
       const int64_t slot = (int64_t)k * c.rk + sd.slot_uni + r2;
       c.keys[slot] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
-      c.vals[slot] = (uint32_t)slot;
+      c.vals[slot] = sd.uni_direct ? (uint32_t)(sd.uni_row0 + kc * sd.nn + sd.nb + uu) : (uint32_t)slot;
     }
     if (sd.op_uniform && c.op == PBG_OP_LINEAR) {
       row_store<NVH>(sd.xraw + ((int64_t)k * sd.op_rows + c.B + r2) * D, x, D, H, lane);
@@ -839,6 +844,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       row_store<NVH>(out, dx, D, H, lane);
     }
   } else {
+    if (sd.uni_direct) return;  // the GEMM's row is the gradient row
     const int r2 = r - c.B;
     const int cc = r2 / sd.u, uu = r2 % sd.u;
     const int64_t kc = (int64_t)k * c.C + cc;
@@ -1880,7 +1886,7 @@ __global__ __launch_bounds__(kGlobalHalves * 32) void global_grad_kernel(StepCtx
     const int col = c0 + lane * 4;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int r = begin + slice * kGlobalHalves + hw; r < end; r += slices * kGlobalHalves) {
-      const float* row = c.gr + ((int64_t)k * c.rk + r) * D;
+      const float* row = c.gr + (int64_t)c.vals[(int64_t)k * c.rk + r] * D;  // (a uniform negative's row may be the GEMM's)
       if (vec) {
         if (col < D) {
           const float4 v = *reinterpret_cast<const float4*>(row + col);
@@ -2080,13 +2086,28 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.rk = slot;
   c.kbits = bits_for((uint64_t)(K - 1));
 
+  // gradient rows, and behind them (so that one 32-bit row number reaches both) the negatives' gradient
+  // matrices of the sides whose uniform rows need no work after the GEMM
+  const int64_t npairs = (int64_t)K * c.rk;
+  int64_t block_rows = npairs;
+  for (int s = 0; s < 2; ++s) {
+    SideCtx& sd = c.side[s];
+    sd.uni_direct = sd.u > 0 && c.cmp == PBG_CMP_DOT && !sd.op_uniform && !c.bias &&
+                    block_rows + KC * sd.nn < ((int64_t)1 << 32);
+    if (sd.uni_direct) {
+      sd.uni_row0 = block_rows;
+      block_rows += KC * sd.nn;
+    }
+  }
+  c.gr = takef((size_t)block_rows * D);
+
   for (int s = 0; s < 2; ++s) {
     SideCtx& sd = c.side[s];
     const SideCtx& so = c.side[1 - s];
     // prepared operands and their gradients
     if (sd.nn > 0) {
       sd.xn = takef(KC * sd.nn * D);
-      sd.dxn = takef(KC * sd.nn * D);
+      sd.dxn = sd.uni_direct ? (c.gr ? c.gr + sd.uni_row0 * D : nullptr) : takef(KC * sd.nn * D);
       if (need_aux) sd.an = takef(KC * sd.nn);
       sd.s = takef(KC * P * sd.nn);
       if (is_distance(c.cmp)) sd.rs = takef(KC * P);
@@ -2178,10 +2199,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     }
   }
 
-  const int64_t npairs = (int64_t)K * c.rk;
   plan->max_norm = d->max_norm > 0.f ? d->max_norm : 0.f;
   if (plan->max_norm > 0.f) plan->renorm_scale = takef((size_t)npairs);
-  c.gr = takef((size_t)npairs * D);
   c.keys = (uint64_t*)take(npairs, 8);
   plan->keys_b = (uint64_t*)take(npairs, 8);
   c.vals = (uint32_t*)take(npairs, 4);
