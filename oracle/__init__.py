@@ -25,7 +25,12 @@ Modules
 Parity pinning (what each function is checked against before it is trusted):
 operators, comparators, gather and losses replay every literal vector of the
 reference's test/test_model.py and test/test_losses.py (tests/golden/*.json);
-the chunk/mask logic is pinned by ``brute`` and by closed-form invariants;
+the chunk/mask logic is pinned by ``brute`` and by closed-form invariants
+(all_negs also by its equality with uniform-only negatives over every entity,
+the bias inside the step also by its reduction to the base comparator and by
+the shift of all scores under a shift of all biases; the N3 regularizer by
+numpy complex arithmetic, closed forms and central differences; the global
+embeddings by the shifted-table identity);
 RowAdagrad by its reduction to torch.optim.Adagrad on constant-row gradients
 and on dim 1, and by pre-summed duplicates; AsyncAdagrad by torch.optim.Adagrad;
 reverse_permutation / shuffle / sub_bucket by the reference's own util.cpp
