@@ -56,6 +56,9 @@ struct SideCtx {
   // with the dot comparator and no operator on them the raw-row gradient IS that row.
   int uni_direct;
   int64_t uni_row0;
+  // (operator side, element-wise operator, dot comparator:) the gradient at the operator's output of a uniform
+  // negative IS its row of dxn; it is not copied to dz, the parameter gradient reads it there
+  int uni_dz_direct;
   int has_op;           // an operator acts on this side's positives
   int op_uniform;       // ... and on its uniform negatives (standard mode)
   const float *p0, *p1; // operator parameters
@@ -858,7 +861,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
     if (c.bias) add_to_first<NVH>(dz, stored * column_sum(sd.s, kc, c.P, sd.nn, col, lane), lane);
     if (sd.op_uniform) {
       const int64_t rel = clamp_index(c.rel[k], c.num_relations);
-      if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D, dz, D, H, lane);
+      if (keep_dz && !sd.uni_dz_direct) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D, dz, D, H, lane);
       if (c.op != PBG_OP_LINEAR)
         row_store<NVH>(out, op_backward<NVH>(c.op, dz, sd.p0, sd.p1, rel, D, H, lane), D, H, lane);
     } else {
@@ -884,8 +887,25 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
   const int D = c.D, H = D / 2;
   float acc = 0.f;
   if (e < D) {
-    for (int r = slice * kParamGroups + rg; r < sd.op_rows; r += slices * kParamGroups) {
+    // chunk and column of the uniform negative the loop is at, kept without a division per row
+    const int step = slices * kParamGroups;
+    int cc = 0, uu = 0;
+    bool in_uniform = false;
+    for (int r = slice * kParamGroups + rg; r < sd.op_rows; r += step) {
       const float* dz = sd.dz + ((int64_t)k * sd.op_rows + r) * D;
+      if (sd.uni_dz_direct && r >= c.B) {
+        if (!in_uniform) {
+          in_uniform = true;
+          cc = (r - c.B) / sd.u;
+          uu = (r - c.B) % sd.u;
+        }
+        dz = sd.dxn + (((int64_t)k * c.C + cc) * sd.nn + sd.nb + uu) * D;
+        uu += step;
+        while (uu >= sd.u) {
+          uu -= sd.u;
+          ++cc;
+        }
+      }
       if (c.op == PBG_OP_TRANSLATION) {
         acc += dz[e];
         continue;
@@ -894,8 +914,7 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
       if (r < c.B) {
         id = sd.idx[(int64_t)k * c.B + r];
       } else {
-        const int r2 = r - c.B;
-        id = uniform_negative(sd, s, ((int64_t)k * c.C + r2 / sd.u) * sd.u + r2 % sd.u);
+        id = uniform_negative(sd, s, (int64_t)k * c.C * sd.u + (r - c.B));  // = (k C + chunk) u + column
       }
       const float* x = sd.w + clamp_index(id, sd.num_rows) * D;
       const float* gl = sd.glob;  // the operator's input is the row plus the global embedding
@@ -2094,6 +2113,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     SideCtx& sd = c.side[s];
     sd.uni_direct = sd.u > 0 && c.cmp == PBG_CMP_DOT && !sd.op_uniform && !c.bias &&
                     block_rows + KC * sd.nn < ((int64_t)1 << 32);
+    sd.uni_dz_direct = sd.u > 0 && c.cmp == PBG_CMP_DOT && sd.op_uniform && !c.bias && c.op != PBG_OP_LINEAR;
     if (sd.uni_direct) {
       sd.uni_row0 = block_rows;
       block_rows += KC * sd.nn;
@@ -2210,6 +2230,10 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
   // (the regularizer's terms live in the staged kernels only)
   plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && getenv("PBG_DISABLE_FUSED") == nullptr;
+  if (plan->fused) {  // the fused kernel writes every gradient row and every dz itself
+    c.side[0].uni_direct = c.side[1].uni_direct = 0;
+    c.side[0].uni_dz_direct = c.side[1].uni_dz_direct = 0;
+  }
 
   if (b) {
     c.side[0].w = b->w_lhs;
