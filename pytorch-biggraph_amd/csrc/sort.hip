@@ -164,7 +164,9 @@ template <int NW, int BITS, int KPT>
 __device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, const uint64_t* __restrict__ keys_in,
                                                    const uint32_t* __restrict__ vals_in,
                                                    uint64_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
-                                                   int64_t begin, int64_t end, int shift, uint32_t mask) {
+                                                   int64_t begin, int64_t end, int shift, uint32_t mask,
+                                                   const uint64_t* first_keys = nullptr,
+                                                   const uint32_t* first_vals = nullptr) {
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   constexpr int kSlice = NW * 64 * KPT;
   const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -179,7 +181,15 @@ __device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, con
       val_next[q] = i < end ? vals_in[i] : 0u;
     }
   };
-  fetch(begin);
+  if (first_keys) {  // the caller fetched the first slice already (wide_fetch)
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+      key_next[q] = first_keys[q];
+      val_next[q] = first_vals[q];
+    }
+  } else {
+    fetch(begin);
+  }
   for (int64_t base = begin; base < end; base += kSlice) {
 #pragma unroll
     for (int q = 0; q < KPT; ++q) {
@@ -233,6 +243,19 @@ __device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, con
   }
 }
 
+// This thread's keys of the slice that starts at `base`, in scatter_range_wide's layout.
+template <int KPT>
+__device__ __forceinline__ void wide_fetch(const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
+                                           int64_t base, int64_t end, uint64_t* k, uint32_t* v) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int q = 0; q < KPT; ++q) {
+    const int64_t i = base + (int64_t)wave * (64 * KPT) + q * 64 + lane;
+    k[q] = i < end ? keys_in[i] : 0ull;
+    v[q] = i < end ? vals_in[i] : 0u;
+  }
+}
+
 // The global pass.  Block 0 also writes the bucket offsets (digit d's keys end up
 // in [bucket_off[d], bucket_off[d + 1])).
 __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
@@ -246,12 +269,10 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
-  uint64_t key_next = 0;
-  uint32_t val_next = 0;
-  if (begin + t < end) {
-    key_next = keys_in[begin + t];
-    val_next = vals_in[begin + t];
-  }
+  constexpr int kGlobalKpt = 4;  // a tile is at least 4096 keys: one slice of 4 keys per thread
+  uint64_t first_keys[kGlobalKpt];
+  uint32_t first_vals[kGlobalKpt];
+  wide_fetch<kGlobalKpt>(keys_in, vals_in, begin, end, first_keys, first_vals);
   // offset of digit d for this block = keys with a smaller digit anywhere
   //                                  + keys with digit d in earlier blocks;
   // two threads per digit, each over every other block, 16 loads in flight
@@ -286,8 +307,8 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
   }
   if (me == 0 && t == 0) bucket_off[kMaxDigits] = grand;
   __syncthreads();
-  scatter_range<kGlobalWaves, kMaxDigitBits>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift,
-                                             (1u << digit_bits) - 1u, key_next, val_next);
+  scatter_range_wide<kGlobalWaves, kMaxDigitBits, kGlobalKpt>(st, keys_in, vals_in, keys_out, vals_out, begin, end,
+                                                              shift, (1u << digit_bits) - 1u, first_keys, first_vals);
 }
 
 // A local pass: block b sorts bucket b (positions [bucket_off[b], bucket_off[b + 1]))
