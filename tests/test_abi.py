@@ -51,3 +51,44 @@ def test_argument_errors_need_no_gpu(pbg):
     d.dim = 6
     assert lib.pbg_train_step_workspace_bytes(ctypes.byref(d)) > 0
     assert lib.pbg_row_adagrad_sparse_workspace_bytes(1000) > 1000 * 24
+
+
+def test_newer_step_fields_are_validated_without_a_gpu(pbg):
+    import ctypes
+
+    L = pbg._lib
+    lib = L.lib()
+
+    def desc(**kw):
+        d = L.StepDesc()
+        d.dim, d.num_workers, d.batch_size = 8, 1, 10
+        d.num_batch_negs, d.num_uniform_negs = 2, 2
+        d.num_relations, d.num_lhs_rows, d.num_rhs_rows = 1, 100, 100
+        d.shared_table = 1
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return d
+
+    size = lambda d: lib.pbg_train_step_workspace_bytes(ctypes.byref(d))
+    plain = size(desc())
+    assert plain > 0
+    # bias: not with l2, not with a regularizer, not with a single coordinate
+    assert size(desc(bias=1)) > 0
+    assert size(desc(bias=1, comparator=L.COMPARATOR_CODES["l2"])) == 0 and b"bias" in lib.pbg_last_error()
+    assert size(desc(bias=1, regularization_coef=0.1, op=L.OPERATOR_CODES["diagonal"])) == 0
+    assert size(desc(bias=1, dim=1)) == 0
+    # affine: two parameter slots, no regularizer (operators.py:40)
+    assert size(desc(op=L.OPERATOR_CODES["affine"])) > plain
+    assert size(desc(op=L.OPERATOR_CODES["affine"], regularization_coef=0.1)) == 0
+    assert size(desc(op=6)) == 0 and b"unknown operator" in lib.pbg_last_error()
+    # all_negs: needs no negatives' counts; the score matrices grow with the tables
+    assert size(desc(all_negs=1, num_batch_negs=0, num_uniform_negs=0)) > plain
+    assert size(desc(num_batch_negs=0, num_uniform_negs=0)) == 0
+    assert size(desc(all_negs=1, num_lhs_rows=1 << 25, num_rhs_rows=1 << 25)) == 0
+    # max_norm adds the per-slot scales
+    assert size(desc(max_norm=1.0)) > plain
+    # the renormalisation entry point
+    assert lib.pbg_embedding_renorm_workspace_bytes(1000, 100) >= 1000 * 101 * 4
+    assert lib.pbg_embedding_renorm(None, 10, 4, None, 0, 1.0, None, 0, None) == L.PBG_OK
+    assert lib.pbg_embedding_renorm(None, 10, 4, None, 3, 1.0, None, 0, None) == L.PBG_ERR_INVALID
+    assert lib.pbg_embedding_renorm(None, 10, 4, None, 3, 0.0, None, 0, None) == L.PBG_ERR_INVALID
