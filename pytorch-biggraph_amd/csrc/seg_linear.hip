@@ -256,23 +256,7 @@ __global__ void run_start_kernel(const uint64_t* __restrict__ keys, const uint32
   run_start[i] = (uint32_t)(b == num_batches ? hi : lower_bound(keys, lo, hi, (rel << kbits) | (uint64_t)b));
 }
 
-// A workgroup streams ALL edges of its relation, kStage sorted positions per
-// step, whatever batch they belong to; the rows of step s + 1 are requested
-// before the products of step s and written to LDS after them.  A step that
-// holds edges of several batches is swept once per batch with the other
-// batches' rows masked in the A operand; whenever the batch changes, the
-// finished batch's gradient tile gets its Adagrad step and the accumulators
-// start over.  The kernel is kept small on purpose (dynamic loops, one copy of
-// every phase): most workgroups live for a few steps only, and code that does
-// not stay in the instruction cache is paid for by each of them.
-constexpr int kStage = 32;  // edges per step
-
-//
-// RUNS = false, grid (relation in rel_order, tile): as above; for a hot relation
-// the gradient tiles of its runs are read from `part` instead of being computed.
-// RUNS = true, grid ((slot * num_batches + batch) * splits + split, tile): the
-// gradient tile of one part of one run of a hot relation, written to
-// part[(blockIdx.x * tiles^2 + tile) * 256 + thread][16] in the MFMA result layout.
+// Where the gradient tiles of the hot relations' runs are, and how the relations are walked.
 struct HotRuns {
   const uint32_t* rel_order;  // [num_relations]
   const uint32_t* hot_slot;   // [num_relations], kNone: not hot
@@ -282,6 +266,24 @@ struct HotRuns {
   float* part;                // null: no relation is hot
   int num_batches, splits;
 };
+
+// A workgroup streams ALL edges of its relation, kStage sorted positions per
+// step, whatever batch they belong to; the rows of step s + 1 are requested
+// before the products of step s and written to LDS after them.  A step that
+// holds edges of several batches is swept once per batch with the other
+// batches' rows masked in the A operand; whenever the batch changes, the
+// finished batch's gradient tile gets its Adagrad step and the accumulators
+// start over.  The kernel is kept small on purpose (dynamic loops, one copy of
+// every phase): most workgroups live for a few steps only, and code that does
+// not stay in the instruction cache is paid for by each of them.
+//
+// RUNS = false, grid (relation in rel_order, tile): as above; for a hot relation
+// the gradient tiles of its runs are read from `part` instead of being computed.
+// RUNS = true, grid ((slot * num_batches + batch) * splits + split, tile): the
+// gradient tile of one part of one run of a hot relation, streamed the same way
+// and written to part[(blockIdx.x * tiles^2 + tile) * 256 + thread][16] in the
+// MFMA result layout.
+constexpr int kStage = 32;  // edges per step
 
 template <bool VEC, bool RUNS>
 __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
