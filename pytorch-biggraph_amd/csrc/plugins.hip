@@ -326,8 +326,9 @@ __global__ __launch_bounds__(kRowThreads) void loss_rows_kernel(int loss, float 
       dp += (sigmoidf(s) - 1.0f) * up;
     }
     for (int j = lane; j < N; j += kWave) {
-      acc += softplusf(row[j]) * inv_n;
-      if (drow) drow[j] = sigmoidf(row[j]) * inv_n * up;
+      float sg;
+      acc += softplus_sigmoid(row[j], &sg) * inv_n;
+      if (drow) drow[j] = sg * inv_n * up;
     }
   } else {
     float mx = s;

@@ -283,5 +283,11 @@ __device__ __forceinline__ float sigmoidf(float z) {
   const float e = expf(z);
   return e / (1.0f + e);
 }
+// softplus(z) and sigmoid(z) from one exponential (the same values as the two functions above)
+__device__ __forceinline__ float softplus_sigmoid(float z, float* sigmoid) {
+  const float e = expf(-fabsf(z));
+  *sigmoid = (z >= 0.f ? 1.0f : e) / (1.0f + e);
+  return fmaxf(z, 0.f) + log1pf(e);
+}
 
 }  // namespace pbg

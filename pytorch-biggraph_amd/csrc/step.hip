@@ -530,8 +530,9 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
       g = (x >= 0.f) ? w : 0.f;
       dpos_part -= g;
     } else if (loss == PBG_LOSS_LOGISTIC) {
-      *loss_acc += softplusf(t) * inv_nn;
-      g = sigmoidf(t) * inv_nn * w;
+      float sg;
+      *loss_acc += softplus_sigmoid(t, &sg) * inv_nn;
+      g = sg * inv_nn * w;
     } else {
       g = expf(t - mx) * inv_z * w;
     }
@@ -1117,8 +1118,9 @@ __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at
           g = (x >= 0.f) ? w : 0.f;
           dpos_part -= g;
         } else {
-          loss_acc += softplusf(te) * inv_nn;
-          g = sigmoidf(te) * inv_nn * w;
+          float sg;
+          loss_acc += softplus_sigmoid(te, &sg) * inv_nn;
+          g = sg * inv_nn * w;
         }
         if (te > pos) ++viol;
         // t = -sqrt(q): dLoss/dq = g * 0.5 / t; stored as -2 dLoss/dq
@@ -1207,8 +1209,9 @@ __device__ __forceinline__ void quad_side_loss(float* lds, int row_at, int bn_at
       g = (x >= 0.f) ? w : 0.f;
       dpos_part -= g;
     } else if (LOSS == PBG_LOSS_LOGISTIC) {
-      loss_acc += softplusf(te) * inv_nn;
-      g = sigmoidf(te) * inv_nn * w;
+      float sg;
+      loss_acc += softplus_sigmoid(te, &sg) * inv_nn;
+      g = sg * inv_nn * w;
     } else {
       g = expf(te - mx) * inv_z * w;
     }
