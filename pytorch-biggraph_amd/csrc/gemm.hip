@@ -469,7 +469,8 @@ int gemm_f32(const GemmArgs& g, hipStream_t stream) {
   // k, and the contiguous axis of a k-major operand, are multiples of 4
   const bool dma_ok = a_vec && b_vec && g.k % 4 == 0 && g.k >= BK && (!g.a_kmajor || (g.m % 4 == 0 && g.m >= 4)) &&
                       (!g.b_kmajor || (g.n % 4 == 0 && g.n >= 4));
-  if (g.m <= 96 || g.n <= 96) {
+  // (a product of at most 64 values of k is bound by writing its output: the smaller tile pads less)
+  if (g.m <= 96 || g.n <= 96 || (!dma_ok && g.k <= 64)) {
     launch<64, 64>(g, a_vec, b_vec, stream);
   } else if (dma_ok) {
     launch_dma(g, stream);
