@@ -7,3 +7,30 @@ def test_smoke_entry_point():
     import __graft_entry__
 
     __graft_entry__.smoke()
+
+
+@pytest.mark.gpu
+def test_bench_line_has_the_contract_fields():
+    """A short bench.py run prints ONE JSON line with the fields the driver reads."""
+    import json
+    import pathlib
+    import subprocess
+    import sys
+
+    root = pathlib.Path(__file__).resolve().parent.parent
+    out = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "1", "--steps", "256", "--warmup", "64",
+                          "--cpu-seconds", "0", "--no-sequential"], capture_output=True, text=True, timeout=240, cwd=root)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [ln for ln in out.stdout.splitlines() if ln.startswith("{")]
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 256 and line["unit"] == "edges/s" and line["value"] > 0
+    assert line["vs_baseline"] is None and line["dtype"] == "f32" and "workload" in line["config"]
+    roof = line["roofline"]
+    for key in ("bound", "achieved", "peak", "unit", "frac", "traffic"):
+        assert key in roof, key
+    assert roof["bound"] in ("hbm", "mfma") and 0 < roof["frac"] < 1
+    assert roof["frac"] == pytest.approx(roof["achieved"] / roof["peak"], rel=1e-6)

@@ -246,3 +246,14 @@ def test_model_argument_errors(pbg):
     bad.set_embeddings("e", pbg.types.Side.RHS, w)
     with pytest.raises(RuntimeError, match="right-hand side operator"):
         bad(ED(edges.lhs, edges.rhs, torch.tensor(0)))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import pathlib
+    import subprocess
+    import sys
+
+    root = pathlib.Path(__file__).resolve().parent.parent
+    out = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 2
+    assert "ONE GPU" in out.stderr
