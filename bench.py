@@ -1,14 +1,14 @@
 #!/usr/bin/env python3
 """Throughput of the PBG training step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1] [--workers 64]
+    python bench.py [--gpus 1] [--steps N] [--warmup W] [--workload cfg1] [--workers 64]
 
-A "step" is one batch of `batch_size` edges through the whole hot path (gather,
-operator, scoring against batch + uniform negatives, loss, backward, RowAdagrad
-and operator Adagrad).  Batches are issued `workers` at a time through
-pbg_train_step, which processes them like `workers` HOGWILD processes in
-lock-step (all read, then all write in order); `--workers 1` is the strictly
-sequential single-process order.  Prints ONE JSON line.
+A "step" is one call of pbg_train_step: `workers` batches of `batch_size` edges
+through the whole hot path (gather, operator, scoring against batch + uniform
+negatives, loss, backward, RowAdagrad and operator Adagrad), processed like
+`workers` HOGWILD processes in lock-step (all read, then all write in order).
+`--steps` and `--warmup` count calls and never change `workers`; `--workers 1` is
+the strictly sequential single-process order.  Prints ONE JSON line.
 """
 import argparse
 import json
@@ -24,9 +24,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
-# HBM bytes per launch of (workload, kernel) at the default --workers, from the
-# rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under profiles/ (not measured live).
-TRAFFIC = {("cfg1", "fused_chunk"): 231.4e6}  # 64 workers
+# HBM bytes per launch of (workload, kernel, workers), from the rocprofv3 FETCH_SIZE /
+# WRITE_SIZE runs summarised under profiles/ (not measured live); any other
+# combination reports null.
+TRAFFIC = {("cfg1", "fused_chunk", 64): 231.4e6}
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
@@ -95,7 +96,8 @@ def cpu_baseline(w, seconds):
     on a bounded sample of the same synthetic workload."""
     from oracle import hogwild, step as ostep
 
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)), 16)
+    host = os.cpu_count() or 1
+    cores = min(host, int(os.environ.get("OMP_NUM_THREADS", host)), 16)  # a GPU box grants 16 host cores per GPU
     b, d = w["batch"], w["dim"]
     sample = dict(w)
     sample["entities"] = min(w["entities"], 2_000_000)      # bounded host copy of the table
@@ -118,7 +120,7 @@ def cpu_baseline(w, seconds):
     eps, edges, wall = hogwild.run(cfg, tables[0], lhs, rhs, rel, b, cores, seconds,
                                    w_rhs=tables[1] if len(tables) > 1 else None)
     note = "" if sample["entities"] == w["entities"] else f", first {sample['entities']} table rows"
-    return {"value": eps, "unit": "edges/s", "cores": cores, "kind": "port",
+    return {"value": eps, "unit": "edges/s", "cores": cores, "host_cpu_count": host, "kind": "port",
             "sample": f"{edges} edges in {wall:.1f} s, {cores} HOGWILD processes over shared-memory tables (oracle.hogwild){note}"}
 
 
@@ -218,7 +220,7 @@ def bucket_epoch(args):
     bl = pkg.bucket_loop
     w = WORKLOADS["cfg4"]
     nparts, rows, d, b = 4, w["entities"], w["dim"], w["batch"]
-    per_bucket = args.steps * b if args.steps else 2_000_000
+    per_bucket = args.steps * args.workers * b if args.steps else 2_000_000  # --steps = calls per bucket
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(0)
     t0 = time.perf_counter()
@@ -254,7 +256,8 @@ def bucket_epoch(args):
     best = results[3]
     line = {
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X", "value": best["edges_per_s"], "unit": "edges/s",
-        "n_gpus": 1, "steps": 16 * per_bucket // b, "warmup": 0, "ms_per_step": best["seconds"] / (16 * per_bucket // b) * 1e3,
+        "n_gpus": 1, "steps": 16 * per_bucket // (b * args.workers), "warmup": 0,
+        "ms_per_step": best["seconds"] / max(1, 16 * per_bucket // (b * args.workers)) * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "cfg4-epoch: one pass over 16 buckets of 4 x 4 partitions (10.4M rows x dim 100 each, pinned host "
                                f"memory), {per_bucket} edges per bucket, translation/l2/ranking, partitions swapped between buckets",
@@ -269,8 +272,8 @@ def bucket_epoch(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="timed batches")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed batches")
+    ap.add_argument("--steps", type=int, default=None, help="timed calls of pbg_train_step (each of --workers batches)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed calls")
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS) + ["cfg4-epoch"])
     ap.add_argument("--workers", type=int, default=64,
                     help="batches in flight per call (HOGWILD workers); 64 batches of cfg1 are 1280 chunks = 5 per compute unit")
@@ -361,12 +364,10 @@ def main():
 
     enqueue_s = [0.0]  # host time per call of the last run's timed loop (launches only, no wait)
 
-    def run(workers, batches, warm, profile_calls=0, hip_graph=False):
+    def run(workers, calls, warm_calls, profile_calls=0, hip_graph=False):
         spec, runner = make_runner(workers)
         c, u = spec.num_chunks, w["uniform_negs"]
         per_call = workers * b
-        calls = max(1, batches // workers)
-        warm_calls = max(1, warm // workers)
         n_r = tables[-1].shape[0]
 
         static = None  # inputs of the captured step (hip_graph): the next call's edges and negatives are written into them
@@ -424,23 +425,24 @@ def main():
                 stages = {"fused_chunk": stages["prep"], "loss_reduce": stages["loss"], "params": stages["params"],
                           "sort": stages["sort"], "update": stages["update"]}
         loss = float(runner.loss_out.mean().item()) / b
-        return spec, calls * per_call / dt, dt / (calls * workers) * 1e3, calls * workers, stages, loss
+        return spec, calls * per_call / dt, dt / calls * 1e3, dt, stages, loss
 
-    default_steps = {"cfg1": 64000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
-    steps = args.steps if args.steps is not None else default_steps
-    warmup = args.warmup if args.warmup is not None else max(args.workers, steps // 10)
-    workers = max(1, min(args.workers, steps))
-    spec, eps, ms_per_step, timed, stages, loss = run(workers, steps, warmup, profile_calls=10)
+    workers = max(1, args.workers)
+    default_batches = {"cfg1": 64000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
+    steps = args.steps if args.steps is not None else max(1, default_batches // workers)
+    warmup = args.warmup if args.warmup is not None else max(1, steps // 10)
+    spec, eps, ms_per_step, wall_s, stages, loss = run(workers, steps, warmup, profile_calls=10)
     host_enqueue_ms = enqueue_s[0] * 1e3
 
     seq = None
     if not args.no_sequential and workers > 1:
-        _, seq_eps, seq_ms, seq_timed, _, _ = run(1, max(50, min(steps // 8, 1000)), 20)
-        seq = {"value": seq_eps, "ms_per_step": seq_ms, "steps": seq_timed, "workers": 1}
+        seq_calls = max(50, min(default_batches // 8, 1000))
+        _, seq_eps, seq_ms, _, _, _ = run(1, seq_calls, 20)
+        seq = {"value": seq_eps, "ms_per_step": seq_ms, "steps": seq_calls, "workers": 1}
         # the same single-batch sequence with the step captured in a HIP graph (one launch per step
         # instead of about ten) and the inputs written into the graph's static buffers
-        _, g_eps, g_ms, g_timed, _, _ = run(1, max(50, min(steps // 8, 1000)), 20, hip_graph=True)
-        seq["hip_graph"] = {"value": g_eps, "ms_per_step": g_ms, "steps": g_timed}
+        _, g_eps, g_ms, _, _, _ = run(1, seq_calls, 20, hip_graph=True)
+        seq["hip_graph"] = {"value": g_eps, "ms_per_step": g_ms, "steps": seq_calls}
 
     # roofline of the dominant stage (HIP events around each stage of pbg_train_step, on its stream)
     alg = algorithmic(w, spec)
@@ -455,7 +457,7 @@ def main():
         achieved, peak, unit = units / seconds / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
-        "frac": achieved / peak, "traffic": TRAFFIC.get((args.workload, dominant)), "launches_in_stage": launches,
+        "frac": achieved / peak, "traffic": TRAFFIC.get((args.workload, dominant, workers)), "launches_in_stage": launches,
         "avg_launch_ms": stages[dominant] / launches,
         "stages_ms": stages,
         "all": {k: {"bound": alg[k][0],
@@ -468,11 +470,13 @@ def main():
 
     line = {
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X",
-        "value": eps, "unit": "edges/s", "n_gpus": 1, "steps": timed, "warmup": warmup,
+        "value": eps, "unit": "edges/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
-                   "hogwild_workers": workers, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
+                   "hogwild_workers": workers, "step": f"one pbg_train_step call of {workers} batches",
+                   "timed_calls": steps, "timed_batches": steps * workers, "timed_edges": steps * workers * b,
+                   "timed_wall_seconds": wall_s, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
                    "mean_loss_per_edge_last_call": loss, "host_enqueue_ms_per_call": host_enqueue_ms},
         "sequential": seq,
         "roofline": roofline,

@@ -349,6 +349,10 @@ class StepRunner:
         bufs.w_rhs, bufs.g_rhs = _ptr(self.w_rhs), _ptr(self.g_rhs)
         bufs.lhs, bufs.rhs, bufs.rel = _ptr(lhs), _ptr(rhs), _ptr(rel)
         bufs.uniform_lhs, bufs.uniform_rhs = _ptr(uniform_lhs), _ptr(uniform_rhs)
+        if edge_weight is not None:  # EdgeList.weight (edgelist.py:51-95): one fp32 weight per edge
+            _need(edge_weight, torch.float32, "edge_weight")
+            if edge_weight.numel() != k * b:
+                raise ValueError(f"edge_weight must hold num_workers * batch_size = {k * b} entries")
         bufs.edge_weight = _ptr(edge_weight)
         bufs.relation_weights = _ptr(self.relation_weights)
         p0, p1 = self._op_pair(self.rhs_op)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import step as ostep
-from tests.test_gpu_step import compare_scores, compare_state, make_inputs, pack, say, to_runner
+from tests.test_gpu_step import compare_scores, compare_state, lockstep, make_inputs, pack, say, to_runner
 
 pytestmark = pytest.mark.gpu
 
@@ -59,8 +59,8 @@ def test_random_combination(pbg, index):
         compare_scores(cfg, tuple(t[k] for t in got), want.scores)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches)
-    rtol = 1e-4 if cfg.comparator == "l2" else 1e-5
+    outs, st64 = lockstep(cfg, st, batches)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-5), ("loss", k)
-    compare_state(cfg, runner, st, rtol, "combination")
+    compare_state(cfg, runner, st, rtol, "combination", st64)

@@ -18,7 +18,7 @@ def test_bench_line_has_the_contract_fields():
     import sys
 
     root = pathlib.Path(__file__).resolve().parent.parent
-    out = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "1", "--steps", "256", "--warmup", "64",
+    out = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "1", "--steps", "20", "--warmup", "5",
                           "--cpu-seconds", "0", "--no-sequential"], capture_output=True, text=True, timeout=240, cwd=root)
     assert out.returncode == 0, out.stderr[-2000:]
     lines = [ln for ln in out.stdout.splitlines() if ln.startswith("{")]
@@ -27,8 +27,12 @@ def test_bench_line_has_the_contract_fields():
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in line, key
-    assert line["n_gpus"] == 1 and line["steps"] == 256 and line["unit"] == "edges/s" and line["value"] > 0
+    assert line["n_gpus"] == 1 and line["steps"] == 20 and line["unit"] == "edges/s" and line["value"] > 0
     assert line["vs_baseline"] is None and line["dtype"] == "f32" and "workload" in line["config"]
+    # --steps counts calls; the number of batches per call does not shrink with it
+    cfg = line["config"]
+    assert cfg["hogwild_workers"] == 64 and cfg["timed_calls"] == 20 and cfg["timed_batches"] == 20 * 64
+    assert line["value"] == pytest.approx(cfg["timed_edges"] / cfg["timed_wall_seconds"], rel=1e-6)
     roof = line["roofline"]
     for key in ("bound", "achieved", "peak", "unit", "frac", "traffic"):
         assert key in roof, key

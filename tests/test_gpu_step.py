@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import step as ostep
+from tests.parity import anchored_state, double_state
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -194,7 +195,23 @@ TRAIN_CASES += [
 ]
 
 
-def compare_state(cfg, runner, st, rtol, tag):
+def lockstep(cfg, st, batches, keep_scores=False):
+    """oracle.step.train_lockstep on `st`; for the l2 comparator also on a float64
+    copy, the anchor of compare_state's criterion for that comparator."""
+    st64 = double_state(st) if cfg.comparator == "l2" else None
+    outs = ostep.train_lockstep(cfg, st, batches, keep_scores=keep_scores)
+    if st64 is not None:
+        ostep.train_lockstep(cfg, st64, batches)
+    return outs, st64
+
+
+def compare_state(cfg, runner, st, rtol, tag, st64=None):
+    if st64 is not None:
+        # l2 is -sqrt(||a||^2 - 2ab + ||b||^2) (model.py:215-246): near a zero distance the
+        # expansion, and through the square root's slope the gradient, is rounding noise in
+        # the reference's own fp32 evaluation; there the float64 result is the anchor
+        anchored_state(cfg, runner, st, st64, rtol, tag)
+        return
     assert_close(runner.w_lhs, st.w_lhs, rtol, tag + " w_lhs")
     assert_close(runner.g_lhs, st.g_lhs, rtol, tag + " g_lhs")
     if not st.shared:
@@ -221,6 +238,18 @@ def hinge_ties(cfg, scores, eps=2e-6):
     return n
 
 
+def copy_of(st):
+    """An independent copy of an oracle state (one table stays one table)."""
+    import copy
+
+    other = copy.deepcopy(st)
+    if st.shared:
+        other.w_rhs, other.g_rhs = other.w_lhs, other.g_lhs
+    if st.glob_lhs is not None and st.glob_rhs is st.glob_lhs:
+        other.glob_rhs, other.glob_rhs_sum = other.glob_lhs, other.glob_lhs_sum
+    return other
+
+
 def copy_state(runner, st):
     runner.w_lhs.copy_(st.w_lhs)
     runner.g_lhs.copy_(st.g_lhs)
@@ -241,15 +270,13 @@ def test_train_step(pbg, case, workers):
     num_pos, dim = case.pop("num_pos"), case.pop("dim")
     cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
                            margin=0.1, **case)
-    # plenty of entities: with l2 a repeated entity inside a chunk sits on the
-    # sqrt kink, where the reference's own gradient is rounding noise
-    n_ent = max(200, num_pos * (40 if cfg.comparator == "l2" else 4))
+    n_ent = max(200, num_pos * 4)
     st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=(dim % 2 == 0))
     runner = to_runner(pbg, cfg, st, num_pos, workers)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches, keep_scores=True)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    outs, st64 = lockstep(cfg, st, batches, keep_scores=True)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
         # a negative that IS the positive's entity ties with it up to rounding: the
@@ -260,7 +287,7 @@ def test_train_step(pbg, case, workers):
             p = pos.unsqueeze(1)
             ties = int(((neg - p).abs() <= 2e-5 * p.abs().clamp_min(1e-6)).sum())
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
-    compare_state(cfg, runner, st, rtol, "step")
+    compare_state(cfg, runner, st, rtol, "step", st64)
 
 
 GLOBAL_CASES = [
@@ -302,11 +329,11 @@ def test_train_step_with_global_embeddings(pbg, case, workers):
     runner = to_runner(pbg, cfg, st, num_pos, workers)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    outs, st64 = lockstep(cfg, st, batches)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
-    compare_state(cfg, runner, st, rtol, "step+global")
+    compare_state(cfg, runner, st, rtol, "step+global", st64)
     assert not torch.equal(st.glob_lhs, zero_glob[0])  # it was trained
 
 
@@ -357,11 +384,11 @@ def test_train_step_with_max_norm(pbg, case, workers):
     assert_close(runner.w_lhs, st.w_lhs, 1e-6, "renormalised table")
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    outs, st64 = lockstep(cfg, st, batches)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
-    compare_state(cfg, runner, st, rtol, "step+max_norm")
+    compare_state(cfg, runner, st, rtol, "step+max_norm", st64)
 
 
 # (A translation moves the bias of every row of its side by the same amount, which ranking and softmax do
@@ -460,11 +487,66 @@ def test_train_step_with_all_negs(pbg, case, workers):
         compare_scores(cfg, tuple(t[k] for t in got), want.scores)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    outs, st64 = lockstep(cfg, st, batches)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
-    compare_state(cfg, runner, st, rtol, "step+all_negs")
+    compare_state(cfg, runner, st, rtol, "step+all_negs", st64)
+
+
+WEIGHT_CASES = [
+    # the single-kernel route (chunk in LDS), each loss
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=230, dim=100),
+    dict(operator="translation", comparator="l2", loss="logistic", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=100,
+         shared=False),
+    dict(operator="diagonal", comparator="dot", loss="softmax", num_batch_negs=20, num_uniform_negs=10, num_pos=45, dim=32),
+    # the staged route, each loss
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=100,
+         num_pos=130, dim=400),
+    dict(operator="linear", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=10, num_pos=45, dim=24),
+    dict(operator="diagonal", comparator="squared_l2", loss="ranking", num_batch_negs=0, num_uniform_negs=7, num_pos=30,
+         dim=9, disable_lhs_negs=True),
+    dict(operator="linear", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=10,
+         num_pos=45, dim=24),
+    dict(operator="translation", comparator="dot", loss="ranking", dynamic=True, num_batch_negs=10, num_uniform_negs=5,
+         num_pos=33, dim=16, shared=False),
+]
+
+
+@pytest.mark.parametrize("case", WEIGHT_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_train_step_with_edge_weights(pbg, case, workers):
+    """EdgeList.weight (edgelist.py:51-95) inside the step: every loss scales an edge's
+    term by its weight (losses.py:65-79, 104-113, 147-161)."""
+    say("train+weights", case, workers)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", True)
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01,
+                           margin=0.1, **case)
+    n_ent = max(200, num_pos * (40 if cfg.comparator == "l2" else 4))
+    st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=shared)
+    g = torch.Generator().manual_seed(99)
+    weights = [0.25 + 2.0 * torch.rand(num_pos, generator=g) for _ in batches]
+    weights[0][::7] = 0.0  # (an edge of weight 0 contributes nothing)
+    unweighted = copy_of(st)
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    runner.train(*pack(cfg, batches), edge_weight=torch.stack(weights).to(DEV))
+    torch.cuda.synchronize()
+    outs, st64 = lockstep(cfg, st, [b + (w,) for b, w in zip(batches, weights)])
+    ostep.train_lockstep(cfg, unweighted, batches)
+    rtol = 1e-5
+    for k, out in enumerate(outs):
+        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+    compare_state(cfg, runner, st, rtol, "step+weights", st64)
+    # the weights moved the result: the comparison above would not pass without them
+    assert (st.w_lhs - unweighted.w_lhs).abs().max() > 1e-3 * st.w_lhs.abs().max()
+    # what the binding refuses: a host tensor, another dtype, another length
+    lhs, rhs, rel, ul, ur = pack(cfg, batches)
+    good = torch.stack(weights).to(DEV)
+    for bad, err in ((good.cpu(), TypeError), (good.double(), TypeError), (good.flatten()[:-1], ValueError)):
+        with pytest.raises(err):
+            runner.train(lhs, rhs, rel, ul, ur, edge_weight=bad)
 
 
 def test_bias_is_refused_where_it_is_not_implemented(pbg):
@@ -529,14 +611,14 @@ def test_train_step_with_n3_regularizer(pbg, case, workers):
                                    for k, v in st.__dict__.items() if v is not None})
     if st.shared:
         st_plain.w_rhs, st_plain.g_rhs = st_plain.w_lhs, st_plain.g_lhs
-    outs = ostep.train_lockstep(cfg, st, batches)
+    outs, st64 = lockstep(cfg, st, batches)
     ostep.train_lockstep(plain, st_plain, batches)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
         assert out.reg > 0.0
         assert float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
-    compare_state(cfg, runner, st, rtol, "step+N3")
+    compare_state(cfg, runner, st, rtol, "step+N3", st64)
     # the regularizer moved the result: the comparison above would not pass without it
     assert (st.w_lhs - st_plain.w_lhs).abs().max() > 100 * rtol * (st.w_lhs - before.cpu()).abs().max()
 
@@ -553,15 +635,29 @@ def test_regularizer_is_refused_for_linear(pbg):
     dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=200, dim=100),
     dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=20, num_uniform_negs=30, num_pos=100, dim=40),
     dict(operator="translation", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=10, num_pos=50, dim=16),
+    # cfg4's step: translation, l2, ranking, two tables, power-law ids
+    dict(operator="translation", comparator="l2", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=200, dim=100,
+         shared=False, zipf=1.8),
+    # cfg5's step: linear, cos, logistic, one relation per edge
+    dict(operator="linear", comparator="cos", loss="logistic", dynamic=True, num_batch_negs=50, num_uniform_negs=50,
+         num_pos=100, dim=64),
 ], ids=ids)
 def test_hundred_steps(pbg, case):
     """Updated embeddings, Adagrad state and operator parameters after 100
     sequential steps stay within 1e-4 relative of the CPU path."""
+    from tests.parity import zipf_ids
+
     say("hundred", case)
     case = dict(case)
     num_pos, dim = case.pop("num_pos"), case.pop("dim")
-    cfg = ostep.StepConfig(dim=dim, num_relations=2, relation_weights=[1.0, 1.0], lr=0.1, dynamic=False, **case)
-    st, batches = make_inputs(cfg, num_pos, 2000, 100, seed=1, scale=1e-3 if case["operator"] == "none" else 0.1)
+    shared, zipf = case.pop("shared", True), case.pop("zipf", None)
+    cfg = ostep.StepConfig(dim=dim, num_relations=2, relation_weights=[1.0, 1.0], lr=0.1,
+                           dynamic=case.pop("dynamic", False), **case)
+    st, batches = make_inputs(cfg, num_pos, 2000, 100, seed=1, shared=shared,
+                              scale=1e-3 if case["operator"] == "none" else 0.1)
+    if zipf:
+        g = torch.Generator().manual_seed(2)
+        batches = [(zipf_ids(num_pos, 2000, zipf, g), zipf_ids(num_pos, 2000, zipf, g)) + b[2:] for b in batches]
     runner = to_runner(pbg, cfg, st, num_pos, 1)
     resyncs = 0
     for n, b in enumerate(batches):
@@ -578,6 +674,7 @@ def test_hundred_steps(pbg, case):
             copy_state(runner, st)
             resyncs += 1
     torch.cuda.synchronize()
+    say("  steps restarted from the oracle's state after a hinge tie:", resyncs, "of", len(batches))
     assert resyncs <= 10, resyncs
     compare_state(cfg, runner, st, 1e-4, "100 steps")
 
@@ -694,8 +791,8 @@ def test_fused_kernel_shapes(pbg, case):
     runner = to_runner(pbg, cfg, st, num_pos, 2)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches, keep_scores=True)
-    rtol = 1e-5 if cfg.comparator != "l2" else 1e-4
+    outs, st64 = lockstep(cfg, st, batches, keep_scores=True)
+    rtol = 1e-5
     for k, out in enumerate(outs):
         assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
         sc = out.scores
@@ -704,7 +801,7 @@ def test_fused_kernel_shapes(pbg, case):
             pp = pos.unsqueeze(1)
             ties = int(((neg - pp).abs() <= 2e-5 * pp.abs().clamp_min(1e-6)).sum())
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
-    compare_state(cfg, runner, st, rtol, "step")
+    compare_state(cfg, runner, st, rtol, "step", st64)
 
 
 def test_lockstep_training_learns_like_sequential(pbg):
