@@ -50,7 +50,7 @@ class Census:
         return f"{self.entries} entries, {self.anchored} passed on the float64 anchor only"
 
 
-def anchored_close(got, ref32, exact, rtol, what, census=None, loose=None, loose_bound=0.0):
+def anchored_close(got, ref32, exact, rtol, what, census=None, loose=None, loose_bound=0.0, slack=None):
     """The stated criterion first: `got` within rtol (relative, with a floor of
     rtol/10 of the tensor's largest entry) of the CPU path's fp32 result `ref32`.
     An entry that misses it must be explained by fp32 rounding alone: it lies
@@ -60,7 +60,8 @@ def anchored_close(got, ref32, exact, rtol, what, census=None, loose=None, loose
     batch name sums thousands of gradient rows, and `l2` cancels ||a||^2 - 2ab +
     ||b||^2: their fp32 results depend on the order of summation by more than rtol
     in the reference as much as here.  `loose` marks entries held to `loose_bound`
-    (absolute) instead."""
+    (absolute) instead; `slack` is an absolute allowance per entry on top of both
+    criteria (adagrad_noise_slack)."""
     got = got.detach().cpu().double()
     ref = ref32.detach().double()
     exact = exact.detach().double()
@@ -69,6 +70,8 @@ def anchored_close(got, ref32, exact, rtol, what, census=None, loose=None, loose
         return
     scale = max(ref.abs().max().item(), 1e-30)
     floor = 0.1 * rtol * scale
+    if slack is not None:
+        floor = floor + slack.double()
     plain = (got - ref).abs() <= rtol * ref.abs() + floor
     noise = (ref - exact).abs()
     noise = noise.amax(dim=-1, keepdim=True) if noise.dim() >= 2 else noise.max()
@@ -85,12 +88,34 @@ def anchored_close(got, ref32, exact, rtol, what, census=None, loose=None, loose
                            "scale", scale, "count", int(bad.sum()), "fp32 reference noise", float(noise.max()))
 
 
-def anchored_state(cfg, runner, st, st64, rtol, tag, census=None, loose_rows=None, loose_steps=0):
+def adagrad_noise_slack(grads, lr, rel_noise=2e-7):
+    """How far fp32 rounding of the gradients alone can move a parameter over a
+    sequence of AsyncAdagrad steps (async_adagrad.py:75-85).  `grads`: the exact
+    gradient of each step, in order, leading axis = relation.  A gradient entry is a
+    cancelling sum over a batch; in fp32 it carries an absolute error of about
+    rel_noise times the largest entry of its relation's slice, whatever its own
+    size.  Step k moves an entry by lr * g_k / sqrt(sum_{j<=k} g_j^2), so that error
+    moves it by up to lr * error / sqrt(sum): negligible where the gradients are of
+    ordinary size, a visible fraction of lr where an entry's gradients so far are
+    all tiny (and never more than 2 lr, a flipped sign)."""
+    total = torch.zeros_like(grads[0], dtype=torch.float64)
+    slack = torch.zeros_like(total)
+    for g in grads:
+        g = g.double()
+        total = total + g * g
+        err = rel_noise * g.abs().reshape(g.shape[0], -1).amax(dim=1).reshape(-1, *([1] * (g.dim() - 1)))
+        step = torch.where(total > 0, lr * err / total.sqrt().clamp_min(1e-300), torch.zeros_like(total))
+        slack = slack + step.clamp_max(2 * lr)
+    return slack
+
+
+def anchored_state(cfg, runner, st, st64, rtol, tag, census=None, loose_rows=None, loose_steps=0, param_slack=None):
     """Tables, Adagrad sums, operator parameters and global embeddings of a
     StepRunner against the oracle's fp32 and float64 states.  `loose_rows` =
     (bool[rows of lhs table], bool[rows of rhs table]): rows a hinge tie reaches;
     they, and every operator parameter, may then differ by `loose_steps` Adagrad
-    steps (a step never exceeds the step size); their Adagrad sums are not compared."""
+    steps (a step never exceeds the step size); their Adagrad sums are not compared.
+    `param_slack` = {"rhs_op" | "lhs_op": {name: adagrad_noise_slack(...)}}."""
     rel_lr = cfg.relation_lr if cfg.relation_lr is not None else cfg.lr
     inf = float("inf")
 
@@ -106,16 +131,17 @@ def anchored_state(cfg, runner, st, st64, rtol, tag, census=None, loose_rows=Non
         anchored_close(runner.w_rhs, st.w_rhs, st64.w_rhs, rtol, tag + " w_rhs", census, **rows(1, st.w_rhs, loose_steps * cfg.lr))
         anchored_close(runner.g_rhs, st.g_rhs, st64.g_rhs, rtol, tag + " g_rhs", census, **rows(1, st.g_rhs, inf))
 
-    def params(like, bound):
+    def params(like, bound, slack=None):
         if loose_rows is None:
-            return {}
+            return dict(slack=slack)
         return dict(loose=torch.ones_like(like, dtype=torch.bool), loose_bound=bound)
 
     for name in ("rhs_op", "rhs_op_sum", "lhs_op", "lhs_op_sum"):
         got, want, exact = getattr(runner, name), getattr(st, name), getattr(st64, name)
         for k in want:
+            slack = (param_slack or {}).get(name, {}).get(k)
             anchored_close(got[k], want[k], exact[k], rtol, f"{tag} {name}.{k}", census,
-                           **params(want[k], inf if name.endswith("sum") else loose_steps * rel_lr))
+                           **params(want[k], inf if name.endswith("sum") else loose_steps * rel_lr, slack))
     if st.glob_lhs is not None:
         for i, (w, w64, s, s64) in enumerate(((st.glob_lhs, st64.glob_lhs, st.glob_lhs_sum, st64.glob_lhs_sum),
                                               (st.glob_rhs, st64.glob_rhs, st.glob_rhs_sum, st64.glob_rhs_sum))):
@@ -154,3 +180,11 @@ def hinge_tie_rows(cfg, scores, lhs, rhs, uniform_lhs, uniform_rhs, eps=2e-6):
             else:
                 out[side].append(int(uniform[c, j - (chunk if has_batch_negs else 0)]))
     return out
+
+
+def violator_ties(pos, neg):
+    """Negatives whose score equals the positive's up to fp32 rounding of a score
+    (about 1e-6 of the largest score of the batch): `neg > pos` may fall either way."""
+    p = pos.unsqueeze(1)
+    window = 2e-5 * p.abs() + 2e-6 * max(float(neg.abs().max()) if neg.numel() else 0.0, float(pos.abs().max()))
+    return int(((neg - p).abs() <= window).sum())

@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from oracle import step as ostep
-from tests.parity import Census, anchored_state, double_state, hinge_tie_rows, zipf_ids
+from tests.parity import Census, anchored_state, double_state, adagrad_noise_slack, hinge_tie_rows, violator_ties, zipf_ids
 from tests.test_gpu_step import pack, say, to_runner
 
 pytestmark = pytest.mark.gpu
@@ -135,6 +135,11 @@ def test_many_workers_match_the_lockstep_oracle(pbg, name, workers):
             tied[1].extend(rows[1])
         say("  batches with hinge ties", tied_batches, "rows reached", len(set(tied[0])) + len(set(tied[1])))
         assert tied_batches <= workers // 4 and len(tied[0]) + len(tied[1]) <= 200, "too many ties to say anything"
+    # exact operator-parameter gradients of every batch (all batches read the state as it is on entry)
+    grads64 = [ostep.forward_backward(cfg, st64, *b)[1] for b in batches] if (st.rhs_op or st.lhs_op) else []
+    rel_lr = cfg.relation_lr if cfg.relation_lr is not None else cfg.lr
+    slack = {side: {k: adagrad_noise_slack([getattr(g, side)[k] for g in grads64], rel_lr) for k in getattr(st, side)}
+             for side in ("rhs_op", "lhs_op")} if grads64 else None
     runner = to_runner(pbg, cfg, st, num_pos, workers)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
@@ -147,8 +152,7 @@ def test_many_workers_match_the_lockstep_oracle(pbg, name, workers):
         sc = out.scores
         for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
                                      (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
-            p = pos.unsqueeze(1)
-            ties = int(((neg - p).abs() <= 2e-5 * p.abs().clamp_min(1e-6)).sum())
+            ties = violator_ties(pos, neg)
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
     census = Census()
     loose_rows = None
@@ -160,5 +164,5 @@ def test_many_workers_match_the_lockstep_oracle(pbg, name, workers):
             loose_rows[0] |= loose_rows[1]
             loose_rows[1] = loose_rows[0]
     anchored_state(cfg, runner, st, st64, 1e-5, f"{name} K={workers}", census, loose_rows=loose_rows,
-                   loose_steps=2 * tied_batches)
+                   loose_steps=2 * tied_batches, param_slack=slack)
     say("  ", census)

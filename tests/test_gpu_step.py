@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import step as ostep
-from tests.parity import anchored_state, double_state
+from tests.parity import anchored_state, double_state, violator_ties
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -201,8 +201,19 @@ def lockstep(cfg, st, batches, keep_scores=False):
     st64 = double_state(st) if cfg.comparator == "l2" else None
     outs = ostep.train_lockstep(cfg, st, batches, keep_scores=keep_scores)
     if st64 is not None:
-        ostep.train_lockstep(cfg, st64, batches)
+        for out, exact in zip(outs, ostep.train_lockstep(cfg, st64, batches)):
+            out.exact_loss = exact.loss
     return outs, st64
+
+
+def loss_close(got, out, rtol=1e-5):
+    """The batch's loss within rtol of the CPU path's; with l2, where a zero distance
+    evaluates to rounding noise of about 1e-3 (model.py:215-246), alternatively no
+    further from the float64 loss than three times the CPU path's fp32 loss is."""
+    if got == pytest.approx(out.loss, rel=rtol, abs=1e-6):
+        return True
+    exact = getattr(out, "exact_loss", None)
+    return exact is not None and abs(got - exact) <= rtol * abs(exact) + 1e-6 + 3.0 * abs(out.loss - exact)
 
 
 def compare_state(cfg, runner, st, rtol, tag, st64=None):
@@ -278,14 +289,13 @@ def test_train_step(pbg, case, workers):
     outs, st64 = lockstep(cfg, st, batches, keep_scores=True)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
         # a negative that IS the positive's entity ties with it up to rounding: the
         # count is exact except for such ties
         sc = out.scores
         for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
                                      (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
-            p = pos.unsqueeze(1)
-            ties = int(((neg - p).abs() <= 2e-5 * p.abs().clamp_min(1e-6)).sum())
+            ties = violator_ties(pos, neg)
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
     compare_state(cfg, runner, st, rtol, "step", st64)
 
@@ -332,7 +342,7 @@ def test_train_step_with_global_embeddings(pbg, case, workers):
     outs, st64 = lockstep(cfg, st, batches)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
     compare_state(cfg, runner, st, rtol, "step+global", st64)
     assert not torch.equal(st.glob_lhs, zero_glob[0])  # it was trained
 
@@ -387,7 +397,7 @@ def test_train_step_with_max_norm(pbg, case, workers):
     outs, st64 = lockstep(cfg, st, batches)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
     compare_state(cfg, runner, st, rtol, "step+max_norm", st64)
 
 
@@ -490,7 +500,7 @@ def test_train_step_with_all_negs(pbg, case, workers):
     outs, st64 = lockstep(cfg, st, batches)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
     compare_state(cfg, runner, st, rtol, "step+all_negs", st64)
 
 
@@ -537,7 +547,7 @@ def test_train_step_with_edge_weights(pbg, case, workers):
     ostep.train_lockstep(cfg, unweighted, batches)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
     compare_state(cfg, runner, st, rtol, "step+weights", st64)
     # the weights moved the result: the comparison above would not pass without them
     assert (st.w_lhs - unweighted.w_lhs).abs().max() > 1e-3 * st.w_lhs.abs().max()
@@ -615,7 +625,7 @@ def test_train_step_with_n3_regularizer(pbg, case, workers):
     ostep.train_lockstep(plain, st_plain, batches)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
         assert out.reg > 0.0
         assert float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
     compare_state(cfg, runner, st, rtol, "step+N3", st64)
@@ -794,12 +804,11 @@ def test_fused_kernel_shapes(pbg, case):
     outs, st64 = lockstep(cfg, st, batches, keep_scores=True)
     rtol = 1e-5
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=rtol, abs=1e-6), ("loss", k)
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
         sc = out.scores
         for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
                                      (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
-            pp = pos.unsqueeze(1)
-            ties = int(((neg - pp).abs() <= 2e-5 * pp.abs().clamp_min(1e-6)).sum())
+            ties = violator_ties(pos, neg)
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
     compare_state(cfg, runner, st, rtol, "step", st64)
 
