@@ -83,6 +83,20 @@ size_t pbg_row_adagrad_sparse_workspace_bytes(int64_t n);
 int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
                            const int64_t* idx, float* grad_rows, int64_t n, float lr,
                            void* workspace, size_t workspace_bytes, pbg_stream_t stream);
+/* pbg_row_adagrad_sparse without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it).  It has no counterpart in the reference.  The
+ * sort's keys, values and counters live in a device array built into the library
+ * (32 MiB per GPU, held until the process ends): n is limited to
+ * pbg_row_adagrad_sparse_static_max_indices() = 2^20 indices and a larger n
+ * returns PBG_ERR_WORKSPACE.  The call allocates nothing; the first call on a
+ * device looks the array's address up (make it outside a graph capture).  All
+ * calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * two threads) race.  Results are bit-identical to pbg_row_adagrad_sparse. */
+int64_t pbg_row_adagrad_sparse_static_max_indices(void);
+int pbg_row_adagrad_sparse_static(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
+                                  const int64_t* idx, float* grad_rows, int64_t n, float lr,
+                                  pbg_stream_t stream);
 int pbg_row_adagrad_dense(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
                           const float* grad, float lr, pbg_stream_t stream);
 

@@ -77,6 +77,9 @@ SIGNATURES = {
     "pbg_row_adagrad_sparse_workspace_bytes": (c_size_t, [c_int64]),
     "pbg_row_adagrad_sparse": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64,
                                          c_float, c_void_p, c_size_t, c_void_p]),
+    "pbg_row_adagrad_sparse_static_max_indices": (c_int64, []),
+    "pbg_row_adagrad_sparse_static": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64,
+                                                c_float, c_void_p]),
     "pbg_row_adagrad_dense": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_float, c_void_p]),
     "pbg_async_adagrad_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p]),
     "pbg_gemm_f32": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,

@@ -4,6 +4,7 @@
 // dim % 4 == 0 (lane l owns float4 number l, l + 64, ...), so a 400-byte row
 // (dim 100) is one coalesced request of 25 lanes and a 4 KiB row (dim 1024) is
 // four full-wave requests.
+#include <mutex>
 #include "pbg_internal.h"
 #include "row_ops.h"
 
@@ -816,6 +817,62 @@ extern "C" int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t n
   // out-of-range indices were parked at key == num_rows and are skipped by the update
   return row_adagrad_sorted(skeys, svals, n, 0, grad_rows, dim, weight, state_sum, num_rows, nullptr,
                             nullptr, 0, lr, s);
+}
+
+// ---------------------------------------------------------------------------
+// The same step for callers that cannot allocate (HIP graph capture, serving loops):
+// the sort's keys, values and counters live in a file-scope device array instead of
+// a caller-provided workspace.  Every GPU holds its own copy of the array at its own
+// address, looked up once per device; all calls on a GPU share it.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr int64_t kStaticMaxIndices = (int64_t)1 << 20;
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;  // 24 bytes per index + the sort's counters
+constexpr int kMaxDevices = 64;
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (the symbol's name is a host-side
+// stand-in, not an address a kernel can use).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail(PBG_ERR_LAUNCH, "pbg_row_adagrad_sparse_static: hipGetDevice: %s", hipGetErrorString(err));
+  if (dev < 0 || dev >= kMaxDevices) return fail(PBG_ERR_UNSUPPORTED, "pbg_row_adagrad_sparse_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr)
+      return fail(PBG_ERR_LAUNCH, "pbg_row_adagrad_sparse_static: hipGetSymbolAddress: %s", hipGetErrorString(err));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PBG_OK;
+}
+}  // namespace
+
+extern "C" int64_t pbg_row_adagrad_sparse_static_max_indices(void) { return kStaticMaxIndices; }
+
+extern "C" int pbg_row_adagrad_sparse_static(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
+                                             const int64_t* idx, float* grad_rows, int64_t n, float lr,
+                                             pbg_stream_t stream) {
+  if (n > kStaticMaxIndices)
+    return fail(PBG_ERR_WORKSPACE, "pbg_row_adagrad_sparse_static: n = %lld exceeds the built-in scratch (at most %lld indices); "
+                "use pbg_row_adagrad_sparse with a workspace", (long long)n, (long long)kStaticMaxIndices);
+  if (n > 0 && carve_sparse(nullptr, n).total > kStaticScratchBytes)
+    return fail(PBG_ERR_WORKSPACE, "pbg_row_adagrad_sparse_static: n = %lld needs more than the built-in scratch", (long long)n);
+  void* ptr = nullptr;
+  int rc = static_scratch(&ptr);
+  if (rc != PBG_OK) return rc;
+  // The sort clears its own counters and overwrites keys and values before it reads
+  // them, so what the previous call left in the array does not matter.
+  return pbg_row_adagrad_sparse(weight, state_sum, num_rows, dim, idx, grad_rows, n, lr, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int pbg_row_adagrad_dense(float* weight, float* state_sum, int64_t num_rows, int32_t dim,
