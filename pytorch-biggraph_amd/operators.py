@@ -4,7 +4,7 @@ Same registries (``OPERATORS`` / ``DYNAMIC_OPERATORS``), class names,
 constructor signatures, parameter names, shapes and initial values as the
 reference; ``forward`` runs in libpbg_hip (pbg_operator_forward / _backward)
 and is differentiable.  Each class also carries the operator code the fused
-training step uses.  ``affine`` is not provided.
+training step uses.
 """
 from abc import ABC, abstractmethod
 from typing import Optional, Union
