@@ -1246,31 +1246,47 @@ __device__ __forceinline__ void for_each_out(const float4v* acc, int q, F&& fn) 
 // flight while the MFMAs of the current one issue; reads run up to 16 k past the
 // end (the caller's buffers keep finite values there).
 template <int NCT>
-__device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_at, int ldb, int kq, int m, int groups,
-                                             int rest, float4v* acc) {
-  a_at += 4 * kq;
-  b_at += 4 * kq * ldb;
-  float4 a = *reinterpret_cast<const float4*>(&lds[a_at]);
+struct RowOperands {
+  float4 a;
   float b[4][NCT];
+  __device__ __forceinline__ void load(const float* lds, int a_at, int b_at, int ldb, int m) {
+    a = *reinterpret_cast<const float4*>(&lds[a_at]);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + r * ldb, m, b[r]);
-  for (int gk = 0; gk < groups; ++gk) {
-    a_at += 16;
-    b_at += 16 * ldb;
-    const float4 an = *reinterpret_cast<const float4*>(&lds[a_at]);
-    float bn[4][NCT];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + r * ldb, m, bn[r]);
+    for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + r * ldb, m, b[r]);
+  }
+  __device__ __forceinline__ void mma(float4v* acc) const {
     const float av[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
     for (int r = 0; r < 4; ++r)
 #pragma unroll
       for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[r][t], av[r], acc[t], 0, 0, 0);
-    a = an;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int t = 0; t < NCT; ++t) b[r][t] = bn[r][t];
+  }
+};
+
+template <int NCT>
+__device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_at, int ldb, int kq, int m, int groups,
+                                             int rest, float4v* acc) {
+  a_at += 4 * kq;
+  b_at += 4 * kq * ldb;
+  RowOperands<NCT> x, y;  // two operand sets taking turns, see mfma_sweep_k16
+  x.load(lds, a_at, b_at, ldb, m);
+  int gk = 0;
+  for (; gk + 2 <= groups; gk += 2) {
+    y.load(lds, a_at + 16, b_at + 16 * ldb, ldb, m);
+    __builtin_amdgcn_sched_barrier(0);
+    x.mma(acc);
+    __builtin_amdgcn_sched_barrier(0);
+    a_at += 32;
+    b_at += 32 * ldb;
+    x.load(lds, a_at, b_at, ldb, m);
+    __builtin_amdgcn_sched_barrier(0);
+    y.mma(acc);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (gk < groups) {
+    x.mma(acc);
+    a_at += 16;
+    b_at += 16 * ldb;
   }
   a_at -= 3 * kq;
   b_at -= 3 * kq * ldb;
@@ -1288,27 +1304,38 @@ __device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_a
 // acc += A B with A's k along LDS rows too (the transposed score block of the
 // uniform negatives' gradient): the lane's A element of step ks is at a_at +
 // (4 ks + kq) * lda.  Returns the sum of the A elements the lane has fed (its
-// share of a column sum of the score block).
+// share of a column sum of the score block).  Reads up to two steps past the end.
 template <int NCT>
 __device__ __forceinline__ float sweep_a_cols(const float* lds, int a_at, int lda, int b_at, int ldb, int kq, int m,
                                               int ksteps, float4v* acc) {
   a_at += kq * lda;
   b_at += kq * ldb;
-  float a = lds[a_at], asum = 0.f;
-  float b[NCT];
-  load_b<NCT>(lds, b_at, m, b);
-  for (int ks = 0; ks < ksteps; ++ks) {
-    a_at += 4 * lda;
-    b_at += 4 * ldb;
-    const float an = lds[a_at];
-    float bn[NCT];
-    load_b<NCT>(lds, b_at, m, bn);
+  float ax = lds[a_at], ay, asum = 0.f;
+  float bx[NCT], by[NCT];
+  load_b<NCT>(lds, b_at, m, bx);
+  int ks = 0;
+  for (; ks + 2 <= ksteps; ks += 2) {
+    ay = lds[a_at + 4 * lda];
+    load_b<NCT>(lds, b_at + 4 * ldb, m, by);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[t], a, acc[t], 0, 0, 0);
-    asum += a;
-    a = an;
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], ax, acc[t], 0, 0, 0);
+    asum += ax;
+    __builtin_amdgcn_sched_barrier(0);
+    a_at += 8 * lda;
+    b_at += 8 * ldb;
+    ax = lds[a_at];
+    load_b<NCT>(lds, b_at, m, bx);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < NCT; ++t) b[t] = bn[t];
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(by[t], ay, acc[t], 0, 0, 0);
+    asum += ay;
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (ks < ksteps) {
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], ax, acc[t], 0, 0, 0);
+    asum += ax;
   }
   return asum;
 }
@@ -1322,15 +1349,14 @@ __device__ __forceinline__ float sweep_a_cols(const float* lds, int a_at, int ld
 // a_at / b_at address element (row, 0).  Reads up to 15 floats past the last k of
 // a row (never used: the groups cover whole multiples of 16 only).
 template <int T>
-__device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b_at, int b_tile, int groups, int rest,
-                                               int kq, float4v* acc) {
-  a_at += 4 * kq;
-  b_at += 4 * kq;
-  for (int gk = 0; gk < groups; ++gk) {
-    const float4 a = *reinterpret_cast<const float4*>(&lds[a_at]);
-    float4 b[T];
+struct K16Operands {
+  float4 a, b[T];
+  __device__ __forceinline__ void load(const float* lds, int a_at, int b_at, int b_tile) {
+    a = *reinterpret_cast<const float4*>(&lds[a_at]);
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) b[ct] = *reinterpret_cast<const float4*>(&lds[b_at + ct * b_tile]);
+  }
+  __device__ __forceinline__ void mma(float4v* acc) const {
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].x, a.x, acc[ct], 0, 0, 0);
 #pragma unroll
@@ -1339,18 +1365,47 @@ __device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b
     for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].z, a.z, acc[ct], 0, 0, 0);
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].w, a.w, acc[ct], 0, 0, 0);
+  }
+};
+
+template <int T>
+__device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b_at, int b_tile, int groups, int rest,
+                                               int kq, float4v* acc) {
+  a_at += 4 * kq;
+  b_at += 4 * kq;
+  // Two operand sets take turns: the operands of group g + 1 are requested before the
+  // matrix instructions of group g issue, and nothing is copied between the sets.  The
+  // scheduling barriers keep the compiler from sinking the loads down to their first
+  // use, which would expose the LDS latency once per group.
+  K16Operands<T> x, y;
+  x.load(lds, a_at, b_at, b_tile);
+  int gk = 0;
+  for (; gk + 2 <= groups; gk += 2) {
+    y.load(lds, a_at + 16, b_at + 16, b_tile);
+    __builtin_amdgcn_sched_barrier(0);
+    x.mma(acc);
+    __builtin_amdgcn_sched_barrier(0);
+    a_at += 32;
+    b_at += 32;
+    x.load(lds, a_at, b_at, b_tile);
+    __builtin_amdgcn_sched_barrier(0);
+    y.mma(acc);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (gk < groups) {
+    x.mma(acc);
     a_at += 16;
     b_at += 16;
   }
   a_at -= 3 * kq;  // single steps: slot kq holds k = 16 groups + 4 step + kq
   b_at -= 3 * kq;
   for (int ks = 0; ks < rest; ++ks) {
-    const float a = lds[a_at];
-    float b[T];
+    const float a1 = lds[a_at];
+    float b1[T];
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) b[ct] = lds[b_at + ct * b_tile];
+    for (int ct = 0; ct < T; ++ct) b1[ct] = lds[b_at + ct * b_tile];
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct], a, acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b1[ct], a1, acc[ct], 0, 0, 0);
     a_at += 4;
     b_at += 4;
   }
