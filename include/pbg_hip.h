@@ -160,8 +160,7 @@ typedef struct pbg_step_desc {
                              * first renormalised IN THE TABLE to at most this 2-norm (pbg_model_forward
                              * included, as in the reference); 0 = off */
   int32_t bias;             /* config.bias: BiasedComparator around `comparator` (model.py:306-344,902-903): a
-                             * row's first coordinate stays out of the comparator and is added to its scores.
-                             * Not implemented for l2 or with a regularizer (PBG_ERR_UNSUPPORTED) */
+                             * row's first coordinate stays out of the comparator and is added to its scores */
   int32_t all_negs;         /* RelationSchema.all_negs (config.py:123-131; model.py:648-650,582-618): one chunk of all
                              * B positives, negatives = EVERY entity of the side's type in table order (lhs_neg
                              * is [K, B, num_lhs_rows]), the edge's own entity masked; num_batch_negs,

@@ -47,6 +47,7 @@ struct SideCtx {
   float *an, *ap, *aa;  // per-row aux of the above: 1/norm (cos) or squared norm (l2)
   float *bn, *bp, *ba;  // with config.bias: the rows' biases (their first coordinates; the rows hold 0 there)
   float* bs;            // with config.bias: [K*C*P] row sums of dLoss/dscore of this side's score matrix
+  float* gs;            // with config.bias and l2: [K*C, P, nn] dLoss/dscore itself (s then holds -2 dLoss/d squared distance, from which it cannot be read back)
   float *dxn, *dxp, *dxa;
   float* s;             // [K*C, P, nn] scores against this side's negatives, then dLoss/dS
   float* rs;            // [K*C*P] row sums of dLoss/d(squared distance) (l2)
@@ -374,6 +375,8 @@ struct ScoreRow {
     *live = ok;
     return t;
   }
+  // the comparator's own part of a live column's score t: without the pair's biases
+  __device__ __forceinline__ float without_bias(int j, float t) const { return cb ? t - (rb + cb[j]) : t; }
 };
 
 __device__ __forceinline__ void positive_scores(const StepCtx& c, int64_t kc, int i, int lane, float* posv) {
@@ -444,7 +447,7 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
 template <class R>
 __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
                                           float pos, float w, int first, float* loss_acc, float* dpos_out,
-                                          int* viol_out, float* rowsum_out, float* gsum_out) {
+                                          int* viol_out, float* rowsum_out, float* gsum_out, float* gout = nullptr) {
   float dpos_part = 0.f, rowsum = 0.f;
   float gsum = 0.f;  // row sum of dLoss/dscore: the gradient of the positive operand's bias (config.bias)
   int viol = 0;
@@ -498,8 +501,9 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
         if (t > pos) ++viol;
         if (!live_u) g = 0.f;
         gsum += g;
+        if (gout) gout[j] = g;
         if (is_distance(cmp)) {
-          const float dq = !live_u ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / t : -g);
+          const float dq = !live_u ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / sr.without_bias(j, t) : -g);
           rowsum += dq;
           out[j] = -2.0f * dq;
         } else {
@@ -539,11 +543,12 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
     if (t > pos) ++viol;
     if (!live) g = 0.f;
     gsum += g;
+    if (gout) gout[j] = g;
     if (is_distance(cmp)) {
       // t = -sqrt(q): dLoss/dq = g * 0.5 / t (squared_l2, t = -q: -g); stored as
       // -2 dLoss/dq so that the backward GEMMs produce the cross terms of
       // ||a||^2 - 2ab + ||b||^2
-      const float dq = !live ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / t : -g);
+      const float dq = !live ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / sr.without_bias(j, t) : -g);
       rowsum += dq;
       out[j] = -2.0f * dq;
     } else {
@@ -569,6 +574,8 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
       const SideCtx& sd = c.side[s];
       float* row = sd.s + (kc * c.P + i) * sd.nn;
       for (int j = lane; j < sd.nn; j += kWave) row[j] = 0.f;
+      if (sd.gs)
+        for (int j = lane; j < sd.nn; j += kWave) sd.gs[(kc * c.P + i) * sd.nn + j] = 0.f;
       if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = 0.f;
       if (sd.bs && lane == 0) sd.bs[kc * c.P + i] = 0.f;
     }
@@ -608,7 +615,7 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     float* out = sd.s + (kc * c.P + i) * nn;
     float rowsum, gsum;
     side_loss<WaveReduce>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum,
-                          &gsum);
+                          &gsum, sd.gs ? sd.gs + (kc * c.P + i) * nn : nullptr);
     if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = rowsum;
     if (sd.bs && lane == 0) sd.bs[kc * c.P + i] = gsum;
   }
@@ -743,6 +750,13 @@ __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos,
   }
 }
 
+// config.bias: sum over a chunk's rows of dLoss/dscore in column `col` of side sd's score matrix
+// (squared_l2 stores 2 dLoss/dscore in the matrix, l2 keeps dLoss/dscore in a matrix of its own)
+__device__ __forceinline__ float bias_column_sum(const StepCtx& c, const SideCtx& sd, int64_t kc, int col, int lane) {
+  if (sd.gs) return column_sum(sd.gs, kc, c.P, sd.nn, col, lane);
+  return (c.cmp == PBG_CMP_SQUARED_L2 ? 0.5f : 1.0f) * column_sum(sd.s, kc, c.P, sd.nn, col, lane);
+}
+
 template <int NVH>
 __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
   const int lane = threadIdx.x & 63;
@@ -763,8 +777,9 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
   // config.bias: a row's bias enters every score of the row (model.py:332-342), so its gradient is
   // the sum of dLoss/dscore over them: a row sum where the row is the positive operand, a column sum
   // where it is a negative, plus the positive pair's.  It joins the gradient after comparator.prepare,
-  // which passes the first coordinate through.  (squared_l2 stores 2 dLoss/dscore in the matrix.)
-  const float stored = c.cmp == PBG_CMP_SQUARED_L2 ? 0.5f : 1.0f;
+  // which passes the first coordinate through.  With a regularizer the bias is a coordinate of the
+  // regularized row like the others (BiasedComparator.prepare keeps it in the row, model.py:311-314):
+  // it is put back for the N3 term, whose gradient at that coordinate joins the bias's.
 
   if (r < c.B) {
     const int cc = r / c.P, i = r % c.P;
@@ -785,15 +800,21 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
         row_axpy<NVH>(dy, coef, y1);
       }
       const RowV<NVH> other = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
-      add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq]);
+      // (the positive score carries the pair's two biases; the distance's gradient needs the distance)
+      const float pair_bias = c.bias ? sd.bp[kc * sd.stride_p + i] + so.bp[kc * so.stride_p + i] : 0.f;
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq] - pair_bias);
+      float breg = 0.f;
       if (c.reg_coef != 0.f) {  // src_pos / dst_pos of the regularizer are these prepared rows (model.py:784-785,854)
-        const float cubes = wave_sum(n3_term<NVH>(c.op, c.reg_coef, dy, y1));
+        RowV<NVH> yb = y1;
+        if (c.bias) add_to_first<NVH>(yb, sd.bp[kc * sd.stride_p + i], lane);
+        const float cubes = wave_sum(n3_term<NVH>(c.op, c.reg_coef, dy, yb));
+        if (c.bias) breg = take_bias<NVH>(dy, lane);  // (dy carried 0 there: the operand rows do)
         if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
       }
       RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
       if (c.bias) {
-        float db = c.dpos[0][pq];
-        if (sd.nb > 0) db += stored * column_sum(sd.s, kc, c.P, sd.nn, i, lane);
+        float db = c.dpos[0][pq] + breg;
+        if (sd.nb > 0) db += bias_column_sum(c, sd, kc, i, lane);
         if (so.nn > 0) db += so.bs[kc * c.P + i];
         add_to_first<NVH>(dz, db, lane);
       }
@@ -813,15 +834,21 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
         if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, i, lane), y1);
       }
       const RowV<NVH> other = row_load<NVH>(so.xa + (kc * c.P + i) * D, D, H, lane);
-      add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq]);
+      const float pair_bias = c.bias ? sd.bp[kc * sd.stride_p + i] + so.ba[kc * c.P + i] : 0.f;
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq] - pair_bias);
       // the plain row is src_pos of one direction's regularizer, the operated row
       // dst_pos of the other's (model.py:722-754)
-      float cubes = 0.f;
-      if (c.reg_coef != 0.f) cubes = n3_term<NVH>(c.op, c.reg_coef, dy, y1);
+      float cubes = 0.f, breg = 0.f, breg2 = 0.f;
+      if (c.reg_coef != 0.f) {
+        RowV<NVH> yb = y1;
+        if (c.bias) add_to_first<NVH>(yb, sd.bp[kc * sd.stride_p + i], lane);
+        cubes = n3_term<NVH>(c.op, c.reg_coef, dy, yb);
+        if (c.bias) breg = take_bias<NVH>(dy, lane);
+      }
       RowV<NVH> dx = prepare_backward<NVH>(c.cmp, dy, y1, aux1);
       if (c.bias) {
-        float db = c.dpos[s][pq];
-        if (sd.alias) db += stored * column_sum(sd.s, kc, c.P, sd.nn, i, lane);
+        float db = c.dpos[s][pq] + breg;
+        if (sd.alias) db += bias_column_sum(c, sd, kc, i, lane);
         add_to_first<NVH>(dx, db, lane);
       }
       // role 2: the operated row f(op(x)), scored against the other side's negatives
@@ -833,13 +860,18 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
         if (l2) row_axpy<NVH>(dy2, 2.0f * so.rs[kc * c.P + i], y2);
       }
       const RowV<NVH> other2 = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
-      add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq]);
+      const float pair_bias2 = c.bias ? sd.ba[kc * c.P + i] + so.bp[kc * so.stride_p + i] : 0.f;
+      add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq] - pair_bias2);
       if (c.reg_coef != 0.f) {
-        cubes = wave_sum(cubes + n3_term<NVH>(c.op, c.reg_coef, dy2, y2));
+        RowV<NVH> yb2 = y2;
+        if (c.bias) add_to_first<NVH>(yb2, sd.ba[kc * c.P + i], lane);
+        cubes = wave_sum(cubes + n3_term<NVH>(c.op, c.reg_coef, dy2, yb2));
+        if (c.bias) breg2 = take_bias<NVH>(dy2, lane);
         if (lane == 0) c.regrow[((int64_t)k * 2 + s) * c.B + r] = cubes;
       }
       RowV<NVH> dz2 = prepare_backward<NVH>(c.cmp, dy2, y2, aux2);
-      if (c.bias) add_to_first<NVH>(dz2, c.dpos[1 - s][pq] + (sd.opd_written ? so.bs[kc * c.P + i] : 0.f), lane);
+      if (c.bias)
+        add_to_first<NVH>(dz2, c.dpos[1 - s][pq] + breg2 + (sd.opd_written ? so.bs[kc * c.P + i] : 0.f), lane);
       if (keep_dz) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + r) * D, dz2, D, H, lane);
       if (c.op != PBG_OP_LINEAR) {
         const RowV<NVH> dx2 = op_backward<NVH>(c.op, dz2, sd.p0, sd.p1, rel, D, H, lane);
@@ -859,7 +891,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
     RowV<NVH> dy = row_load<NVH>(sd.dxn + (kc * sd.nn + col) * D, D, H, lane);
     if (l2) row_axpy<NVH>(dy, -column_sum(sd.s, kc, c.P, sd.nn, col, lane), y);
     RowV<NVH> dz = prepare_backward<NVH>(c.cmp, dy, y, sd.an ? sd.an[kc * sd.nn + col] : 0.f);
-    if (c.bias) add_to_first<NVH>(dz, stored * column_sum(sd.s, kc, c.P, sd.nn, col, lane), lane);
+    if (c.bias) add_to_first<NVH>(dz, bias_column_sum(c, sd, kc, col, lane), lane);
     if (sd.op_uniform) {
       const int64_t rel = clamp_index(c.rel[k], c.num_relations);
       if (keep_dz && !sd.uni_dz_direct) row_store<NVH>(sd.dz + ((int64_t)k * sd.op_rows + c.B + r2) * D, dz, D, H, lane);
@@ -2275,10 +2307,6 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->num_lhs_rows < 1 || d->num_rhs_rows < 1) return fail(PBG_ERR_INVALID, "step: empty table");
   if (d->bias) {
     if (d->dim < 2) return fail(PBG_ERR_INVALID, "step: bias needs at least two coordinates");
-    // -sqrt(q) stores dLoss/dq in the score matrix, from which the sums of dLoss/dscore cannot be read back
-    if (d->comparator == PBG_CMP_L2) return fail(PBG_ERR_UNSUPPORTED, "step: bias is not implemented for the l2 comparator");
-    // (the regularizer would need the bias coordinate of the prepared rows, which is kept aside)
-    if (d->regularization_coef != 0.f) return fail(PBG_ERR_UNSUPPORTED, "step: bias is not implemented with a regularizer");
   }
   return PBG_OK;
 }
@@ -2376,6 +2404,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
       if (c.bias) {
         sd.bn = takef(KC * sd.nn);
         sd.bs = takef(KC * P);
+        if (c.cmp == PBG_CMP_L2) sd.gs = takef(KC * P * sd.nn);
       }
     }
     if (sd.alias) {

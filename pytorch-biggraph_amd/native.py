@@ -212,7 +212,7 @@ class StepSpec:
     relation_lr: Optional[float] = None
     regularization_coef: float = 0.0  # config.regularization_coef of the N3 regularizer; 0 = none
     max_norm: Optional[float] = None  # config.max_norm: looked-up rows are first renormalised in the table
-    bias: bool = False  # config.bias: BiasedComparator around the comparator (not with l2 or a regularizer)
+    bias: bool = False  # config.bias: BiasedComparator around the comparator
     # RelationSchema.all_negs: one chunk, every entity of a side's type is a negative (model.py:648-650,582-618)
     all_negs: bool = False
 

@@ -72,11 +72,12 @@ def test_newer_step_fields_are_validated_without_a_gpu(pbg):
     size = lambda d: lib.pbg_train_step_workspace_bytes(ctypes.byref(d))
     plain = size(desc())
     assert plain > 0
-    # bias: not with l2, not with a regularizer, not with a single coordinate
-    assert size(desc(bias=1)) > 0
-    assert size(desc(bias=1, comparator=L.COMPARATOR_CODES["l2"])) == 0 and b"bias" in lib.pbg_last_error()
-    assert size(desc(bias=1, regularization_coef=0.1, op=L.OPERATOR_CODES["diagonal"])) == 0
-    assert size(desc(bias=1, dim=1)) == 0
+    # bias: with every comparator (l2 keeps dLoss/dscore in a matrix of its own) and with a regularizer,
+    # not with a single coordinate
+    assert size(desc(bias=1)) > plain
+    assert size(desc(bias=1, comparator=L.COMPARATOR_CODES["l2"])) > size(desc(bias=1, comparator=L.COMPARATOR_CODES["squared_l2"]))
+    assert size(desc(bias=1, regularization_coef=0.1, op=L.OPERATOR_CODES["diagonal"])) > 0
+    assert size(desc(bias=1, dim=1)) == 0 and b"bias" in lib.pbg_last_error()
     # affine: two parameter slots, no regularizer (operators.py:40)
     assert size(desc(op=L.OPERATOR_CODES["affine"])) > plain
     assert size(desc(op=L.OPERATOR_CODES["affine"], regularization_coef=0.1)) == 0

@@ -17,13 +17,14 @@ from tests.test_gpu_step import compare_scores, compare_state, lockstep, make_in
 pytestmark = pytest.mark.gpu
 
 
-def sample_case(rng):
+def sample_case(rng, wide=False):
+    """wide: also bias with l2 and bias with the regularizer."""
     op = rng.choice(ostep.OPERATOR_NAMES)
     cmp_ = rng.choice(ostep.COMPARATOR_NAMES)
     dyn = rng.random() < 0.4
-    bias = rng.random() < 0.3 and cmp_ != "l2"
+    bias = rng.random() < (0.5 if wide else 0.3) and (wide or cmp_ != "l2")
     glob = (not dyn) and rng.random() < 0.3
-    reg = 0.02 if (rng.random() < 0.2 and op not in ("linear", "affine", "none") and not bias) else 0.0
+    reg = 0.02 if (rng.random() < (0.4 if wide else 0.2) and op not in ("linear", "affine", "none") and (wide or not bias)) else 0.0
     dim = rng.choice([6, 8, 12, 16, 24, 32, 100, 128])
     nb, nu = rng.choice([0, 4, 10, 50]), rng.choice([0, 3, 10, 50])
     if nb == 0 and nu == 0:
@@ -41,10 +42,12 @@ def sample_case(rng):
 
 def cases():
     rng = random.Random(20240607)
-    return [sample_case(rng) for _ in range(120)]
+    first = [sample_case(rng) for _ in range(120)]
+    rng = random.Random(20241125)
+    return first + [sample_case(rng, wide=True) for _ in range(40)]
 
 
-@pytest.mark.parametrize("index", range(120))
+@pytest.mark.parametrize("index", range(160))
 def test_random_combination(pbg, index):
     kw, extra = cases()[index]
     say("combination", index, kw, extra)

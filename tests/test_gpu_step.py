@@ -421,6 +421,26 @@ BIAS_CASES = [
          dim=9, disable_lhs_negs=True),
     dict(operator="none", comparator="dot", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
          global_emb=True),  # (a global embedding's first element is such a common shift too)
+    # l2: the score matrix holds dLoss/d(squared distance), so dLoss/dscore is kept beside it for the biases' sums
+    dict(operator="none", comparator="l2", loss="logistic", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=100, shared=False),
+    dict(operator="diagonal", comparator="l2", loss="ranking", num_batch_negs=20, num_uniform_negs=10, num_pos=45, dim=32),
+    dict(operator="complex_diagonal", comparator="l2", loss="softmax", num_batch_negs=10, num_uniform_negs=100, num_pos=33, dim=16,
+         shared=False),
+    dict(operator="linear", comparator="l2", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=10, num_pos=45,
+         dim=24),
+    dict(operator="diagonal", comparator="l2", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=6, num_pos=21,
+         dim=10, disable_lhs_negs=True),
+    # with the N3 regularizer: the bias is a coordinate of the regularized row (model.py:311-314, regularizers.py:82-97)
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=100, num_pos=130,
+         dim=400, regularization_coef=1e-3),
+    dict(operator="diagonal", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
+         regularization_coef=0.05, shared=False),
+    dict(operator="diagonal", comparator="l2", loss="ranking", num_batch_negs=8, num_uniform_negs=4, num_pos=30, dim=10,
+         regularization_coef=0.05),
+    dict(operator="complex_diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=20, num_uniform_negs=10,
+         num_pos=70, dim=32, regularization_coef=1e-2),
+    dict(operator="translation", comparator="squared_l2", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=0,
+         num_pos=45, dim=12, regularization_coef=0.02, disable_rhs_negs=True),
     # one relation per edge
     dict(operator="translation", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=5,
          num_pos=33, dim=16),
@@ -457,10 +477,12 @@ def test_train_step_with_bias(pbg, case, workers):
         compare_scores(cfg, tuple(t[k] for t in got), want.scores)
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs = ostep.train_lockstep(cfg, st, batches)
+    outs, st64 = lockstep(cfg, st, batches)
     for k, out in enumerate(outs):
-        assert float(runner.loss_out[k]) == pytest.approx(out.loss, rel=1e-5, abs=1e-6), ("loss", k)
-    compare_state(cfg, runner, st, 1e-5, "step+bias")
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
+        if cfg.regularization_coef:
+            assert out.reg > 0.0 and float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
+    compare_state(cfg, runner, st, 1e-5, "step+bias", st64)
 
 
 ALL_NEGS_CASES = [
@@ -557,15 +579,6 @@ def test_train_step_with_edge_weights(pbg, case, workers):
     for bad, err in ((good.cpu(), TypeError), (good.double(), TypeError), (good.flatten()[:-1], ValueError)):
         with pytest.raises(err):
             runner.train(lhs, rhs, rel, ul, ur, edge_weight=bad)
-
-
-def test_bias_is_refused_where_it_is_not_implemented(pbg):
-    w = torch.randn(20, 8, device=DEV)
-    for kw in (dict(comparator="l2"), dict(regularization_coef=0.1, operator="diagonal")):
-        spec = pbg.StepSpec(dim=8, batch_size=10, bias=True, **kw)
-        op = {"diagonal": torch.ones(1, 8, device=DEV)} if "operator" in kw else {}
-        with pytest.raises(NotImplementedError, match="bias is not implemented"):
-            pbg.StepRunner(spec, w, torch.zeros(20, device=DEV), rhs_op=op, rhs_op_sum={k: torch.zeros_like(v) for k, v in op.items()})
 
 
 def test_global_embeddings_are_refused_for_dynamic_relations(pbg):
