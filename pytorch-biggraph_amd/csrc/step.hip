@@ -438,83 +438,83 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   return sr;
 }
 
-// Loss of one positive against one side's nn negatives, computed by the group
-// of lanes R describes (a wave, or a quad); `first` is the lane's index in the
-// group.  Adds the unweighted per-lane loss partial to *loss_acc, overwrites the
-// score row with dLoss/dscore (l2: -2 dLoss/d squared distance) and returns the
-// group-reduced dLoss/dpos, violator count and (l2) row sum of dLoss/d squared
-// distance.
-template <class R>
-__device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
-                                          float pos, float w, int first, float* loss_acc, float* dpos_out,
-                                          int* viol_out, float* rowsum_out, float* gsum_out, float* gout = nullptr) {
-  float dpos_part = 0.f, rowsum = 0.f;
-  float gsum = 0.f;  // row sum of dLoss/dscore: the gradient of the positive operand's bias (config.bias)
-  int viol = 0;
-  float mx = pos, inv_z = 0.f;
-  const float inv_nn = 1.0f / (float)nn;
-  // softmax makes three passes over the row; a wave keeps a row of up to
-  // kWave * kSoftmaxCache scores in registers after the first
-  constexpr int kSoftmaxCache = 20;
-  const bool cached = loss == PBG_LOSS_SOFTMAX && R::kStep == kWave && nn <= kWave * kSoftmaxCache;
-  float held[kSoftmaxCache];
-  unsigned held_live = 0u;
-  if (loss == PBG_LOSS_SOFTMAX) {
-    bool live;
-    if (cached) {
+// Loss of one positive against one side's nn negatives, computed by one wave
+// (lane `first` owns columns first, first + 64, ...).  Adds the unweighted per-lane
+// loss partial to *loss_acc, overwrites the score row with dLoss/dscore (l2: -2
+// dLoss/d squared distance) and returns the wave-reduced dLoss/dpos, violator count,
+// (l2) row sum of dLoss/d squared distance and row sum of dLoss/dscore.
+//
+// Rows of up to 64 * DEPTH columns are read ONCE, with all of a lane's loads in
+// flight together: the loads are issued from straight-line code at clamped
+// (always valid) columns and what lies past the row is dropped afterwards -- a load
+// inside a branch would make the code after the branch wait for it, one load
+// after the other.  Every pass of the loss then runs over registers.
+template <int DEPTH, bool DIST>  // DIST: a distance comparator (l2, squared_l2)
+__device__ __forceinline__ void side_loss_held(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
+                                               float pos, float w, int first, float* loss_acc, float* dpos_out,
+                                               int* viol_out, float* rowsum_out, float* gsum_out, float* gout) {
+  float t[DEPTH];
+  float half_inv[DIST ? DEPTH : 1];  // l2: 0.5 / (the distance score without the pair's biases), the slope of -sqrt
+  unsigned live_bits = 0u;
+  {
+    float raw[DEPTH];
 #pragma unroll
-      for (int u = 0; u < kSoftmaxCache; ++u) {
-        const int j = first + u * kWave;
-        held[u] = -INFINITY;
-        if (j < nn) {
-          held[u] = sr.at(j, &live);
-          held_live |= live ? 1u << u : 0u;
-          mx = fmaxf(mx, held[u]);
+    for (int u = 0; u < DEPTH; ++u) raw[u] = sr.raw[min(first + u * kWave, nn - 1)];
+    if (DIST) {
+      float bn[DEPTH];
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) bn[u] = sr.bn[min(first + u * kWave, nn - 1)];
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) {
+        const float qd = fmaf(-2.0f, raw[u], bn[u]) + sr.a2;
+        if (cmp == PBG_CMP_L2) {
+          if (qd >= 1e-30f) live_bits |= 1u << u;
+          raw[u] = -sqrtf(fmaxf(qd, 1e-30f));
+          half_inv[DIST ? u : 0] = 0.5f / raw[u];
+        } else {
+          live_bits |= 1u << u;
+          raw[u] = -qd;
         }
       }
     } else {
-      for (int j = first; j < nn; j += R::kStep) mx = fmaxf(mx, sr.at(j, &live));
+      live_bits = 0xffffffffu;
     }
-    mx = R::max(mx);
-    float z = 0.f;
-    if (cached) {
+    if (sr.cb) {  // model.py:338-342
+      float cb[DEPTH];
 #pragma unroll
-      for (int u = 0; u < kSoftmaxCache; ++u)
-        if (first + u * kWave < nn) z += expf(held[u] - mx);
-    } else {
-      for (int j = first; j < nn; j += R::kStep) z += expf(sr.at(j, &live) - mx);
+      for (int u = 0; u < DEPTH; ++u) cb[u] = sr.cb[min(first + u * kWave, nn - 1)];
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) raw[u] += sr.rb + cb[u];
     }
-    z = R::sum(z) + expf(pos - mx);
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const int j = first + u * kWave;
+      t[u] = raw[u];
+      if ((j < sr.nb && (j == sr.i || j >= sr.masked_from)) || j == sr.own) {
+        t[u] = -1e9f;
+        live_bits &= ~(1u << u);
+      }
+      if (j >= nn) {  // past the row: a score of -inf adds nothing to any loss
+        t[u] = -INFINITY;
+        live_bits &= ~(1u << u);
+      }
+    }
+  }
+  float dpos_part = 0.f, rowsum = 0.f, gsum = 0.f, mx = pos, inv_z = 0.f;
+  int viol = 0;
+  const float inv_nn = 1.0f / (float)nn;
+  if (loss == PBG_LOSS_SOFTMAX) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) mx = fmaxf(mx, t[u]);
+    mx = wave_max(mx);
+    float z = 0.f;
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) z += expf(t[u] - mx);
+    z = wave_sum(z) + expf(pos - mx);
     inv_z = 1.0f / z;
     if (first == 0) {
       *loss_acc += (mx + logf(z)) - pos;
       dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
-    }
-    if (cached) {  // third pass from the registers
-#pragma unroll
-      for (int u = 0; u < kSoftmaxCache; ++u) {
-        const int j = first + u * kWave;
-        if (j >= nn) continue;
-        const float t = held[u];
-        const bool live_u = (held_live >> u) & 1u;
-        float g = expf(t - mx) * inv_z * w;
-        if (t > pos) ++viol;
-        if (!live_u) g = 0.f;
-        gsum += g;
-        if (gout) gout[j] = g;
-        if (is_distance(cmp)) {
-          const float dq = !live_u ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / sr.without_bias(j, t) : -g);
-          rowsum += dq;
-          out[j] = -2.0f * dq;
-        } else {
-          out[j] = g;
-        }
-      }
-      *dpos_out = R::sum(dpos_part);
-      *rowsum_out = R::sum(rowsum);
-      *gsum_out = R::sum(gsum);
-      *viol_out = R::sum_int(viol);
-      return;
     }
   } else if (loss == PBG_LOSS_LOGISTIC) {
     if (first == 0) {
@@ -522,13 +522,78 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
       dpos_part += (sigmoidf(pos) - 1.0f) * w;
     }
   }
-  for (int j = first; j < nn; j += R::kStep) {
-    bool live;
-    const float t = sr.at(j, &live);
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) {
+    const int j = first + u * kWave;
+    const float tu = t[u];
+    const bool live = (live_bits >> u) & 1u;
     float g;
     if (loss == PBG_LOSS_RANKING) {
       // F.margin_ranking_loss(neg, pos, target=-1): max(0, (t - pos) + margin); the
       // clamp lets the gradient through at exactly 0
+      const float x = (tu - pos) + margin;
+      if (x > 0.f) *loss_acc += x;
+      g = (x >= 0.f) ? w : 0.f;
+      dpos_part -= g;
+    } else if (loss == PBG_LOSS_LOGISTIC) {
+      float sg;
+      *loss_acc += softplus_sigmoid(tu, &sg) * inv_nn;
+      g = sg * inv_nn * w;
+    } else {
+      g = expf(tu - mx) * inv_z * w;
+    }
+    if (tu > pos) ++viol;
+    if (!live) g = 0.f;
+    gsum += g;
+    float stored = g;
+    if (DIST) {
+      // t = -sqrt(q): dLoss/dq = g * 0.5 / t (squared_l2, t = -q: -g); stored as
+      // -2 dLoss/dq so that the backward GEMMs produce the cross terms of
+      // ||a||^2 - 2ab + ||b||^2
+      const float dq = !live ? 0.f : (cmp == PBG_CMP_L2 ? g * half_inv[DIST ? u : 0] : -g);
+      rowsum += dq;
+      stored = -2.0f * dq;
+    }
+    if (j < nn) {
+      out[j] = stored;
+      if (gout) gout[j] = g;
+    }
+  }
+  *dpos_out = wave_sum(dpos_part);
+  *rowsum_out = wave_sum(rowsum);
+  *gsum_out = wave_sum(gsum);
+  *viol_out = wave_sum_int(viol);
+}
+
+// The same for rows of any length: the row is read once per pass of the loss.
+__device__ __forceinline__ void side_loss_long(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn,
+                                               float pos, float w, int first, float* loss_acc, float* dpos_out,
+                                               int* viol_out, float* rowsum_out, float* gsum_out, float* gout) {
+  float dpos_part = 0.f, rowsum = 0.f, gsum = 0.f, mx = pos, inv_z = 0.f;
+  int viol = 0;
+  const float inv_nn = 1.0f / (float)nn;
+  bool live;
+  if (loss == PBG_LOSS_SOFTMAX) {
+    for (int j = first; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
+    mx = wave_max(mx);
+    float z = 0.f;
+    for (int j = first; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
+    z = wave_sum(z) + expf(pos - mx);
+    inv_z = 1.0f / z;
+    if (first == 0) {
+      *loss_acc += (mx + logf(z)) - pos;
+      dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+    }
+  } else if (loss == PBG_LOSS_LOGISTIC) {
+    if (first == 0) {
+      *loss_acc += softplusf(-pos);
+      dpos_part += (sigmoidf(pos) - 1.0f) * w;
+    }
+  }
+  for (int j = first; j < nn; j += kWave) {
+    const float t = sr.at(j, &live);
+    float g;
+    if (loss == PBG_LOSS_RANKING) {
       const float x = (t - pos) + margin;
       if (x > 0.f) *loss_acc += x;
       g = (x >= 0.f) ? w : 0.f;
@@ -545,9 +610,6 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
     gsum += g;
     if (gout) gout[j] = g;
     if (is_distance(cmp)) {
-      // t = -sqrt(q): dLoss/dq = g * 0.5 / t (squared_l2, t = -q: -g); stored as
-      // -2 dLoss/dq so that the backward GEMMs produce the cross terms of
-      // ||a||^2 - 2ab + ||b||^2
       const float dq = !live ? 0.f : (cmp == PBG_CMP_L2 ? g * 0.5f / sr.without_bias(j, t) : -g);
       rowsum += dq;
       out[j] = -2.0f * dq;
@@ -555,12 +617,28 @@ __device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const
       out[j] = g;
     }
   }
-  *dpos_out = R::sum(dpos_part);
-  *rowsum_out = R::sum(rowsum);
-  *gsum_out = R::sum(gsum);
-  *viol_out = R::sum_int(viol);
+  *dpos_out = wave_sum(dpos_part);
+  *rowsum_out = wave_sum(rowsum);
+  *gsum_out = wave_sum(gsum);
+  *viol_out = wave_sum_int(viol);
 }
 
+// DEPTH: 0 = rows of any length, else rows of at most 64 * DEPTH columns
+template <int DEPTH, bool DIST>
+__device__ __forceinline__ void side_loss(int loss, float margin, int cmp, const ScoreRow& sr, float* out, int nn, float pos,
+                                          float w, int first, float* loss_acc, float* dpos_out, int* viol_out,
+                                          float* rowsum_out, float* gsum_out, float* gout) {
+  if (DEPTH > 0)
+    side_loss_held<(DEPTH > 0 ? DEPTH : 1), DIST>(loss, margin, cmp, sr, out, nn, pos, w, first, loss_acc, dpos_out, viol_out,
+                                                  rowsum_out, gsum_out, gout);
+  else
+    side_loss_long(loss, margin, cmp, sr, out, nn, pos, w, first, loss_acc, dpos_out, viol_out, rowsum_out, gsum_out, gout);
+}
+
+// One kernel per row length class and comparator class: a lane's registers (and with
+// them the number of waves a compute unit keeps in flight to hide the memory latency
+// of the per-edge reads) follow the longest row the kernel accepts.
+template <int DEPTH, bool DIST>
 __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
   const int lane = threadIdx.x & 63;
   const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
@@ -614,7 +692,7 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
     ScoreRow sr = score_row(c, s, kc, cc, i);
     float* out = sd.s + (kc * c.P + i) * nn;
     float rowsum, gsum;
-    side_loss<WaveReduce>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum,
+    side_loss<DEPTH, DIST>(c.loss, c.margin, c.cmp, sr, out, nn, pos, w, lane, &loss_acc, &dposv[s], &violv[s], &rowsum,
                           &gsum, sd.gs ? sd.gs + (kc * c.P + i) * nn : nullptr);
     if (sd.rs && lane == 0) sd.rs[kc * c.P + i] = rowsum;
     if (sd.bs && lane == 0) sd.bs[kc * c.P + i] = gsum;
@@ -2905,6 +2983,21 @@ int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s) {
             : launch_fused_loss<8, PBG_CMP_DOT, 0>(plan, lds_bytes, s);
 }
 
+template <int DEPTH>
+void launch_loss_depth(const StepCtx& c, hipStream_t s) {
+  const dim3 grid = wave_grid((int64_t)c.K * c.C * c.P);
+  if (is_distance(c.cmp)) hipLaunchKernelGGL((loss_kernel<DEPTH, true>), grid, dim3(kRowThreads), 0, s, c);
+  else hipLaunchKernelGGL((loss_kernel<DEPTH, false>), grid, dim3(kRowThreads), 0, s, c);
+}
+
+void launch_loss(const StepCtx& c, hipStream_t s) {
+  const int nn = c.side[0].nn > c.side[1].nn ? c.side[0].nn : c.side[1].nn;
+  if (nn <= 4 * kWave) launch_loss_depth<4>(c, s);
+  else if (nn <= 8 * kWave) launch_loss_depth<8>(c, s);
+  else if (nn <= 20 * kWave) launch_loss_depth<20>(c, s);
+  else launch_loss_depth<0>(c, s);
+}
+
 int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_t s, hipEvent_t* ev) {
   int rc = validate(desc, true);
   if (rc != PBG_OK) return rc;
@@ -2937,7 +3030,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(2);
     if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
     mark(3);
-    hipLaunchKernelGGL(loss_kernel, wave_grid((int64_t)c.K * c.C * c.P), dim3(kRowThreads), 0, s, c);
+    launch_loss(c, s);
     hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
     mark(4);
     if ((rc = run_backward_dn(plan, s)) != PBG_OK) return rc;
