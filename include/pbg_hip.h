@@ -234,6 +234,18 @@ int pbg_train_step_num_stages(void);
  * stage 0 is that kernel and stages 1-6 are empty), 0 when it runs the staged
  * kernels.  No counterpart in the reference. */
 int pbg_train_step_is_fused(const pbg_step_desc* desc);
+/* Which kernels pbg_train_step runs for this configuration (-1: the descriptor
+ * is invalid): the staged chain, the one fused kernel above, or the streaming
+ * route -- a chunk's positives resident in LDS, its negatives gathered raw from
+ * the table and streamed past them in tiles, twice (scores and loss statistics,
+ * then both gradient products), with stage 0 the per-edge preparation, stage 2
+ * that kernel and stage 6 the per-edge finish.  A call whose buffers carry global
+ * embeddings runs the staged chain where this says streaming.  No counterpart in
+ * the reference. */
+#define PBG_ROUTE_STAGED 0
+#define PBG_ROUTE_FUSED 1
+#define PBG_ROUTE_STREAM 2
+int pbg_train_step_route(const pbg_step_desc* desc);
 int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,
                            float* stage_ms);
 

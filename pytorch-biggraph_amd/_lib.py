@@ -91,6 +91,7 @@ SIGNATURES = {
     "pbg_train_step": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p]),
     "pbg_train_step_num_stages": (c_int32, []),
     "pbg_train_step_is_fused": (c_int32, [POINTER(StepDesc)]),
+    "pbg_train_step_route": (c_int32, [POINTER(StepDesc)]),
     "pbg_train_step_profile": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, POINTER(c_float)]),
     "pbg_model_forward": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),

@@ -24,86 +24,15 @@
 
 #include "pbg_internal.h"
 #include "row_ops.h"
+#include "step_ctx.h"
+#include "mfma_tiles.h"
+#include "stream.h"
 
 namespace pbg {
 namespace {
 
 constexpr int kRowThreads = 256;
 constexpr int kWavesPerBlock = kRowThreads / kWave;
-
-struct SideCtx {
-  const float* w;       // embedding table of this side
-  const float* glob;    // global embedding of this side's entity type [D], or null
-  const int64_t* idx;   // [K, B] positive entities
-  const int64_t* uidx;  // [K, C, U] uniform negatives (null if u == 0, or if they are drawn in the step)
-  uint64_t useed;       // seed of the in-step draw (uidx == null)
-  int64_t key_base;     // offset of this table in the sort-key row space
-  int64_t num_rows;
-  int all;              // RelationSchema.all_negs: the negatives are the table's rows 0 .. num_rows - 1 (u == num_rows)
-  int nb, u, nn;        // batch-negative / uniform / total negative columns of this side
-  int stride_p;         // rows per chunk of the buffer that holds the positives
-  int alias;            // positives are the first P rows of the negatives matrix
-  float *xn, *xp, *xa;  // prepared negatives matrix, positives, operated positives (dynamic)
-  float *an, *ap, *aa;  // per-row aux of the above: 1/norm (cos) or squared norm (l2)
-  float *bn, *bp, *ba;  // with config.bias: the rows' biases (their first coordinates; the rows hold 0 there)
-  float* bs;            // with config.bias: [K*C*P] row sums of dLoss/dscore of this side's score matrix
-  float* gs;            // with config.bias and l2: [K*C, P, nn] dLoss/dscore itself (s then holds -2 dLoss/d squared distance, from which it cannot be read back)
-  float *dxn, *dxp, *dxa;
-  float* s;             // [K*C, P, nn] scores against this side's negatives, then dLoss/dS
-  float* rs;            // [K*C*P] row sums of dLoss/d(squared distance) (l2)
-  int slot_pos, slot_uni;
-  // The gradient rows of this side's uniform negatives are read where the backward GEMM wrote them
-  // (dxn, which then lies behind gr in one block; uni_row0 = row number of dxn's first row counted from gr):
-  // with the dot comparator and no operator on them the raw-row gradient IS that row.
-  int uni_direct;
-  int64_t uni_row0;
-  // (operator side, element-wise operator, dot comparator:) the gradient at the operator's output of a uniform
-  // negative IS its row of dxn; it is not copied to dz, the parameter gradient reads it there
-  int uni_dz_direct;
-  int has_op;           // an operator acts on this side's positives
-  int op_uniform;       // ... and on its uniform negatives (standard mode)
-  const float *p0, *p1; // operator parameters
-  float *xraw, *z, *dz; // [K, op_rows, D] staging of operator inputs / outputs / output grads
-  int op_rows;
-  // N3 regularizer, dynamic relations: per relation, the gradient of the parameter
-  // term per edge [num_relations, D] and the term itself [num_relations], both
-  // from the parameters as they are before the call's updates
-  float *reg_pgrad, *reg_pcube;
-  int plain_written, opd_written;  // dxp / dxa were produced by a GEMM
-};
-
-struct StepCtx {
-  int D, K, B, P, C, U, last, dynamic, op, cmp, loss, num_relations;
-  int bias;    // config.bias: BiasedComparator around the comparator (model.py:306-344,902-903)
-  int affine;  // op == PBG_OP_LINEAR with a translation added to the product (operators.py:103-115, 272-293)
-  float margin;
-  SideCtx side[2];
-  const int64_t* rel;
-  const float* edge_weight;
-  const float* rel_weights;
-  float* pos[2];   // [K*C*P] positive score paired with lhs negatives / rhs negatives
-  float* dpos[2];  // gradients of the above (standard mode: only [0], already summed)
-  float* lossrow;  // [K*C*P]
-  int* violrow;    // [K*C*P, 2] violators of each edge (lhs, rhs)
-  int rk;          // gradient rows per batch
-  int kbits;
-  float* gr;       // [K*rk, D] gradient rows
-  uint64_t* keys;
-  uint32_t* vals;
-  unsigned long long* violators;  // [K, 2]
-  float* loss_out;                // [K]
-  float reg_coef;  // N3 regularizer weight (0: none)
-  float* regrow;   // [K, 2, B] sum of cubed moduli of each positive's prepared row(s), per side
-  float* reg_out;  // [K] or null
-};
-
-// Uniform negative number flat = (k * C + chunk) * U + u of side s: given by the
-// caller or drawn here (model.py:70-75).
-__device__ __forceinline__ int64_t uniform_negative(const SideCtx& sd, int s, int64_t flat) {
-  if (sd.all) return flat % sd.u;  // (one chunk: flat = batch * u + entity)
-  if (sd.uidx) return sd.uidx[flat];
-  return sampled_row(sd.useed, (uint64_t)flat, (uint32_t)s, sd.num_rows);
-}
 
 // x + the global embedding of the side's entity type (model.py:486-492)
 template <int NVH>
@@ -1160,7 +1089,6 @@ __global__ __launch_bounds__(kRowThreads) void param_update_wave_kernel(StepCtx 
 // The kernel is instantiated per comparator and loss and keeps its straight-line
 // parts short: a workgroup runs every instruction once, so code that does not
 // fit the instruction cache is paid for in fetch stalls by every workgroup.
-typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kFusedThreads = 512;
 constexpr int kFusedIds = 256;  // slots of the row id array: 8 waves x 16 rounds x 2 half-waves
 constexpr int kFusedSide = kFusedIds / 2;  // ... per side
@@ -1172,20 +1100,6 @@ struct FusedLayout {
   int ids;                       // int32 row ids of the 2N operand rows (-1: padding), kFusedIds slots; last block
   int total;                     // floats
 };
-
-// reductions over 8 adjacent lanes, result in every lane of the group
-__device__ __forceinline__ float oct_sum(float v) {
-  v = quad_sum(v);
-  return v + dpp_f<kDppRowHalfMirror>(0.f, v);  // lane i of a half-row takes lane 7 - i: the other quad
-}
-__device__ __forceinline__ float oct_max(float v) {
-  v = quad_max(v);
-  return fmaxf(v, dpp_f<kDppRowHalfMirror>(v, v));
-}
-__device__ __forceinline__ int oct_sum_int(int v) {
-  v = quad_sum_int(v);
-  return v + dpp_i<kDppRowHalfMirror, 0xf, 0xf>(0, v);
-}
 
 // Loss of one positive against one side's negatives for a score row held in LDS
 // and spread over 8 adjacent lanes: lane qd owns columns qd, qd + 8, ..., `ne` of
@@ -1300,227 +1214,6 @@ __device__ __forceinline__ void fused_row_loss(float* lds, int row_at, int bn_at
   *viol_out = oct_sum_int(viol);
 }
 
-// ---- MFMA products of the fused kernel ----
-// Every product is formed as (B^T A^T): the instruction's first operand comes
-// from B, so a lane ends up with four consecutive values of ONE row of A B.
-//
-// B operand of one k-step when k runs along B's LDS rows (the gradient products:
-// B = a side's operand rows, columns = embedding coordinates).  A wave covers NCT
-// column tiles starting at a multiple of 16.  Which 16 columns form a tile is
-// free as long as the results are read back the same way, so lane m = lane & 15
-// reads NCT consecutive floats with ONE wide load, at a place chosen so that the
-// results leave the wave in 64-byte runs: the instruction's row index i = m ends
-// up as i = 4q + r in lane group q, result register r, and a lane stores four
-// results of four registers as one 128-bit word.
-//   4-tile part: lane m reads columns 16 (m & 3) + 4 (m >> 2) + t, t = 0..3 (tile t)
-//                -> register r of tile t holds column 16 r + 4 q + t
-//   2-tile part: lane m reads columns 16 ((m & 3) >> 1) + 4 (m >> 2) + 2 (m & 1) + t
-//                -> register r of tile t holds column 16 (r >> 1) + 4 q + 2 (r & 1) + t
-//   1-tile part: lane m reads column m -> register r holds column 4 q + r
-// NCT = 3 is a 2-tile part followed by a 1-tile part 32 columns on.
-template <int NCT>
-__device__ __forceinline__ void load_b(const float* lds, int at, int m, float* b) {
-  if constexpr (NCT == 4) {
-    const float4 v = *reinterpret_cast<const float4*>(&lds[at + 16 * (m & 3) + 4 * (m >> 2)]);
-    b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
-  } else if constexpr (NCT >= 2) {
-    const float2 v = *reinterpret_cast<const float2*>(&lds[at + 16 * ((m & 3) >> 1) + 4 * (m >> 2) + 2 * (m & 1)]);
-    b[0] = v.x; b[1] = v.y;
-    if constexpr (NCT == 3) b[2] = lds[at + 32 + m];
-  } else {
-    b[0] = lds[at + m];
-  }
-}
-
-// The results of such a product: fn(column offset from the wave's first column,
-// four consecutive values of the lane's row), q = lane >> 4.
-template <int NCT, class F>
-__device__ __forceinline__ void for_each_out(const float4v* acc, int q, F&& fn) {
-  if constexpr (NCT == 4) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) fn(16 * r + 4 * q, make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]));
-  } else if constexpr (NCT >= 2) {
-    fn(4 * q, make_float4(acc[0][0], acc[1][0], acc[0][1], acc[1][1]));
-    fn(16 + 4 * q, make_float4(acc[0][2], acc[1][2], acc[0][3], acc[1][3]));
-    if constexpr (NCT == 3) fn(32 + 4 * q, make_float4(acc[2][0], acc[2][1], acc[2][2], acc[2][3]));
-  } else {
-    fn(4 * q, make_float4(acc[0][0], acc[0][1], acc[0][2], acc[0][3]));
-  }
-}
-
-// acc += A B with A's k along its LDS row (a_at = element (row, 0) of the lane's A
-// row): a lane reads four consecutive k as one 128-bit word, so the k slots of
-// step r of group g hold k = 16 g + 4 kq + r, kq = lane >> 4; B's rows k start at
-// b_at + k * ldb.  `groups` groups of 16 k, then `rest` single steps (slot kq
-// holds k = 16 groups + 4 step + kq).  The operands of the next group are in
-// flight while the MFMAs of the current one issue; reads run up to 16 k past the
-// end (the caller's buffers keep finite values there).
-template <int NCT>
-struct RowOperands {
-  float4 a;
-  float b[4][NCT];
-  __device__ __forceinline__ void load(const float* lds, int a_at, int b_at, int ldb, int m) {
-    a = *reinterpret_cast<const float4*>(&lds[a_at]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + r * ldb, m, b[r]);
-  }
-  __device__ __forceinline__ void mma(float4v* acc) const {
-    const float av[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[r][t], av[r], acc[t], 0, 0, 0);
-  }
-};
-
-template <int NCT>
-__device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_at, int ldb, int kq, int m, int groups,
-                                             int rest, float4v* acc) {
-  a_at += 4 * kq;
-  b_at += 4 * kq * ldb;
-  RowOperands<NCT> x, y;  // two operand sets taking turns, see mfma_sweep_k16
-  x.load(lds, a_at, b_at, ldb, m);
-  int gk = 0;
-  for (; gk + 2 <= groups; gk += 2) {
-    y.load(lds, a_at + 16, b_at + 16 * ldb, ldb, m);
-    __builtin_amdgcn_sched_barrier(0);
-    x.mma(acc);
-    __builtin_amdgcn_sched_barrier(0);
-    a_at += 32;
-    b_at += 32 * ldb;
-    x.load(lds, a_at, b_at, ldb, m);
-    __builtin_amdgcn_sched_barrier(0);
-    y.mma(acc);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (gk < groups) {
-    x.mma(acc);
-    a_at += 16;
-    b_at += 16 * ldb;
-  }
-  a_at -= 3 * kq;
-  b_at -= 3 * kq * ldb;
-  for (int ks = 0; ks < rest; ++ks) {
-    const float a1 = lds[a_at];
-    float b1[NCT];
-    load_b<NCT>(lds, b_at, m, b1);
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b1[t], a1, acc[t], 0, 0, 0);
-    a_at += 4;
-    b_at += 4 * ldb;
-  }
-}
-
-// acc += A B with A's k along LDS rows too (the transposed score block of the
-// uniform negatives' gradient): the lane's A element of step ks is at a_at +
-// (4 ks + kq) * lda.  Returns the sum of the A elements the lane has fed (its
-// share of a column sum of the score block).  Reads up to two steps past the end.
-template <int NCT>
-__device__ __forceinline__ float sweep_a_cols(const float* lds, int a_at, int lda, int b_at, int ldb, int kq, int m,
-                                              int ksteps, float4v* acc) {
-  a_at += kq * lda;
-  b_at += kq * ldb;
-  float ax = lds[a_at], ay, asum = 0.f;
-  float bx[NCT], by[NCT];
-  load_b<NCT>(lds, b_at, m, bx);
-  int ks = 0;
-  for (; ks + 2 <= ksteps; ks += 2) {
-    ay = lds[a_at + 4 * lda];
-    load_b<NCT>(lds, b_at + 4 * ldb, m, by);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], ax, acc[t], 0, 0, 0);
-    asum += ax;
-    __builtin_amdgcn_sched_barrier(0);
-    a_at += 8 * lda;
-    b_at += 8 * ldb;
-    ax = lds[a_at];
-    load_b<NCT>(lds, b_at, m, bx);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(by[t], ay, acc[t], 0, 0, 0);
-    asum += ay;
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (ks < ksteps) {
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], ax, acc[t], 0, 0, 0);
-    asum += ax;
-  }
-  return asum;
-}
-
-// The same product for operands whose k runs along the LDS rows (both operands
-// of the score products): a lane reads FOUR consecutive k of its row as one
-// 128-bit word and feeds them to four MFMAs, so the k slots of step r hold
-// k = 16 g + 4 (lane >> 4) + r for group g -- any assignment of k to slots is
-// right as long as both operands use the same one.  A quarter of the LDS
-// instructions of mfma_sweep; `groups` groups of 16 k, then `rest` single steps.
-// a_at / b_at address element (row, 0).  Reads up to 15 floats past the last k of
-// a row (never used: the groups cover whole multiples of 16 only).
-template <int T>
-struct K16Operands {
-  float4 a, b[T];
-  __device__ __forceinline__ void load(const float* lds, int a_at, int b_at, int b_tile) {
-    a = *reinterpret_cast<const float4*>(&lds[a_at]);
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) b[ct] = *reinterpret_cast<const float4*>(&lds[b_at + ct * b_tile]);
-  }
-  __device__ __forceinline__ void mma(float4v* acc) const {
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].x, a.x, acc[ct], 0, 0, 0);
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].y, a.y, acc[ct], 0, 0, 0);
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].z, a.z, acc[ct], 0, 0, 0);
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].w, a.w, acc[ct], 0, 0, 0);
-  }
-};
-
-template <int T>
-__device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b_at, int b_tile, int groups, int rest,
-                                               int kq, float4v* acc) {
-  a_at += 4 * kq;
-  b_at += 4 * kq;
-  // Two operand sets take turns: the operands of group g + 1 are requested before the
-  // matrix instructions of group g issue, and nothing is copied between the sets.  The
-  // scheduling barriers keep the compiler from sinking the loads down to their first
-  // use, which would expose the LDS latency once per group.
-  K16Operands<T> x, y;
-  x.load(lds, a_at, b_at, b_tile);
-  int gk = 0;
-  for (; gk + 2 <= groups; gk += 2) {
-    y.load(lds, a_at + 16, b_at + 16, b_tile);
-    __builtin_amdgcn_sched_barrier(0);
-    x.mma(acc);
-    __builtin_amdgcn_sched_barrier(0);
-    a_at += 32;
-    b_at += 32;
-    x.load(lds, a_at, b_at, b_tile);
-    __builtin_amdgcn_sched_barrier(0);
-    y.mma(acc);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (gk < groups) {
-    x.mma(acc);
-    a_at += 16;
-    b_at += 16;
-  }
-  a_at -= 3 * kq;  // single steps: slot kq holds k = 16 groups + 4 step + kq
-  b_at -= 3 * kq;
-  for (int ks = 0; ks < rest; ++ks) {
-    const float a1 = lds[a_at];
-    float b1[T];
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) b1[ct] = lds[b_at + ct * b_tile];
-#pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b1[ct], a1, acc[ct], 0, 0, 0);
-    a_at += 4;
-    b_at += 4;
-  }
-}
-
 // Geometry of one chunk, the same for both roles.
 struct FusedGeom {
   int D, P, U, N, ldx, lds, xn0, xn1, sc0, sc1, sq0, sq1, rs0, rs1, cs0, cs1;
@@ -1560,14 +1253,6 @@ __device__ __forceinline__ void fused_load_ids(const StepCtx& c, const FusedGeom
 }
 
 constexpr int kFusedRounds = kFusedIds / 16;  // rows per half-wave of the 8 helper waves
-
-// v, or zeros: by a bit mask (a select between a loaded value and a constant makes
-// the compiler index a two-entry stack array).
-__device__ __forceinline__ float4 keep_if(float4 v, bool keep) {
-  const int m = keep ? -1 : 0;
-  return make_float4(__int_as_float(__float_as_int(v.x) & m), __int_as_float(__float_as_int(v.y) & m),
-                     __int_as_float(__float_as_int(v.z) & m), __int_as_float(__float_as_int(v.w) & m));
-}
 
 // What a chunk's rows need besides themselves: the relation's operator parameters
 // and the two global embeddings at this lane's four columns.
@@ -1731,12 +1416,6 @@ __device__ __forceinline__ void fused_scores(float* lds, const FusedGeom& g, int
 // A step's 4 row tiles x T column tiles are split over the 8 compute waves as
 // (row tile, first ceil(T/2) or last floor(T/2) column tiles), two waves per SIMD,
 // so every SIMD carries T tiles per step.
-// Workgroup barrier of the fused kernel.  Only LDS traffic has to be ordered across
-// it: the waves exchange data through LDS alone, rows on their way from HBM into
-// registers and results on their way to HBM belong to one wave each.
-// __syncthreads() would also wait for those (its fences drain the vector memory
-// counter), which puts the latency of the gather on every step's critical path.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 //
 // LD != 0: both LDS row strides (operand rows, score rows) equal LD, known at compile
@@ -2030,14 +1709,6 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       lds_barrier();  // (f), (g)
     }
   }
-}
-
-// Row stride >= n (a multiple of 4) that keeps both MFMA access patterns
-// (16 rows x 4 columns, and 4 rows x 16 columns) at most 3-way bank conflicted.
-int lds_stride(int n) {
-  int ld = (n + 3) / 4 * 4;
-  while (ld % 32 != 12 && ld % 32 != 20) ld += 4;
-  return ld;
 }
 
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
@@ -2352,6 +2023,8 @@ struct Plan {
   int pslices[2]; // partial sums per batch of the element-wise parameter gradients
   bool fused;          // the chunk fits the LDS-resident kernel
   FusedLayout fl;
+  bool stream;         // the chunk's positives fit LDS and its negatives are streamed past them
+  StreamPlan sp;
   // dynamic relations: (relation, batch) keys of the positives and their sort buffers
   uint64_t *rkeys_a, *rkeys_b;
   uint32_t *rvals_a, *rvals_b;
@@ -2575,7 +2248,6 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.vals = (uint32_t*)take(npairs, 4);
   plan->vals_b = (uint32_t*)take(npairs, 4);
   plan->sort_temp = take(sort_temp_bytes(npairs), 1);
-  plan->bytes = off;
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
   // (the regularizer's terms live in the staged kernels only)
   plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && getenv("PBG_DISABLE_FUSED") == nullptr;
@@ -2583,6 +2255,24 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     c.side[0].uni_direct = c.side[1].uni_direct = 0;
     c.side[0].uni_dz_direct = c.side[1].uni_dz_direct = 0;
   }
+  // The streaming route's own buffers lie behind the staged ones: a call with global
+  // embeddings (known only from its buffers) takes the staged route on the same workspace.
+  plan->stream = !plan->fused && stream_geometry(c, &plan->sp) && getenv("PBG_DISABLE_STREAM") == nullptr;
+  if (plan->stream) {
+    StreamPlan& sp = plan->sp;
+    const size_t ne = (size_t)K * c.B;
+    for (int s = 0; s < 2; ++s) {
+      sp.sa[s] = takef(ne * D);
+      sp.sdb[s] = takef(ne * D);
+      sp.spos[s] = takef(ne);
+      sp.sloss[s] = takef((size_t)K * CP);
+      // dynamic relations: the operand's gradient IS the operator-output gradient of the side the operand came from
+      float* dz = c.side[1 - s].dz;
+      sp.sda[s] = (c.dynamic && c.op != PBG_OP_NONE) ? dz : takef(ne * D);
+    }
+    sp.scratch = takef(stream_scratch_floats(sp));
+  }
+  plan->bytes = off;
 
   if (b) {
     c.side[0].w = b->w_lhs;
@@ -2807,8 +2497,10 @@ int run_rowback(const Plan& plan, hipStream_t stream) {
   return check_launch("step rowback");
 }
 
+// `edge_terms`: (streaming route, standard mode) dz holds every edge's term of the parameter
+// gradient itself, so the gradient is a column sum
 int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& plan, hipStream_t stream,
-               RelOrder* ro) {
+               RelOrder* ro, bool edge_terms) {
   const StepCtx& c = plan.c;
   if (c.op == PBG_OP_NONE) return PBG_OK;
   const int D = c.D, K = c.K;
@@ -2867,8 +2559,10 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
       h.m = D; h.n = D; h.k = sd.op_rows; h.batch = K; h.alpha = 1.f; h.beta = 0.f;
       if ((rc = gemm_f32(h, stream)) != PBG_OK) return rc;
     } else {
+      StepCtx cg = c;
+      if (edge_terms) cg.op = PBG_OP_TRANSLATION;  // (whose gradient is the column sum of dz)
       hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
-                         dim3(kParamGroups * 64), 0, stream, c, s, plan.dth[s], plan.pslices[s]);
+                         dim3(kParamGroups * 64), 0, stream, cg, s, plan.dth[s], plan.pslices[s]);
     }
     if (c.affine) {  // the translation: column sums of dz, then its own Adagrad steps (parameters in the second slot)
       StepCtx ct = c;
@@ -3004,14 +2698,33 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   Plan plan;
   make_plan(desc, bufs, &plan);
   if ((rc = check_buffers(desc, bufs, plan, true)) != PBG_OK) return rc;
+  const bool stream = plan.stream && !bufs->lhs_global;
+  if (stream) {  // every gradient row is written in its final form; the operator-output gradients cover the positives only
+    for (int side = 0; side < 2; ++side) {
+      plan.c.side[side].uni_direct = plan.c.side[side].uni_dz_direct = 0;
+      if (plan.c.side[side].has_op) plan.c.side[side].op_rows = plan.c.B;
+    }
+  }
   const StepCtx& c = plan.c;
   RelOrder rel_order;
   auto mark = [&](int i) {
-    if (ev) hipEventRecord(ev[i], s);
+    if (ev) (void)hipEventRecord(ev[i], s);
   };
   mark(0);
   if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
-  if (plan.fused) {
+  if (stream) {
+    if ((rc = stream_prep(c, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
+    mark(1);
+    mark(2);
+    if ((rc = stream_chunks(c, plan.sp, s)) != PBG_OK) return rc;
+    mark(3);
+    mark(4);
+    mark(5);
+    mark(6);
+    if ((rc = stream_finish(c, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+    mark(7);
+  } else if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
     const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
     if ((rc = launch_fused(plan, lds_bytes, s)) != PBG_OK) return rc;
@@ -3046,7 +2759,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     }
     mark(7);
   }
-  if ((rc = run_params(desc, bufs, plan, s, &rel_order)) != PBG_OK) return rc;
+  if ((rc = run_params(desc, bufs, plan, s, &rel_order, stream)) != PBG_OK) return rc;
   if (bufs->lhs_global) {  // the raw-row gradients are complete and still one per gathered row
     hipLaunchKernelGGL(global_grad_kernel, dim3((unsigned)c.K, (unsigned)(2 * plan.gslices)), dim3(kGlobalHalves * 32), 0,
                        s, c, plan.gth, plan.gslices);
@@ -3088,6 +2801,13 @@ extern "C" int pbg_train_step_is_fused(const pbg_step_desc* desc) {
   Plan plan;
   make_plan(desc, nullptr, &plan);
   return plan.fused ? 1 : 0;
+}
+
+extern "C" int pbg_train_step_route(const pbg_step_desc* desc) {
+  if (validate(desc, true) != PBG_OK) return -1;
+  Plan plan;
+  make_plan(desc, nullptr, &plan);
+  return plan.fused ? PBG_ROUTE_FUSED : (plan.stream ? PBG_ROUTE_STREAM : PBG_ROUTE_STAGED);
 }
 
 extern "C" int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_stream_t stream,

@@ -402,6 +402,12 @@ class StepRunner:
         """True when the step runs as the single LDS-resident chunk kernel."""
         return bool(_lib.lib().pbg_train_step_is_fused(ctypes.byref(self.desc)))
 
+    @property
+    def route(self) -> str:
+        """Which kernels the step runs: "staged", "fused" (one LDS-resident chunk
+        kernel) or "stream" (positives in LDS, negatives streamed past them)."""
+        return ("staged", "fused", "stream")[_lib.lib().pbg_train_step_route(ctypes.byref(self.desc))]
+
     def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None,
                        uniform_seed=None) -> List[float]:
         """train() with HIP events between the stages; synchronises and returns

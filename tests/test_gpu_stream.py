@@ -1,0 +1,150 @@
+"""The streaming route of the training step (a chunk's positives resident in LDS,
+its negatives gathered raw and streamed past them) against the oracle's lock-step
+training: every operator the route takes x every loss x both relation modes, the
+three row lengths it is built for, partial last chunks, edge weights, negatives
+drawn in the step, and the staged route on the same inputs."""
+import itertools
+import os
+
+import pytest
+import torch
+
+from oracle import step as ostep
+from tests.parity import double_state, violator_ties
+from tests.test_gpu_step import DEV, compare_state, copy_of, loss_close, make_inputs, pack, say, to_runner
+
+pytestmark = pytest.mark.gpu
+
+CASES = []
+for op, loss, dyn in itertools.product(("none", "diagonal", "complex_diagonal"), ostep.LOSS_NAMES, (False, True)):
+    CASES.append(dict(operator=op, loss=loss, dynamic=dyn, num_batch_negs=50, num_uniform_negs=100, num_pos=130, dim=128))
+CASES += [
+    # the headline shape of the route: dim 400, chunks of 50, 1000 uniform negatives; a partial last chunk
+    dict(operator="complex_diagonal", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=1000, num_pos=173,
+         dim=400),
+    dict(operator="complex_diagonal", loss="softmax", dynamic=True, num_batch_negs=50, num_uniform_negs=1000, num_pos=120,
+         dim=400),
+    dict(operator="complex_diagonal", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=300, num_pos=100,
+         dim=400, shared=False),
+    dict(operator="diagonal", loss="logistic", dynamic=False, num_batch_negs=50, num_uniform_negs=70, num_pos=64, dim=400),
+    # dim 256; chunks of 64, 37 and 8 rows; a negatives count that is no multiple of the tile
+    dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=64, num_uniform_negs=200, num_pos=200, dim=256),
+    dict(operator="none", loss="ranking", dynamic=False, num_batch_negs=37, num_uniform_negs=91, num_pos=100, dim=256,
+         shared=False),
+    dict(operator="complex_diagonal", loss="logistic", dynamic=True, num_batch_negs=8, num_uniform_negs=64, num_pos=30,
+         dim=256, shared=False),
+    # no batch negatives: the chunk is as long as the uniform draw (model.py:648-650)
+    dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64, num_pos=150, dim=128),
+    dict(operator="none", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=64, dim=256),
+]
+
+
+def ids(case):
+    return "-".join(f"{v}" for v in case.values())
+
+
+def lockstep64(cfg, st, batches, keep_scores=False):
+    """oracle.step.train_lockstep on `st` and on a float64 copy of it.  A row that is
+    a negative of many chunks sums hundreds of gradient terms of mixed sign, and a
+    score row of a thousand negatives sums a thousand exponentials: the CPU path's own
+    fp32 result then lies further from the exact one than the tolerance (3e-5 against
+    1e-5 at dim 400 with 1000 negatives), so the float64 result anchors the comparison
+    (tests.parity.anchored_close)."""
+    st64 = double_state(st)
+    outs = ostep.train_lockstep(cfg, st, batches, keep_scores=keep_scores)
+    for out, exact in zip(outs, ostep.train_lockstep(cfg, st64, batches)):
+        out.exact_loss = exact.loss
+    return outs, st64
+
+
+def build(pbg, case, workers, seed_shift=0):
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    shared = case.pop("shared", True)
+    cfg = ostep.StepConfig(dim=dim, comparator="dot", num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1,
+                           relation_lr=0.01, margin=0.1, **case)
+    st, batches = make_inputs(cfg, num_pos, max(300, num_pos * 4), workers, seed=num_pos + dim + seed_shift, shared=shared)
+    return cfg, st, batches, num_pos
+
+
+@pytest.mark.parametrize("case", CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_stream_route_matches_the_oracle(pbg, case, workers):
+    say("stream", case, workers)
+    cfg, st, batches, num_pos = build(pbg, case, workers)
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    assert runner.route == "stream"
+    runner.train(*pack(cfg, batches))
+    torch.cuda.synchronize()
+    outs, st64 = lockstep64(cfg, st, batches, keep_scores=True)
+    for k, out in enumerate(outs):
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
+        sc = out.scores
+        for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
+                                     (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
+            ties = violator_ties(pos, neg)
+            assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
+    compare_state(cfg, runner, st, 1e-5, "stream", st64)
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[5], CASES[18], CASES[23]], ids=ids)
+def test_stream_route_with_edge_weights(pbg, case):
+    say("stream+weights", case)
+    cfg, st, batches, num_pos = build(pbg, case, 2)
+    g = torch.Generator().manual_seed(7)
+    weights = [0.25 + 2.0 * torch.rand(num_pos, generator=g) for _ in batches]
+    weights[0][::5] = 0.0
+    unweighted = copy_of(st)
+    runner = to_runner(pbg, cfg, st, num_pos, 2)
+    assert runner.route == "stream"
+    runner.train(*pack(cfg, batches), edge_weight=torch.stack(weights).to(DEV))
+    torch.cuda.synchronize()
+    outs, st64 = lockstep64(cfg, st, [b + (w,) for b, w in zip(batches, weights)])
+    ostep.train_lockstep(cfg, unweighted, batches)
+    for k, out in enumerate(outs):
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
+    compare_state(cfg, runner, st, 1e-5, "stream+weights", st64)
+    assert (st.w_lhs - unweighted.w_lhs).abs().max() > 1e-3 * st.w_lhs.abs().max()
+
+
+@pytest.mark.parametrize("case", [CASES[3], CASES[19]], ids=ids)
+def test_stream_route_draws_its_negatives(pbg, case):
+    """A call that draws its uniform negatives from a seed equals, bit for bit, the call
+    that is handed the same draw."""
+    say("stream, in-step negatives", case)
+    from pytorch_biggraph_amd import native
+
+    cfg, st, batches, num_pos = build(pbg, case, 3)
+    lhs, rhs, rel, _, _ = pack(cfg, batches)
+    a = to_runner(pbg, cfg, st, num_pos, 3)
+    b = to_runner(pbg, cfg, st, num_pos, 3)
+    assert a.route == "stream"
+    seed = 0x0FEDCBA987654321
+    shape = (3, a.spec.num_chunks, cfg.num_uniform_negs)
+    ul = native.sample_uniform_negatives(seed, 0, st.w_lhs.shape[0], shape, DEV)
+    ur = native.sample_uniform_negatives(seed, 1, st.w_rhs.shape[0], shape, DEV)
+    a.train(lhs, rhs, rel, ul, ur)
+    b.train(lhs, rhs, rel, uniform_seed=seed)
+    torch.cuda.synchronize()
+    assert torch.equal(a.loss_out, b.loss_out) and torch.equal(a.violators_out, b.violators_out)
+    assert torch.equal(a.w_lhs, b.w_lhs) and torch.equal(a.g_lhs, b.g_lhs)
+    for k in a.rhs_op:
+        assert torch.equal(a.rhs_op[k], b.rhs_op[k])
+
+
+def test_twenty_calls_on_the_stream_route(pbg):
+    """20 training calls of 2 batches each, the state carried from call to call."""
+    case = dict(operator="complex_diagonal", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=200, num_pos=100,
+                dim=128)
+    say("stream, 20 calls", case)
+    cfg, st, _, num_pos = build(pbg, case, 2)
+    runner = to_runner(pbg, cfg, st, num_pos, 2)
+    assert runner.route == "stream"
+    st64 = double_state(st)
+    for call in range(20):
+        _, batches = make_inputs(cfg, num_pos, st.w_lhs.shape[0], 2, seed=1000 + call, shared=True)
+        runner.train(*pack(cfg, batches))
+        ostep.train_lockstep(cfg, st, batches)
+        ostep.train_lockstep(cfg, st64, batches)
+    torch.cuda.synchronize()
+    compare_state(cfg, runner, st, 1e-4, "stream x20", st64)  # 1e-4 after many steps
