@@ -2266,6 +2266,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
       sp.sdb[s] = takef(ne * D);
       sp.spos[s] = takef(ne);
       sp.sloss[s] = takef((size_t)K * CP);
+      sp.colid[s] = (int*)take((size_t)KC * (c.P + c.side[s].u), sizeof(int));
       // dynamic relations: the operand's gradient IS the operator-output gradient of the side the operand came from
       float* dz = c.side[1 - s].dz;
       sp.sda[s] = (c.dynamic && c.op != PBG_OP_NONE) ? dz : takef(ne * D);

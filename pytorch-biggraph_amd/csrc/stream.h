@@ -11,7 +11,7 @@ struct StreamPlan {
   int pr;      // rows kept of the positives' operand block: P rounded up to 4
   int ntiles;  // tiles of 32 negatives per (chunk, side)
   int grid;    // workgroups
-  int n_at, a_at, g_at, id_at, total;  // LDS offsets and size, in floats
+  int n_at, a_at, g_at, total;  // LDS offsets and size, in floats
   // Per side s, indexed by edge (k * B + position): the operand row that edge's OTHER
   // side contributes to the scores against side s's negatives, that row's gradient,
   // and the gradient of the edge's own side-s row as a batch negative of its chunk.
@@ -21,6 +21,7 @@ struct StreamPlan {
   float* spos[2];   // [K * B] positive score paired with side s's negatives
   float* sloss[2];  // [K * C * P] weighted loss against side s's negatives
   float* scratch;   // [grid, ntiles, 2048] score tiles between the two sweeps
+  int* colid[2];    // [K * C, P + U] row id of every column of side s's negatives (-1: padded position)
 };
 
 // Whether the route takes this configuration; fills the geometry (not the pointers).

@@ -95,25 +95,38 @@ __global__ __launch_bounds__(kRowThreads) void stream_prep_kernel(StepCtx c, Str
 // ---------------------------------------------------------------------------
 // the chunk kernel
 // ---------------------------------------------------------------------------
-// Row id of column j of an item's negatives (-1: a padded position of a partial
-// last chunk, or a column past the last negative), and the sort key of a uniform
-// negative's gradient row.
-__device__ __forceinline__ int stream_column_id(const StepCtx& c, const SideCtx& sd, int s, int k, int cc, int kc, int valid,
-                                                int j, bool write_key) {
-  const int P = c.P, U = sd.u;
-  const bool is_pos = j < P;
-  const int q = cc * P + j, u = min(max(j - P, 0), U - 1);
-  const bool real = is_pos ? j < valid : j < P + U;
+// One thread per (chunk, side, column): the row id of that column of the item's negatives
+// (-1: a padded position of a partial last chunk), as 32 bits in the order the chunk kernel
+// walks them, and the sort key of a uniform negative's gradient row.  Drawing the ids here
+// (Philox, 40 quarter-rate multiplies per id) keeps that arithmetic out of the chunk kernel,
+// whose helper waves share their vector ALUs with the matrix instructions.
+__global__ __launch_bounds__(256) void stream_ids_kernel(StepCtx c, StreamPlan a) {
+  const int P = c.P, U = c.side[0].u, ncols = P + U;
+  const int64_t per_side = (int64_t)c.K * c.C * ncols;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= 2 * per_side) return;
+  const int s = t >= per_side;
+  const int64_t r = t - (s ? per_side : 0);
+  const int kc = (int)(r / ncols), j = (int)(r - (int64_t)kc * ncols);
+  const int k = kc / c.C, cc = kc - k * c.C;
+  const int valid = (cc == c.C - 1) ? c.last : P;
+  const SideCtx& sd = c.side[s];
   int64_t id;
-  if (is_pos) id = sd.idx[(int64_t)k * c.B + min(q, c.B - 1)];
-  else id = uniform_negative(sd, s, (int64_t)kc * U + u);
+  bool real;
+  if (j < P) {
+    real = j < valid;
+    id = sd.idx[(int64_t)k * c.B + min(cc * P + j, c.B - 1)];
+  } else {
+    real = true;
+    id = uniform_negative(sd, s, (int64_t)kc * U + (j - P));
+  }
   id = clamp_index(id, sd.num_rows);
-  if (write_key && real && !is_pos) {
-    const int64_t pair = (int64_t)k * c.rk + sd.slot_uni + (int64_t)cc * U + u;
+  if (j >= P) {
+    const int64_t pair = (int64_t)k * c.rk + sd.slot_uni + (int64_t)cc * U + (j - P);
     c.keys[pair] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
     c.vals[pair] = (uint32_t)pair;
   }
-  return real ? (int)id : -1;
+  (s ? a.colid[1] : a.colid[0])[r] = real ? (int)id : -1;
 }
 
 // Half a wave per 128 columns of a row, 128-bit loads, the whole tile in flight:
@@ -123,10 +136,17 @@ template <int NSEG>
 struct TileRows {
   float4 v[2 * NSEG];
   int id0, id1;
-  __device__ __forceinline__ void issue(const float* w, int D, const int* ids, int ht, bool active) {
-    const int hw = ht >> 5, c4 = (ht & 31) << 2;
-    id0 = active ? ids[hw] : -1;
-    id1 = active ? ids[hw + 16] : -1;
+  // the two ids of this thread's rows of the tile that starts at column j0 (-1 past the last column)
+  static __device__ __forceinline__ void fetch_ids(const int* colid, int j0, int ncols, int ht, int* a0, int* a1) {
+    const int hw = ht >> 5;
+    const int x0 = colid[min(j0 + hw, ncols - 1)], x1 = colid[min(j0 + hw + 16, ncols - 1)];
+    *a0 = j0 + hw < ncols ? x0 : -1;
+    *a1 = j0 + hw + 16 < ncols ? x1 : -1;
+  }
+  __device__ __forceinline__ void issue(const float* w, int D, int row0, int row1, int ht) {
+    const int c4 = (ht & 31) << 2;
+    id0 = row0;
+    id1 = row1;
     const uint32_t row_bytes = (uint32_t)D * 4u;
     const char* base = reinterpret_cast<const char*>(w);
     const char* r0 = base + (uint64_t)(uint32_t)max(id0, 0) * row_bytes;
@@ -138,37 +158,105 @@ struct TileRows {
       v[2 * seg + 1] = *reinterpret_cast<const float4*>(r1 + col * 4);
     }
   }
-  __device__ __forceinline__ void store(float* lds, int n_at, int lda, int D, int ht) const {
+  // `absent`: the tile may hold absent rows (the same for the whole workgroup)
+  __device__ __forceinline__ void store(float* lds, int n_at, int lda, int D, int ht, bool absent) const {
     const int hw = ht >> 5, c4 = (ht & 31) << 2;
 #pragma unroll
     for (int seg = 0; seg < NSEG; ++seg) {
       const int col = seg * 128 + c4;
       if (col < D) {
-        *reinterpret_cast<float4*>(&lds[n_at + hw * lda + col]) = keep_if(v[2 * seg], id0 >= 0);
-        *reinterpret_cast<float4*>(&lds[n_at + (hw + 16) * lda + col]) = keep_if(v[2 * seg + 1], id1 >= 0);
+        float4 v0 = v[2 * seg], v1 = v[2 * seg + 1];
+        if (absent) {
+          v0 = keep_if(v0, id0 >= 0);
+          v1 = keep_if(v1, id1 >= 0);
+        }
+        *reinterpret_cast<float4*>(&lds[n_at + hw * lda + col]) = v0;
+        *reinterpret_cast<float4*>(&lds[n_at + (hw + 16) * lda + col]) = v1;
       }
     }
   }
 };
 
-// NCT column tiles of dA += G_t N_t for the lane's row of the score tile: a_at = that row's first
-// element + 4 kq, b_at = the tile's row 4 kq at the part's first column.  The k slots of
-// step r of group g hold k = 16 g + 4 kq + r in both operands; LDA is known at compile
-// time, so every address below is one register plus an immediate.  The other compute wave
-// of the SIMD issues its matrix instructions while this one waits for its operands.
+// B operand of one k-step for NCT column tiles (k along the LDS rows, columns = embedding
+// coordinates), with the 16 columns of a tile chosen so that the reads are free of bank
+// conflicts: lane m = lane & 15 reads NCT consecutive floats at column NCT * m (eight lanes
+// of a 128-bit read cover 32 consecutive banks), tile t taking the t-th of them.  The
+// instruction's row index i = m comes back as i = 4 q + r in lane group q, register r, so
+//   4 tiles: register r of tile t holds column 16 q + 4 r + t -> four 128-bit words per lane, one 64-byte run
+//   2 tiles: register r of tile t holds column 8 q + 2 r + t
+//   1 tile:  register r holds column 4 q + r
+// NCT = 3 is a 2-tile part followed by a 1-tile part 32 columns on.
+template <int NCT>
+__device__ __forceinline__ void tile_b(const float* lds, int at, int m, float* b) {
+  if constexpr (NCT == 4) {
+    const float4 v = *reinterpret_cast<const float4*>(&lds[at + 4 * m]);
+    b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+  } else if constexpr (NCT >= 2) {
+    const float2 v = *reinterpret_cast<const float2*>(&lds[at + 2 * m]);
+    b[0] = v.x; b[1] = v.y;
+    if constexpr (NCT == 3) b[2] = lds[at + 32 + m];
+  } else {
+    b[0] = lds[at + m];
+  }
+}
+// fn(column offset from the first tile's first column, four consecutive values of the lane's row)
+template <int NCT, class F>
+__device__ __forceinline__ void tile_out(const float4v* acc, int q, F&& fn) {
+  if constexpr (NCT == 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) fn(16 * q + 4 * r, make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]));
+  } else if constexpr (NCT >= 2) {
+    fn(8 * q, make_float4(acc[0][0], acc[1][0], acc[0][1], acc[1][1]));
+    fn(8 * q + 4, make_float4(acc[0][2], acc[1][2], acc[0][3], acc[1][3]));
+    if constexpr (NCT == 3) fn(32 + 4 * q, make_float4(acc[2][0], acc[2][1], acc[2][2], acc[2][3]));
+  } else {
+    fn(4 * q, make_float4(acc[0][0], acc[0][1], acc[0][2], acc[0][3]));
+  }
+}
+
+// dA[N column tiles] += G_t N_t for the lane's row of the score tile: a_at = that row's first
+// element + 4 kq, b_at = the tile's row 4 kq at the wave's first column.  The work is cut into
+// units of (up to 4 column tiles) x (8 k): two of the tile's rows feed 8 matrix
+// instructions, the score row's four k values of a group of 16 k come with one 128-bit read
+// per two units; the k slots of step r of group g hold k = 16 g + 4 kq + r in both operands.
+// Two operand sets take turns, the reads of the next unit pinned above the matrix
+// instructions of the current one; LDA is known at compile time, so every address is one
+// register plus an immediate.
+template <int NCT>
+struct DaOperands {
+  float b[2][NCT];
+  template <int LDA>
+  __device__ __forceinline__ void load(const float* lds, int b_at, int m16) {
+    tile_b<NCT>(lds, b_at, m16, b[0]);
+    tile_b<NCT>(lds, b_at + LDA, m16, b[1]);
+  }
+  __device__ __forceinline__ void mma(float a0, float a1, float4v* acc) const {
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[0][t], a0, acc[t], 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[1][t], a1, acc[t], 0, 0, 0);
+  }
+};
+// unit u of a part: k group u / 2, rows 2 (u % 2) and 2 (u % 2) + 1 of the group's four
 template <int NCT, int LDA>
 __device__ __forceinline__ void stream_da_part(const float* lds, int a_at, int b_at, int m16, float4v* acc) {
+  constexpr int units = 2 * (kTile / 16);
+  DaOperands<NCT> x, y;
+  float4 a = *reinterpret_cast<const float4*>(&lds[a_at]), an = a;
+  x.template load<LDA>(lds, b_at, m16);
 #pragma unroll
-  for (int g = 0; g < kTile / 16; ++g) {
-    const float4 av4 = *reinterpret_cast<const float4*>(&lds[a_at + 16 * g]);
-    const float av[4] = {av4.x, av4.y, av4.z, av4.w};
-    float b[4][NCT];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + (16 * g + r) * LDA, m16, b[r]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[r][t], av[r], acc[t], 0, 0, 0);
+  for (int u = 0; u < units; ++u) {
+    DaOperands<NCT>& cur = (u & 1) ? y : x;
+    DaOperands<NCT>& nxt = (u & 1) ? x : y;
+    if (u + 1 < units) {
+      nxt.template load<LDA>(lds, b_at + (16 * ((u + 1) / 2) + 2 * ((u + 1) & 1)) * LDA, m16);
+      if (((u + 1) & 1) == 0) an = *reinterpret_cast<const float4*>(&lds[a_at + 16 * ((u + 1) / 2)]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (u & 1) cur.mma(a.z, a.w, acc);
+    else cur.mma(a.x, a.y, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    if (u & 1) a = an;
   }
 }
 template <int N, int LDA>
@@ -183,31 +271,81 @@ __device__ __forceinline__ void stream_da_store(const float4v* acc, int kq, floa
   constexpr int full = N / 4, rem = N % 4;
 #pragma unroll
   for (int p = 0; p < full; ++p)
-    for_each_out<4>(acc + 4 * p, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * p + col) = v; });
+    tile_out<4>(acc + 4 * p, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * p + col) = v; });
   if constexpr (rem > 0)
-    for_each_out<rem>(acc + 4 * full, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * full + col) = v; });
+    tile_out<rem>(acc + 4 * full, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * full + col) = v; });
 }
 
 // NCT column tiles from `ct` on of dN_t = G_t^T A for the lane's negative, stored at dst (or
 // dropped): g_at = the negative's column of G_t in row kq, a_at = row kq of A at column 0.
+// One k step = one element of G_t's column and, per tile, one float of A's row per lane;
+// two operand sets take turns as above.  Here a tile is 16 ADJACENT columns (lane m reads
+// column m of each tile: 32-bit reads without bank conflicts), so that a lane's four results
+// of a tile are one 128-bit word and the four lanes of a row write 64 bytes in one piece:
+// these rows are the bulk of what the kernel writes to HBM, and a store instruction
+// whose 16-byte pieces lie 64 bytes apart costs four times the requests.
+// Reads one step past the last (the rows behind both blocks exist).
 template <int NCT, int LDA>
 __device__ __forceinline__ void stream_dn_part(const float* lds, int g_at, int a_at, int ct, int ksteps, int kq, int m16,
                                                float* dst) {
   float4v acc[NCT];
 #pragma unroll
   for (int t = 0; t < NCT; ++t) acc[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-  a_at += ct * 16;
-#pragma unroll 2
-  for (int ks = 0; ks < ksteps; ++ks) {
-    const float g = lds[g_at];
-    float b[NCT];
-    load_b<NCT>(lds, a_at, m16, b);
+  a_at += ct * 16 + m16;
+  float gx = lds[g_at], gy;
+  float bx[NCT], by[NCT];
 #pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[t], g, acc[t], 0, 0, 0);
-    g_at += 4 * kLdg;
-    a_at += 4 * LDA;
+  for (int t = 0; t < NCT; ++t) bx[t] = lds[a_at + 16 * t];
+  int ks = 0;
+  for (; ks + 2 <= ksteps; ks += 2) {
+    gy = lds[g_at + 4 * kLdg];
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) by[t] = lds[a_at + 4 * LDA + 16 * t];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], gx, acc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    g_at += 8 * kLdg;
+    a_at += 8 * LDA;
+    gx = lds[g_at];
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) bx[t] = lds[a_at + 16 * t];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(by[t], gy, acc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
   }
-  if (dst) for_each_out<NCT>(acc, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + ct * 16 + col) = v; });
+  if (ks < ksteps) {
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bx[t], gx, acc[t], 0, 0, 0);
+  }
+  if (dst) {
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+      *reinterpret_cast<float4*>(dst + (ct + t) * 16 + 4 * kq) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+  }
+}
+
+// The helpers' arithmetic competes with the compute waves' matrix instructions for the
+// same issue slots (fp32 matrix products run on the vector ALUs, and a wave that wants one
+// vector instruction waits for a gap between another wave's matrix instructions), so the
+// per-element work uses the hardware's exp2 / log2 / rcp (1 ulp) with one multiply or fma
+// around them instead of the library's correctly rounded sequences.  e^(x - m) is formed as
+// 2^((x - m) log2 e) with the subtraction FIRST: its relative error is then about 1e-7 |x - m|,
+// nothing for the scores near the maximum that carry the sum.  (Folding the subtraction into
+// one fma with -m log2 e rounds that constant to 1e-7 |m| instead, and an edge whose own
+// entity is also drawn as its negative has two score-sized terms, e^(t - m) / Z and the
+// positive's 1 - e^(pos - m) / Z, that must cancel to the last bits.)
+constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
+__device__ __forceinline__ float exp_of_difference(float x, float m) {
+  return __builtin_amdgcn_exp2f((x - m) * kLog2e);
+}
+// sigmoid(z) and (through *softplus) softplus(z) from one exponential
+__device__ __forceinline__ float fast_sigmoid(float z, float* softplus) {
+  const float e = __builtin_amdgcn_exp2f(-fabsf(z) * kLog2e);
+  const float r = __builtin_amdgcn_rcpf(1.0f + e);
+  if (softplus) *softplus = fmaxf(z, 0.f) + __builtin_amdgcn_logf(1.0f + e) * kLn2;
+  return (z >= 0.f ? 1.0f : e) * r;
 }
 
 // Statistics of one row of the score matrix, spread over the 8 threads that own the row.
@@ -216,19 +354,17 @@ struct RowLoss {
   float m, z;     // softmax: running maximum (starts at the positive score) and sum of exp(score - m)
   float acc;      // ranking: sum of hinges; logistic: sum of softplus(score)
   float gsum;     // ranking: sum of dLoss/dscore
-  int viol;
   __device__ __forceinline__ void start(float pos) {
     m = pos;
     z = 0.f;
     acc = 0.f;
     gsum = 0.f;
-    viol = 0;
   }
   __device__ __forceinline__ void add(const float* t, float pos, float w, float margin) {
     if (LOSS == PBG_LOSS_SOFTMAX) {
-      const float mt = fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3]));
-      const float mn = fmaxf(m, mt);
-      z = z * expf(m - mn) + ((expf(t[0] - mn) + expf(t[1] - mn)) + (expf(t[2] - mn) + expf(t[3] - mn)));
+      const float mn = fmaxf(fmaxf(m, t[0]), fmaxf(fmaxf(t[1], t[2]), t[3]));
+      z = z * exp_of_difference(m, mn) + ((exp_of_difference(t[0], mn) + exp_of_difference(t[1], mn)) +
+                                          (exp_of_difference(t[2], mn) + exp_of_difference(t[3], mn)));
       m = mn;
     }
 #pragma unroll
@@ -240,9 +376,10 @@ struct RowLoss {
         acc += fmaxf(x, 0.f);
         gsum += (x >= 0.f) ? w : 0.f;
       } else if (LOSS == PBG_LOSS_LOGISTIC) {
-        acc += softplusf(t[e]);
+        float sp;
+        fast_sigmoid(t[e], &sp);
+        acc += sp;
       }
-      if (t[e] > pos) ++viol;
     }
   }
 };
@@ -253,12 +390,13 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int D = NT * 16, D4 = D / 4, NSEG = (D + 127) / 128;
   constexpr int lda = lds_stride(D);               // (= a.lda)
-  constexpr int T0 = (NT + 1) / 2, T1 = NT - T0;  // column tiles of dA per wave group
+  // column tiles of dA per wave group: [0, T0) and [NT - T0, NT) -- with NT odd the middle tile is formed by
+  // both groups (bit-identical values, one code path for the two groups)
+  constexpr int T0 = (NT + 1) / 2;
   const int wave16 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wave = wave16 & 7, ht = threadIdx.x & (kHelpers - 1);
   const int P = c.P, C = c.C, U = c.side[0].u, ncols = P + U, nt = a.ntiles, pr = a.pr;
   const int CP = C * P;
-  int* idbuf = reinterpret_cast<int*>(lds + a.id_at);
   float* scr = a.scratch + (size_t)blockIdx.x * nt * (kHelpers * 4) + ht * 4;
   const bool helper = wave16 >= 8;
   if (helper) __builtin_amdgcn_s_setprio(3);
@@ -278,10 +416,6 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
         const float4 v = *reinterpret_cast<const float4*>(src + (int64_t)min(row, valid - 1) * D + c4);
         *reinterpret_cast<float4*>(&lds[a.a_at + row * lda + c4]) = keep_if(v, row < valid);
       }
-      if (threadIdx.x < 64) {
-        const int b = threadIdx.x >> 5, tile = b < nt ? b : 0;
-        idbuf[threadIdx.x] = stream_column_id(c, sd, s, k, cc, kc, valid, tile * kTile + (threadIdx.x & 31), b < nt);
-      }
     }
     lds_barrier();  // (p1)
 
@@ -297,9 +431,17 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
       const bool has_nb = sd.nb > 0;
       const float inv_nn = 1.0f / (float)sd.nn;
 
+      // a tile with columns that are masked or absent: the chunk's own rows, and the columns past the last negative
+      auto edge_tile = [&](int tile) { return tile * kTile < P || (tile + 1) * kTile > ncols; };
+      // The ids of a tile's rows are fetched one step before the rows themselves, so that
+      // neither load waits for the other inside a step.
+      const int* colid = (s ? a.colid[1] : a.colid[0]) + (int64_t)kc * ncols;
       TileRows<NSEG> rows;
-      rows.issue(sd.w, D, idbuf, ht, true);
-      rows.store(lds, a.n_at, lda, D, ht);
+      int nid0, nid1;
+      TileRows<NSEG>::fetch_ids(colid, 0, ncols, ht, &nid0, &nid1);
+      rows.issue(sd.w, D, nid0, nid1, ht);
+      TileRows<NSEG>::fetch_ids(colid, nt > 1 ? kTile : 0, ncols, ht, &nid0, &nid1);
+      rows.store(lds, a.n_at, lda, D, ht, true);
       lds_barrier();  // (p2) tile 0 in LDS
 
       RowLoss<LOSS> st;
@@ -308,12 +450,14 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
       auto absorb = [&](int tile, int gbuf) {
         const float4 sv = *reinterpret_cast<const float4*>(&lds[gbuf + hrow * kLdg + hc]);
         float t[4] = {sv.x, sv.y, sv.z, sv.w};
-        const int j0 = tile * kTile + hc;
+        if (edge_tile(tile)) {
+          const int j0 = tile * kTile + hc;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int j = j0 + e;
-          if (j < P && (!has_nb || j == hrow || j >= valid)) t[e] = -1e9f;
-          if (j >= ncols) t[e] = -INFINITY;
+          for (int e = 0; e < 4; ++e) {
+            const int j = j0 + e;
+            if (j < P && (!has_nb || j == hrow || j >= valid)) t[e] = -1e9f;
+            if (j >= ncols) t[e] = -INFINITY;
+          }
         }
         *reinterpret_cast<float4*>(scr + (size_t)tile * (kHelpers * 4)) = make_float4(t[0], t[1], t[2], t[3]);
         st.add(t, pos, w, c.margin);
@@ -322,11 +466,11 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
       // ---- sweep 1 ----
       for (int q = 0; q < nt; ++q) {
         const int tn = q + 1 == nt ? 0 : q + 1, t2 = tn + 1 == nt ? 0 : tn + 1;
-        rows.issue(sd.w, D, idbuf + ((q + 1) & 1) * kTile, ht, true);
-        if (ht < kTile) idbuf[(q & 1) * kTile + ht] = stream_column_id(c, sd, s, k, cc, kc, valid, t2 * kTile + ht, q + 2 < nt);
+        rows.issue(sd.w, D, nid0, nid1, ht);  // tile tn
+        TileRows<NSEG>::fetch_ids(colid, t2 * kTile, ncols, ht, &nid0, &nid1);
         if (q >= 1) absorb(q - 1, a.g_at + ((q - 1) & 1) * kTileFloats);
         lds_barrier();  // (A) S_q complete, tile q no longer read
-        rows.store(lds, a.n_at, lda, D, ht);
+        rows.store(lds, a.n_at, lda, D, ht, edge_tile(tn));
         lds_barrier();  // (B) tile tn in LDS
       }
       absorb(nt - 1, a.g_at + ((nt - 1) & 1) * kTileFloats);
@@ -349,41 +493,48 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
         dpos = (sigmoidf(pos) - 1.0f) * w;
         scale = inv_nn * w;
       }
-      const int viol = oct_sum_int(st.viol);
-      if ((ht & 7) == 0 && hrow < P) {
-        const int64_t job = (int64_t)k * CP + cc * P + hrow;
-        (s ? a.sloss[1] : a.sloss[0])[job] = row_live ? loss_w : 0.f;
-        c.violrow[job * 2 + s] = row_live ? viol : 0;
-      }
-      // dLoss/dS of this thread's four columns of a tile; the positive's gradient on the diagonal
-      auto grad_tile = [&](int tile, int gbuf) {
-        const float4 sv = *reinterpret_cast<const float4*>(scr + (size_t)tile * (kHelpers * 4));
+      // dLoss/dS of this thread's four columns of a tile, the positive's gradient on the diagonal;
+      // the violators are counted on the way (masked and absent columns score -1e9 / -inf)
+      int viol = 0;
+      auto parked = [&](int tile) { return *reinterpret_cast<const float4*>(scr + (size_t)tile * (kHelpers * 4)); };
+      auto grad_tile = [&](int tile, int gbuf, float4 sv) {
         const float t[4] = {sv.x, sv.y, sv.z, sv.w};
         float g[4];
-        const int j0 = tile * kTile + hc;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if (LOSS == PBG_LOSS_SOFTMAX) g[e] = expf(t[e] - mx) * scale;
+          if (LOSS == PBG_LOSS_SOFTMAX) g[e] = exp_of_difference(t[e], mx) * scale;
           else if (LOSS == PBG_LOSS_RANKING) g[e] = ((t[e] - pos) + c.margin >= 0.f) ? w : 0.f;
-          else g[e] = sigmoidf(t[e]) * scale;
-          if (j0 + e == hrow && hrow < P) g[e] = dpos;
+          else g[e] = fast_sigmoid(t[e], nullptr) * scale;
+          viol += t[e] > pos ? 1 : 0;
+        }
+        if (tile * kTile < P) {
+          const int j0 = tile * kTile + hc;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (j0 + e == hrow && hrow < P) g[e] = dpos;
         }
         *reinterpret_cast<float4*>(&lds[gbuf + hrow * kLdg + hc]) = make_float4(g[0], g[1], g[2], g[3]);
       };
-      grad_tile(0, a.g_at + (nt & 1) * kTileFloats);
+      grad_tile(0, a.g_at + (nt & 1) * kTileFloats, parked(0));
       lds_barrier();  // (T) G_0 in LDS
 
       // ---- sweep 2 ----
       for (int q = nt; q < 2 * nt; ++q) {
         const int t = q - nt;
         const bool more = t + 1 < nt;
-        rows.issue(sd.w, D, idbuf + ((q + 1) & 1) * kTile, ht, more);
-        if (ht < kTile && t + 2 < nt)
-          idbuf[(q & 1) * kTile + ht] = stream_column_id(c, sd, s, k, cc, kc, valid, (t + 2) * kTile + ht, false);
-        if (more) grad_tile(t + 1, a.g_at + ((q + 1) & 1) * kTileFloats);
+        const float4 sv = parked(min(t + 1, nt - 1));  // asked for first: loads come back in the order they were issued
+        rows.issue(sd.w, D, nid0, nid1, ht);  // tile t + 1 (with `more`; else rows that are not stored)
+        TileRows<NSEG>::fetch_ids(colid, min(t + 2, nt - 1) * kTile, ncols, ht, &nid0, &nid1);
+        if (more) grad_tile(t + 1, a.g_at + ((q + 1) & 1) * kTileFloats, sv);
         lds_barrier();  // (A) dA has taken tile t
-        if (more) rows.store(lds, a.n_at, lda, D, ht);
+        if (more) rows.store(lds, a.n_at, lda, D, ht, edge_tile(t + 1));
         lds_barrier();  // (B) tile t + 1 and G_(t+1) in LDS, G_t no longer read
+      }
+      viol = oct_sum_int(viol);
+      if ((ht & 7) == 0 && hrow < P) {
+        const int64_t job = (int64_t)k * CP + cc * P + hrow;
+        (s ? a.sloss[1] : a.sloss[0])[job] = row_live ? loss_w : 0.f;
+        c.violrow[job * 2 + s] = row_live ? viol : 0;
       }
     } else {
       // ================= compute role =================
@@ -424,8 +575,7 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
         const int m16 = lane_ & 15, kq = lane_ >> 4;
         {  // dA += G_t N_t: this wave's row tile, its half of the column tiles
           const int a_at = gbuf + (rt * 16 + m16) * kLdg + 4 * kq, b_at = a.n_at + 4 * kq * lda;
-          if (grp == 0) stream_da_product<T0, lda>(lds, a_at, b_at, m16, dA);
-          else if (T1 > 0) stream_da_product<(T1 > 0 ? T1 : 1), lda>(lds, a_at, b_at + T0 * 16, m16, dA);
+          stream_da_product<T0, lda>(lds, a_at, b_at + (grp ? (NT - T0) * 16 : 0), m16, dA);
         }
         lds_barrier();  // (A)
         {  // dN_t = G_t^T A: 16 negatives x this wave's quarter of the column tiles
@@ -449,9 +599,8 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
       const int m16 = lane_ & 15, kq = lane_ >> 4;
       const int i = rt * 16 + m16;
       if (i < valid) {
-        float* dst = (s ? a.sda[1] : a.sda[0]) + (e0 + i) * D + (grp ? T0 * 16 : 0);
-        if (grp == 0) stream_da_store<T0>(dA, kq, dst);
-        else if (T1 > 0) stream_da_store<(T1 > 0 ? T1 : 1)>(dA, kq, dst);
+        float* dst = (s ? a.sda[1] : a.sda[0]) + (e0 + i) * D + (grp ? (NT - T0) * 16 : 0);
+        stream_da_store<T0>(dA, kq, dst);
       }
     }
   }
@@ -573,8 +722,7 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
   sp->n_at = 0;
   sp->a_at = kTile * sp->lda;
   sp->g_at = sp->a_at + sp->pr * sp->lda;
-  sp->id_at = sp->g_at + 2 * kTileFloats;
-  sp->total = sp->id_at + 2 * kTile + kSlack;
+  sp->total = sp->g_at + 2 * kTileFloats + kSlack;
   if ((size_t)sp->total * sizeof(float) > 160 * 1024 - 512) return false;
   static int cus = 0;
   if (cus == 0) {
@@ -591,6 +739,8 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
 int stream_prep(const StepCtx& c, const StreamPlan& sp, int nvh, hipStream_t stream) {
   if (nvh > 4) return fail(PBG_ERR_UNSUPPORTED, "step: streaming route needs dim <= 512");
   PBG_STREAM_ROWS(nvh, stream_prep_kernel, (int64_t)c.K * 2 * c.B, stream, c, sp);
+  const int64_t columns = 2 * (int64_t)c.K * c.C * (c.P + c.side[0].u);
+  hipLaunchKernelGGL(stream_ids_kernel, dim3((unsigned)ceil_div(columns, 256)), dim3(256), 0, stream, c, sp);
   return check_launch("step streaming prep");
 }
 
