@@ -5,6 +5,8 @@
 // (dim 100) is one coalesced request of 25 lanes and a 4 KiB row (dim 1024) is
 // four full-wave requests.
 #include <mutex>
+#include <cstdlib>
+
 #include "pbg_internal.h"
 #include "row_ops.h"
 
@@ -406,6 +408,106 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   }
 }
 
+// One wave per TABLE row, for calls whose gradient rows outnumber the tables' rows many
+// times over (a small entity table under a thousand uniform negatives per chunk and 64
+// workers: every row has a run in nearly every worker's batch).  Walking the sorted
+// positions from their side (row_update_kernel) then spends its time in the chain
+// of dependent loads along a row's runs.  Here the wave finds its row's first position
+// by a 64-ary search, then walks the row's stretch of sorted positions window by
+// window: the rows to read -- the head row of every run, or all rows of a short run that
+// tile_reduce left alone (folded_run) -- are known from the keys of the window alone, so
+// R of them are in flight at a time whatever run they belong to, and the runs' Adagrad
+// steps follow in worker order on registers.
+template <int NV, bool VEC, int R>
+__global__ __launch_bounds__(kRowThreads) void row_walk_kernel(
+    const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
+    const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
+    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
+  if (row >= rows0 + rows1) return;
+  const uint64_t target = (uint64_t)row << kbits;
+  // first position whose key is >= target; every round the 64 lanes probe the range at equal distances
+  int64_t lo = 0, hi = n;
+  while (hi > lo) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t p = lo + (int64_t)(lane + 1) * step - 1;
+    const bool below = p < hi && keys[p] < target;
+    const int cnt = __popcll(__ballot(below));  // the keys are sorted: the probes below the target are the first cnt
+    const int64_t nhi = lo + (int64_t)(cnt + 1) * step - 1;
+    lo += (int64_t)cnt * step;
+    hi = nhi < hi ? nhi : hi;
+  }
+  const int64_t s = lo;
+  if (s >= n || (keys[s] >> kbits) != (uint64_t)row) return;
+  const int nv = VEC ? (dim >> 2) : dim;
+  const float fdim = (float)dim;
+  float* wrow = row < rows0 ? w0 + row * dim : w1 + (row - rows0) * dim;
+  float* gptr = row < rows0 ? g0 + row : g1 + (row - rows0);
+  RowRegs<NV, VEC> w, acc;
+  w.load(wrow, nv, lane);
+  float gsum = *gptr;
+  acc.zero();
+  for (int64_t wb = s & ~(int64_t)(kWave - 1);; wb += kWave) {
+    const int64_t p = wb + lane;
+    const bool inb = p < n;
+    const uint64_t key = inb ? keys[p] : ~0ull;
+    const uint32_t val = inb ? vals[p] : 0u;
+    const bool in_row = inb && p >= s && (key >> kbits) == (uint64_t)row;
+    const uint64_t m_in = __ballot(in_row);
+    if (m_in == 0ull) break;
+    // the keys just outside the window (only looked at where a neighbour inside is in the row)
+    const uint64_t key_before = wb > 0 ? keys[wb - 1] : ~key;
+    const uint64_t key_after = wb + kWave < n ? keys[wb + kWave] : ~0ull;
+    uint64_t prev = __shfl_up(key, 1, 64), next = __shfl_down(key, 1, 64);
+    if (lane == 0) prev = key_before;
+    if (lane == kWave - 1) next = key_after;
+    const uint64_t starts = __ballot(in_row && (p == 0 || prev != key));   // first position of a run
+    const uint64_t lasts = __ballot(in_row && (p == n - 1 || next != key));  // last position of a run
+    // the rows to read, and the positions after which a run is complete
+    uint64_t todo = 0ull, done = 0ull;
+    for (uint64_t st = starts; st != 0ull; st &= st - 1) {
+      const int a = __ffsll((unsigned long long)st) - 1;
+      const uint64_t from = lasts & (~0ull << a);
+      const int e = from != 0ull ? __ffsll((unsigned long long)from) - 1 : -1;  // -1: the run goes on past the window
+      const int len = e - a + 1;
+      if (e >= 0 && len >= 2 && len <= kShort && (a / kTile) == (e / kTile)) {  // folded_run: the window starts at a multiple of kTile
+        todo |= ((2ull << e) - 1) & (~0ull << a);
+        done |= 1ull << e;
+      } else {  // the run's sum is in its first row (tile_reduce, run_combine)
+        todo |= 1ull << a;
+        done |= 1ull << a;
+      }
+    }
+    while (todo != 0ull) {
+      int pos[R];
+      const int first = __ffsll((unsigned long long)todo) - 1;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        pos[r] = todo != 0ull ? __ffsll((unsigned long long)todo) - 1 : -1;
+        todo &= todo - 1;  // (0 stays 0)
+      }
+      // all R loads are issued before the first is used; slots past the end read the first row again and are dropped
+      RowRegs<NV, VEC> x[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        x[r].load(grad_rows + (int64_t)lane_u32(val, pos[r] >= 0 ? pos[r] : first) * dim, nv, lane);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (pos[r] < 0) break;
+        acc.add(x[r]);
+        if ((done >> pos[r]) & 1ull) {
+          gsum = adagrad_apply(w, acc, gsum, fdim, lr);
+          acc.zero();
+        }
+      }
+    }
+    if (!(m_in >> (kWave - 1))) break;  // the row's stretch ended inside the window
+  }
+  w.store(wrow, nv, lane);
+  if (lane == 0) *gptr = gsum;
+}
+
 // The same for rows of at most 128 floats (dim % 4 == 0): half a wave per sorted
 // position, one 128-bit word per lane, so a wave keeps twice as many rows in
 // flight for the same registers.  The two halves of a wave run the same code on
@@ -630,13 +732,21 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
   const int64_t borders = ceil_div(n, kTile) - 1;
   const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
+  // gradient rows outnumbering the tables' rows 16 times over: a wave per table row (row_walk_kernel)
+  const int64_t table_rows = rows0 + rows1;
+  const bool walk = kbits > 0 && table_rows > 0 && n >= 16 * table_rows && getenv("PBG_DISABLE_ROW_WALK") == nullptr;
+  const dim3 walk_grid((unsigned)ceil_div(table_rows > 0 ? table_rows : 1, wpb));
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim,       \
-                       (int)(kbits == 0));                                                                      \
+                       (int)(kbits == 0 || walk));                                                              \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
-    if (VEC && dim <= 128) {                                                                                       \
+    if (walk) {                                                                                                    \
+      constexpr int R = NV <= 2 ? 8 : (NV <= 4 ? 4 : 2);                                                           \
+      hipLaunchKernelGGL((row_walk_kernel<NV, VEC, R>), walk_grid, block, 0, stream, keys, vals, n, kbits, grad_rows,  \
+                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+    } else if (VEC && dim <= 128) {                                                                                \
       constexpr int R = 4;                                                                                         \
       const dim3 hgrid((unsigned)ceil_div(ceil_div(n, R) * 32, kRowThreads));                                      \
       hipLaunchKernelGGL((row_update_half_kernel<R>), hgrid, block, 0, stream, keys, vals, n, kbits, grad_rows,    \
