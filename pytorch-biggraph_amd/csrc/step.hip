@@ -1771,67 +1771,108 @@ __device__ __forceinline__ int64_t block_scan_end(const uint64_t* __restrict__ k
   }
 }
 
-// Element-wise operators: one workgroup per (relation present in the call, 64-element slice).
-// It walks the relation's runs (one per batch, ascending), sums each run's parameter
-// gradient over the run's edges in a fixed order and applies AsyncAdagrad
-// (async_adagrad.py:75-85) before the next run: the K batches' updates in order.
-__global__ __launch_bounds__(256) void dyn_param_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
-                                                        const uint32_t* __restrict__ vals, float* p0, float* p1,
-                                                        float* s0, float* s1, float lr) {
+// Element-wise operators, in two kernels.  A relation's runs (its edges of one batch each,
+// ascending) update its parameters one after the other (AsyncAdagrad,
+// async_adagrad.py:75-85: the K batches' updates in order), but a run's gradient depends
+// on nothing but the tables as they were on entry:
+//   grad    one workgroup per (run, 64-element slice) sums the run's parameter gradient over
+//           its edges in a fixed order and leaves it at the run's first sorted position;
+//   apply   one wave per (relation present in the call, 64-element slice) walks the
+//           relation's runs and applies their gradients in order.
+// With relation frequencies following a power law the busiest relation owns a tenth of a
+// call's edges: walking its runs AND their edges in one chain of dependent loads would take
+// longer than everything else in the call together.
+__device__ __forceinline__ float dyn_param_term(const StepCtx& c, const SideCtx& sd, int64_t edge, int e, int H) {
+  const int D = c.D;
+  const float* dz = sd.dz + edge * D;
+  if (c.op == PBG_OP_TRANSLATION) return dz[e];
+  const float* x = sd.w + clamp_index(sd.idx[edge], sd.num_rows) * D;
+  if (c.op == PBG_OP_DIAGONAL) return x[e] * dz[e];
+  if (e < H) return x[e] * dz[e] + x[e + H] * dz[e + H];
+  const int h = e - H;
+  return x[h] * dz[h + H] - x[h + H] * dz[h];
+}
+
+__global__ __launch_bounds__(256) void dyn_param_grad_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
+                                                             const uint32_t* __restrict__ vals, float* __restrict__ grun) {
   __shared__ float sh[4][64];
   __shared__ int64_t sh_end;
   const SideCtx& sd = c.side[s];
   const int64_t n = (int64_t)c.K * c.B;
   const int64_t i = blockIdx.x;
-  const uint64_t rel = keys[i] >> c.kbits;
-  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;
+  const uint64_t key = keys[i];
+  if (i > 0 && keys[i - 1] == key) return;  // not the first position of a run
   const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
   const int e = blockIdx.y * 64 + lane;
   const int D = c.D, H = D / 2;
-  float* p;
-  float* st;
-  if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
-    p = (e < H) ? p0 + rel * H + e : p1 + rel * H + (e - H);
-    st = (e < H) ? s0 + rel * H + e : s1 + rel * H + (e - H);
-  } else {
-    p = p0 + rel * D + e;
-    st = s0 + rel * D + e;
+  const int64_t end = block_scan_end(keys, i, n, key, 0, &sh_end);
+  float acc = 0.f;
+  if (e < D) {
+    int64_t r = i + rg;
+    for (; r + 4 < end; r += 8) {  // two edges' chains of loads (value -> index -> rows) in flight
+      const int64_t e0 = vals[r], e1 = vals[r + 4];
+      const float t0 = dyn_param_term(c, sd, e0, e, H), t1 = dyn_param_term(c, sd, e1, e, H);
+      acc += t0;
+      acc += t1;
+    }
+    if (r < end) acc += dyn_param_term(c, sd, vals[r], e, H);
   }
+  sh[rg][lane] = acc;
+  __syncthreads();
+  if (rg == 0 && e < D) {
+    float g = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
+    // N3 on the parameters of the run's edges (regularizers.py:73-76), from the values before this call
+    if (c.reg_coef != 0.f) g += (float)(end - i) * sd.reg_pgrad[(key >> c.kbits) * D + e];
+    grun[i * D + e] = g;
+  }
+}
+
+__global__ __launch_bounds__(64) void dyn_param_apply_kernel(StepCtx c, const uint64_t* __restrict__ keys,
+                                                             const float* __restrict__ grun, float* p0, float* p1, float* s0,
+                                                             float* s1, float lr) {
+  const int64_t n = (int64_t)c.K * c.B;
+  const int64_t i = blockIdx.x;
+  const uint64_t rel = keys[i] >> c.kbits;
+  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;  // not the first position of a relation
+  const int lane = threadIdx.x;
+  const int e = blockIdx.y * 64 + lane;
+  const int D = c.D, H = D / 2;
+  const bool on = e < D;
+  float* p = nullptr;
+  float* st = nullptr;
+  if (on) {
+    if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+      p = (e < H) ? p0 + rel * H + e : p1 + rel * H + (e - H);
+      st = (e < H) ? s0 + rel * H + e : s1 + rel * H + (e - H);
+    } else {
+      p = p0 + rel * D + e;
+      st = s0 + rel * D + e;
+    }
+  }
+  float pv = on ? *p : 0.f, sum = on ? *st : 0.f;
   int64_t j = i;
-  while (j < n && (keys[j] >> c.kbits) == rel) {
-    const int64_t end = block_scan_end(keys, j, n, keys[j], 0, &sh_end);
-    float acc = 0.f;
-    if (e < D) {
-      for (int64_t r = j + rg; r < end; r += 4) {
-        const int64_t edge = vals[r];
-        const float* dz = sd.dz + edge * D;
-        if (c.op == PBG_OP_TRANSLATION) {
-          acc += dz[e];
-          continue;
-        }
-        const float* x = sd.w + clamp_index(sd.idx[edge], sd.num_rows) * D;
-        if (c.op == PBG_OP_DIAGONAL) {
-          acc += x[e] * dz[e];
-        } else if (e < H) {
-          acc += x[e] * dz[e] + x[e + H] * dz[e + H];
-        } else {
-          const int h = e - H;
-          acc += x[h] * dz[h + H] - x[h + H] * dz[h];
-        }
+  while (true) {
+    const float g = on ? grun[j * D + e] : 0.f;
+    // the next run: the first later position with another key (all lanes scan together)
+    const uint64_t key = keys[j];
+    int64_t base = j + 1, next;
+    while (true) {
+      const int64_t q = base + lane;
+      const uint64_t m = __ballot(q < n && keys[q] == key);
+      if (m != ~0ull) {
+        next = base + (__ffsll((unsigned long long)~m) - 1);
+        break;
       }
+      base += 64;
     }
-    sh[rg][lane] = acc;
-    __syncthreads();
-    if (rg == 0 && e < D) {
-      float g = (sh[0][lane] + sh[1][lane]) + (sh[2][lane] + sh[3][lane]);
-      // N3 on the parameters of the run's edges (regularizers.py:73-76), from the values before this call
-      if (c.reg_coef != 0.f) g += (float)(end - j) * sd.reg_pgrad[rel * D + e];
-      const float sum = *st + g * g;
-      *st = sum;
-      *p += -lr * (g / (sqrtf(sum) + 1e-10f));
-    }
-    __syncthreads();
-    j = end;
+    sum += g * g;
+    pv += -lr * (g / (sqrtf(sum) + 1e-10f));
+    if (next >= n || (keys[next] >> c.kbits) != rel) break;
+    j = next;
+  }
+  if (on) {
+    *st = sum;
+    *p = pv;
   }
 }
 
@@ -2030,6 +2071,7 @@ struct Plan {
   uint32_t *rvals_a, *rvals_b;
   void* rsort_temp;
   void* rel_start;  // first sorted position of every relation (`linear` only)
+  float* dyn_grun;  // element-wise operators: the parameter gradient of every (relation, batch) run, at the run's first sorted position [K * B, D]
   int nvh;
   float* gth;   // partial sums of the global embeddings' gradients [2, K, gslices, D]
   int gslices;
@@ -2225,6 +2267,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     plan->rvals_b = (uint32_t*)take(ne, 4);
     plan->rsort_temp = take(sort_temp_bytes(ne), 1);
     if (c.op == PBG_OP_LINEAR) plan->rel_start = take(seg_linear_update_temp_bytes(c.num_relations, ne, D, K), 1);
+    if (c.op != PBG_OP_LINEAR || c.affine) plan->dyn_grun = takef((size_t)ne * D);
   }
   for (int s = 0; s < 2; ++s) {
     plan->pslices[s] = 1;
@@ -2528,12 +2571,16 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
         if (c.affine) {  // the translations: the element-wise kernel on dz, parameters in the second slot
           StepCtx ct = c;
           ct.op = PBG_OP_TRANSLATION;
-          hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, ct,
-                             s, rkeys, rvals, p1, nullptr, s1, nullptr, d->relation_lr);
+          hipLaunchKernelGGL(dyn_param_grad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream,
+                             ct, s, rkeys, rvals, plan.dyn_grun);
+          hipLaunchKernelGGL(dyn_param_apply_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(64), 0, stream,
+                             ct, rkeys, plan.dyn_grun, p1, nullptr, s1, nullptr, d->relation_lr);
         }
       } else {
-        hipLaunchKernelGGL(dyn_param_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
-                           rkeys, rvals, p0, p1, s0, s1, d->relation_lr);
+        hipLaunchKernelGGL(dyn_param_grad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c,
+                           s, rkeys, rvals, plan.dyn_grun);
+        hipLaunchKernelGGL(dyn_param_apply_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(64), 0, stream, c,
+                           rkeys, plan.dyn_grun, p0, p1, s0, s1, d->relation_lr);
       }
     }
     return check_launch("step params (dynamic)");
