@@ -153,6 +153,13 @@ def algorithmic(w, spec):
     # cores are the roofline that bounds it.
     out["fused_chunk"] = ("mfma", 3 * 2.0 * (b * d + 2 * c * p * n * d))
     out["fused_chunk_bytes"] = rows * (2 * 4 * d + 8) + 3 * b * 8
+    # The streaming chunk kernel (positives in LDS, negatives streamed past them twice): the three products of
+    # both sides, every score matrix with the chunk's P own rows as its first columns (their diagonal carries
+    # the positive pair).  Its HBM side: every negative's raw row read in both sweeps (from the table, by id),
+    # its gradient row written once, the positives' operand rows read and their gradients written.
+    ns = p + u
+    out["stream_chunk"] = ("mfma", 3 * 2.0 * 2 * c * p * ns * d)
+    out["stream_chunk_bytes"] = 2 * c * ns * (3 * 4 * d + 4) + 2 * b * (3 * 4 * d)
     return out
 
 
@@ -363,6 +370,7 @@ def main():
         rel_edges[:full] = rel_edges[:full].view(-1, b).sort(dim=1).values.reshape(-1)
 
     enqueue_s = [0.0]  # host time per call of the last run's timed loop (launches only, no wait)
+    route_of = {}      # workers -> which kernels pbg_train_step ran ("staged", "fused", "stream")
 
     def run(workers, calls, warm_calls, profile_calls=0, hip_graph=False):
         spec, runner = make_runner(workers)
@@ -420,11 +428,16 @@ def main():
                 ms = one_call(warm_calls + calls + i, profiled=True)
                 acc = ms if acc is None else [a + m for a, m in zip(acc, ms)]
             stages = dict(zip(runner.STAGES, [a / profile_calls for a in acc]))
-            if runner.fused:
+            if runner.route == "fused":
                 # one kernel covers stages "prep" .. "rowback"; "loss" holds the per-batch reduction of the statistics
                 stages = {"fused_chunk": stages["prep"], "loss_reduce": stages["loss"], "params": stages["params"],
                           "sort": stages["sort"], "update": stages["update"]}
+            elif runner.route == "stream":
+                # per-edge preparation + column ids | the chunk kernel | per-edge finish + the statistics' reduction
+                stages = {"stream_prep": stages["prep"], "stream_chunk": stages["scores"], "stream_finish": stages["rowback"],
+                          "params": stages["params"], "sort": stages["sort"], "update": stages["update"]}
         loss = float(runner.loss_out.mean().item()) / b
+        route_of[workers] = runner.route
         return spec, calls * per_call / dt, dt / calls * 1e3, dt, stages, loss
 
     workers = max(1, args.workers)
@@ -433,6 +446,7 @@ def main():
     warmup = args.warmup if args.warmup is not None else max(1, steps // 10)
     spec, eps, ms_per_step, wall_s, stages, loss = run(workers, steps, warmup, profile_calls=10)
     host_enqueue_ms = enqueue_s[0] * 1e3
+    route = route_of[workers]
 
     seq = None
     if not args.no_sequential and workers > 1:
@@ -464,9 +478,9 @@ def main():
                     "achieved": (alg[k][1] * workers / (stages[k] * 1e-3) / (1e9 if alg[k][0] == "hbm" else 1e12)) if stages[k] > 0 else None}
                 for k in stages if k in alg},
     }
-    if dominant == "fused_chunk":
+    if dominant in ("fused_chunk", "stream_chunk"):
         # the same launch against the other roofline: rows read once + gradient rows written once
-        roofline["algorithmic_hbm_gbs"] = alg["fused_chunk_bytes"] * workers / seconds / 1e9
+        roofline["algorithmic_hbm_gbs"] = alg[dominant + "_bytes"] * workers / seconds / 1e9
 
     line = {
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X",
@@ -474,7 +488,7 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
-                   "hogwild_workers": workers, "step": f"one pbg_train_step call of {workers} batches",
+                   "hogwild_workers": workers, "step": f"one pbg_train_step call of {workers} batches", "route": route,
                    "timed_calls": steps, "timed_batches": steps * workers, "timed_edges": steps * workers * b,
                    "timed_wall_seconds": wall_s, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
                    "mean_loss_per_edge_last_call": loss, "host_enqueue_ms_per_call": host_enqueue_ms},
