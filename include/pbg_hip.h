@@ -172,6 +172,12 @@ typedef struct pbg_step_buffers {
   float* g_lhs;               /* [num_lhs_rows]  RowAdagrad state["sum"] */
   float* w_rhs;               /* [num_rhs_rows, D] */
   float* g_rhs;               /* [num_rhs_rows] */
+  /* Entity and relation ids are NOT validated on the device: an id outside
+   * [0, num_*_rows) (or [0, num_relations)) is clamped to the nearest valid one, so the
+   * step reads and updates row 0 or the last row instead, where the reference's
+   * F.embedding raises IndexError (model.py:60-61).  A caller that cannot vouch for
+   * its ids checks them first (pytorch_biggraph_amd.native.StepRunner.train(check_ids=True)
+   * does, with one device reduction per array). */
   const int64_t* lhs;         /* [K, B] */
   const int64_t* rhs;         /* [K, B] */
   const int64_t* rel;         /* standard: [K]; dynamic: [K, B] */

@@ -373,13 +373,36 @@ class StepRunner:
         bufs.uniform_seed = (uniform_seed or 0) & (2**64 - 1)
         return bufs
 
-    def train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None, uniform_seed=None) -> None:
+    def train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None, uniform_seed=None,
+              check_ids: bool = False) -> None:
         """One lock-step training step over num_workers batches; statistics land
         in self.loss_out / self.violators_out (device, no sync).  The uniform
         negatives are either given ([K, C, U] per side) or drawn inside the step
-        from `uniform_seed` (sample_uniform_negatives shows which)."""
+        from `uniform_seed` (sample_uniform_negatives shows which).
+
+        The kernels clamp an id outside its table instead of failing.  With
+        `check_ids` the ids are range-checked first (one reduction per array and
+        one host synchronisation) and an IndexError is raised as F.embedding does
+        in the reference (model.py:60-61)."""
+        if check_ids:
+            self._check_ids(lhs, rhs, rel, uniform_lhs, uniform_rhs)
         bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight, uniform_seed)
         check(_lib.lib().pbg_train_step(ctypes.byref(self.desc), ctypes.byref(bufs), _stream()))
+
+    def _check_ids(self, lhs, rhs, rel, uniform_lhs, uniform_rhs) -> None:
+        bounds = []
+        for name, ids, limit in (("lhs", lhs, self.w_lhs.shape[0]), ("rhs", rhs, self.w_rhs.shape[0]),
+                                 ("rel", rel, self.spec.num_relations), ("uniform_lhs", uniform_lhs, self.w_lhs.shape[0]),
+                                 ("uniform_rhs", uniform_rhs, self.w_rhs.shape[0])):
+            if ids is not None and ids.numel() > 0:
+                lo, hi = torch.aminmax(ids)
+                bounds.append((name, limit, lo, hi))
+        if not bounds:
+            return
+        found = torch.stack([torch.stack((lo, hi)) for _, _, lo, hi in bounds]).tolist()
+        for (name, limit, _, _), (lo, hi) in zip(bounds, found):
+            if lo < 0 or hi >= limit:
+                raise IndexError(f"{name}: index out of range ({lo if lo < 0 else hi} not in [0, {limit}))")
 
     def capture_train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None) -> "torch.cuda.CUDAGraph":
         """Records one train() call into a HIP graph and returns it.  The tensors

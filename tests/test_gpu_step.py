@@ -581,6 +581,29 @@ def test_train_step_with_edge_weights(pbg, case, workers):
             runner.train(lhs, rhs, rel, ul, ur, edge_weight=bad)
 
 
+def test_ids_out_of_range_are_found_when_asked(pbg):
+    """The kernels clamp ids; StepRunner.train(check_ids=True) raises the IndexError
+    the reference's F.embedding raises (model.py:60-61), before anything is trained."""
+    say("check_ids")
+    cfg = ostep.StepConfig(dim=16, operator="translation", comparator="dot", loss="ranking", num_relations=3,
+                           num_batch_negs=5, num_uniform_negs=5, lr=0.1, relation_lr=0.01, margin=0.1)
+    st, batches = make_inputs(cfg, 20, 50, 2, seed=5, shared=True)
+    runner = to_runner(pbg, cfg, st, 20, 2)
+    lhs, rhs, rel, ul, ur = pack(cfg, batches)
+    before = runner.w_lhs.clone()
+    runner.train(lhs, rhs, rel, ul, ur, check_ids=True)  # in range: trains
+    torch.cuda.synchronize()
+    assert not torch.equal(before, runner.w_lhs)
+    after = runner.w_lhs.clone()
+    for which, value in ((0, 50), (1, -1), (2, 3), (3, 50), (4, -7)):
+        args = [lhs.clone(), rhs.clone(), rel.clone(), ul.clone(), ur.clone()]
+        args[which].view(-1)[-1] = value
+        with pytest.raises(IndexError):
+            runner.train(*args, check_ids=True)
+    torch.cuda.synchronize()
+    assert torch.equal(after, runner.w_lhs)
+
+
 def test_global_embeddings_are_refused_for_dynamic_relations(pbg):
     spec = pbg.StepSpec(dim=8, batch_size=10, dynamic=True, num_relations=2)
     w = torch.randn(20, 8, device=DEV)
