@@ -60,6 +60,10 @@ WORKLOADS = {
                   entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=1000,
                   operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=True,
                   init_scale=1e-3, zipf=1.1, two_tables=False),
+    "fb15k": dict(desc="the reference's FB15k example as configured (examples/configs/fb15k_config_cpu.py): 1345 relations (dynamic), complex_diagonal/dot/softmax, dim 400, 14951 entities, B=1000, chunk 50 + 1000 uniform negatives, N3 regularizer 1e-3",
+                  entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=1000,
+                  operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=True,
+                  init_scale=1e-3, zipf=1.1, two_tables=False, regularization_coef=1e-3),
 }
 
 
@@ -117,7 +121,8 @@ def cpu_baseline(w, seconds):
         rel = power_law_ids(n, w["relations"], s_rel, gen, "cpu") if s_rel else torch.randint(0, w["relations"], (n,), generator=gen)
     cfg = ostep.StepConfig(dim=d, operator=w["operator"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
                            num_batch_negs=w["batch_negs"], num_uniform_negs=w["uniform_negs"], dynamic=w["dynamic"],
-                           num_relations=w["relations"], lr=0.1, relation_weights=[1.0] * w["relations"])
+                           num_relations=w["relations"], lr=0.1, relation_weights=[1.0] * w["relations"],
+                           regularization_coef=w.get("regularization_coef", 0.0))
     eps, edges, wall = hogwild.run(cfg, tables[0], lhs, rhs, rel, b, cores, seconds,
                                    w_rhs=tables[1] if len(tables) > 1 else None)
     note = "" if sample["entities"] == w["entities"] else f", first {sample['entities']} table rows"
@@ -330,7 +335,7 @@ def main():
         spec = pkg.StepSpec(dim=d, batch_size=b, num_workers=workers, num_batch_negs=w["batch_negs"],
                             num_uniform_negs=w["uniform_negs"], operator=w["operator"], dynamic=w["dynamic"],
                             num_relations=w["relations"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
-                            lr=0.1)
+                            lr=0.1, regularization_coef=w.get("regularization_coef", 0.0))
         ws = [t.clone() for t in tables]
         gs = [torch.zeros(t.shape[0], device=dev) for t in tables]
         rhs_op, rhs_sum = {}, {}
@@ -442,7 +447,7 @@ def main():
         return spec, calls * per_call / dt, dt / calls * 1e3, dt, stages, loss
 
     workers = max(1, args.workers)
-    default_batches = {"cfg1": 64000, "cfg2": 400, "cfg2d": 400, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
+    default_batches = {"cfg1": 64000, "cfg2": 400, "cfg2d": 400, "fb15k": 400, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
     steps = args.steps if args.steps is not None else max(1, default_batches // workers)
     warmup = args.warmup if args.warmup is not None else max(1, steps // 10)
     spec, eps, ms_per_step, wall_s, stages, loss = run(workers, steps, warmup, profile_calls=10)

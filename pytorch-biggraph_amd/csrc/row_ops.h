@@ -243,6 +243,31 @@ __device__ __forceinline__ RowV<NVH> op_backward(int op, const RowV<NVH>& dz, co
   return dx;
 }
 
+// N3 regularizer (regularizers.py:51-97) on one prepared row y: adds
+// d (coef * sum m^3) / dy = 3 coef m y to dy and returns this lane's share of
+// sum m^3, where m is the modulus of a complex coordinate (y[e], y[e + D/2]) for
+// complex_diagonal (operators.py:154-157) and |y[e]| otherwise (operators.py:42-43).
+template <int NVH>
+__device__ __forceinline__ float n3_term(int op, float coef, RowV<NVH>& dy, const RowV<NVH>& y) {
+  float cubes = 0.f;
+  const float c3 = 3.0f * coef;
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    if (op == PBG_OP_COMPLEX_DIAGONAL) {
+      const float m = sqrtf(y.a[0][v] * y.a[0][v] + y.a[1][v] * y.a[1][v]);
+      dy.a[0][v] += c3 * m * y.a[0][v];
+      dy.a[1][v] += c3 * m * y.a[1][v];
+      cubes += m * m * m;
+    } else {
+      const float m0 = fabsf(y.a[0][v]), m1 = fabsf(y.a[1][v]);
+      dy.a[0][v] += c3 * m0 * y.a[0][v];
+      dy.a[1][v] += c3 * m1 * y.a[1][v];
+      cubes += m0 * m0 * m0 + m1 * m1 * m1;
+    }
+  }
+  return cubes;
+}
+
 // comparator.prepare (model.py:161-162,187-192,251-252), in place; returns the
 // per-row aux value: 1/norm for cos, norm^2 for l2 (model.py:228-229).
 template <int NVH>

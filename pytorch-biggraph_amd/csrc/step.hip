@@ -713,31 +713,6 @@ __device__ __forceinline__ float column_sum(const float* __restrict__ s, int64_t
   return wave_sum(acc);
 }
 
-// N3 regularizer (regularizers.py:51-97) on one prepared row y: adds
-// d (coef * sum m^3) / dy = 3 coef m y to dy and returns this lane's share of
-// sum m^3, where m is the modulus of a complex coordinate (y[e], y[e + D/2]) for
-// complex_diagonal (operators.py:154-157) and |y[e]| otherwise (operators.py:42-43).
-template <int NVH>
-__device__ __forceinline__ float n3_term(int op, float coef, RowV<NVH>& dy, const RowV<NVH>& y) {
-  float cubes = 0.f;
-  const float c3 = 3.0f * coef;
-#pragma unroll
-  for (int v = 0; v < NVH; ++v) {
-    if (op == PBG_OP_COMPLEX_DIAGONAL) {
-      const float m = sqrtf(y.a[0][v] * y.a[0][v] + y.a[1][v] * y.a[1][v]);
-      dy.a[0][v] += c3 * m * y.a[0][v];
-      dy.a[1][v] += c3 * m * y.a[1][v];
-      cubes += m * m * m;
-    } else {
-      const float m0 = fabsf(y.a[0][v]), m1 = fabsf(y.a[1][v]);
-      dy.a[0][v] += c3 * m0 * y.a[0][v];
-      dy.a[1][v] += c3 * m1 * y.a[1][v];
-      cubes += m0 * m0 * m0 + m1 * m1 * m1;
-    }
-  }
-  return cubes;
-}
-
 // dy += dpos * d kappa(self, other) / d self
 template <int NVH>
 __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos, const RowV<NVH>& self,
@@ -917,8 +892,10 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
 // of the parameter gradient of element e: diagonal x.dz, translation dz,
 // complex_diagonal (real | imag).  Fixed summation order, no atomics.
 constexpr int kParamGroups = 16;
+// `reg_op`: the operator whose parameters the N3 term is taken over (c.op, except where the caller
+// has set c.op to translation to get plain column sums of rows that hold finished gradient terms).
 __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c, int s, float* __restrict__ dth,
-                                                                        int slices) {
+                                                                        int slices, int reg_op) {
   __shared__ float sh[kParamGroups][64];
   const SideCtx& sd = c.side[s];
   const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
@@ -979,7 +956,7 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
       // m = |p| (operators.py:69-70,83-84) or the modulus of (real, imag) (operators.py:151-152)
       const int64_t r = clamp_index(c.rel[k], c.num_relations);
       const float c3 = 3.0f * c.reg_coef * (float)c.C;
-      if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+      if (reg_op == PBG_OP_COMPLEX_DIAGONAL) {
         const int h = e < H ? e : e - H;
         const float re = sd.p0[r * H + h], im = sd.p1[r * H + h];
         total += c3 * sqrtf(re * re + im * im) * (e < H ? re : im);
@@ -2610,14 +2587,14 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
       StepCtx cg = c;
       if (edge_terms) cg.op = PBG_OP_TRANSLATION;  // (whose gradient is the column sum of dz)
       hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
-                         dim3(kParamGroups * 64), 0, stream, cg, s, plan.dth[s], plan.pslices[s]);
+                         dim3(kParamGroups * 64), 0, stream, cg, s, plan.dth[s], plan.pslices[s], c.op);
     }
     if (c.affine) {  // the translation: column sums of dz, then its own Adagrad steps (parameters in the second slot)
       StepCtx ct = c;
       ct.op = PBG_OP_TRANSLATION;
       const int sl = plan.pslices_t[s];
       hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)sl),
-                         dim3(kParamGroups * 64), 0, stream, ct, s, plan.dth_t[s], sl);
+                         dim3(kParamGroups * 64), 0, stream, ct, s, plan.dth_t[s], sl, PBG_OP_TRANSLATION);
       if (K <= kWave) {
         hipLaunchKernelGGL(param_update_wave_kernel, dim3((unsigned)ceil_div(D, kWavesPerBlock)), dim3(kRowThreads), 0,
                            stream, ct, s, plan.dth_t[s], sl, (int64_t)D, p1, nullptr, s1, nullptr, d->relation_lr);
@@ -2740,6 +2717,16 @@ void launch_loss(const StepCtx& c, hipStream_t s) {
   else launch_loss_depth<0>(c, s);
 }
 
+// The regularizer's parameter terms and per-batch value, once the positives' cubes are written.
+// Reads the operator parameters: before run_params updates them.
+void launch_reg(const StepCtx& c, hipStream_t s) {
+  if (c.reg_coef == 0.f) return;
+  if (c.dynamic && c.op != PBG_OP_NONE)
+    for (int side = 0; side < 2; ++side)
+      hipLaunchKernelGGL(reg_factor_kernel, wave_grid(c.num_relations), dim3(kRowThreads), 0, s, c, side);
+  hipLaunchKernelGGL(reg_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+}
+
 int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_t s, hipEvent_t* ev) {
   int rc = validate(desc, true);
   if (rc != PBG_OK) return rc;
@@ -2771,6 +2758,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(6);
     if ((rc = stream_finish(c, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
     hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
+    launch_reg(c, s);
     mark(7);
   } else if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
@@ -2799,12 +2787,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if ((rc = run_backward_da(plan, s)) != PBG_OK) return rc;
     mark(6);
     if ((rc = run_rowback(plan, s)) != PBG_OK) return rc;
-    if (c.reg_coef != 0.f) {  // reads the operator parameters: before run_params updates them
-      if (c.dynamic && c.op != PBG_OP_NONE)
-        for (int side = 0; side < 2; ++side)
-          hipLaunchKernelGGL(reg_factor_kernel, wave_grid(c.num_relations), dim3(kRowThreads), 0, s, c, side);
-      hipLaunchKernelGGL(reg_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
-    }
+    launch_reg(c, s);
     mark(7);
   }
   if ((rc = run_params(desc, bufs, plan, s, &rel_order, stream)) != PBG_OK) return rc;

@@ -612,7 +612,8 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
 // One wave per edge: the two raw-row gradients of the pair from the four partial
 // rows the items left (the row as the other item's operand, mapped back through
 // the operator, plus the row as a batch negative of its own side), the edge's loss,
-// and (standard mode) the edge's term of the operator's parameter gradient.
+// the N3 regularizer's terms of the edge's rows, and (standard mode) the edge's term
+// of the operator's parameter gradient.
 template <int NVH>
 __global__ __launch_bounds__(kRowThreads) void stream_finish_kernel(StepCtx c, StreamPlan a) {
   const int lane = threadIdx.x & 63;
@@ -629,10 +630,41 @@ __global__ __launch_bounds__(kRowThreads) void stream_finish_kernel(StepCtx c, S
   const int64_t e = (int64_t)k * c.B + q;
   const SideCtx& s0 = c.side[0];
   const SideCtx& s1 = c.side[1];
-  const RowV<NVH> a0 = row_load<NVH>(a.sda[0] + e * D, D, H, lane);  // gradient at the operand derived from the rhs row
-  const RowV<NVH> a1 = row_load<NVH>(a.sda[1] + e * D, D, H, lane);  // ... from the lhs row
+  RowV<NVH> a0 = row_load<NVH>(a.sda[0] + e * D, D, H, lane);  // gradient at the operand derived from the rhs row
+  RowV<NVH> a1 = row_load<NVH>(a.sda[1] + e * D, D, H, lane);  // ... from the lhs row
   RowV<NVH> gl = row_load<NVH>(a.sdb[0] + e * D, D, H, lane);
   RowV<NVH> gr = row_load<NVH>(a.sdb[1] + e * D, D, H, lane);
+  const bool reg = c.reg_coef != 0.f;
+  RowV<NVH> xl, xr;
+  if (reg || (c.op != PBG_OP_NONE && !c.dynamic)) {
+    xl = row_load<NVH>(s0.w + clamp_index(s0.idx[e], s0.num_rows) * D, D, H, lane);
+    xr = row_load<NVH>(s1.w + clamp_index(s1.idx[e], s1.num_rows) * D, D, H, lane);
+  }
+  if (reg) {
+    // N3 over the rows the model hands the regularizer (model.py:784-785,845-854): the lhs row
+    // and op(rhs row); with one relation per edge each side's row in one direction and its
+    // operated row in the other (model.py:722-758).  The term of an operated row joins the
+    // gradient at that row, which then flows through the operator like the scores' part.
+    float cubes0 = n3_term<NVH>(c.op, c.reg_coef, gl, xl), cubes1;
+    const RowV<NVH> zr = row_load<NVH>(a.sa[0] + e * D, D, H, lane);  // op(rhs row)
+    if (c.dynamic) {
+      const RowV<NVH> zl = row_load<NVH>(a.sa[1] + e * D, D, H, lane);  // the lhs operator's op(lhs row)
+      cubes0 += n3_term<NVH>(c.op, c.reg_coef, a1, zl);
+      cubes1 = n3_term<NVH>(c.op, c.reg_coef, gr, xr) + n3_term<NVH>(c.op, c.reg_coef, a0, zr);
+      if (c.op != PBG_OP_NONE) {  // these rows are the operator-output gradients the parameter stage reads
+        row_store<NVH>(a.sda[0] + e * D, a0, D, H, lane);
+        row_store<NVH>(a.sda[1] + e * D, a1, D, H, lane);
+      }
+    } else {
+      cubes1 = n3_term<NVH>(c.op, c.reg_coef, a0, zr);
+    }
+    cubes0 = wave_sum(cubes0);
+    cubes1 = wave_sum(cubes1);
+    if (lane == 0) {
+      c.regrow[((int64_t)k * 2 + 0) * c.B + q] = cubes0;
+      c.regrow[((int64_t)k * 2 + 1) * c.B + q] = cubes1;
+    }
+  }
   if (c.op == PBG_OP_NONE) {
     row_axpy<NVH>(gl, 1.0f, a1);
     row_axpy<NVH>(gr, 1.0f, a0);
@@ -646,8 +678,6 @@ __global__ __launch_bounds__(kRowThreads) void stream_finish_kernel(StepCtx c, S
     row_axpy<NVH>(gr, 1.0f, op_backward<NVH>(c.op, a0, s1.p0, s1.p1, rel, D, H, lane));
     // d/d parameter of <lhs, op(rhs)>-shaped scores: through op(rhs) with gradient a0, and through
     // op^T(lhs) with gradient a1 (operators.py:59-84,128-157)
-    const RowV<NVH> xl = row_load<NVH>(s0.w + clamp_index(s0.idx[e], s0.num_rows) * D, D, H, lane);
-    const RowV<NVH> xr = row_load<NVH>(s1.w + clamp_index(s1.idx[e], s1.num_rows) * D, D, H, lane);
     RowV<NVH> t;
 #pragma unroll
     for (int v = 0; v < NVH; ++v) {
@@ -707,7 +737,7 @@ bool stream_dim_built(int D) { return D == 128 || D == 256 || D == 400; }
 
 bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
   memset(sp, 0, sizeof(*sp));
-  if (c.cmp != PBG_CMP_DOT || c.bias || c.affine || c.reg_coef != 0.f) return false;
+  if (c.cmp != PBG_CMP_DOT || c.bias || c.affine) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_DIAGONAL && c.op != PBG_OP_COMPLEX_DIAGONAL) return false;
   if (!stream_dim_built(c.D) || c.P > 64) return false;
   for (int s = 0; s < 2; ++s) {

@@ -1,8 +1,8 @@
 """The streaming route of the training step (a chunk's positives resident in LDS,
 its negatives gathered raw and streamed past them) against the oracle's lock-step
 training: every operator the route takes x every loss x both relation modes, the
-three row lengths it is built for, partial last chunks, edge weights, negatives
-drawn in the step, and the staged route on the same inputs."""
+three row lengths it is built for, partial last chunks, the N3 regularizer,
+edge weights and negatives drawn in the step."""
 import itertools
 import os
 
@@ -36,6 +36,20 @@ CASES += [
     # no batch negatives: the chunk is as long as the uniform draw (model.py:648-650)
     dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64, num_pos=150, dim=128),
     dict(operator="none", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=64, dim=256),
+    # the N3 regularizer (regularizers.py:51-97); the first is the reference's FB15k example
+    # (examples/configs/fb15k_config_cpu.py: ComplEx, one relation per edge, 1000 uniform negatives, coefficient 1e-3)
+    dict(operator="complex_diagonal", loss="softmax", dynamic=True, num_batch_negs=50, num_uniform_negs=1000, num_pos=120,
+         dim=400, regularization_coef=1e-3),
+    dict(operator="complex_diagonal", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=100, num_pos=130,
+         dim=128, regularization_coef=0.05),
+    dict(operator="diagonal", loss="logistic", dynamic=False, num_batch_negs=37, num_uniform_negs=91, num_pos=100, dim=256,
+         regularization_coef=0.02, shared=False),
+    dict(operator="diagonal", loss="softmax", dynamic=True, num_batch_negs=50, num_uniform_negs=100, num_pos=130, dim=128,
+         regularization_coef=0.05),
+    dict(operator="none", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=100, num_pos=130, dim=128,
+         regularization_coef=0.05),
+    dict(operator="none", loss="ranking", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=70, dim=128,
+         regularization_coef=0.05),
 ]
 
 
@@ -84,6 +98,8 @@ def test_stream_route_matches_the_oracle(pbg, case, workers):
                                      (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
             ties = violator_ties(pos, neg)
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
+        if cfg.regularization_coef:
+            assert out.reg > 0.0 and float(runner.reg_out[k]) == pytest.approx(out.reg, rel=1e-5), ("reg", k)
     compare_state(cfg, runner, st, 1e-5, "stream", st64)
 
 
