@@ -1054,7 +1054,7 @@ __global__ __launch_bounds__(kRowThreads) void param_update_wave_kernel(StepCtx 
 // chunk in one workgroup, operands resident in LDS
 // ---------------------------------------------------------------------------
 // Eligible shapes (standard mode, operator none / translation / diagonal,
-// comparator dot / l2, batch + uniform negatives on both sides, D <= 128,
+// comparator dot / cos / l2, batch + uniform negatives on both sides, D <= 128,
 // P <= 64, U <= 64) keep a chunk's 2(P+U) prepared rows and its two score
 // matrices in LDS (132 KB at P = U = 50, D = 100).  Eight waves: phase 0 gathers
 // and applies the operator; phase 1 forms S = A N^T with fp32 MFMA (one row tile
@@ -1074,6 +1074,7 @@ struct FusedLayout {
   int ldx, lds;                  // row strides (floats) of the operand rows and of the score rows
   int xn[2], sc[2], sq[2], rs[2], cs[2], pos, dpos;  // offsets in floats
   int part;                      // [2 sides][dLoss/dpos, weighted loss, violators][P] per-side results of the loss phase
+  int xch;                       // cos: [2 column groups][64 rows] partial <row, gradient row> of the product being written out
   int ids;                       // int32 row ids of the 2N operand rows (-1: padding), kFusedIds slots; last block
   int total;                     // floats
 };
@@ -1272,7 +1273,8 @@ __device__ __forceinline__ void fused_issue_rows(const StepCtx& c, const FusedGe
   x->glob1 = keep_if(g1, has_g1);
 }
 
-// Operator (rhs side) and, for l2, the squared norms; the rows of side S land in LDS.
+// Operator (rhs side) and, for l2, the squared norms (cos: the normalisation and the
+// reciprocal norms); the rows of side S land in LDS.
 // Only columns below D are written (the pad columns behind them were zeroed once,
 // when the kernel started).  `pads`: the chunk has padded positives (a partial last
 // chunk), whose rows are zeros.
@@ -1300,6 +1302,15 @@ __device__ __forceinline__ void fused_store_side(const StepCtx& c, const FusedGe
         y.x += x.par.x; y.y += x.par.y; y.z += x.par.z; y.w += x.par.w;
       }
     }
+    if (CMP == PBG_CMP_COS) {  // comparator.prepare: the row times the reciprocal of its norm (model.py:187-192)
+      const float sq = col_ok ? y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w : 0.f;
+      const float part = half_sum_at_31(sq);  // complete in lanes 31 and 63
+      const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part), 31));
+      const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part), 63));
+      const float inv = 1.0f / sqrtf(half ? hi : lo);
+      y.x *= inv; y.y *= inv; y.z *= inv; y.w *= inv;
+      if ((lane & 31) == 31) lds[(S ? g.sq1 : g.sq0) + j] = inv;
+    }
     if (pads && idv[S * (kFusedRounds / 2) + u] < 0) y = make_float4(0.f, 0.f, 0.f, 0.f);
     if (col_ok) *reinterpret_cast<float4*>(&lds[at]) = y;
     if (CMP == PBG_CMP_L2) {
@@ -1317,11 +1328,28 @@ struct FusedOut {
   const float* par;  // diagonal operator: its parameters at the wave's first column, or null
   int self_at, other_at;  // l2: LDS offsets of the row's own operand row and of its partner's, at the wave's first column
   float coef, pcoef;      // l2: v += coef * self + pcoef * (self - other)
+                          // cos: v = pcoef * (v - coef * self), the gradient through the normalisation
+                          // (pcoef = 1 / norm, coef = <self, v over the whole row>)
 };
 
-template <bool L2>
+// This lane's share of <own operand row, gradient row> over the columns it holds.
+__device__ __forceinline__ void fused_self_dot(const float* lds, int self_at, int col, int cols_left, float4 v, float* acc) {
+  if (col >= cols_left) return;
+  const float4 self = *reinterpret_cast<const float4*>(&lds[self_at + col]);
+  *acc += (self.x * v.x + self.y * v.y) + (self.z * v.z + self.w * v.w);
+}
+
+template <int CMP>
 __device__ __forceinline__ void fused_emit(const float* lds, const FusedOut& o, int col, int cols_left, float4 v) {
   if (col >= cols_left) return;  // past D (a multiple of 4)
+  constexpr bool L2 = CMP == PBG_CMP_L2;
+  if (CMP == PBG_CMP_COS) {
+    const float4 self = *reinterpret_cast<const float4*>(&lds[o.self_at + col]);
+    v.x = o.pcoef * (v.x - o.coef * self.x);
+    v.y = o.pcoef * (v.y - o.coef * self.y);
+    v.z = o.pcoef * (v.z - o.coef * self.z);
+    v.w = o.pcoef * (v.w - o.coef * self.w);
+  }
   if (L2) {
     const float4 self = *reinterpret_cast<const float4*>(&lds[o.self_at + col]);
     float4 other = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1406,6 +1434,10 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
   // array turns into a global load.
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool l2 = CMP == PBG_CMP_L2;
+  // cos: a gradient row goes back through the normalisation, dz = (dy - y <y, dy>) / norm, and the
+  // row is spread over the two waves that share its row tile: they exchange their shares of
+  // <y, dy> through LDS, one more barrier per product, which the helpers keep as well.
+  constexpr bool cosn = CMP == PBG_CMP_COS;
   constexpr int T0 = (T + 1) / 2, T1 = T - T0;
   constexpr int kLossCols = 2 * T;  // score columns per lane of the 8 lanes that share a row
   const int lane = threadIdx.x & 63;
@@ -1518,6 +1550,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
             lds[g.cs0 + j] = acc;
           }
         }
+        if (cosn && s == 1) lds_barrier();  // the exchange of step 3
         lds_barrier();  // (c) after side 0, (d) after side 1
       }
 
@@ -1563,16 +1596,19 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
           }
         }
       }
+      if (cosn) lds_barrier();  // the exchange of step 4
       lds_barrier();  // (e)
 
       // ---- step 5: the next chunk's rows into registers; they have two products' time to arrive ----
       fused_issue_rows(c, g, ids, rel_next, wave, ln, v, idv, &extras, more);
+      if (cosn) lds_barrier();  // the exchange of step 5
       lds_barrier();  // (f) the products no longer read the side-1 rows (dot)
 
       // ---- step 6 ----
-      side1_stored = !l2 && more;
+      side1_stored = CMP == PBG_CMP_DOT && more;  // (l2 and cos still read the rows' own values while writing gradients out)
       pads = c.last < P && cc_next == C - 1;  // of the chunk whose rows are in the registers now
       if (side1_stored) fused_store_side<CMP, 1>(c, g, lds, wave, ln, v, idv, extras, pads);
+      if (cosn) lds_barrier();  // the exchange of step 6
       lds_barrier();  // (g) the products have let go of all operand rows
     }
     return;
@@ -1622,6 +1658,20 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       }
       if (l2 && m == 1) lds_barrier();  // (e') of the helpers
       const int u = rt * 16 + m16;
+      float row_dot_ = 0.f;
+      if (cosn) {
+        const int self_at = xs + (P + min(u, U - 1)) * ldx + ct0 * 16, left = D - ct0 * 16;
+        float part = 0.f;
+        if (live) {
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+        }
+        part += __shfl_xor(part, 16);
+        part += __shfl_xor(part, 32);
+        if (kq == 0) lds[f.xch + grp * 64 + rt * 16 + m16] = part;
+        lds_barrier();
+        row_dot_ = part + lds[f.xch + (1 - grp) * 64 + rt * 16 + m16];
+      }
       if (live && u < U) {
         const int r2 = cc * U + u;
         FusedOut o;
@@ -1637,9 +1687,13 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
           asum += __shfl_xor(asum, 32);
           o.coef = -asum;
         }
+        if (cosn) {
+          o.coef = row_dot_;
+          o.pcoef = lds[(m ? g.sq1 : g.sq0) + P + u];
+        }
         const int left = D - ct0 * 16;
-        if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<l2>(lds, o, col, left, v4); });
-        else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<l2>(lds, o, col, left, v4); });
+        if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
+        else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
       }
       lds_barrier();  // (d), (e)
     }
@@ -1651,17 +1705,34 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       const int bx = m ? xn0 : xn1, xs = m ? xn1 : xn0;
       const int rs_o = m ? g.rs0 : g.rs1, cs_m = m ? g.cs1 : g.cs0;
       const bool has_op = m == 1 && c.op != PBG_OP_NONE;
-      if (rt * 16 < P && ct0 * 16 < D) {
+      const bool live = rt * 16 < P && ct0 * 16 < D;
+      float4v acc[T0];
+#pragma unroll
+      for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      if (live) {
         // The k index runs past N up to the next multiple of 4: the score blocks keep
         // zero pad columns there, so those terms vanish.
-        float4v acc[T0];
-#pragma unroll
-        for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int ar = min(rt * 16 + m16, P - 1);
         const int ksteps = (N + 3) >> 2;
         const int a_at = dsa + ar * lds_, b_at = bx + ct0 * 16;
         if (grp == 0) sweep_a_rows<T0>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
         else if (T1 > 0) sweep_a_rows<(T1 > 0 ? T1 : 1)>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
+      }
+      float row_dot_ = 0.f;
+      if (cosn) {
+        const int self_at = xs + min(rt * 16 + m16, P - 1) * ldx + ct0 * 16, left = D - ct0 * 16;
+        float part = 0.f;
+        if (live) {
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+        }
+        part += __shfl_xor(part, 16);
+        part += __shfl_xor(part, 32);
+        if (kq == 0) lds[f.xch + grp * 64 + rt * 16 + m16] = part;
+        lds_barrier();
+        row_dot_ = part + lds[f.xch + (1 - grp) * 64 + rt * 16 + m16];
+      }
+      if (live) {
         const int i = rt * 16 + m16;
         if (i < valid) {
           const int q = cc * P + i;
@@ -1678,9 +1749,13 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
             o.coef = 2.0f * lds[rs_o + i] - lds[cs_m + i];
             o.pcoef = pz * pz > 2e-30f ? dpz / pz : 0.f;
           }
+          if (cosn) {
+            o.coef = row_dot_;
+            o.pcoef = lds[(m ? g.sq1 : g.sq0) + i];
+          }
           const int left = D - ct0 * 16;
-          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<l2>(lds, o, col, left, v4); });
-          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<l2>(lds, o, col, left, v4); });
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
         }
       }
       lds_barrier();  // (f), (g)
@@ -1691,7 +1766,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.dynamic) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
-  if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2) return false;
+  if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
   if (c.D > 128 || c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;
   for (int s = 0; s < 2; ++s)
@@ -1712,6 +1787,7 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   f->pos = take(c.P);
   f->dpos = take(c.P);
   f->part = take(6 * c.P);
+  f->xch = take(c.cmp == PBG_CMP_COS ? 128 : 0);
   f->ids = take(kFusedIds);
   f->total = off;
   return (size_t)off * sizeof(float) <= 160 * 1024 - 512;
@@ -2686,20 +2762,22 @@ int launch_fused_loss(const Plan& plan, size_t lds_bytes, hipStream_t s) {
   }
 }
 
+template <int T, int LD>
+int launch_fused_cmp(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+  switch (plan.c.cmp) {
+    case PBG_CMP_L2: return launch_fused_loss<T, PBG_CMP_L2, LD>(plan, lds_bytes, s);
+    case PBG_CMP_COS: return launch_fused_loss<T, PBG_CMP_COS, LD>(plan, lds_bytes, s);
+    default: return launch_fused_loss<T, PBG_CMP_DOT, LD>(plan, lds_bytes, s);
+  }
+}
+
 int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s) {
   const StepCtx& c = plan.c;
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
-  const bool l2 = c.cmp == PBG_CMP_L2;
   // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 108 floats)
-  if (small_tiles && plan.fl.ldx == 108 && plan.fl.lds == 108)
-    return l2 ? launch_fused_loss<7, PBG_CMP_L2, 108>(plan, lds_bytes, s)
-              : launch_fused_loss<7, PBG_CMP_DOT, 108>(plan, lds_bytes, s);
-  if (small_tiles) {
-    return l2 ? launch_fused_loss<7, PBG_CMP_L2, 0>(plan, lds_bytes, s)
-              : launch_fused_loss<7, PBG_CMP_DOT, 0>(plan, lds_bytes, s);
-  }
-  return l2 ? launch_fused_loss<8, PBG_CMP_L2, 0>(plan, lds_bytes, s)
-            : launch_fused_loss<8, PBG_CMP_DOT, 0>(plan, lds_bytes, s);
+  if (small_tiles && plan.fl.ldx == 108 && plan.fl.lds == 108) return launch_fused_cmp<7, 108>(plan, lds_bytes, s);
+  if (small_tiles) return launch_fused_cmp<7, 0>(plan, lds_bytes, s);
+  return launch_fused_cmp<8, 0>(plan, lds_bytes, s);
 }
 
 template <int DEPTH>

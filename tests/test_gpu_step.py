@@ -823,7 +823,28 @@ def _fused_shape_cases():
     return cases
 
 
-@pytest.mark.parametrize("case", _fused_shape_cases(), ids=ids)
+def _fused_cos_cases():
+    """The same kind of sample for the cos comparator (the reference's default,
+    config.py:185-190), whose rows are normalised on their way into LDS and whose
+    gradient rows go back through the normalisation on their way out."""
+    import random
+
+    rng = random.Random(11)
+    cases = [dict(operator="none", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50,
+                  num_pos=173, dim=100)]
+    for _ in range(26):
+        p = rng.choice([1, 2, 3, 15, 16, 17, 31, 33, 48, 50, 63, 64])
+        u = rng.choice([1, 2, 5, 16, 17, 49, 50, 64])
+        d = rng.choice([4, 8, 12, 36, 60, 64, 100, 116, 124, 128])
+        chunks = rng.choice([1, 2, 3])
+        num_pos = max(1, p * chunks - rng.choice([0, 0, 1, p // 2]))
+        cases.append(dict(operator=rng.choice(["none", "translation", "diagonal"]), comparator="cos",
+                          loss=rng.choice(["ranking", "logistic", "softmax"]), dynamic=False, num_batch_negs=p,
+                          num_uniform_negs=u, num_pos=num_pos, dim=d))
+    return cases
+
+
+@pytest.mark.parametrize("case", _fused_shape_cases() + _fused_cos_cases(), ids=ids)
 def test_fused_kernel_shapes(pbg, case):
     """Chunk sizes, negative counts, dims and partial last chunks around the
     tile borders of the fused chunk kernel, two batches per call."""
@@ -835,6 +856,8 @@ def test_fused_kernel_shapes(pbg, case):
     n_ent = max(300, num_pos * (60 if cfg.comparator == "l2" else 4))
     st, batches = make_inputs(cfg, num_pos, n_ent, 2, seed=num_pos * 131 + dim, shared=(dim % 8 == 0))
     runner = to_runner(pbg, cfg, st, num_pos, 2)
+    if cfg.comparator == "cos" and cfg.num_batch_negs + cfg.num_uniform_negs <= 100:  # (the largest shapes do not fit LDS)
+        assert runner.route == "fused"
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
     outs, st64 = lockstep(cfg, st, batches, keep_scores=True)
