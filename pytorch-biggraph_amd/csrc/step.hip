@@ -2774,8 +2774,8 @@ int launch_fused_cmp(const Plan& plan, size_t lds_bytes, hipStream_t s) {
 int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s) {
   const StepCtx& c = plan.c;
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
-  // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 108 floats)
-  if (small_tiles && plan.fl.ldx == 108 && plan.fl.lds == 108) return launch_fused_cmp<7, 108>(plan, lds_bytes, s);
+  // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 104 floats)
+  if (small_tiles && plan.fl.ldx == 104 && plan.fl.lds == 104) return launch_fused_cmp<7, 104>(plan, lds_bytes, s);
   if (small_tiles) return launch_fused_cmp<7, 0>(plan, lds_bytes, s);
   return launch_fused_cmp<8, 0>(plan, lds_bytes, s);
 }
