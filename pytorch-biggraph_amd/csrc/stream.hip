@@ -239,14 +239,15 @@ __device__ __forceinline__ void tile_out(const float4v* acc, int q, F&& fn) {
 // Two operand sets take turns, the reads of the next unit pinned above the matrix
 // instructions of the current one; LDA is known at compile time, so every address is one
 // register plus an immediate.
-template <int NCT>
+// The operands of one unit: two of the tile's rows for up to 4 column tiles.
 struct DaOperands {
-  float b[2][NCT];
-  template <int LDA>
+  float b[2][4];
+  template <int NCT, int LDA>
   __device__ __forceinline__ void load(const float* lds, int b_at, int m16) {
     tile_b<NCT>(lds, b_at, m16, b[0]);
     tile_b<NCT>(lds, b_at + LDA, m16, b[1]);
   }
+  template <int NCT>
   __device__ __forceinline__ void mma(float a0, float a1, float4v* acc) const {
 #pragma unroll
     for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[0][t], a0, acc[t], 0, 0, 0);
@@ -254,34 +255,39 @@ struct DaOperands {
     for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[1][t], a1, acc[t], 0, 0, 0);
   }
 };
-// unit u of a part: steps 4 (u / 2) + 2 (u % 2) and the next
-template <int NCT, int LDA>
-__device__ __forceinline__ void stream_da_part(const float* lds, int a_at, int b_at, int m16, float4v* acc) {
-  constexpr int units = 2 * (kTile / 16);
-  DaOperands<NCT> x, y;
-  float4 a = *reinterpret_cast<const float4*>(&lds[a_at]), an = a;
-  x.template load<LDA>(lds, b_at, m16);
-#pragma unroll
-  for (int u = 0; u < units; ++u) {
-    DaOperands<NCT>& cur = (u & 1) ? y : x;
-    DaOperands<NCT>& nxt = (u & 1) ? x : y;
-    if (u + 1 < units) {
-      nxt.template load<LDA>(lds, b_at + (4 * ((u + 1) / 2) + 2 * ((u + 1) & 1)) * LDA, m16);
-      if (((u + 1) & 1) == 0) an = *reinterpret_cast<const float4*>(&lds[a_at + 8 * ((u + 1) / 2)]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (u & 1) cur.mma(a.z, a.w, acc);
-    else cur.mma(a.x, a.y, acc);
-    __builtin_amdgcn_sched_barrier(0);
-    if (u & 1) a = an;
-  }
-}
+// All N column tiles as one pipeline of units: part p = column tiles 4 p .. 4 p + 3 (the last
+// part may hold fewer), unit u of a part = steps 4 (u / 2) + 2 (u % 2) and the next.  The reads
+// of the next unit -- of the next part after a part's last unit -- are pinned above the matrix
+// instructions of the current one, so the wave never waits for a read that it has only just issued.
 template <int N, int LDA>
 __device__ __forceinline__ void stream_da_product(const float* lds, int a_at, int b_at, int m16, float4v* acc) {
-  constexpr int full = N / 4, rem = N % 4;
+  constexpr int full = N / 4, rem = N % 4, parts = full + (rem > 0 ? 1 : 0);
+  constexpr int upp = 2 * (kTile / 16);  // units per part
+  constexpr int units = parts * upp;
+  DaOperands x, y;
+  auto load_unit = [&](DaOperands& ops, int idx) {
+    const int part = idx / upp, u = idx % upp;
+    const int at = b_at + 64 * part + (4 * (u / 2) + 2 * (u & 1)) * LDA;
+    if (part < full) ops.template load<4, LDA>(lds, at, m16);
+    else ops.template load<(rem > 0 ? rem : 1), LDA>(lds, at, m16);
+  };
+  float4 a = *reinterpret_cast<const float4*>(&lds[a_at]), an = a;
+  load_unit(x, 0);
 #pragma unroll
-  for (int p = 0; p < full; ++p) stream_da_part<4, LDA>(lds, a_at, b_at + 64 * p, m16, acc + 4 * p);
-  if constexpr (rem > 0) stream_da_part<rem, LDA>(lds, a_at, b_at + 64 * full, m16, acc + 4 * full);
+  for (int idx = 0; idx < units; ++idx) {
+    DaOperands& cur = (idx & 1) ? y : x;
+    DaOperands& nxt = (idx & 1) ? x : y;
+    if (idx + 1 < units) {
+      load_unit(nxt, idx + 1);
+      if (((idx + 1) & 1) == 0) an = *reinterpret_cast<const float4*>(&lds[a_at + 8 * (((idx + 1) % upp) / 2)]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const float a0 = (idx & 1) ? a.z : a.x, a1 = (idx & 1) ? a.w : a.y;
+    if (idx / upp < full) cur.template mma<4>(a0, a1, acc + 4 * (idx / upp));
+    else cur.template mma<(rem > 0 ? rem : 1)>(a0, a1, acc + 4 * full);
+    __builtin_amdgcn_sched_barrier(0);
+    if (idx & 1) a = an;
+  }
 }
 template <int N>
 __device__ __forceinline__ void stream_da_store(const float4v* acc, int kq, float* dst) {
@@ -535,18 +541,26 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
         *reinterpret_cast<float4*>(&lds[gbuf + hrow * kLdg + swap23(hc)]) = make_float4(g[0], g[1], g[2], g[3]);
       };
       grad_tile(0, a.g_at + (nt & 1) * kTileFloats, parked(0));
+      // The parked scores come back from beyond the L2 (a workgroup parks 270 KB per item): those of
+      // tile t + 1 are asked for a whole tile ahead, or the round trip would sit between the
+      // helpers and barrier (A) in every tile.
+      float4 sv = parked(min(1, nt - 1));
       lds_barrier();  // (T) G_0 in LDS
 
       // ---- sweep 2 ----
       for (int q = nt; q < 2 * nt; ++q) {
         const int t = q - nt;
         const bool more = t + 1 < nt;
-        const float4 sv = parked(min(t + 1, nt - 1));  // asked for first: loads come back in the order they were issued
+        const float4 sv_next = parked(min(t + 2, nt - 1));
         rows.issue(sd.w, D, nid0, nid1, ht);  // tile t + 1 (with `more`; else rows that are not stored)
         TileRows<NSEG>::fetch_ids(colid, min(t + 2, nt - 1) * kTile, ncols, ht, &nid0, &nid1);
-        if (more) grad_tile(t + 1, a.g_at + ((q + 1) & 1) * kTileFloats, sv);
         lds_barrier();  // (A) dA has taken tile t
         if (more) rows.store(lds, a.n_at, lda, D, ht, edge_tile(t + 1));
+        // G_(t+1) goes into the buffer that dN_(t-1) was the last to read.  It is formed on this side of (A):
+        // every vector instruction of a helper waits for a gap between matrix instructions, and up to (A) the
+        // helpers' loads above are all that stands between them and the barrier.
+        if (more) grad_tile(t + 1, a.g_at + ((q + 1) & 1) * kTileFloats, sv);
+        sv = sv_next;
         lds_barrier();  // (B) tile t + 1 and G_(t+1) in LDS, G_t no longer read
       }
       viol = oct_sum_int(viol);
@@ -596,18 +610,29 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
           const int a_at = gbuf + (rt * 16 + m16) * kLdg + 16 * (kq >> 1) + 4 * (kq & 1), b_at = a.n_at + 8 * kq * lda;
           stream_da_product<T0, lda>(lds, a_at, b_at + (grp ? (NT - T0) * 16 : 0), m16, dA);
         }
+        // (where dN_t goes: worked out on this side of the barrier, while other waves still multiply)
+        const int j = t * kTile + rt2 * 16 + m16;
+        float* dst = nullptr;
+        if (j < P) {
+          if (j < valid) dst = sdb + (int64_t)j * D;
+        } else if (j < ncols) {
+          dst = uni + (int64_t)(j - P) * D;
+        }
+        const int k0 = 2 * (kq & 1) + (kq >> 1);
+        const int g_at = gbuf + k0 * kLdg + rt2 * 16 + swap23(m16), a_at = a.a_at + k0 * lda;
         lds_barrier();  // (A)
         {  // dN_t = G_t^T A: 16 negatives x this wave's quarter of the column tiles
-          const int j = t * kTile + rt2 * 16 + m16;
-          float* dst = nullptr;
-          if (j < P) {
-            if (j < valid) dst = sdb + (int64_t)j * D;
-          } else if (j < ncols) {
-            dst = uni + (int64_t)(j - P) * D;
-          }
-          const int k0 = 2 * (kq & 1) + (kq >> 1);
-          const int g_at = gbuf + k0 * kLdg + rt2 * 16 + swap23(m16), a_at = a.a_at + k0 * lda;
+          // The two compute waves of a SIMD (wave and wave + 4) take their parts in opposite orders, so that
+          // one is in the middle of a part while the other drains its accumulators and refills its operands.
           int ct = dn_ct0, left = dn_cnt;
+          const int small = left & 3;
+          if (qtr >= 2 && small) {
+            if (small == 3) stream_dn_part<3, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
+            else if (small == 2) stream_dn_part<2, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
+            else stream_dn_part<1, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
+            ct += small;
+            left -= small;
+          }
           for (; left >= 4; left -= 4, ct += 4) stream_dn_part<4, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
           if (left == 3) stream_dn_part<3, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
           else if (left == 2) stream_dn_part<2, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
