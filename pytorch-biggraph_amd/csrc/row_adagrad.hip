@@ -114,7 +114,9 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_multi_kernel(const fl
 // alone by tile_reduce (and never concerns run_combine) and summed, in position
 // order, by the update kernel as it reads it, with the loads of the same phase.
 // (With several workers a row has a run per worker and the update kernels' loop
-// over them is latency bound: the extra loads cost more there than they save.)
+// over them is latency bound: the extra loads cost more there than they save.
+// row_walk_kernel, which streams a table row's whole stretch anyway, takes every
+// whole run that lies inside one tile, whatever its length.)
 constexpr int kTile = 32;
 constexpr int kShort = 4;
 // [s, s + len) in sorted positions: summed by the update kernels themselves (single-worker calls)
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
     heads &= heads - 1;
     const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
     if (b - a < 2) continue;
-    if (leave_short && b - a <= kShort) {  // a short run inside the tile is the update kernel's (folded_run)
+    if (b - a <= leave_short) {  // a whole run of at most leave_short positions inside the tile is the update kernel's
       const uint64_t kp = lane_u64(key, a);
       const bool whole = (a > 0 || !has_before || key_before != kp) && (b < (int)(end - begin) || !has_after || key_after != kp);
       if (whole) continue;
@@ -471,7 +473,7 @@ __global__ __launch_bounds__(kRowThreads) void row_walk_kernel(
       const uint64_t from = lasts & (~0ull << a);
       const int e = from != 0ull ? __ffsll((unsigned long long)from) - 1 : -1;  // -1: the run goes on past the window
       const int len = e - a + 1;
-      if (e >= 0 && len >= 2 && len <= kShort && (a / kTile) == (e / kTile)) {  // folded_run: the window starts at a multiple of kTile
+      if (e >= 0 && len >= 2 && (a / kTile) == (e / kTile)) {  // a whole run inside one tile (the window starts at a multiple of kTile): summed here
         todo |= ((2ull << e) - 1) & (~0ull << a);
         done |= 1ull << e;
       } else {  // the run's sum is in its first row (tile_reduce, run_combine)
@@ -739,7 +741,7 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim,       \
-                       (int)(kbits == 0 || walk));                                                              \
+                       walk ? kTile : (kbits == 0 ? kShort : 0));                                                              \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
     if (walk) {                                                                                                    \
