@@ -173,11 +173,14 @@ struct TileRows {
       v[2 * seg + 1] = *reinterpret_cast<const float4*>(r1 + col * 4);
     }
   }
-  // `absent`: the tile may hold absent rows (the same for the whole workgroup)
-  __device__ __forceinline__ void store(float* lds, int n_at, int lda, int D, int ht, bool absent) const {
+  // `absent`: the tile may hold absent rows (the same for the whole workgroup).  `paced`: the writes are
+  // spread out in time -- a burst of LDS writes holds up every read that arrives behind it, and in the
+  // second sweep those are the operand reads of a running product while the helpers have time to spare.
+  __device__ __forceinline__ void store(float* lds, int n_at, int lda, int D, int ht, bool absent, bool paced = false) const {
     const int hw = ht >> 5, c4 = (ht & 31) << 2;
 #pragma unroll
     for (int seg = 0; seg < NSEG; ++seg) {
+      if (paced && seg > 0) __builtin_amdgcn_s_sleep(6);
       const int col = seg * 128 + c4;
       if (col < D) {
         float4 v0 = v[2 * seg], v1 = v[2 * seg + 1];
@@ -186,6 +189,7 @@ struct TileRows {
           v1 = keep_if(v1, id1 >= 0);
         }
         *reinterpret_cast<float4*>(&lds[n_at + hw * lda + col]) = v0;
+        if (paced) __builtin_amdgcn_s_sleep(6);
         *reinterpret_cast<float4*>(&lds[n_at + (hw + 16) * lda + col]) = v1;
       }
     }
@@ -555,7 +559,7 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
         rows.issue(sd.w, D, nid0, nid1, ht);  // tile t + 1 (with `more`; else rows that are not stored)
         TileRows<NSEG>::fetch_ids(colid, min(t + 2, nt - 1) * kTile, ncols, ht, &nid0, &nid1);
         lds_barrier();  // (A) dA has taken tile t
-        if (more) rows.store(lds, a.n_at, lda, D, ht, edge_tile(t + 1));
+        if (more) rows.store(lds, a.n_at, lda, D, ht, edge_tile(t + 1), true);
         // G_(t+1) goes into the buffer that dN_(t-1) was the last to read.  It is formed on this side of (A):
         // every vector instruction of a helper waits for a gap between matrix instructions, and up to (A) the
         // helpers' loads above are all that stands between them and the barrier.
