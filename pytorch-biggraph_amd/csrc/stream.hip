@@ -791,7 +791,8 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
   if (!stream_dim_built(c.D) || c.P > 64) return false;
   for (int s = 0; s < 2; ++s) {
     const SideCtx& sd = c.side[s];
-    if (sd.all || sd.u < 64 || sd.u != c.side[0].u || sd.num_rows >= ((int64_t)1 << 31)) return false;
+    // (measured at dim 400 with 50 + 50 negatives: 50.8 M edges/s here against 34.5 M on the staged kernels)
+    if (sd.all || sd.u < 8 || sd.u != c.side[0].u || sd.num_rows >= ((int64_t)1 << 31)) return false;
     if (sd.nb != 0 && sd.nb != c.P) return false;
   }
   sp->pr = (c.P + 3) / 4 * 4;

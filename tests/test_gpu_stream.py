@@ -33,6 +33,12 @@ CASES += [
          shared=False),
     dict(operator="complex_diagonal", loss="logistic", dynamic=True, num_batch_negs=8, num_uniform_negs=64, num_pos=30,
          dim=256, shared=False),
+    # the reference's default negatives (50 + 50, config.py:323-337) at dims beyond the LDS-resident kernel; very few negatives
+    dict(operator="complex_diagonal", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=50, num_pos=173,
+         dim=400),
+    dict(operator="diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=50, num_pos=100, dim=256),
+    dict(operator="none", loss="logistic", dynamic=False, num_batch_negs=20, num_uniform_negs=8, num_pos=50, dim=400,
+         shared=False),
     # no batch negatives: the chunk is as long as the uniform draw (model.py:648-650)
     dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64, num_pos=150, dim=128),
     dict(operator="none", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=64, dim=256),
