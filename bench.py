@@ -72,6 +72,10 @@ WORKLOADS = {
                  entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=50,
                  operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=False,
                  init_scale=1e-3, zipf=1.1, two_tables=False),
+    "d200": dict(desc="as d400 at dim 200 (13 column tiles, the last half padding)",
+                 entities=14_951, edges=483_142, dim=200, batch=1000, batch_negs=50, uniform_negs=50,
+                 operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=False,
+                 init_scale=1e-3, zipf=1.1, two_tables=False),
     "fb15k": dict(desc="the reference's FB15k example as configured (examples/configs/fb15k_config_cpu.py): 1345 relations (dynamic), complex_diagonal/dot/softmax, dim 400, 14951 entities, B=1000, chunk 50 + 1000 uniform negatives, N3 regularizer 1e-3",
                   entities=14_951, edges=483_142, dim=400, batch=1000, batch_negs=50, uniform_negs=1000,
                   operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=True,
@@ -459,7 +463,7 @@ def main():
         return spec, calls * per_call / dt, dt / calls * 1e3, dt, stages, loss
 
     workers = max(1, args.workers)
-    default_batches = {"cfg1": 64000, "cfg1cos": 64000, "cfg2": 400, "cfg2d": 400, "fb15k": 400, "d400": 6400, "livejournal": 3200, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
+    default_batches = {"cfg1": 64000, "cfg1cos": 64000, "cfg2": 400, "cfg2d": 400, "fb15k": 400, "d400": 6400, "d200": 6400, "livejournal": 3200, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
     steps = args.steps if args.steps is not None else max(1, default_batches // workers)
     warmup = args.warmup if args.warmup is not None else max(1, steps // 10)
     spec, eps, ms_per_step, wall_s, stages, loss = run(workers, steps, warmup, profile_calls=10)

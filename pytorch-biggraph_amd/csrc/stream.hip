@@ -293,14 +293,19 @@ __device__ __forceinline__ void stream_da_product(const float* lds, int a_at, in
     if (idx & 1) a = an;
   }
 }
-template <int N>
-__device__ __forceinline__ void stream_da_store(const float4v* acc, int kq, float* dst) {
+// `cols`: the row's columns from dst on (ALL: every column the tiles cover exists)
+template <int N, bool ALL>
+__device__ __forceinline__ void stream_da_store(const float4v* acc, int kq, float* dst, int cols) {
   constexpr int full = N / 4, rem = N % 4;
 #pragma unroll
   for (int p = 0; p < full; ++p)
-    tile_out<4>(acc + 4 * p, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * p + col) = v; });
+    tile_out<4>(acc + 4 * p, kq, [&](int col, float4 v) {
+      if (ALL || 64 * p + col < cols) *reinterpret_cast<float4*>(dst + 64 * p + col) = v;
+    });
   if constexpr (rem > 0)
-    tile_out<rem>(acc + 4 * full, kq, [&](int col, float4 v) { *reinterpret_cast<float4*>(dst + 64 * full + col) = v; });
+    tile_out<rem>(acc + 4 * full, kq, [&](int col, float4 v) {
+      if (ALL || 64 * full + col < cols) *reinterpret_cast<float4*>(dst + 64 * full + col) = v;
+    });
 }
 
 // NCT column tiles from `ct` on of dN_t = G_t^T A for the lane's negative, stored at dst (or
@@ -314,9 +319,9 @@ __device__ __forceinline__ void stream_da_store(const float4v* acc, int kq, floa
 // these rows are the bulk of what the kernel writes to HBM, and a store instruction
 // whose 16-byte pieces lie 64 bytes apart costs four times the requests.
 // Reads one step past the last (the rows behind both blocks exist).
-template <int NCT, int LDA>
+template <int NCT, int LDA, bool ALL>
 __device__ __forceinline__ void stream_dn_part(const float* lds, int g_at, int a_at, int ct, int ksteps, int kq, int m16,
-                                               float* dst) {
+                                               float* dst, int cols) {
   float4v acc[NCT];
 #pragma unroll
   for (int t = 0; t < NCT; ++t) acc[t] = (float4v){0.f, 0.f, 0.f, 0.f};
@@ -351,7 +356,8 @@ __device__ __forceinline__ void stream_dn_part(const float* lds, int g_at, int a
   if (dst) {
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
-      *reinterpret_cast<float4*>(dst + (ct + t) * 16 + 4 * kq) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (ALL || (ct + t) * 16 + 4 * kq < cols)
+        *reinterpret_cast<float4*>(dst + (ct + t) * 16 + 4 * kq) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
   }
 }
 
@@ -417,8 +423,12 @@ struct RowLoss {
 template <int NT, int LOSS>
 __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, StreamPlan a, int num_items) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int D = NT * 16, D4 = D / 4, NSEG = (D + 127) / 128;
-  constexpr int lda = lds_stride(D);            // (= a.lda)
+  // The rows are NT tiles of 16 columns wide in LDS; kExact: that is the embedding dimension itself (and a
+  // compile-time constant), else the last tile is partly padding that stays zero from the start of the kernel.
+  constexpr int DP = NT * 16, NSEG = (DP + 127) / 128;
+  constexpr bool kExact = NT == 8 || NT == 16 || NT == 25;
+  constexpr int lda = lds_stride(DP);           // (= a.lda)
+  const int D = kExact ? DP : c.D, D4 = D >> 2;
   // column tiles of dA per wave group: [0, T0) and [NT - T0, NT) -- with NT odd the middle tile is formed by
   // both groups (bit-identical values, one code path for the two groups)
   constexpr int T0 = (NT + 1) / 2;
@@ -428,6 +438,11 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
   const int CP = C * P;
   float* scr = a.scratch + (size_t)blockIdx.x * nt * (kHelpers * 4) + ht * 4;
   const bool helper = wave16 >= 8;
+  if (!kExact) {
+    for (int i = threadIdx.x * 4; i < a.total; i += 2 * kHelpers * 4)
+      *reinterpret_cast<float4*>(&lds[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
+    lds_barrier();
+  }
   if (helper) __builtin_amdgcn_s_setprio(3);
 
   for (int item = blockIdx.x; item < num_items; item += gridDim.x) {
@@ -631,16 +646,16 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
           int ct = dn_ct0, left = dn_cnt;
           const int small = left & 3;
           if (qtr >= 2 && small) {
-            if (small == 3) stream_dn_part<3, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
-            else if (small == 2) stream_dn_part<2, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
-            else stream_dn_part<1, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
+            if (small == 3) stream_dn_part<3, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
+            else if (small == 2) stream_dn_part<2, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
+            else stream_dn_part<1, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
             ct += small;
             left -= small;
           }
-          for (; left >= 4; left -= 4, ct += 4) stream_dn_part<4, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
-          if (left == 3) stream_dn_part<3, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
-          else if (left == 2) stream_dn_part<2, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
-          else if (left == 1) stream_dn_part<1, lda>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst);
+          for (; left >= 4; left -= 4, ct += 4) stream_dn_part<4, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
+          if (left == 3) stream_dn_part<3, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
+          else if (left == 2) stream_dn_part<2, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
+          else if (left == 1) stream_dn_part<1, lda, kExact>(lds, g_at, a_at, ct, pr >> 2, kq, m16, dst, D);
         }
         lds_barrier();  // (B)
       }
@@ -648,8 +663,8 @@ __global__ __launch_bounds__(2 * kHelpers) void stream_chunk_kernel(StepCtx c, S
       const int m16 = lane_ & 15, kq = lane_ >> 4;
       const int i = rt * 16 + m16;
       if (i < valid) {
-        float* dst = (s ? a.sda[1] : a.sda[0]) + (e0 + i) * D + (grp ? (NT - T0) * 16 : 0);
-        stream_da_store<T0>(dA, kq, dst);
+        const int first = grp ? (NT - T0) * 16 : 0;
+        stream_da_store<T0, kExact>(dA, kq, (s ? a.sda[1] : a.sda[0]) + (e0 + i) * D + first, D - first);
       }
     }
   }
@@ -772,7 +787,13 @@ int launch_chunk_loss(const StepCtx& c, const StreamPlan& sp, hipStream_t s) {
   }
 }
 
-bool stream_dim_built(int D) { return D == 128 || D == 256 || D == 400; }
+// Column tiles of 16 per row for which the chunk kernel is built: the exact dims 128, 256, 400, and
+// 13 / 19 tiles for any dim (a multiple of 4) in (192, 208] / (288, 304]; 0: not built.
+int stream_tiles(int D) {
+  if (D == 128 || D == 256 || D == 400) return D / 16;
+  const int nt = (D + 15) / 16;
+  return (D % 4 == 0 && (nt == 13 || nt == 19)) ? nt : 0;
+}
 
 #define PBG_STREAM_ROWS(nvh, KERNEL, jobs, stream, ...)                                                                  \
   do {                                                                                                                   \
@@ -788,7 +809,7 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
   memset(sp, 0, sizeof(*sp));
   if (c.cmp != PBG_CMP_DOT || c.bias || c.affine) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_DIAGONAL && c.op != PBG_OP_COMPLEX_DIAGONAL) return false;
-  if (!stream_dim_built(c.D) || c.P > 64) return false;
+  if (stream_tiles(c.D) == 0 || c.P > 64) return false;
   for (int s = 0; s < 2; ++s) {
     const SideCtx& sd = c.side[s];
     // (measured at dim 400 with 50 + 50 negatives: 50.8 M edges/s here against 34.5 M on the staged kernels)
@@ -796,7 +817,7 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
     if (sd.nb != 0 && sd.nb != c.P) return false;
   }
   sp->pr = (c.P + 3) / 4 * 4;
-  sp->lda = lds_stride(c.D);
+  sp->lda = lds_stride(stream_tiles(c.D) * 16);
   sp->ntiles = (int)ceil_div(c.P + c.side[0].u, kTile);
   // the tile first: the products' reads past its last row then land in the rows behind it
   sp->n_at = 0;
@@ -826,10 +847,12 @@ int stream_prep(const StepCtx& c, const StreamPlan& sp, int nvh, hipStream_t str
 
 int stream_chunks(const StepCtx& c, const StreamPlan& sp, hipStream_t stream) {
   int rc;
-  switch (c.D) {
-    case 128: rc = launch_chunk_loss<8>(c, sp, stream); break;
-    case 256: rc = launch_chunk_loss<16>(c, sp, stream); break;
-    case 400: rc = launch_chunk_loss<25>(c, sp, stream); break;
+  switch (stream_tiles(c.D)) {
+    case 8: rc = launch_chunk_loss<8>(c, sp, stream); break;
+    case 13: rc = launch_chunk_loss<13>(c, sp, stream); break;
+    case 16: rc = launch_chunk_loss<16>(c, sp, stream); break;
+    case 19: rc = launch_chunk_loss<19>(c, sp, stream); break;
+    case 25: rc = launch_chunk_loss<25>(c, sp, stream); break;
     default: return fail(PBG_ERR_UNSUPPORTED, "step: streaming route not built for dim %d", c.D);
   }
   if (rc != PBG_OK) return rc;

@@ -39,6 +39,15 @@ CASES += [
     dict(operator="diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=50, num_pos=100, dim=256),
     dict(operator="none", loss="logistic", dynamic=False, num_batch_negs=20, num_uniform_negs=8, num_pos=50, dim=400,
          shared=False),
+    # dims that are no multiple of 16: the last column tile of a row is partly padding
+    dict(operator="complex_diagonal", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=50, num_pos=120,
+         dim=200),
+    dict(operator="diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=100, num_pos=100, dim=300),
+    dict(operator="none", loss="logistic", dynamic=False, num_batch_negs=33, num_uniform_negs=70, num_pos=70, dim=196,
+         shared=False),
+    dict(operator="complex_diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=200, num_pos=130,
+         dim=292, regularization_coef=0.02),
+    dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=64, num_uniform_negs=40, num_pos=128, dim=208),
     # no batch negatives: the chunk is as long as the uniform draw (model.py:648-650)
     dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64, num_pos=150, dim=128),
     dict(operator="none", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=64, dim=256),
