@@ -160,6 +160,24 @@ __device__ __forceinline__ void scatter_range(SliceState<NW, BITS>& st, const ui
 // the rounds in its own row of wave_count (no other wave touches it, so the
 // rounds need no barrier), and the two barriers and the walk over the waves'
 // counts are paid once per KPT * NW * 64 keys instead of once per NW * 64.
+// The lanes of the wave whose key has the same digit as this lane's (valid lanes only).  A bucket
+// is swollen by ONE hot key, so most rounds of 64 consecutive keys carry a single digit value: that
+// case costs two ballots instead of one per bit.
+template <int BITS>
+__device__ __forceinline__ uint64_t digit_peers(uint32_t digit, bool valid) {
+  const uint64_t all = __ballot(valid);
+  const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)digit);
+  if ((all & 1ull) && __ballot(valid && digit == first) == all) return all;
+  uint64_t peers = all;
+#pragma unroll
+  for (int b = 0; b < BITS; ++b) {
+    const bool bit = (digit >> b) & 1u;
+    const uint64_t m = __ballot(valid && bit);
+    peers &= bit ? m : ~m;
+  }
+  return peers;
+}
+
 template <int NW, int BITS, int KPT>
 __device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, const uint64_t* __restrict__ keys_in,
                                                    const uint32_t* __restrict__ vals_in,
@@ -204,13 +222,7 @@ __device__ __forceinline__ void scatter_range_wide(SliceState<NW, BITS>& st, con
       const int64_t i = base + (int64_t)wave * (64 * KPT) + q * 64 + lane;
       valid[q] = i < end;
       digit[q] = (uint32_t)(key[q] >> shift) & mask;
-      uint64_t peers = __ballot(valid[q]);
-#pragma unroll
-      for (int b = 0; b < BITS; ++b) {
-        const bool bit = (digit[q] >> b) & 1u;
-        const uint64_t m = __ballot(valid[q] && bit);
-        peers &= bit ? m : ~m;
-      }
+      const uint64_t peers = digit_peers<BITS>(digit[q], valid[q]);
       const int rank_in_round = __popcll(peers & below);
       const uint32_t prior = valid[q] ? st.wave_count[parity][wave][digit[q]] : 0u;  // this wave's earlier rounds
       rank[q] = prior + (uint32_t)rank_in_round;
@@ -355,13 +367,7 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
       for (int q = 0; q < kInFlight; ++q) {
         const bool valid = base + (int64_t)q * kBucketWaves * 64 + t < end;
         const uint32_t digit = (uint32_t)(kq[q] >> shift) & mask;
-        uint64_t peers = __ballot(valid);
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-          const bool bit = (digit >> b) & 1u;
-          const uint64_t m = __ballot(valid && bit);
-          peers &= bit ? m : ~m;
-        }
+        const uint64_t peers = digit_peers<8>(digit, valid);
         if (valid && (peers & below) == 0ull) atomicAdd(&st.cursor[digit], (uint32_t)__popcll(peers));
       }
     }
