@@ -34,7 +34,12 @@ CASES = {
                          num_uniform_negs=50, entities=20000, scale=0.1, zipf=1.8, shared=False, ks=(64,)),
     # cfg2: complex_diagonal, dot, softmax, dim 400, wide negative sets, Zipf(1.1) entities and relations
     "cfg2": dict(operator="complex_diagonal", comparator="dot", loss="softmax", dim=400, num_pos=200, num_batch_negs=50,
-                 num_uniform_negs=300, entities=3000, relations=12, scale=0.1, zipf=1.1, rel_zipf=1.1, ks=(20, 64, 65)),
+                 num_uniform_negs=300, entities=3000, relations=12, scale=0.1, zipf=1.1, rel_zipf=1.1, ks=(20, 64, 65, 256)),
+    # ... with one relation per edge, at a dim the streaming kernels take (the run's parameter gradient and the
+    # relation's K Adagrad steps come from two kernels of their own there)
+    "cfg2-dynamic-dim256": dict(operator="complex_diagonal", comparator="dot", loss="softmax", dim=256, num_pos=200,
+                                dynamic=True, num_batch_negs=50, num_uniform_negs=100, entities=3000, relations=12, scale=0.1,
+                                zipf=1.1, rel_zipf=1.1, ks=(20, 64, 65)),
     "cfg2-dynamic": dict(operator="complex_diagonal", comparator="dot", loss="softmax", dim=64, num_pos=200, dynamic=True,
                          num_batch_negs=50, num_uniform_negs=100, entities=3000, relations=12, scale=0.1, zipf=1.1,
                          rel_zipf=1.1, ks=(20, 65)),
