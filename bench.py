@@ -8,7 +8,10 @@ through the whole hot path (gather, operator, scoring against batch + uniform
 negatives, loss, backward, RowAdagrad and operator Adagrad), processed like
 `workers` HOGWILD processes in lock-step (all read, then all write in order).
 `--steps` and `--warmup` count calls and never change `workers`; `--workers 1` is
-the strictly sequential single-process order.  Prints ONE JSON line.
+the strictly sequential single-process order.  Before the warm-up calls the device
+is kept busy for `--preheat-ms` (200) with the same calls on a scratch copy of the
+state, so that a short run is not timed while the clocks still settle.  Prints ONE
+JSON line.
 """
 import argparse
 import json
@@ -303,6 +306,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed calls of pbg_train_step (each of --workers batches)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed calls")
+    ap.add_argument("--preheat-ms", type=float, default=200.0,
+                    help="untimed calls on a scratch copy of the state before the warm-up calls, until this much time has passed")
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS) + ["cfg4-epoch"])
     ap.add_argument("--workers", type=int, default=64,
                     help="batches in flight per call (HOGWILD workers); 64 batches of cfg1 are 1280 chunks = 5 per compute unit")
@@ -393,6 +398,7 @@ def main():
 
     enqueue_s = [0.0]  # host time per call of the last run's timed loop (launches only, no wait)
     route_of = {}      # workers -> which kernels pbg_train_step ran ("staged", "fused", "stream")
+    preheat_s = [args.preheat_ms / 1e3]
 
     def run(workers, calls, warm_calls, profile_calls=0, hip_graph=False):
         spec, runner = make_runner(workers)
@@ -434,6 +440,22 @@ def main():
                     torch.zeros((workers, c, u), dtype=torch.int64, device=dev),
                     torch.zeros((workers, c, u), dtype=torch.int64, device=dev)]
             static = (*s_in, runner.capture_train(*s_in))
+        if preheat_s[0] > 0 and not hip_graph:
+            # The device's clocks take some milliseconds of load to settle, and `--steps 20 --warmup 5` would be
+            # over before they have: untimed calls on a scratch copy of the state until preheat_s has passed.
+            # They do not touch the state that the warm-up and timed calls train.
+            _, scratch = make_runner(workers)
+            t_end = time.perf_counter() + preheat_s[0]
+            j = 0
+            while time.perf_counter() < t_end:
+                for _ in range(4):
+                    off = (j * per_call) % (n_edges - per_call + 1) // b * b
+                    rel = rel_edges[off:off + per_call] if rel_edges is not None else rel_pool[(j * workers) % (4096 - workers + 1):][:workers]
+                    scratch.train(lhs_all[off:off + per_call], rhs_all[off:off + per_call], rel, uniform_seed=0x0BAD0000 + j)
+                    j += 1
+                torch.cuda.synchronize()
+            del scratch
+            preheat_s[0] = 0.0  # once per process
         for i in range(warm_calls):
             one_call(i)
         torch.cuda.synchronize()
@@ -512,7 +534,7 @@ def main():
         "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
                    "hogwild_workers": workers, "step": f"one pbg_train_step call of {workers} batches", "route": route,
                    "timed_calls": steps, "timed_batches": steps * workers, "timed_edges": steps * workers * b,
-                   "timed_wall_seconds": wall_s, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
+                   "timed_wall_seconds": wall_s, "preheat_ms_on_scratch_state": args.preheat_ms, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",
                    "mean_loss_per_edge_last_call": loss, "host_enqueue_ms_per_call": host_enqueue_ms},
         "sequential": seq,
         "roofline": roofline,
