@@ -48,6 +48,9 @@ CASES += [
     dict(operator="complex_diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=200, num_pos=130,
          dim=292, regularization_coef=0.02),
     dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=64, num_uniform_negs=40, num_pos=128, dim=208),
+    # fewer positives than a chunk holds; a single positive
+    dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=100, num_pos=30, dim=128),
+    dict(operator="complex_diagonal", loss="ranking", dynamic=True, num_batch_negs=50, num_uniform_negs=64, num_pos=1, dim=256),
     # no batch negatives: the chunk is as long as the uniform draw (model.py:648-650)
     dict(operator="diagonal", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64, num_pos=150, dim=128),
     dict(operator="none", loss="logistic", dynamic=True, num_batch_negs=0, num_uniform_negs=64, num_pos=64, dim=256),
