@@ -28,6 +28,9 @@
 #include "mfma_tiles.h"
 #include "stream.h"
 
+#include <atomic>
+#include <mutex>
+
 namespace pbg {
 namespace {
 
@@ -1207,9 +1210,15 @@ struct FusedGeom {
 // Row ids and sort keys of chunk kc = (k, cc).  The id array has kFusedSide slots
 // per side (slot s * kFusedSide + j = row j of side s's operand rows, -1 from row N
 // on), so that the side is the same for a whole wave and everything chosen by it
-// stays in scalar registers; thread t < kFusedIds owns slot t.
+// stays in scalar registers; thread t < kFusedIds owns slot t.  When the call's keys
+// are sorted beside this kernel, fused_ids_kernel has made ids and keys beforehand
+// (c.fused_rowid) and the ids are only fetched here.
 __device__ __forceinline__ void fused_load_ids(const StepCtx& c, const FusedGeom& g, int kc, int k, int cc, int t, int* ids) {
   if (t >= kFusedIds) return;
+  if (c.fused_rowid) {
+    ids[t] = c.fused_rowid[(int64_t)kc * kFusedIds + t];
+    return;
+  }
   const int s = __builtin_amdgcn_readfirstlane(t >> 7), j = t & (kFusedSide - 1);
   const SideCtx& sd = c.side[s];
   const bool is_pos = j < g.P;
@@ -1763,6 +1772,30 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
   }
 }
 
+// One thread per operand-row slot of every chunk (kFusedIds per chunk, see fused_load_ids): the slot's
+// row id (-1: a slot past the operand rows or a padded position of the last chunk) and, for real
+// slots, the sort key and value of the slot's gradient row.  Nothing here depends on the
+// embeddings, so the sort of the keys can run beside the chunk kernel.
+__global__ __launch_bounds__(kFusedIds) void fused_ids_kernel(StepCtx c) {
+  const int kc = blockIdx.x, t = threadIdx.x;
+  const int P = c.P, U = c.U, N = P + U;
+  const int k = kc / c.C, cc = kc - k * c.C;
+  const int s = t >> 7, j = t & (kFusedSide - 1);
+  const SideCtx& sd = c.side[s];
+  const bool is_pos = j < P;
+  const int q = cc * P + j, u = min(max(j - P, 0), U - 1);
+  const bool real = j < N && (!is_pos || q < c.B);
+  const int64_t flat = (int64_t)kc * U + u;
+  int64_t id = is_pos ? sd.idx[(int64_t)k * c.B + min(q, c.B - 1)] : uniform_negative(sd, s, flat);
+  id = clamp_index(id, sd.num_rows);
+  if (real) {
+    const int64_t pair = (int64_t)k * c.rk + (is_pos ? sd.slot_pos + q : sd.slot_uni + cc * U + u);
+    c.keys[pair] = ((uint64_t)(sd.key_base + id) << c.kbits) | (uint64_t)k;
+    c.vals[pair] = (uint32_t)pair;
+  }
+  c.fused_rowid[(int64_t)kc * kFusedIds + t] = real ? (int)id : -1;
+}
+
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.dynamic) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
@@ -2010,7 +2043,9 @@ __global__ __launch_bounds__(256) void reg_reduce_kernel(StepCtx c) {
 // r = slice (mod slices) of side s in batch k of gr[k, r, :].  Half a wave per
 // row, 128-bit loads; fixed order, no atomics.
 constexpr int kGlobalHalves = 8;  // half-waves per workgroup
-__global__ __launch_bounds__(kGlobalHalves * 32) void global_grad_kernel(StepCtx c, float* __restrict__ gth, int slices) {
+// `direct`: gradient row r of batch k is row k * rk + r (the fused route; its value array may already be sorted)
+__global__ __launch_bounds__(kGlobalHalves * 32) void global_grad_kernel(StepCtx c, float* __restrict__ gth, int slices,
+                                                                          int direct) {
   __shared__ float4 sh[kGlobalHalves][32];
   const int lane = threadIdx.x & 31, hw = threadIdx.x >> 5;
   const int k = blockIdx.x, s = blockIdx.y / slices, slice = blockIdx.y % slices;
@@ -2022,7 +2057,8 @@ __global__ __launch_bounds__(kGlobalHalves * 32) void global_grad_kernel(StepCtx
     const int col = c0 + lane * 4;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int r = begin + slice * kGlobalHalves + hw; r < end; r += slices * kGlobalHalves) {
-      const float* row = c.gr + (int64_t)c.vals[(int64_t)k * c.rk + r] * D;  // (a uniform negative's row may be the GEMM's)
+      const int64_t slot = (int64_t)k * c.rk + r;
+      const float* row = c.gr + (direct ? slot : (int64_t)c.vals[slot]) * D;  // (a uniform negative's row may be the GEMM's)
       if (vec) {
         if (col < D) {
           const float4 v = *reinterpret_cast<const float4*>(row + col);
@@ -2116,6 +2152,7 @@ struct Plan {
   int64_t psize;  // floats of parameter gradient per batch
   int pslices[2]; // partial sums per batch of the element-wise parameter gradients
   bool fused;          // the chunk fits the LDS-resident kernel
+  int* fused_rowid;    // ... and this is where fused_ids_kernel leaves its row ids [K*C, kFusedIds]
   FusedLayout fl;
   bool stream;         // the chunk's positives fit LDS and its negatives are streamed past them
   StreamPlan sp;
@@ -2350,6 +2387,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   if (plan->fused) {  // the fused kernel writes every gradient row and every dz itself
     c.side[0].uni_direct = c.side[1].uni_direct = 0;
     c.side[0].uni_dz_direct = c.side[1].uni_dz_direct = 0;
+    plan->fused_rowid = (int*)take((size_t)KC * kFusedIds, sizeof(int));
   }
   // The streaming route's own buffers lie behind the staged ones: a call with global
   // embeddings (known only from its buffers) takes the staged route on the same workspace.
@@ -2731,7 +2769,7 @@ constexpr int kStages = 10;
 // One instantiation of the fused kernel per (tile count, comparator, loss); each
 // raises its dynamic LDS limit the first time it needs more than it was given.
 template <int T, int CMP, int LOSS, int LD>
-int launch_fused_as(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+int launch_fused_as(const Plan& plan, size_t lds_bytes, hipStream_t s, int blocks) {
   static size_t lds_allowed = 0;
   if (lds_bytes > lds_allowed) {
     if (hipFuncSetAttribute((const void*)fused_chunk_kernel<T, CMP, LOSS, LD>,
@@ -2739,7 +2777,31 @@ int launch_fused_as(const Plan& plan, size_t lds_bytes, hipStream_t s) {
       return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
     lds_allowed = lds_bytes;
   }
-  // one persistent workgroup per compute unit (the LDS footprint allows no more)
+  const int chunks = plan.c.K * plan.c.C;
+  hipLaunchKernelGGL((fused_chunk_kernel<T, CMP, LOSS, LD>), dim3((unsigned)blocks), dim3(2 * kFusedThreads), lds_bytes, s,
+                     plan.c, plan.fl, chunks);
+  return PBG_OK;
+}
+
+template <int T, int CMP, int LD>
+int launch_fused_loss(const Plan& plan, size_t lds_bytes, hipStream_t s, int blocks) {
+  switch (plan.c.loss) {
+    case PBG_LOSS_RANKING: return launch_fused_as<T, CMP, PBG_LOSS_RANKING, LD>(plan, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_fused_as<T, CMP, PBG_LOSS_LOGISTIC, LD>(plan, lds_bytes, s, blocks);
+    default: return launch_fused_as<T, CMP, PBG_LOSS_SOFTMAX, LD>(plan, lds_bytes, s, blocks);
+  }
+}
+
+template <int T, int LD>
+int launch_fused_cmp(const Plan& plan, size_t lds_bytes, hipStream_t s, int blocks) {
+  switch (plan.c.cmp) {
+    case PBG_CMP_L2: return launch_fused_loss<T, PBG_CMP_L2, LD>(plan, lds_bytes, s, blocks);
+    case PBG_CMP_COS: return launch_fused_loss<T, PBG_CMP_COS, LD>(plan, lds_bytes, s, blocks);
+    default: return launch_fused_loss<T, PBG_CMP_DOT, LD>(plan, lds_bytes, s, blocks);
+  }
+}
+
+int compute_units() {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0;
@@ -2747,37 +2809,47 @@ int launch_fused_as(const Plan& plan, size_t lds_bytes, hipStream_t s) {
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
       cus = 256;
   }
-  const int chunks = plan.c.K * plan.c.C;
-  hipLaunchKernelGGL((fused_chunk_kernel<T, CMP, LOSS, LD>), dim3((unsigned)(chunks < cus ? chunks : cus)),
-                     dim3(2 * kFusedThreads), lds_bytes, s, plan.c, plan.fl, chunks);
-  return PBG_OK;
+  return cus;
 }
 
-template <int T, int CMP, int LD>
-int launch_fused_loss(const Plan& plan, size_t lds_bytes, hipStream_t s) {
-  switch (plan.c.loss) {
-    case PBG_LOSS_RANKING: return launch_fused_as<T, CMP, PBG_LOSS_RANKING, LD>(plan, lds_bytes, s);
-    case PBG_LOSS_LOGISTIC: return launch_fused_as<T, CMP, PBG_LOSS_LOGISTIC, LD>(plan, lds_bytes, s);
-    default: return launch_fused_as<T, CMP, PBG_LOSS_SOFTMAX, LD>(plan, lds_bytes, s);
+// The library's own second stream per device, on which the sort of a call's keys runs beside the
+// chunk kernel (the keys do not depend on the embeddings).  A call forks it from the caller's stream
+// with one event and joins it back with another before the update reads the sorted keys; a ring of
+// event pairs, so that consecutive calls do not share one.  Default priority, like every stream here.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork[8], join[8];
+  std::atomic<unsigned> next{0};
+  bool ok = false;
+};
+SideStream* side_stream() {
+  constexpr int kMaxDevices = 16;
+  static SideStream tab[kMaxDevices];
+  static bool tried[kMaxDevices];
+  static std::mutex mu;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  SideStream& ss = tab[dev];
+  if (!tried[dev]) {
+    tried[dev] = true;
+    bool ok = hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking) == hipSuccess;
+    for (int i = 0; ok && i < 8; ++i)
+      ok = hipEventCreateWithFlags(&ss.fork[i], hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&ss.join[i], hipEventDisableTiming) == hipSuccess;
+    ss.ok = ok;
+    if (!ok) (void)hipGetLastError();
   }
+  return ss.ok ? &ss : nullptr;
 }
 
-template <int T, int LD>
-int launch_fused_cmp(const Plan& plan, size_t lds_bytes, hipStream_t s) {
-  switch (plan.c.cmp) {
-    case PBG_CMP_L2: return launch_fused_loss<T, PBG_CMP_L2, LD>(plan, lds_bytes, s);
-    case PBG_CMP_COS: return launch_fused_loss<T, PBG_CMP_COS, LD>(plan, lds_bytes, s);
-    default: return launch_fused_loss<T, PBG_CMP_DOT, LD>(plan, lds_bytes, s);
-  }
-}
-
-int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s) {
+int launch_fused(const Plan& plan, size_t lds_bytes, hipStream_t s, int blocks) {
   const StepCtx& c = plan.c;
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
   // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 104 floats)
-  if (small_tiles && plan.fl.ldx == 104 && plan.fl.lds == 104) return launch_fused_cmp<7, 104>(plan, lds_bytes, s);
-  if (small_tiles) return launch_fused_cmp<7, 0>(plan, lds_bytes, s);
-  return launch_fused_cmp<8, 0>(plan, lds_bytes, s);
+  if (small_tiles && plan.fl.ldx == 104 && plan.fl.lds == 104) return launch_fused_cmp<7, 104>(plan, lds_bytes, s, blocks);
+  if (small_tiles) return launch_fused_cmp<7, 0>(plan, lds_bytes, s, blocks);
+  return launch_fused_cmp<8, 0>(plan, lds_bytes, s, blocks);
 }
 
 template <int DEPTH>
@@ -2823,6 +2895,13 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   auto mark = [&](int i) {
     if (ev) (void)hipEventRecord(ev[i], s);
   };
+  const int64_t npairs = (int64_t)c.K * c.rk;
+  const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
+  // gradient rows are numbered batch by batch, so a stable sort on the row bits alone orders them by (row, batch)
+  const int sort_bits = bits_for(rows - 1) + c.kbits;
+  uint64_t* skeys = nullptr;
+  uint32_t* svals = nullptr;
+  hipEvent_t sort_done = nullptr;  // set: the sort was queued on the side stream and ends with this event
   mark(0);
   if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
   if (stream) {
@@ -2841,7 +2920,43 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   } else if (plan.fused) {
     // gather -> operator -> scores -> loss -> backward -> raw-row gradients in one kernel per chunk
     const size_t lds_bytes = (size_t)plan.fl.total * sizeof(float);
-    if ((rc = launch_fused(plan, lds_bytes, s)) != PBG_OK) return rc;
+    // One persistent workgroup per compute unit (the LDS footprint allows no more); workgroup b takes chunks
+    // b, b + grid, ...: `rounds` of them at most.
+    const int cus = compute_units(), chunks = c.K * c.C;
+    const int rounds = (int)ceil_div(chunks, cus);
+    int blocks = chunks < cus ? chunks : cus;
+    // The sort keys do not depend on the embeddings: made by a kernel of their own first, they can be sorted
+    // on the side stream while the chunk kernel runs -- on the compute units that it leaves alone (its
+    // workgroups would otherwise hold every one of them until the last chunk is done).  That is free when
+    // fewer workgroups finish in the same number of rounds, and pays for a round more when the sort is a
+    // long one (two or more passes inside the buckets: tables beyond 2^17 rows, where hot rows make them long).
+    // A small call keeps everything on one stream: two events cost more there than its sort.
+    SideStream* ss = nullptr;
+    if (chunks >= 128 && cus > 1 && getenv("PBG_DISABLE_SIDE_STREAM") == nullptr) {
+      const int rounds_beside = (int)ceil_div(chunks, cus - 1);
+      if (rounds_beside == rounds || sort_bits - c.kbits > 17) {
+        ss = side_stream();
+        if (ss) blocks = (int)ceil_div(chunks, rounds_beside);
+      }
+    }
+    unsigned slot = 0;
+    if (ss) {
+      plan.c.fused_rowid = plan.fused_rowid;
+      hipLaunchKernelGGL(fused_ids_kernel, dim3((unsigned)chunks), dim3(kFusedIds), 0, s, c);
+      slot = ss->next.fetch_add(1) & 7u;
+      if (hipEventRecord(ss->fork[slot], s) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
+    }
+    if ((rc = launch_fused(plan, lds_bytes, s, blocks)) != PBG_OK) return rc;  // (queued first: it is to find the machine empty)
+    if (ss) {
+      if (hipStreamWaitEvent(ss->stream, ss->fork[slot], 0) != hipSuccess)
+        return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
+      if ((rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, ss->stream,
+                           &skeys, &svals)) != PBG_OK)
+        return rc;
+      if (hipEventRecord(ss->join[slot], ss->stream) != hipSuccess)
+        return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
+      sort_done = ss->join[slot];
+    }
     mark(1);
     mark(2);
     mark(3);
@@ -2871,21 +2986,19 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   if ((rc = run_params(desc, bufs, plan, s, &rel_order, stream)) != PBG_OK) return rc;
   if (bufs->lhs_global) {  // the raw-row gradients are complete and still one per gathered row
     hipLaunchKernelGGL(global_grad_kernel, dim3((unsigned)c.K, (unsigned)(2 * plan.gslices)), dim3(kGlobalHalves * 32), 0,
-                       s, c, plan.gth, plan.gslices);
+                       s, c, plan.gth, plan.gslices, plan.fused ? 1 : 0);
     hipLaunchKernelGGL(global_update_kernel, wave_grid(c.D), dim3(kRowThreads), 0, s, c, plan.gth, plan.gslices,
                        bufs->lhs_global == bufs->rhs_global ? 1 : 0, bufs->lhs_global, bufs->lhs_global_sum,
                        bufs->rhs_global, bufs->rhs_global_sum, desc->relation_lr);
     if ((rc = check_launch("step global embeddings")) != PBG_OK) return rc;
   }
   mark(8);
-  const int64_t npairs = (int64_t)c.K * c.rk;
-  const uint64_t rows = (uint64_t)desc->num_lhs_rows + (desc->shared_table ? 0 : (uint64_t)desc->num_rhs_rows);
-  // gradient rows are numbered batch by batch, so a stable sort on the row bits alone orders them by (row, batch)
-  uint64_t* skeys;
-  uint32_t* svals;
-  rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, bits_for(rows - 1) + c.kbits,
-                  plan.sort_temp, s, &skeys, &svals);
-  if (rc != PBG_OK) return rc;
+  if (sort_done) {
+    if (hipStreamWaitEvent(s, sort_done, 0) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot join the side stream");
+  } else {
+    rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, s, &skeys, &svals);
+    if (rc != PBG_OK) return rc;
+  }
   mark(9);
   if (desc->shared_table) {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,

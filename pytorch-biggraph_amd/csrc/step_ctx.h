@@ -71,6 +71,7 @@ struct StepCtx {
   float reg_coef;  // N3 regularizer weight (0: none)
   float* regrow;   // [K, 2, B] sum of cubed moduli of each positive's prepared row(s), per side
   float* reg_out;  // [K] or null
+  int* fused_rowid;  // fused route: [K*C, 256] row id of every operand-row slot of a chunk (-1: none), see fused_ids_kernel
 };
 
 // Uniform negative number flat = (k * C + chunk) * U + u of side s: given by the

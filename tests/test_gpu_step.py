@@ -725,23 +725,28 @@ def test_hundred_steps(pbg, case):
     compare_state(cfg, runner, st, 1e-4, "100 steps")
 
 
-def test_hip_graph_replays_match_eager(pbg):
+@pytest.mark.parametrize("workers", [1, 8])
+def test_hip_graph_replays_match_eager(pbg, workers):
     """A captured step replayed with new inputs does what the eager call does:
     two runners from the same state, one eager, one replaying its graph, with
-    eager work and synchronisations between the replays, stay bit-identical."""
-    say("hip graph")
+    eager work and synchronisations between the replays, stay bit-identical.
+    With 8 batches of 1000 edges the call has 160 chunks, enough for the sort of
+    its keys to run on the library's side stream beside the chunk kernel: the
+    capture then holds a fork and a join."""
+    say("hip graph", workers)
     cfg = ostep.StepConfig(dim=100, operator="translation", comparator="l2", loss="ranking", num_batch_negs=50,
                            num_uniform_negs=50, lr=0.1, num_relations=3, relation_weights=[1.0, 0.5, 2.0])
-    num_pos, steps = 230, 4
-    st, batches = make_inputs(cfg, num_pos, 3000, steps + 1, seed=5)
-    eager = to_runner(pbg, cfg, st, num_pos, 1)
-    graphed = to_runner(pbg, cfg, st, num_pos, 1)
-    static = [t.clone() for t in pack(cfg, [batches[0]])]
+    num_pos, steps = (230, 4) if workers == 1 else (1000, 3)
+    st, all_batches = make_inputs(cfg, num_pos, 3000 if workers == 1 else 40000, (steps + 1) * workers, seed=5)
+    batches = [all_batches[i * workers:(i + 1) * workers] for i in range(steps + 1)]
+    eager = to_runner(pbg, cfg, st, num_pos, workers)
+    graphed = to_runner(pbg, cfg, st, num_pos, workers)
+    static = [t.clone() for t in pack(cfg, batches[0])]
     graph = graphed.capture_train(*static)  # runs batch 0 twice (set-up call + capture is not a run) ...
     copy_state(graphed, st)                 # ... so start again from the common state
     graphed.loss_out.zero_()
     for b in batches[1:]:
-        inputs = pack(cfg, [b])
+        inputs = pack(cfg, b)
         eager.train(*inputs)
         for dst, src in zip(static, inputs):
             dst.copy_(src)
