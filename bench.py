@@ -30,8 +30,8 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of (workload, kernel, workers), from the rocprofv3 FETCH_SIZE /
 # WRITE_SIZE runs summarised in profiles/train_step_pmc_traffic.md (not measured live);
 # any other combination reports null.
-TRAFFIC = {("cfg1", "fused_chunk", 64): 233.3e6, ("cfg4", "fused_chunk", 64): 230.6e6,
-           ("cfg2", "stream_chunk", 64): 13961.0e6}
+TRAFFIC = {("cfg1", "fused_chunk", 64): 233.3e6, ("cfg4", "fused_chunk", 64): 225.5e6,
+           ("cfg2", "stream_chunk", 64): 13960.2e6}
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
