@@ -761,6 +761,38 @@ def test_hip_graph_replays_match_eager(pbg, workers):
             assert torch.equal(eager.rhs_op_sum[k], graphed.rhs_op_sum[k])
 
 
+def test_two_streams_share_the_side_stream(pbg):
+    """Two runners train on two streams at once, each call large enough for the sort of
+    its keys to run on the library's side stream: the results are those of the same
+    calls made one after the other."""
+    say("two streams")
+    cfg = ostep.StepConfig(dim=100, operator="none", comparator="dot", loss="ranking", num_batch_negs=50,
+                           num_uniform_negs=50, lr=0.1)
+    workers, num_pos, calls = 8, 1000, 6
+    states, inputs = [], []
+    for r in range(2):
+        st, batches = make_inputs(cfg, num_pos, 50000, workers * calls, seed=11 + r)
+        states.append(st)
+        inputs.append([pack(cfg, batches[i * workers:(i + 1) * workers]) for i in range(calls)])
+    alone = [to_runner(pbg, cfg, st, num_pos, workers) for st in states]
+    for r in range(2):
+        for inp in inputs[r]:
+            alone[r].train(*inp)
+    torch.cuda.synchronize()
+    together = [to_runner(pbg, cfg, st, num_pos, workers) for st in states]
+    streams = [torch.cuda.Stream(device=DEV) for _ in range(2)]
+    torch.cuda.synchronize()
+    for i in range(calls):
+        for r in range(2):
+            with torch.cuda.stream(streams[r]):
+                together[r].train(*inputs[r][i])
+    torch.cuda.synchronize()
+    for r in range(2):
+        assert together[r].route == "fused"
+        assert torch.equal(alone[r].w_lhs, together[r].w_lhs) and torch.equal(alone[r].g_lhs, together[r].g_lhs)
+        assert torch.equal(alone[r].loss_out, together[r].loss_out)
+
+
 @pytest.mark.parametrize("case", [
     dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50,
          num_pos=230, dim=100),                                                  # fused chunk kernel
