@@ -132,7 +132,7 @@ int pbg_gemm_f32(const float* a, const float* b, float* c, int32_t batch, int32_
  * (train_cpu.py:849-884) in the one interleaving that is deterministic.
  * ---------------------------------------------------------------------- */
 typedef struct pbg_step_desc {
-  int32_t dim;              /* D */
+  int32_t dim;              /* D, 1 .. 4096 (config.py:142-150 sets no limit; the per-row kernels keep a row in one wave's registers) */
   int32_t num_workers;      /* K >= 1 */
   int32_t batch_size;       /* B >= 1, edges per batch */
   int32_t num_batch_negs;   /* config.num_batch_negs; 0 selects uniform-only negatives (model.py:651-656) */

@@ -10,6 +10,9 @@
 namespace pbg {
 
 constexpr int kWave = 64;
+// Largest embedding dimension: the per-row kernels keep a row in the registers of one wave,
+// 64 floats per lane at this width.
+constexpr int kMaxDim = 4096;
 
 // Records `msg` for pbg_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);

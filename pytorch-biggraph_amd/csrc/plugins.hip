@@ -18,7 +18,9 @@ dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 
     if ((nvh) <= 1) hipLaunchKernelGGL((KERNEL<1>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);        \
     else if ((nvh) <= 2) hipLaunchKernelGGL((KERNEL<2>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);   \
     else if ((nvh) <= 4) hipLaunchKernelGGL((KERNEL<4>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);   \
-    else hipLaunchKernelGGL((KERNEL<8>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);                   \
+    else if ((nvh) <= 8) hipLaunchKernelGGL((KERNEL<8>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);   \
+    else if ((nvh) <= 16) hipLaunchKernelGGL((KERNEL<16>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__); \
+    else hipLaunchKernelGGL((KERNEL<32>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);                  \
   } while (0)
 
 int nvh_for(int dim) { return (int)ceil_div((dim + 1) / 2, kWave); }
@@ -400,7 +402,7 @@ extern "C" int pbg_operator_forward(int32_t op, int32_t dim, int64_t n_rows, con
                                     const float* p1, const int64_t* rel, int64_t num_ops, float* y,
                                     pbg_stream_t stream) {
   if (!valid_op(op)) return fail(PBG_ERR_INVALID, "pbg_operator_forward: unknown operator %d", op);
-  if (dim <= 0 || dim > 1024 || n_rows < 0) return fail(PBG_ERR_INVALID, "pbg_operator_forward: bad sizes");
+  if (dim <= 0 || dim > kMaxDim || n_rows < 0) return fail(PBG_ERR_INVALID, "pbg_operator_forward: bad sizes");
   if (op == PBG_OP_COMPLEX_DIAGONAL && dim % 2 != 0)
     return fail(PBG_ERR_INVALID, "Need even dimension as 1st half is real and 2nd half is imaginary coordinates");
   if (n_rows == 0) return PBG_OK;
@@ -433,7 +435,7 @@ extern "C" int pbg_operator_backward(int32_t op, int32_t dim, int64_t n_rows, co
                                      const float* p0, const float* p1, const int64_t* rel, int64_t num_ops, float* dx,
                                      float* dp0, float* dp1, pbg_stream_t stream) {
   if (!valid_op(op)) return fail(PBG_ERR_INVALID, "pbg_operator_backward: unknown operator %d", op);
-  if (dim <= 0 || dim > 1024 || n_rows < 0) return fail(PBG_ERR_INVALID, "pbg_operator_backward: bad sizes");
+  if (dim <= 0 || dim > kMaxDim || n_rows < 0) return fail(PBG_ERR_INVALID, "pbg_operator_backward: bad sizes");
   if (n_rows == 0) return PBG_OK;
   if (!x || !dy || !dx || (op != PBG_OP_NONE && (!p0 || !dp0)) ||
       ((op == PBG_OP_COMPLEX_DIAGONAL || op == PBG_OP_AFFINE) && (!p1 || !dp1)))
@@ -473,7 +475,7 @@ extern "C" int pbg_operator_backward(int32_t op, int32_t dim, int64_t n_rows, co
 extern "C" int pbg_comparator_prepare(int32_t cmp, int32_t dim, int64_t n, const float* x, float* y, float* aux,
                                       pbg_stream_t stream) {
   if (!valid_cmp(cmp)) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare: unknown comparator %d", cmp);
-  if (dim <= 0 || dim > 1024 || n < 0) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare: bad sizes");
+  if (dim <= 0 || dim > kMaxDim || n < 0) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare: bad sizes");
   if (n == 0) return PBG_OK;
   if (!x || !y) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare: null pointer");
   PBG_DISPATCH_NVH(nvh_for(dim), prepare_kernel, wave_grid(n), (hipStream_t)stream, cmp, dim, n, x, y, aux);
@@ -483,7 +485,7 @@ extern "C" int pbg_comparator_prepare(int32_t cmp, int32_t dim, int64_t n, const
 extern "C" int pbg_comparator_prepare_backward(int32_t cmp, int32_t dim, int64_t n, const float* dy, const float* y,
                                                const float* aux, float* dx, pbg_stream_t stream) {
   if (!valid_cmp(cmp)) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare_backward: unknown comparator %d", cmp);
-  if (dim <= 0 || dim > 1024 || n < 0) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare_backward: bad sizes");
+  if (dim <= 0 || dim > kMaxDim || n < 0) return fail(PBG_ERR_INVALID, "pbg_comparator_prepare_backward: bad sizes");
   if (n == 0) return PBG_OK;
   if (!dy || !y || !dx || (cmp == PBG_CMP_COS && !aux))
     return fail(PBG_ERR_INVALID, "pbg_comparator_prepare_backward: null pointer");
@@ -501,7 +503,7 @@ extern "C" int pbg_comparator_forward(int32_t cmp, int32_t chunks, int32_t p, in
                                       const float* rhs_neg, float* pos, float* lhs_neg_scores, float* rhs_neg_scores,
                                       void* workspace, size_t workspace_bytes, pbg_stream_t stream) {
   if (!valid_cmp(cmp)) return fail(PBG_ERR_INVALID, "pbg_comparator_forward: unknown comparator %d", cmp);
-  if (chunks < 0 || p < 0 || ln < 0 || rn < 0 || dim <= 0 || dim > 1024)
+  if (chunks < 0 || p < 0 || ln < 0 || rn < 0 || dim <= 0 || dim > kMaxDim)
     return fail(PBG_ERR_INVALID, "pbg_comparator_forward: bad sizes");
   if (chunks == 0 || p == 0) return PBG_OK;
   if (!lhs_pos || !rhs_pos || !pos || (ln > 0 && (!lhs_neg || !lhs_neg_scores)) ||
@@ -548,7 +550,7 @@ extern "C" int pbg_comparator_backward(int32_t cmp, int32_t chunks, int32_t p, i
                                        const float* drhs_neg_scores, float* dlhs_pos, float* drhs_pos, float* dlhs_neg,
                                        float* drhs_neg, void* workspace, size_t workspace_bytes, pbg_stream_t stream) {
   if (!valid_cmp(cmp)) return fail(PBG_ERR_INVALID, "pbg_comparator_backward: unknown comparator %d", cmp);
-  if (chunks < 0 || p < 0 || ln < 0 || rn < 0 || dim <= 0 || dim > 1024)
+  if (chunks < 0 || p < 0 || ln < 0 || rn < 0 || dim <= 0 || dim > kMaxDim)
     return fail(PBG_ERR_INVALID, "pbg_comparator_backward: bad sizes");
   if (chunks == 0) return PBG_OK;
   if (!lhs_pos || !rhs_pos || !pos || !dpos || !dlhs_pos || !drhs_pos)

@@ -15,7 +15,6 @@ namespace {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kRowThreads = 256;  // 4 waves per block, one row per wave
-constexpr int kMaxV4 = 4;         // float4 per lane: covers dim <= 1024
 
 
 // ---- gather ----------------------------------------------------------------
@@ -765,7 +764,11 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   else if (nvec <= 4) PBG_LAUNCH(4);
   else if (nvec <= 8) PBG_LAUNCH(8);
   else if (nvec <= 16) PBG_LAUNCH(16);
-  else return fail(PBG_ERR_UNSUPPORTED, "row_adagrad: dim %d too large", dim);
+  else if constexpr (!VEC) {  // (a dim that is no multiple of 4: one float per lane and register)
+    if (nvec <= 32) PBG_LAUNCH(32);
+    else if (nvec <= 64) PBG_LAUNCH(64);
+    else return fail(PBG_ERR_UNSUPPORTED, "row_adagrad: dim %d too large", dim);
+  } else return fail(PBG_ERR_UNSUPPORTED, "row_adagrad: dim %d too large", dim);
 #undef PBG_LAUNCH
   return PBG_OK;
 }

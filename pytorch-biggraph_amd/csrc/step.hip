@@ -1396,7 +1396,8 @@ struct Plan {
 
 int validate(const pbg_step_desc* d, bool training) {
   if (!d) return fail(PBG_ERR_INVALID, "step: null descriptor");
-  if (d->dim <= 0 || d->dim > 1024) return fail(PBG_ERR_UNSUPPORTED, "step: dim must be in [1, 1024], got %d", d->dim);
+  if (d->dim <= 0 || d->dim > kMaxDim)
+    return fail(PBG_ERR_UNSUPPORTED, "step: dim must be in [1, %d], got %d", kMaxDim, d->dim);
   if (d->num_workers < 1 || d->num_workers > 256) return fail(PBG_ERR_INVALID, "step: num_workers must be in [1, 256]");
   if (d->batch_size < 1) return fail(PBG_ERR_INVALID, "step: batch_size must be positive");
   if (d->num_batch_negs < 0 || d->num_uniform_negs < 0) return fail(PBG_ERR_INVALID, "step: negative negatives count");
@@ -1716,7 +1717,9 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
     if ((nvh) <= 1) hipLaunchKernelGGL((KERNEL<1>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);          \
     else if ((nvh) <= 2) hipLaunchKernelGGL((KERNEL<2>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);     \
     else if ((nvh) <= 4) hipLaunchKernelGGL((KERNEL<4>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);     \
-    else hipLaunchKernelGGL((KERNEL<8>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);                     \
+    else if ((nvh) <= 8) hipLaunchKernelGGL((KERNEL<8>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);     \
+    else if ((nvh) <= 16) hipLaunchKernelGGL((KERNEL<16>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);   \
+    else hipLaunchKernelGGL((KERNEL<32>), grid, dim3(kRowThreads), 0, stream, __VA_ARGS__);                    \
   } while (0)
 
 dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 1, kWavesPerBlock)); }

@@ -50,6 +50,12 @@ def test_argument_errors_need_no_gpu(pbg):
     assert b"even dimension" in lib.pbg_last_error()
     d.dim = 6
     assert lib.pbg_train_step_workspace_bytes(ctypes.byref(d)) > 0
+    # rows of up to 4096 floats are taken; the next even width is refused with a message that says so
+    d.dim = 4096
+    assert lib.pbg_train_step_workspace_bytes(ctypes.byref(d)) > 0
+    d.dim = 4098
+    assert lib.pbg_train_step_workspace_bytes(ctypes.byref(d)) == 0
+    assert b"[1, 4096]" in lib.pbg_last_error()
     assert lib.pbg_row_adagrad_sparse_workspace_bytes(1000) > 1000 * 24
 
 

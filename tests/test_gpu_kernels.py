@@ -15,7 +15,7 @@ def say(*a):
     print(*a, flush=True)
 
 
-@pytest.mark.parametrize("dim,n_rows,n", [(100, 1000, 4000), (3, 7, 20), (1024, 300, 513), (400, 64, 1), (6, 5, 0)])
+@pytest.mark.parametrize("dim,n_rows,n", [(100, 1000, 4000), (3, 7, 20), (1024, 300, 513), (400, 64, 1), (6, 5, 0), (4096, 40, 100), (2050, 30, 64)])
 def test_gather_bit_exact(pbg, dim, n_rows, n):
     say("gather", dim, n_rows, n)
     g = torch.Generator().manual_seed(dim)
@@ -70,7 +70,7 @@ def test_bmm_nt_unaligned_dim(pbg):
 
 
 @pytest.mark.parametrize("dim,n_rows,n", [(100, 500, 4000), (1, 9, 30), (4, 50, 1), (1024, 40, 300), (10, 100000, 5000),
-                                          (400, 3, 700)])
+                                          (400, 3, 700), (4096, 30, 200), (2048, 5, 300), (2050, 20, 100), (1030, 9, 64)])
 def test_row_adagrad_sparse(pbg, dim, n_rows, n):
     say("row_adagrad_sparse", dim, n_rows, n)
     g = torch.Generator().manual_seed(n)

@@ -65,6 +65,14 @@ CASES = {
                            num_batch_negs=20, num_uniform_negs=20, entities=1500, relations=5, scale=0.3, ks=(20, 65)),
     "diagonal-dynamic": dict(operator="diagonal", comparator="dot", loss="logistic", dim=32, num_pos=100, dynamic=True,
                              num_batch_negs=20, num_uniform_negs=20, entities=1500, relations=5, scale=0.3, ks=(64, 65)),
+    # `linear` on rows wider than 1024 floats: every output coordinate sums that many products (the float64 anchor
+    # and the Adagrad slack of this file's criterion are for exactly such sums)
+    "linear-dim1536-dynamic": dict(operator="linear", comparator="dot", loss="logistic", dim=1536, num_pos=24, dynamic=True,
+                                   num_batch_negs=8, num_uniform_negs=5, entities=300, relations=3, scale=0.03, ks=(1, 3)),
+    "linear-dim1100": dict(operator="linear", comparator="cos", loss="softmax", dim=1100, num_pos=24, num_batch_negs=8,
+                           num_uniform_negs=5, entities=300, relations=3, scale=0.03, ks=(1, 3)),
+    "affine-dim2048": dict(operator="affine", comparator="l2", loss="ranking", dim=2048, num_pos=24, num_batch_negs=8,
+                           num_uniform_negs=5, entities=300, relations=2, scale=0.03, shared=False, ks=(2,)),
     # global embeddings: their update walks the batches in blocks of 64
     "global-fused": dict(operator="none", comparator="dot", loss="logistic", dim=100, num_pos=200, num_batch_negs=50,
                          num_uniform_negs=50, entities=3000, scale=0.1, global_emb=True, ks=(64, 65, 130)),

@@ -245,6 +245,9 @@ MODEL_CASES = [
     dict(operator="diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=20, num_pos=40,
          dim=16, max_norm=1.2),
     dict(operator="affine", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=9),
+    # rows wider than 1024 floats through the plugin classes
+    dict(operator="complex_diagonal", comparator="cos", loss="softmax", dynamic=False, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=2048),
+    dict(operator="translation", comparator="l2", loss="ranking", dynamic=True, num_batch_negs=8, num_uniform_negs=8, num_pos=24, dim=4096),
     dict(operator="affine", comparator="l2", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
     dict(operator="none", comparator="dot", loss="softmax", dynamic=True, num_batch_negs=10, num_uniform_negs=5, num_pos=25, dim=8),
     # with the N3 regularizer (the reference's FB15k example uses 1e-3 on ComplEx)

@@ -128,6 +128,10 @@ FORWARD_CASES += [
     dict(operator="translation", comparator="l2", dynamic=True, num_batch_negs=4, num_uniform_negs=3,
          num_pos=9, dim=8, disable_rhs_negs=True),
     dict(operator="none", comparator="dot", dynamic=False, num_batch_negs=16, num_uniform_negs=2, num_pos=5, dim=7),
+    # rows wider than 1024 floats: 32 and 64 floats of a row per lane
+    dict(operator="complex_diagonal", comparator="cos", dynamic=False, num_batch_negs=8, num_uniform_negs=5, num_pos=24, dim=2048),
+    dict(operator="translation", comparator="l2", dynamic=True, num_batch_negs=8, num_uniform_negs=5, num_pos=24, dim=4096),
+    dict(operator="diagonal", comparator="dot", dynamic=False, num_batch_negs=8, num_uniform_negs=5, num_pos=24, dim=2050),
 ]
 
 
@@ -192,6 +196,15 @@ TRAIN_CASES += [
          num_uniform_negs=50, num_pos=173, dim=100),
     dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=0,
          num_uniform_negs=9, num_pos=40, dim=9, disable_lhs_negs=True),
+    # rows wider than 1024 floats (the largest dimension is 4096), also where the dimension is no multiple of 4
+    dict(operator="complex_diagonal", comparator="cos", loss="softmax", dynamic=False, num_batch_negs=8,
+         num_uniform_negs=5, num_pos=24, dim=2048),
+    dict(operator="translation", comparator="l2", loss="ranking", dynamic=True, num_batch_negs=8,
+         num_uniform_negs=5, num_pos=24, dim=4096),
+    dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=8,
+         num_uniform_negs=5, num_pos=24, dim=1030),
+    dict(operator="none", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=8,
+         num_uniform_negs=5, num_pos=24, dim=2050),
 ]
 
 
