@@ -743,13 +743,9 @@ __global__ __launch_bounds__(kFusedIds) void fused_ids_kernel(StepCtx c) {
 // raises its dynamic LDS limit the first time it needs more than it was given.
 template <int T, int CMP, int LOSS, int LD>
 int launch_fused_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
-  static size_t lds_allowed = 0;
-  if (lds_bytes > lds_allowed) {
-    if (hipFuncSetAttribute((const void*)fused_chunk_kernel<T, CMP, LOSS, LD>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-      return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
-    lds_allowed = lds_bytes;
-  }
+  static LdsLimit limit;
+  const int rc = reserve_lds((const void*)fused_chunk_kernel<T, CMP, LOSS, LD>, &limit, lds_bytes);
+  if (rc != PBG_OK) return rc;
   const int chunks = c.K * c.C;
   hipLaunchKernelGGL((fused_chunk_kernel<T, CMP, LOSS, LD>), dim3((unsigned)blocks), dim3(2 * kFusedThreads), lds_bytes, s,
                      c, fl, chunks);

@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/pbg_hip.h"
 
 namespace pbg {
@@ -18,6 +20,17 @@ constexpr int kMaxDim = 4096;
 int fail(int code, const char* fmt, ...);
 // Turns the pending HIP launch error (if any) into a pbg_status.
 int check_launch(const char* what);
+
+// Per-device state of the library is kept for devices 0 .. kMaxDevices - 1.
+constexpr int kMaxDevices = 16;
+// The dynamic LDS limit a kernel has been given so far, per device.
+struct LdsLimit {
+  std::atomic<size_t> allowed[kMaxDevices];
+};
+// Raises `kernel`'s dynamic LDS limit on the current device to `bytes` unless it is that high already.
+int reserve_lds(const void* kernel, LdsLimit* limit, size_t bytes);
+// Compute units of the current device.
+int compute_units();
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

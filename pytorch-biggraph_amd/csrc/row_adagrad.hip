@@ -943,7 +943,6 @@ extern "C" int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t n
 namespace {
 constexpr int64_t kStaticMaxIndices = (int64_t)1 << 20;
 constexpr size_t kStaticScratchBytes = (size_t)32 << 20;  // 24 bytes per index + the sort's counters
-constexpr int kMaxDevices = 64;
 }  // namespace
 
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];

@@ -1996,17 +1996,6 @@ namespace {
 // prep | operator forward | score GEMMs | loss | dN GEMMs | dA GEMMs | rowback | params | sort | update
 constexpr int kStages = 10;
 
-int compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-  }
-  return cus;
-}
-
 // The library's own second stream per device, on which the sort of a call's keys runs beside the
 // chunk kernel (the keys do not depend on the embeddings).  A call forks it from the caller's stream
 // with one event and joins it back with another before the update reads the sorted keys; a ring of
@@ -2018,7 +2007,6 @@ struct SideStream {
   bool ok = false;
 };
 SideStream* side_stream() {
-  constexpr int kMaxDevices = 16;
   static SideStream tab[kMaxDevices];
   static bool tried[kMaxDevices];
   static std::mutex mu;

@@ -765,13 +765,9 @@ __global__ __launch_bounds__(kRowThreads) void stream_finish_kernel(StepCtx c, S
 template <int NT, int LOSS>
 int launch_chunk_as(const StepCtx& c, const StreamPlan& sp, hipStream_t s) {
   const size_t lds_bytes = (size_t)sp.total * sizeof(float);
-  static size_t lds_allowed = 0;
-  if (lds_bytes > lds_allowed) {
-    if (hipFuncSetAttribute((const void*)stream_chunk_kernel<NT, LOSS>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess)
-      return fail(PBG_ERR_LAUNCH, "step: cannot reserve %zu bytes of LDS", lds_bytes);
-    lds_allowed = lds_bytes;
-  }
+  static LdsLimit limit;
+  const int rc = reserve_lds((const void*)stream_chunk_kernel<NT, LOSS>, &limit, lds_bytes);
+  if (rc != PBG_OK) return rc;
   const int items = 2 * c.K * c.C;
   hipLaunchKernelGGL((stream_chunk_kernel<NT, LOSS>), dim3((unsigned)(items < sp.grid ? items : sp.grid)),
                      dim3(2 * kHelpers), lds_bytes, s, c, sp, items);
