@@ -118,6 +118,14 @@ int pbg_gemm_f32(const float* a, const float* b, float* c, int32_t batch, int32_
                  int32_t lda, int32_t ldb, int32_t ldc, int64_t stride_a, int64_t stride_b,
                  int64_t stride_c, int32_t a_kmajor, int32_t b_kmajor, float alpha, float beta,
                  pbg_stream_t stream);
+/* The same product for operands whose every value is a float16 number (held as fp32), as torch.bmm
+ * computes it on Half tensors: the comparators' call sites under config.half_precision
+ * (model.py:504-505 then :179-180,209-210).  Runs on the fp16 matrix instructions, sums in fp32,
+ * and stores C rounded to float16 numbers (still as fp32). */
+int pbg_gemm_f16(const float* a, const float* b, float* c, int32_t batch, int32_t m, int32_t n, int32_t k,
+                 int32_t lda, int32_t ldb, int32_t ldc, int64_t stride_a, int64_t stride_b,
+                 int64_t stride_c, int32_t a_kmajor, int32_t b_kmajor, float alpha, float beta,
+                 pbg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * The training step.  Replaces Trainer._process_one_batch (train_cpu.py:86-112):
@@ -165,6 +173,13 @@ typedef struct pbg_step_desc {
                              * B positives, negatives = EVERY entity of the side's type in table order (lhs_neg
                              * is [K, B, num_lhs_rows]), the edge's own entity masked; num_batch_negs,
                              * num_uniform_negs and the uniform index arrays are ignored */
+  int32_t half_precision;   /* config.half_precision (config.py:496-498; model.py:504-505,827-829): every embedding
+                             * is cast to float16 once it is prepared for the comparator, so the negatives' scores
+                             * are float16 products and the prepared embeddings' gradients float16 tensors; positive
+                             * scores, losses, operators and both optimizers stay fp32.  Tables, scores and gradients
+                             * are still fp32 arrays here (holding float16 numbers where the reference holds Half
+                             * tensors); the products run on the fp16 matrix instructions.  dot and cos comparators,
+                             * without bias and regularizer (anything else: PBG_ERR_UNSUPPORTED) */
 } pbg_step_desc;
 
 typedef struct pbg_step_buffers {

@@ -53,6 +53,12 @@ class StepConfig:
     # RelationSchema.all_negs (config.py:123-131): the negatives of an edge are ALL entities of the
     # side's type, in one chunk (model.py:648-650,582-618)
     all_negs: bool = False
+    # config.py:496-498 "Use half-precision training (GPU ONLY)": every embedding is cast to
+    # float16 once it is prepared for the comparator (model.py:504-505), so the negative scores are
+    # float16 products cast back (model.py:827-829) and the gradient of every prepared embedding is a
+    # float16 tensor.  The reference only casts on a CUDA device; here the same statements run on
+    # the CPU's Half tensors.
+    half_precision: bool = False
 
     def chunking(self, num_pos: int) -> Tuple[int, int, str]:
         """(chunk_size, num_chunks, mode) as model.py:648-656 and :787."""
@@ -331,7 +337,7 @@ class Scores:
 
 
 def _adjust(cfg: StepConfig, embs, rel, op_params, glob=None) -> torch.Tensor:
-    """model.py:478-506 without half precision: global embedding of the entity
+    """model.py:478-506: global embedding of the entity
     type (``glob``, None = disabled), operator, comparator.prepare.
     ``op_params is None`` means "no operator"."""
     if glob is not None:
@@ -340,7 +346,10 @@ def _adjust(cfg: StepConfig, embs, rel, op_params, glob=None) -> torch.Tensor:
         embs = embs + glob
     if op_params is not None:
         embs = apply_operator(cfg.operator, embs, op_params, rel)
-    return (biased_prepare if cfg.bias else comparator_prepare)(cfg.comparator, embs)
+    embs = (biased_prepare if cfg.bias else comparator_prepare)(cfg.comparator, embs)
+    if cfg.half_precision and embs.dtype == torch.float32:  # model.py:504-505 (without its is_cuda condition)
+        embs = embs.half()
+    return embs
 
 
 def _direction_agnostic(

@@ -47,6 +47,7 @@ class StepDesc(ctypes.Structure):
         ("max_norm", c_float),
         ("bias", c_int32),
         ("all_negs", c_int32),
+        ("half_precision", c_int32),
     ]
 
 
@@ -83,6 +84,8 @@ SIGNATURES = {
     "pbg_row_adagrad_dense": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_float, c_void_p]),
     "pbg_async_adagrad_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p]),
     "pbg_gemm_f32": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                               c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_float, c_float, c_void_p]),
+    "pbg_gemm_f16": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_float, c_float, c_void_p]),
     "pbg_sizeof_step_desc": (c_size_t, []),
     "pbg_sizeof_step_buffers": (c_size_t, []),

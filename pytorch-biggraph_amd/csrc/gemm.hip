@@ -12,12 +12,42 @@
 // an operand whose other axis is contiguous is kept as tile[k][r].  All operand
 // values of a depth-16 tile are read into registers before the 64 MFMAs of the
 // tile, which then issue back to back.
+//
+// HALF variants (config.half_precision: both operands hold float16 numbers): the same
+// tiles and the same lanes' values, converted to fp16 in registers (exactly) after the LDS
+// read and contracted by ONE v_mfma_f32_16x16x16_f16 per depth-16 tile instead of four
+// fp32 steps: lane group g holds k = 4 g .. 4 g + 3 in both layouts.  Sums stay fp32; the
+// result is rounded to a float16 number when it is stored.
 #include "pbg_internal.h"
 
 namespace pbg {
 namespace {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// acc[i][j] += A-tile i (rows) x B-tile j (columns) over the 16 values of k the lanes hold in fa / fb
+template <bool HALF, int TM, int TN>
+__device__ __forceinline__ void tile_products(const float4v (&fa)[TM], const float4v (&fb)[TN], float4v (&acc)[TM][TN]) {
+  if constexpr (HALF) {
+    half4v ha[TM], hb[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) ha[i] = (half4v){(_Float16)fa[i][0], (_Float16)fa[i][1], (_Float16)fa[i][2], (_Float16)fa[i][3]};
+#pragma unroll
+    for (int j = 0; j < TN; ++j) hb[j] = (half4v){(_Float16)fb[j][0], (_Float16)fb[j][1], (_Float16)fb[j][2], (_Float16)fb[j][3]};
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(ha[i], hb[j], acc[i][j], 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+  }
+}
 
 constexpr int kGemmThreads = 256;
 constexpr int BK = 16;
@@ -116,7 +146,7 @@ struct TileLoader {
   }
 };
 
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR>
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, bool HALF>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g, int a_vec, int b_vec) {
   constexpr int TM = BM / 2 / 16;  // MFMA tiles per wave along m
   constexpr int TN = BN / 2 / 16;
@@ -178,13 +208,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g, int a
       for (int i = 0; i < TM; ++i) fa[i] = LoadA::operand(lds_a[cur], wm0 + i * 16 + (lane & 15), lane >> 4);
 #pragma unroll
       for (int j = 0; j < TN; ++j) fb[j] = LoadB::operand(lds_b[cur], wn0 + j * 16 + (lane & 15), lane >> 4);
-#pragma unroll
-      for (int s = 0; s < 4; ++s)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+      tile_products<HALF, TM, TN>(fa, fb, acc);
       if ((kt & (kFoldTiles - 1)) == kFoldTiles - 1) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -214,7 +238,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g, int a
             float* dst = c + (int64_t)row * g.ldc + col;
             float v = g.alpha * (tot[i][j][r] + acc[i][j][r]);
             if (g.beta != 0.f) v += g.beta * *dst;
-            *dst = v;
+            *dst = HALF ? (float)(_Float16)v : v;
           }
         }
       }
@@ -308,7 +332,7 @@ struct DmaTile {
 // bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima).
 #define PBG_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
-template <bool A_KMAJOR, bool B_KMAJOR>
+template <bool A_KMAJOR, bool B_KMAJOR, bool HALF>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dma_kernel(GemmArgs g) {
   constexpr int TM = 4, TN = 4;
   __shared__ __attribute__((aligned(16))) float lds_a[kDmaStages][kDmaTileFloats];
@@ -383,13 +407,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dma_kernel(GemmArgs g) {
           for (int j = 0; j < TN; ++j) fb[j][s] = live ? fb[j][s] : 0.f;
         }
       }
-#pragma unroll
-      for (int s = 0; s < 4; ++s)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+      tile_products<HALF, TM, TN>(fa, fb, acc);
       if ((kt & (kFoldTiles - 1)) == kFoldTiles - 1) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -418,7 +436,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dma_kernel(GemmArgs g) {
             float* dst = c + (int64_t)row * g.ldc + col;
             float v = g.alpha * (tot[i][j][r] + acc[i][j][r]);
             if (g.beta != 0.f) v += g.beta * *dst;
-            *dst = v;
+            *dst = HALF ? (float)(_Float16)v : v;
           }
         }
       }
@@ -426,32 +444,33 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dma_kernel(GemmArgs g) {
   }
 }
 
+template <bool HALF>
 void launch_dma(const GemmArgs& g, hipStream_t stream) {
   dim3 grid((unsigned)ceil_div(g.n, kDmaTile), (unsigned)ceil_div(g.m, kDmaTile),
             (unsigned)(g.batch < 65535 ? g.batch : 65535));
   dim3 block(kGemmThreads);
   if (!g.a_kmajor && !g.b_kmajor)
-    hipLaunchKernelGGL((gemm_dma_kernel<false, false>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_dma_kernel<false, false, HALF>), grid, block, 0, stream, g);
   else if (!g.a_kmajor && g.b_kmajor)
-    hipLaunchKernelGGL((gemm_dma_kernel<false, true>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_dma_kernel<false, true, HALF>), grid, block, 0, stream, g);
   else if (g.a_kmajor && !g.b_kmajor)
-    hipLaunchKernelGGL((gemm_dma_kernel<true, false>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_dma_kernel<true, false, HALF>), grid, block, 0, stream, g);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<true, true>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_dma_kernel<true, true, HALF>), grid, block, 0, stream, g);
 }
 
-template <int BM, int BN>
+template <int BM, int BN, bool HALF>
 void launch(const GemmArgs& g, int a_vec, int b_vec, hipStream_t stream) {
   dim3 grid((unsigned)ceil_div(g.n, BN), (unsigned)ceil_div(g.m, BM), (unsigned)(g.batch < 65535 ? g.batch : 65535));
   dim3 block(kGemmThreads);
   if (!g.a_kmajor && !g.b_kmajor)
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, false, false>), grid, block, 0, stream, g, a_vec, b_vec);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, false, false, HALF>), grid, block, 0, stream, g, a_vec, b_vec);
   else if (!g.a_kmajor && g.b_kmajor)
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, false, true>), grid, block, 0, stream, g, a_vec, b_vec);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, false, true, HALF>), grid, block, 0, stream, g, a_vec, b_vec);
   else if (g.a_kmajor && !g.b_kmajor)
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, true, false>), grid, block, 0, stream, g, a_vec, b_vec);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, true, false, HALF>), grid, block, 0, stream, g, a_vec, b_vec);
   else
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, true, true>), grid, block, 0, stream, g, a_vec, b_vec);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, true, true, HALF>), grid, block, 0, stream, g, a_vec, b_vec);
 }
 
 bool quad_aligned(const float* p, int ld, int64_t stride) {
@@ -470,12 +489,15 @@ int gemm_f32(const GemmArgs& g, hipStream_t stream) {
   const bool dma_ok = a_vec && b_vec && g.k % 4 == 0 && g.k >= BK && (!g.a_kmajor || (g.m % 4 == 0 && g.m >= 4)) &&
                       (!g.b_kmajor || (g.n % 4 == 0 && g.n >= 4));
   // (a product of at most 64 values of k is bound by writing its output: the smaller tile pads less)
-  if (g.m <= 96 || g.n <= 96 || (!dma_ok && g.k <= 64)) {
-    launch<64, 64>(g, a_vec, b_vec, stream);
-  } else if (dma_ok) {
-    launch_dma(g, stream);
+  const bool small = g.m <= 96 || g.n <= 96 || (!dma_ok && g.k <= 64);
+  if (g.half) {
+    if (small) launch<64, 64, true>(g, a_vec, b_vec, stream);
+    else if (dma_ok) launch_dma<true>(g, stream);
+    else launch<128, 128, true>(g, a_vec, b_vec, stream);
   } else {
-    launch<128, 128>(g, a_vec, b_vec, stream);
+    if (small) launch<64, 64, false>(g, a_vec, b_vec, stream);
+    else if (dma_ok) launch_dma<false>(g, stream);
+    else launch<128, 128, false>(g, a_vec, b_vec, stream);
   }
   return check_launch("gemm_f32");
 }
@@ -496,5 +518,23 @@ extern "C" int pbg_gemm_f32(const float* a, const float* b, float* c, int32_t ba
   g.m = m; g.n = n; g.k = k; g.batch = batch;
   g.a_kmajor = a_kmajor; g.b_kmajor = b_kmajor;
   g.alpha = alpha; g.beta = beta;
+  return pbg::gemm_f32(g, (hipStream_t)stream);
+}
+
+extern "C" int pbg_gemm_f16(const float* a, const float* b, float* c, int32_t batch, int32_t m, int32_t n, int32_t k,
+                            int32_t lda, int32_t ldb, int32_t ldc, int64_t stride_a, int64_t stride_b,
+                            int64_t stride_c, int32_t a_kmajor, int32_t b_kmajor, float alpha, float beta,
+                            pbg_stream_t stream) {
+  if (batch < 0 || m < 0 || n < 0 || k < 0) return pbg::fail(PBG_ERR_INVALID, "pbg_gemm_f16: negative size");
+  if (batch == 0 || m == 0 || n == 0) return PBG_OK;
+  if (!a || !b || !c) return pbg::fail(PBG_ERR_INVALID, "pbg_gemm_f16: null pointer");
+  pbg::GemmArgs g{};
+  g.a = a; g.b = b; g.c = c;
+  g.stride_a = stride_a; g.stride_b = stride_b; g.stride_c = stride_c;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.m = m; g.n = n; g.k = k; g.batch = batch;
+  g.a_kmajor = a_kmajor; g.b_kmajor = b_kmajor;
+  g.alpha = alpha; g.beta = beta;
+  g.half = 1;
   return pbg::gemm_f32(g, (hipStream_t)stream);
 }

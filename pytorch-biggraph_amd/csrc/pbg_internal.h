@@ -74,6 +74,9 @@ struct GemmArgs {
   // floats further (one operator matrix per relation)
   const int64_t* b_index = nullptr;
   int64_t b_index_stride = 0;
+  // 1: every value of A and B is a float16 number (held as fp32): the products run on the fp16 matrix
+  // instructions, still summed in fp32, and C is rounded to float16 numbers (torch.bmm on Half tensors)
+  int half = 0;
 };
 int gemm_f32(const GemmArgs& args, hipStream_t stream);
 

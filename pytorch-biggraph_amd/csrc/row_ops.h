@@ -163,6 +163,17 @@ __device__ __forceinline__ void row_store(float* __restrict__ p, const RowV<NVH>
     if (h < H && H + h < D) p[H + h] = r.a[1][v];
   }
 }
+// The value a float16 tensor would hold for x (round to nearest even; beyond 65504: infinity), as fp32.
+__device__ __forceinline__ float half_round(float x) { return (float)(_Float16)x; }
+// config.half_precision: the prepared row as `embs.half()` leaves it (model.py:504-505)
+template <int NVH>
+__device__ __forceinline__ void row_round_half(RowV<NVH>& y) {
+#pragma unroll
+  for (int v = 0; v < NVH; ++v) {
+    y.a[0][v] = half_round(y.a[0][v]);
+    y.a[1][v] = half_round(y.a[1][v]);
+  }
+}
 template <int NVH>
 __device__ __forceinline__ float row_dot(const RowV<NVH>& x, const RowV<NVH>& y) {  // per-lane partial
   float acc = 0.f;

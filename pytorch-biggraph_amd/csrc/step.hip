@@ -172,6 +172,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
       RowV<NVH> y = x;
       const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
       const float aux = prepare_row<NVH>(c.cmp, y);
+      if (c.half) row_round_half<NVH>(y);
       row_store<NVH>(xp_row, y, D, H, lane);
       if (ap && lane == 0) *ap = aux;
       if (bp && lane == 0) *bp = b;
@@ -183,6 +184,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
         RowV<NVH> y = op_forward<NVH>(c.op, x, sd.p0, sd.p1, rel, D, H, lane);
         const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
         const float aux = prepare_row<NVH>(c.cmp, y);
+        if (c.half) row_round_half<NVH>(y);
         row_store<NVH>(c.dynamic ? xa_row : xp_row, y, D, H, lane);
         float* auxdst = c.dynamic ? aa : ap;
         if (auxdst && lane == 0) *auxdst = aux;
@@ -212,6 +214,7 @@ __global__ __launch_bounds__(kRowThreads) void prep_kernel(StepCtx c) {
     }
     const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
     const float aux = prepare_row<NVH>(c.cmp, y);
+    if (c.half) row_round_half<NVH>(y);
     row_store<NVH>(sd.xn + (kc * sd.nn + sd.nb + uu) * D, y, D, H, lane);
     if (sd.an && lane == 0) sd.an[kc * sd.nn + sd.nb + uu] = aux;
     if (c.bias && lane == 0) sd.bn[kc * sd.nn + sd.nb + uu] = b;
@@ -235,6 +238,7 @@ __global__ __launch_bounds__(kRowThreads) void prepare_staged_kernel(StepCtx c, 
   }
   const float b = c.bias ? take_bias<NVH>(y, lane) : 0.f;
   const float aux = prepare_row<NVH>(c.cmp, y);
+  if (c.half) row_round_half<NVH>(y);
   if (r < c.B) {
     const int cc = r / c.P, i = r % c.P;
     const int64_t kc = (int64_t)k * c.C + cc;
@@ -287,6 +291,7 @@ struct ScoreRow {
   float rb;          // bias of the positive operand
   int64_t own;       // all_negs: the column of the edge's own entity on this side (masked, model.py:596-618); else -1
   int cmp, nb, i, masked_from;  // batch-negative columns; own column; first padded column
+  int half;  // config.half_precision: dLoss/dscore is stored as the float16 number the cast's backward makes of it (model.py:827-829)
 
   // score of column j as the model returns it (model.py:234-246,836-839); `live`
   // is false where the value is a constant with no gradient
@@ -320,9 +325,10 @@ __device__ __forceinline__ void positive_scores(const StepCtx& c, int64_t kc, in
     // With batch negatives the score block already holds the pair: column i of row i
     // is (rhs positive i) . (lhs positive i), before masking.  (Distances are
     // recomputed from the rows: the block's ||a||^2 - 2ab + ||b||^2 cancels for a close pair.)
-    if (!is_distance(c.cmp) && c.side[0].nb > 0)
+    // (Nor with half_precision: the block then holds float16 numbers, the positive score is an fp32 sum, model.py:177.)
+    if (!is_distance(c.cmp) && !c.half && c.side[0].nb > 0)
       posv[0] = posv[1] = c.side[0].s[(kc * c.P + i) * c.side[0].nn + i];
-    else if (!is_distance(c.cmp) && c.side[1].nb > 0)
+    else if (!is_distance(c.cmp) && !c.half && c.side[1].nb > 0)
       posv[0] = posv[1] = c.side[1].s[(kc * c.P + i) * c.side[1].nn + i];
     else
       posv[0] = posv[1] = kappa(c.cmp, lp, rp, D, lane);
@@ -348,6 +354,7 @@ __device__ __forceinline__ ScoreRow score_row(const StepCtx& c, int s, int64_t k
   ScoreRow sr;
   sr.raw = sd.s + (kc * c.P + i) * sd.nn;
   sr.cmp = c.cmp;
+  sr.half = c.half;
   sr.bn = nullptr;
   sr.a2 = 0.f;
   if (is_distance(c.cmp)) {
@@ -488,7 +495,7 @@ __device__ __forceinline__ void side_loss_held(int loss, float margin, int cmp, 
       stored = -2.0f * dq;
     }
     if (j < nn) {
-      out[j] = stored;
+      out[j] = sr.half ? half_round(stored) : stored;
       if (gout) gout[j] = g;
     }
   }
@@ -547,7 +554,7 @@ __device__ __forceinline__ void side_loss_long(int loss, float margin, int cmp, 
       rowsum += dq;
       out[j] = -2.0f * dq;
     } else {
-      out[j] = g;
+      out[j] = sr.half ? half_round(g) : g;
     }
   }
   *dpos_out = wave_sum(dpos_part);
@@ -718,9 +725,10 @@ __device__ __forceinline__ float column_sum(const float* __restrict__ s, int64_t
 }
 
 // dy += dpos * d kappa(self, other) / d self
+// (`half`: the term and the sum are float16 numbers, as the gradient of a Half tensor that autograd adds up is)
 template <int NVH>
 __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos, const RowV<NVH>& self,
-                                             const RowV<NVH>& other, float pos) {
+                                             const RowV<NVH>& other, float pos, bool half = false) {
   if (is_distance(cmp)) {
     // kappa = -sqrt(max(sum (a-b)^2, 1e-30)); no gradient where the clamp is active.
     // squared_l2: kappa = -sum (a-b)^2
@@ -730,6 +738,12 @@ __device__ __forceinline__ void add_pos_term(int cmp, RowV<NVH>& dy, float dpos,
     for (int v = 0; v < NVH; ++v) {
       dy.a[0][v] += coef * (self.a[0][v] - other.a[0][v]);
       dy.a[1][v] += coef * (self.a[1][v] - other.a[1][v]);
+    }
+  } else if (half) {
+#pragma unroll
+    for (int v = 0; v < NVH; ++v) {
+      dy.a[0][v] = half_round(dy.a[0][v] + half_round(dpos * other.a[0][v]));
+      dy.a[1][v] = half_round(dy.a[1][v] + half_round(dpos * other.a[1][v]));
     }
   } else {
     row_axpy<NVH>(dy, dpos, other);
@@ -788,7 +802,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       const RowV<NVH> other = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
       // (the positive score carries the pair's two biases; the distance's gradient needs the distance)
       const float pair_bias = c.bias ? sd.bp[kc * sd.stride_p + i] + so.bp[kc * so.stride_p + i] : 0.f;
-      add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq] - pair_bias);
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[0][pq], y1, other, c.pos[0][pq] - pair_bias, c.half);
       float breg = 0.f;
       if (c.reg_coef != 0.f) {  // src_pos / dst_pos of the regularizer are these prepared rows (model.py:784-785,854)
         RowV<NVH> yb = y1;
@@ -821,7 +835,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       }
       const RowV<NVH> other = row_load<NVH>(so.xa + (kc * c.P + i) * D, D, H, lane);
       const float pair_bias = c.bias ? sd.bp[kc * sd.stride_p + i] + so.ba[kc * c.P + i] : 0.f;
-      add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq] - pair_bias);
+      add_pos_term<NVH>(c.cmp, dy, c.dpos[s][pq], y1, other, c.pos[s][pq] - pair_bias, c.half);
       // the plain row is src_pos of one direction's regularizer, the operated row
       // dst_pos of the other's (model.py:722-754)
       float cubes = 0.f, breg = 0.f, breg2 = 0.f;
@@ -847,7 +861,7 @@ __global__ __launch_bounds__(kRowThreads) void rowback_kernel(StepCtx c) {
       }
       const RowV<NVH> other2 = row_load<NVH>(so.xp + (kc * so.stride_p + i) * D, D, H, lane);
       const float pair_bias2 = c.bias ? sd.ba[kc * c.P + i] + so.bp[kc * so.stride_p + i] : 0.f;
-      add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq] - pair_bias2);
+      add_pos_term<NVH>(c.cmp, dy2, c.dpos[1 - s][pq], y2, other2, c.pos[1 - s][pq] - pair_bias2, c.half);
       if (c.reg_coef != 0.f) {
         RowV<NVH> yb2 = y2;
         if (c.bias) add_to_first<NVH>(yb2, sd.ba[kc * c.P + i], lane);
@@ -1419,6 +1433,15 @@ int validate(const pbg_step_desc* d, bool training) {
   if (d->bias) {
     if (d->dim < 2) return fail(PBG_ERR_INVALID, "step: bias needs at least two coordinates");
   }
+  if (d->half_precision) {
+    // The distance comparators clamp at 1e-30 before the square root (model.py:244), which is 0 as a
+    // float16: every batch negative that is its own positive's row then has a NaN gradient in the
+    // reference; bias and the regularizer would do their sums in float16.
+    if (d->comparator == PBG_CMP_L2 || d->comparator == PBG_CMP_SQUARED_L2)
+      return fail(PBG_ERR_UNSUPPORTED, "step: half_precision is built for the dot and cos comparators");
+    if (d->bias || d->regularization_coef != 0.f)
+      return fail(PBG_ERR_UNSUPPORTED, "step: half_precision is not built with bias or a regularizer");
+  }
   return PBG_OK;
 }
 
@@ -1450,6 +1473,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   c.op = d->op == PBG_OP_AFFINE ? PBG_OP_LINEAR : d->op;
   c.affine = d->op == PBG_OP_AFFINE;
   c.bias = d->bias != 0;
+  c.half = d->half_precision != 0;
   c.cmp = d->comparator;
   c.loss = d->loss;
   c.margin = d->margin;
@@ -1611,7 +1635,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->sort_temp = take(sort_temp_bytes(npairs), 1);
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
   // (the regularizer's terms live in the staged kernels only)
-  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && getenv("PBG_DISABLE_FUSED") == nullptr;
+  // (half_precision: the staged route only, whose products then run on the fp16 matrix instructions)
+  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && !c.half && getenv("PBG_DISABLE_FUSED") == nullptr;
   if (plan->fused) {  // the fused kernel writes every gradient row and every dz itself
     c.side[0].uni_direct = c.side[1].uni_direct = 0;
     c.side[0].uni_dz_direct = c.side[1].uni_dz_direct = 0;
@@ -1619,7 +1644,7 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   }
   // The streaming route's own buffers lie behind the staged ones: a call with global
   // embeddings (known only from its buffers) takes the staged route on the same workspace.
-  plan->stream = !plan->fused && stream_geometry(c, &plan->sp) && getenv("PBG_DISABLE_STREAM") == nullptr;
+  plan->stream = !plan->fused && !c.half && stream_geometry(c, &plan->sp) && getenv("PBG_DISABLE_STREAM") == nullptr;
   if (plan->stream) {
     StreamPlan& sp = plan->sp;
     const size_t ne = (size_t)K * c.B;
@@ -1808,6 +1833,7 @@ int run_scores(const Plan& plan, hipStream_t stream) {
     g.b = sd.xn; g.stride_b = (int64_t)sd.nn * D; g.ldb = D; g.b_kmajor = 0;
     g.c = sd.s; g.stride_c = (int64_t)P * sd.nn; g.ldc = sd.nn;
     g.m = P; g.n = sd.nn; g.k = D; g.batch = K * C; g.alpha = 1.f; g.beta = 0.f;
+    g.half = c.half;
     if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
   }
   return check_launch("step forward");
@@ -1827,6 +1853,7 @@ int run_backward_dn(const Plan& plan, hipStream_t stream) {
     g.stride_b = (int64_t)(c.dynamic ? P : so.stride_p) * D; g.ldb = D; g.b_kmajor = 1;
     g.c = sd.dxn; g.stride_c = (int64_t)sd.nn * D; g.ldc = D;
     g.m = sd.nn; g.n = D; g.k = P; g.batch = K * C; g.alpha = 1.f; g.beta = 0.f;
+    g.half = c.half;
     if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
   }
   return check_launch("step backward dN");
@@ -1850,6 +1877,7 @@ int run_backward_da(const Plan& plan, hipStream_t stream) {
     }
     g.ldc = D;
     g.m = P; g.n = D; g.k = sd.nn; g.batch = K * C; g.alpha = 1.f;
+    g.half = c.half;
     if ((rc = gemm_f32(g, stream)) != PBG_OK) return rc;
   }
   return check_launch("step backward");

@@ -51,6 +51,7 @@ struct SideCtx {
 struct StepCtx {
   int D, K, B, P, C, U, last, dynamic, op, cmp, loss, num_relations;
   int bias;    // config.bias: BiasedComparator around the comparator (model.py:306-344,902-903)
+  int half;    // config.half_precision: prepared rows, negative scores and their gradients are float16 numbers (model.py:504-505,827-829)
   int affine;  // op == PBG_OP_LINEAR with a translation added to the product (operators.py:103-115, 272-293)
   float margin;
   SideCtx side[2];

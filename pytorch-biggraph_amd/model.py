@@ -15,8 +15,11 @@ autograd on these scores.
 training step takes its weight, ``forward`` returns its value as the reference's
 does.
 
-Not provided (outside the accelerated path): FeaturizedEmbedding,
-half precision.
+``half_precision`` (model.py:504-505: embeddings become float16 once prepared for the
+comparator; "GPU ONLY", config.py:496-498) is taken for the dot and cos comparators
+without bias and regularizer; the step refuses the other combinations.
+
+Not provided (outside the accelerated path): FeaturizedEmbedding.
 """
 from abc import ABC, abstractmethod
 from enum import Enum
@@ -285,8 +288,6 @@ class MultiRelationEmbedder(nn.Module):
         super().__init__()
         if regularizer is not None and not isinstance(regularizer, N3Regularizer):
             raise NotImplementedError("Only the N3 regularizer is supported")
-        if half_precision:
-            raise NotImplementedError("Half precision is not supported")
         if any(e.featurized for e in entities.values()):
             raise NotImplementedError("Featurized entities are not supported")
         self.default_dim = default_dim
@@ -311,7 +312,7 @@ class MultiRelationEmbedder(nn.Module):
                 self.EMB_PREFIX + entity: nn.Parameter(torch.zeros((schema.dimension or default_dim,)))
                 for entity, schema in entities.items()})
         self.max_norm: Optional[float] = max_norm
-        self.half_precision = False
+        self.half_precision = bool(half_precision)
         self.regularizer: Optional[AbstractRegularizer] = regularizer
         self._runners: Dict[tuple, native.StepRunner] = {}
 
@@ -379,7 +380,7 @@ class MultiRelationEmbedder(nn.Module):
             comparator=self.comparator.comparator_name,
             regularization_coef=float(self.regularizer.weight) if self.regularizer is not None else 0.0,
             max_norm=self.max_norm, bias=isinstance(self.comparator, BiasedComparator),
-            all_negs=bool(self.relations[relation_idx].all_negs), **training)
+            all_negs=bool(self.relations[relation_idx].all_negs), half_precision=self.half_precision, **training)
 
     def operator_tensors(self, relation_idx: int):
         """({name: tensor} of the rhs operator, of the lhs operator) in the

@@ -119,8 +119,10 @@ def bmm_nt(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def gemm(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, a_kmajor, b_kmajor,
-         alpha=1.0, beta=0.0) -> None:
-    check(_lib.lib().pbg_gemm_f32(_ptr(a), _ptr(b), _ptr(c), batch, m, n, k, lda, ldb, ldc, stride_a, stride_b,
+         alpha=1.0, beta=0.0, half=False) -> None:
+    """`half`: the operands hold float16 numbers; the product as torch.bmm makes it on Half tensors (pbg_gemm_f16)."""
+    fn = _lib.lib().pbg_gemm_f16 if half else _lib.lib().pbg_gemm_f32
+    check(fn(_ptr(a), _ptr(b), _ptr(c), batch, m, n, k, lda, ldb, ldc, stride_a, stride_b,
                                   stride_c, int(a_kmajor), int(b_kmajor), float(alpha), float(beta), _stream()))
 
 
@@ -215,6 +217,8 @@ class StepSpec:
     bias: bool = False  # config.bias: BiasedComparator around the comparator
     # RelationSchema.all_negs: one chunk, every entity of a side's type is a negative (model.py:648-650,582-618)
     all_negs: bool = False
+    # config.half_precision: embeddings are float16 numbers from comparator.prepare on (model.py:504-505)
+    half_precision: bool = False
 
     @property
     def chunk_size(self) -> int:
@@ -289,6 +293,7 @@ class StepRunner:
         d.max_norm = float(spec.max_norm) if spec.max_norm else 0.0
         d.bias = int(bool(spec.bias))
         d.all_negs = int(bool(spec.all_negs))
+        d.half_precision = int(bool(spec.half_precision))
         self.desc = d
         self.rhs_op = rhs_op or {}
         self.rhs_op_sum = rhs_op_sum or {}

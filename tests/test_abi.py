@@ -25,8 +25,8 @@ def test_header_symbols_are_exported(pbg):
 def test_struct_sizes_match_the_header(pbg):
     import ctypes
 
-    # 15 x 4-byte fields + one 4-byte field, then two int64: 16 * 4 + 16
-    assert ctypes.sizeof(pbg._lib.StepDesc) == 96
+    # 16 4-byte fields, two int64, five 4-byte fields and 4 bytes of padding: 16 * 4 + 16 + 5 * 4 + 4
+    assert ctypes.sizeof(pbg._lib.StepDesc) == 104
     # 22 pointers + workspace_bytes, then sample_uniform (4 + 4 padding) and uniform_seed
     assert ctypes.sizeof(pbg._lib.StepBuffers) == 30 * 8
     lib = pbg._lib.lib()

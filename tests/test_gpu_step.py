@@ -52,7 +52,8 @@ def to_runner(pbg, cfg, st, num_pos, workers):
         num_uniform_negs=cfg.num_uniform_negs, disable_lhs_negs=cfg.disable_lhs_negs,
         disable_rhs_negs=cfg.disable_rhs_negs, operator=cfg.operator, dynamic=cfg.dynamic,
         num_relations=cfg.num_relations, comparator=cfg.comparator, loss=cfg.loss, margin=cfg.margin, lr=cfg.lr,
-        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm, bias=cfg.bias, all_negs=cfg.all_negs)
+        relation_lr=cfg.relation_lr, regularization_coef=cfg.regularization_coef, max_norm=cfg.max_norm, bias=cfg.bias, all_negs=cfg.all_negs,
+        half_precision=cfg.half_precision)
     dev = lambda t: t.clone().to(DEV)
     w_l, g_l = dev(st.w_lhs), dev(st.g_lhs)
     w_r, g_r = (None, None) if st.shared else (dev(st.w_rhs), dev(st.g_rhs))

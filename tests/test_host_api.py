@@ -217,9 +217,10 @@ def test_model_argument_errors(pbg):
     ent = {"e": C.EntitySchema()}
     mk = lambda **kw: M.MultiRelationEmbedder(4, rel, ent, 2, 2, False, False, [None],
                                               [pbg.operators.TranslationOperator(4)], M.DotComparator(), **kw)
-    for kw in (dict(half_precision=True), dict(regularizer=object())):
-        with pytest.raises(NotImplementedError):
-            mk(**kw)
+    with pytest.raises(NotImplementedError):
+        mk(regularizer=object())
+    # model.py:444: kept, and handed on to every step the model describes
+    assert mk(half_precision=True).step_spec(0, 3, 4).half_precision and not mk().step_spec(0, 3, 4).half_precision
     capped = mk(max_norm=1.0)  # model.py:443-451: handed on to every embedding module
     capped.set_embeddings("e", pbg.types.Side.LHS, torch.nn.Parameter(torch.zeros(5, 4)))
     assert capped.lhs_embs["emb_e"].max_norm == 1.0 and capped.step_spec(0, 3, 4).max_norm == 1.0
