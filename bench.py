@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
+FP16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16, what --half-precision's products are priced against
 # HBM bytes per launch of (workload, kernel, workers), from the rocprofv3 FETCH_SIZE /
 # WRITE_SIZE runs summarised in profiles/train_step_pmc_traffic.md (not measured live);
 # any other combination reports null.
@@ -313,6 +314,9 @@ def main():
                     help="batches in flight per call (HOGWILD workers); 64 batches of cfg1 are 1280 chunks = 5 per compute unit")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="length of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-sequential", action="store_true", help="skip the workers=1 measurement")
+    ap.add_argument("--half-precision", action="store_true",
+                    help="the reference's config.half_precision (dot / cos workloads): float16 embeddings from "
+                         "comparator.prepare on, products on the fp16 matrix instructions; never the default line")
     ap.add_argument("--standalone-kernels", action="store_true",
                     help="only measure the stand-alone gather and sparse RowAdagrad kernels on large tables")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -342,6 +346,7 @@ def main():
     # The CPU baseline runs first, before this process opens the GPU: its worker
     # processes each touch the HIP runtime once (autograd asks it for a device
     # count), and the box allows 16 processes on the card at a time.
+    # (the CPU baseline is the reference's CPU path, which has no half precision: fp32 beside either line)
     cpu = cpu_baseline(w, args.cpu_seconds) if args.cpu_seconds > 0 else None
 
     import __graft_entry__
@@ -356,7 +361,8 @@ def main():
         spec = pkg.StepSpec(dim=d, batch_size=b, num_workers=workers, num_batch_negs=w["batch_negs"],
                             num_uniform_negs=w["uniform_negs"], operator=w["operator"], dynamic=w["dynamic"],
                             num_relations=w["relations"], comparator=w["comparator"], loss=w["loss"], margin=0.1,
-                            lr=0.1, regularization_coef=w.get("regularization_coef", 0.0))
+                            lr=0.1, regularization_coef=w.get("regularization_coef", 0.0),
+                            half_precision=args.half_precision)
         ws = [t.clone() for t in tables]
         gs = [torch.zeros(t.shape[0], device=dev) for t in tables]
         rhs_op, rhs_sum = {}, {}
@@ -512,7 +518,7 @@ def main():
     if bound == "hbm":
         achieved, peak, unit = units / seconds / 1e9, HBM_PEAK_GBS, "GB/s"
     else:
-        achieved, peak, unit = units / seconds / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        achieved, peak, unit = units / seconds / 1e12, (FP16_MFMA_PEAK_TFLOPS if args.half_precision else FP32_MFMA_PEAK_TFLOPS), "TFLOP/s"
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
         "frac": achieved / peak, "traffic": TRAFFIC.get((args.workload, dominant, workers)), "launches_in_stage": launches,
@@ -530,8 +536,8 @@ def main():
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X",
         "value": eps, "unit": "edges/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['desc']}", "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
+        "dtype": "f16 products, f32 sums (config.half_precision)" if args.half_precision else "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}" + (", half_precision" if args.half_precision else ""), "batch_size": b, "negatives_per_edge_per_side": spec.chunk_size * (w['batch_negs'] > 0) + w["uniform_negs"],
                    "hogwild_workers": workers, "step": f"one pbg_train_step call of {workers} batches", "route": route,
                    "timed_calls": steps, "timed_batches": steps * workers, "timed_edges": steps * workers * b,
                    "timed_wall_seconds": wall_s, "preheat_ms_on_scratch_state": args.preheat_ms, "uniform_negative_draw": "inside the step (Philox4x32-10, one seed per call)",

@@ -35,7 +35,10 @@ RowAdagrad by its reduction to torch.optim.Adagrad on constant-row gradients
 and on dim 1, and by pre-summed duplicates; AsyncAdagrad by torch.optim.Adagrad;
 reverse_permutation / shuffle / sub_bucket by the reference's own util.cpp
 compiled into oracle/_ref (when built) and by argsort / index_copy / stable
-sort identities.  randperm's bit pattern is not portable (it depends on the
+sort identities; half_precision (no vector in the reference's tests, and its cast
+only happens on a CUDA device) by the fp32 path on inputs whose intermediates are
+all float16 numbers and by a numpy float16 restatement of every rounding point
+(tests/test_oracle_half.py).  randperm's bit pattern is not portable (it depends on the
 thread count): only its contract (a uniform random permutation) is checked,
 so its bits are "parity unpinned" by design.
 """
