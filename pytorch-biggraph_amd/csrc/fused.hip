@@ -36,7 +36,9 @@ constexpr int kFusedSide = kFusedIds / 2;  // ... per side
 // with the matrix instructions of the compute waves for the same issue slots (the
 // fp32 matrix products run on the vector ALUs), so the per-column work is kept
 // to the loss's own arithmetic.
-template <int CMP, int LOSS, int kCols>
+// HALF (config.half_precision): dLoss/dscore goes back through the scores' cast to fp32 (model.py:827-829)
+// and is written as the float16 number that makes of it.
+template <int CMP, int LOSS, int kCols, bool HALF>
 __device__ __forceinline__ void fused_row_loss(float* lds, int row_at, int bn_at, float a2, float margin, float inv_nn, int ne,
                                                float pos, float w, int qd, float* loss_w, float* dpos_out, int* viol_out,
                                                float* rowsum_out) {
@@ -83,7 +85,7 @@ __device__ __forceinline__ void fused_row_loss(float* lds, int row_at, int bn_at
         rowsum += dq;
         g = -2.0f * dq;
       }
-      lds[at + 8 * e] = g;
+      lds[at + 8 * e] = HALF ? half_round(g) : g;
     }
     if (LOSS == PBG_LOSS_RANKING) dpos -= gsum;
   } else {
@@ -129,7 +131,7 @@ __device__ __forceinline__ void fused_row_loss(float* lds, int row_at, int bn_at
         rowsum += dq;
         g = -2.0f * dq;
       }
-      lds[at + 8 * e] = g;
+      lds[at + 8 * e] = HALF ? half_round(g) : g;
     }
   }
   *loss_w = oct_sum(loss_acc) * w;
@@ -230,7 +232,7 @@ __device__ __forceinline__ void fused_issue_rows(const StepCtx& c, const FusedGe
 // Only columns below D are written (the pad columns behind them were zeroed once,
 // when the kernel started).  `pads`: the chunk has padded positives (a partial last
 // chunk), whose rows are zeros.
-template <int CMP, int S>
+template <int CMP, int S, bool HALF>
 __device__ __forceinline__ void fused_store_side(const StepCtx& c, const FusedGeom& g, float* lds, int lwave, int lane,
                                                  const float4* v, const int* idv, const FusedRowExtras& x, bool pads) {
   const int half = lane >> 5, c4 = (lane & 31) << 2;
@@ -263,6 +265,9 @@ __device__ __forceinline__ void fused_store_side(const StepCtx& c, const FusedGe
       y.x *= inv; y.y *= inv; y.z *= inv; y.w *= inv;
       if ((lane & 31) == 31) lds[(S ? g.sq1 : g.sq0) + j] = inv;
     }
+    if (HALF) {  // embs.half() (model.py:504-505)
+      y.x = half_round(y.x); y.y = half_round(y.y); y.z = half_round(y.z); y.w = half_round(y.w);
+    }
     if (pads && idv[S * (kFusedRounds / 2) + u] < 0) y = make_float4(0.f, 0.f, 0.f, 0.f);
     if (col_ok) *reinterpret_cast<float4*>(&lds[at]) = y;
     if (CMP == PBG_CMP_L2) {
@@ -285,15 +290,20 @@ struct FusedOut {
 };
 
 // This lane's share of <own operand row, gradient row> over the columns it holds.
+template <bool HALF>
 __device__ __forceinline__ void fused_self_dot(const float* lds, int self_at, int col, int cols_left, float4 v, float* acc) {
   if (col >= cols_left) return;
+  if (HALF) v = make_float4(half_round(v.x), half_round(v.y), half_round(v.z), half_round(v.w));
   const float4 self = *reinterpret_cast<const float4*>(&lds[self_at + col]);
   *acc += (self.x * v.x + self.y * v.y) + (self.z * v.z + self.w * v.w);
 }
 
-template <int CMP>
+// HALF: the product is the gradient of a Half tensor, a float16 number; what follows (the cast's backward,
+// prepare's, the operator's) is fp32.
+template <int CMP, bool HALF>
 __device__ __forceinline__ void fused_emit(const float* lds, const FusedOut& o, int col, int cols_left, float4 v) {
   if (col >= cols_left) return;  // past D (a multiple of 4)
+  if (HALF) v = make_float4(half_round(v.x), half_round(v.y), half_round(v.z), half_round(v.w));
   constexpr bool L2 = CMP == PBG_CMP_L2;
   if (CMP == PBG_CMP_COS) {
     const float4 self = *reinterpret_cast<const float4*>(&lds[o.self_at + col]);
@@ -323,7 +333,7 @@ __device__ __forceinline__ void fused_emit(const float* lds, const FusedOut& o, 
 // other side, columns = side s's negatives; this wave's row tile rt and NCT column
 // tiles from ct0 on.  dot: the positive score is the diagonal (the i-th batch
 // negative is the i-th positive's own partner row, model.py:177).
-template <int NCT, bool L2>
+template <int NCT, bool L2, bool HALF>
 __device__ __forceinline__ void fused_scores(float* lds, const FusedGeom& g, int s, int rt, int ct0, int lane, int pos_at,
                                              bool write_pos) {
   if (rt * 16 >= g.P || ct0 * 16 >= g.N) return;
@@ -337,7 +347,7 @@ __device__ __forceinline__ void fused_scores(float* lds, const FusedGeom& g, int
   const int a_at = (s ? g.xn0 : g.xn1) + ar * g.ldx;
   const int b_at = (s ? g.xn1 : g.xn0) + (ct0 * 16 + (lane & 15)) * g.ldx;  // column tile ct: 16 rows further down
   const int ksteps = (g.D + 3) >> 2;
-  mfma_sweep_k16<NCT>(lds, a_at, b_at, 16 * g.ldx, ksteps >> 2, ksteps & 3, lane >> 4, acc);
+  mfma_sweep_k16<NCT, HALF>(lds, a_at, b_at, 16 * g.ldx, ksteps >> 2, ksteps & 3, lane >> 4, acc);
   const int row = rt * 16 + (lane & 15);
   if (row >= g.P) return;
   const int at = (s ? g.sc1 : g.sc0) + row * g.lds + ct0 * 16 + 4 * (lane >> 4);
@@ -345,10 +355,14 @@ __device__ __forceinline__ void fused_scores(float* lds, const FusedGeom& g, int
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) {
     const int col = (ct0 + ct) * 16 + 4 * (lane >> 4);
+    // (HALF: a score is the float16 rounding of the fp32 sum, torch.bmm on Half tensors; the positive
+    // score below is the fp32 sum itself, model.py:177)
+    const float s0 = HALF ? half_round(acc[ct][0]) : acc[ct][0], s1 = HALF ? half_round(acc[ct][1]) : acc[ct][1];
+    const float s2 = HALF ? half_round(acc[ct][2]) : acc[ct][2], s3 = HALF ? half_round(acc[ct][3]) : acc[ct][3];
     if (col < n8)  // columns from n8 on stay zero
       *reinterpret_cast<float4*>(&lds[at + ct * 16]) =
-          make_float4(col < g.N ? acc[ct][0] : -INFINITY, col + 1 < g.N ? acc[ct][1] : -INFINITY,
-                      col + 2 < g.N ? acc[ct][2] : -INFINITY, col + 3 < g.N ? acc[ct][3] : -INFINITY);
+          make_float4(col < g.N ? s0 : -INFINITY, col + 1 < g.N ? s1 : -INFINITY, col + 2 < g.N ? s2 : -INFINITY,
+                      col + 3 < g.N ? s3 : -INFINITY);
     if (!L2 && write_pos && row >= col && row < col + 4) {
       const int r = row - col;
       lds[pos_at + row] = r == 0 ? acc[ct][0] : (r == 1 ? acc[ct][1] : (r == 2 ? acc[ct][2] : acc[ct][3]));
@@ -377,7 +391,7 @@ __device__ __forceinline__ void fused_scores(float* lds, const FusedGeom& g, int
 //
 // LD != 0: both LDS row strides (operand rows, score rows) equal LD, known at compile
 // time, so that the products' LDS addresses are one register plus immediates.
-template <int T, int CMP, int LOSS, int LD>
+template <int T, int CMP, int LOSS, int LD, bool HALF>
 __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
   // All LDS accesses index `lds` directly (no pointer tables), so that they
   // compile to ds_read / ds_write rather than flat accesses.  Everything indexed
@@ -429,8 +443,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       int ln = lane, t = tid;
       asm volatile("" : "+v"(ln), "+v"(t));
       // ---- step 7 of the previous chunk ----
-      fused_store_side<CMP, 0>(c, g, lds, wave, ln, v, idv, extras, pads);
-      if (!side1_stored) fused_store_side<CMP, 1>(c, g, lds, wave, ln, v, idv, extras, pads);
+      fused_store_side<CMP, 0, HALF>(c, g, lds, wave, ln, v, idv, extras, pads);
+      if (!side1_stored) fused_store_side<CMP, 1, HALF>(c, g, lds, wave, ln, v, idv, extras, pads);
       lds_barrier();  // (a) operand rows of chunk kc in LDS
 
       const int kn = kc + gridDim.x;
@@ -484,7 +498,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
             if (qd == (i & 7)) lds[row_at + i] = masked;
             if (valid < P)
               for (int j = valid + ((qd - valid) & 7); j < P; j += 8) lds[row_at + j] = masked;
-            fused_row_loss<CMP, LOSS, kLossCols>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f,
+            fused_row_loss<CMP, LOSS, kLossCols, HALF>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f,
                                                    c.margin, 1.0f / (float)N, (N + 7) >> 3, lds[f.pos + i], w_edge, qd, &loss_w,
                                                    &dpos_s, &viol, &rowsum);
           }
@@ -538,6 +552,9 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
           // of steps 5 and 6 then carry dpos_i * rhs_i into the lhs gradient and
           // dpos_i * lhs_i into the rhs one.
           if (!l2 && i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
+          // (HALF: the folded block is an operand of the fp16 products; the sum of its two or three terms is
+          // rounded here, one rounding where autograd's float16 additions make two)
+          if (HALF) sum = half_round(sum);
           lds[sc1 + i * lds_ + j] = sum;
           lds[sc0 + j * lds_ + i] = sum;
           i += di;
@@ -559,7 +576,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       // ---- step 6 ----
       side1_stored = CMP == PBG_CMP_DOT && more;  // (l2 and cos still read the rows' own values while writing gradients out)
       pads = c.last < P && cc_next == C - 1;  // of the chunk whose rows are in the registers now
-      if (side1_stored) fused_store_side<CMP, 1>(c, g, lds, wave, ln, v, idv, extras, pads);
+      if (side1_stored) fused_store_side<CMP, 1, HALF>(c, g, lds, wave, ln, v, idv, extras, pads);
       if (cosn) lds_barrier();  // the exchange of step 6
       lds_barrier();  // (g) the products have let go of all operand rows
     }
@@ -587,8 +604,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 
     // ---- steps 1 and 2: the score blocks ----
     for (int s = 0; s < 2; ++s) {
-      if (grp == 0) fused_scores<T0, l2>(lds, g, s, rt, 0, lane_, f.pos, s == 0);
-      else if (T1 > 0) fused_scores<(T1 > 0 ? T1 : 1), l2>(lds, g, s, rt, T0, lane_, f.pos, s == 0);
+      if (grp == 0) fused_scores<T0, l2, HALF>(lds, g, s, rt, 0, lane_, f.pos, s == 0);
+      else if (T1 > 0) fused_scores<(T1 > 0 ? T1 : 1), l2, HALF>(lds, g, s, rt, T0, lane_, f.pos, s == 0);
       lds_barrier();  // (b), (c)
     }
 
@@ -605,8 +622,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
       if (live) {
         const int au = min(rt * 16 + m16, U - 1);
         const int a_at = dsn + P + au, b_at = bx + ct0 * 16, pk = (P + 3) >> 2;
-        if (grp == 0) asum = sweep_a_cols<T0>(lds, a_at, lds_, b_at, ldx, kq, m16, pk, acc);
-        else if (T1 > 0) asum = sweep_a_cols<(T1 > 0 ? T1 : 1)>(lds, a_at, lds_, b_at, ldx, kq, m16, pk, acc);
+        if (grp == 0) asum = sweep_a_cols<T0, HALF>(lds, a_at, lds_, b_at, ldx, kq, m16, pk, acc);
+        else if (T1 > 0) asum = sweep_a_cols<(T1 > 0 ? T1 : 1), HALF>(lds, a_at, lds_, b_at, ldx, kq, m16, pk, acc);
       }
       if (l2 && m == 1) lds_barrier();  // (e') of the helpers
       const int u = rt * 16 + m16;
@@ -615,8 +632,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         const int self_at = xs + (P + min(u, U - 1)) * ldx + ct0 * 16, left = D - ct0 * 16;
         float part = 0.f;
         if (live) {
-          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
-          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot<HALF>(lds, self_at, col, left, v4, &part); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot<HALF>(lds, self_at, col, left, v4, &part); });
         }
         part += __shfl_xor(part, 16);
         part += __shfl_xor(part, 32);
@@ -644,8 +661,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
           o.pcoef = lds[(m ? g.sq1 : g.sq0) + P + u];
         }
         const int left = D - ct0 * 16;
-        if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
-        else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
+        if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP, HALF>(lds, o, col, left, v4); });
+        else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP, HALF>(lds, o, col, left, v4); });
       }
       lds_barrier();  // (d), (e)
     }
@@ -667,16 +684,16 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
         const int ar = min(rt * 16 + m16, P - 1);
         const int ksteps = (N + 3) >> 2;
         const int a_at = dsa + ar * lds_, b_at = bx + ct0 * 16;
-        if (grp == 0) sweep_a_rows<T0>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
-        else if (T1 > 0) sweep_a_rows<(T1 > 0 ? T1 : 1)>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
+        if (grp == 0) sweep_a_rows<T0, HALF>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
+        else if (T1 > 0) sweep_a_rows<(T1 > 0 ? T1 : 1), HALF>(lds, a_at, b_at, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
       }
       float row_dot_ = 0.f;
       if (cosn) {
         const int self_at = xs + min(rt * 16 + m16, P - 1) * ldx + ct0 * 16, left = D - ct0 * 16;
         float part = 0.f;
         if (live) {
-          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
-          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot(lds, self_at, col, left, v4, &part); });
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_self_dot<HALF>(lds, self_at, col, left, v4, &part); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_self_dot<HALF>(lds, self_at, col, left, v4, &part); });
         }
         part += __shfl_xor(part, 16);
         part += __shfl_xor(part, 32);
@@ -706,8 +723,8 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
             o.pcoef = lds[(m ? g.sq1 : g.sq0) + i];
           }
           const int left = D - ct0 * 16;
-          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
-          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP>(lds, o, col, left, v4); });
+          if (grp == 0) for_each_out<T0>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP, HALF>(lds, o, col, left, v4); });
+          else if (T1 > 0) for_each_out<(T1 > 0 ? T1 : 1)>(acc, kq, [&](int col, float4 v4) { fused_emit<CMP, HALF>(lds, o, col, left, v4); });
         }
       }
       lds_barrier();  // (f), (g)
@@ -739,34 +756,39 @@ __global__ __launch_bounds__(kFusedIds) void fused_ids_kernel(StepCtx c) {
   c.fused_rowid[(int64_t)kc * kFusedIds + t] = real ? (int)id : -1;
 }
 
-// One instantiation of the fused kernel per (tile count, comparator, loss); each
+// One instantiation of the fused kernel per (tile count, comparator, loss, half precision); each
 // raises its dynamic LDS limit the first time it needs more than it was given.
-template <int T, int CMP, int LOSS, int LD>
+template <int T, int CMP, int LOSS, int LD, bool HALF>
 int launch_fused_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   static LdsLimit limit;
-  const int rc = reserve_lds((const void*)fused_chunk_kernel<T, CMP, LOSS, LD>, &limit, lds_bytes);
+  const int rc = reserve_lds((const void*)fused_chunk_kernel<T, CMP, LOSS, LD, HALF>, &limit, lds_bytes);
   if (rc != PBG_OK) return rc;
   const int chunks = c.K * c.C;
-  hipLaunchKernelGGL((fused_chunk_kernel<T, CMP, LOSS, LD>), dim3((unsigned)blocks), dim3(2 * kFusedThreads), lds_bytes, s,
-                     c, fl, chunks);
+  hipLaunchKernelGGL((fused_chunk_kernel<T, CMP, LOSS, LD, HALF>), dim3((unsigned)blocks), dim3(2 * kFusedThreads), lds_bytes,
+                     s, c, fl, chunks);
   return PBG_OK;
 }
 
-template <int T, int CMP, int LD>
+template <int T, int CMP, int LD, bool HALF>
 int launch_fused_loss(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   switch (c.loss) {
-    case PBG_LOSS_RANKING: return launch_fused_as<T, CMP, PBG_LOSS_RANKING, LD>(c, fl, lds_bytes, s, blocks);
-    case PBG_LOSS_LOGISTIC: return launch_fused_as<T, CMP, PBG_LOSS_LOGISTIC, LD>(c, fl, lds_bytes, s, blocks);
-    default: return launch_fused_as<T, CMP, PBG_LOSS_SOFTMAX, LD>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_RANKING: return launch_fused_as<T, CMP, PBG_LOSS_RANKING, LD, HALF>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_fused_as<T, CMP, PBG_LOSS_LOGISTIC, LD, HALF>(c, fl, lds_bytes, s, blocks);
+    default: return launch_fused_as<T, CMP, PBG_LOSS_SOFTMAX, LD, HALF>(c, fl, lds_bytes, s, blocks);
   }
 }
 
 template <int T, int LD>
 int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
+  if (c.half) {  // (dot and cos only: the step's validation has refused the rest)
+    if (c.cmp == PBG_CMP_COS) return launch_fused_loss<T, PBG_CMP_COS, LD, true>(c, fl, lds_bytes, s, blocks);
+    if (c.cmp == PBG_CMP_DOT) return launch_fused_loss<T, PBG_CMP_DOT, LD, true>(c, fl, lds_bytes, s, blocks);
+    return fail(PBG_ERR_UNSUPPORTED, "step: half_precision on the fused route is built for dot and cos");
+  }
   switch (c.cmp) {
-    case PBG_CMP_L2: return launch_fused_loss<T, PBG_CMP_L2, LD>(c, fl, lds_bytes, s, blocks);
-    case PBG_CMP_COS: return launch_fused_loss<T, PBG_CMP_COS, LD>(c, fl, lds_bytes, s, blocks);
-    default: return launch_fused_loss<T, PBG_CMP_DOT, LD>(c, fl, lds_bytes, s, blocks);
+    case PBG_CMP_L2: return launch_fused_loss<T, PBG_CMP_L2, LD, false>(c, fl, lds_bytes, s, blocks);
+    case PBG_CMP_COS: return launch_fused_loss<T, PBG_CMP_COS, LD, false>(c, fl, lds_bytes, s, blocks);
+    default: return launch_fused_loss<T, PBG_CMP_DOT, LD, false>(c, fl, lds_bytes, s, blocks);
   }
 }
 

@@ -1,6 +1,12 @@
 // fp32 matrix products of 16 x 16 tiles out of LDS (v_mfma_f32_16x16x4_f32), the
 // reductions over 8 adjacent lanes and the LDS-only workgroup barrier shared by
 // the kernels that keep a chunk in LDS.
+//
+// HALF variants of the products (config.half_precision: every operand value is a
+// float16 number held as fp32): the four values of k that a lane feeds to four
+// fp32 steps go, packed to fp16 (exactly), into ONE v_mfma_f32_16x16x16_f16 --
+// lane group q holds four of the instruction's 16 k in both operands, and which k
+// a slot stands for is free as long as both operands agree.  Sums stay fp32.
 #pragma once
 
 #include "pbg_internal.h"
@@ -9,6 +15,24 @@
 namespace pbg {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef __fp16 fp16x2v __attribute__((ext_vector_type(2)));
+
+// Four float16 numbers held as fp32, packed (the conversion is exact for such values).
+__device__ __forceinline__ half4v pack_half4(float x, float y, float z, float w) {
+  union {
+    struct { fp16x2v lo, hi; } p;
+    half4v h;
+  } u;
+  u.p.lo = __builtin_amdgcn_cvt_pkrtz(x, y);
+  u.p.hi = __builtin_amdgcn_cvt_pkrtz(z, w);
+  return u.h;
+}
+// One k per lane group (a single fp32 step's operands) as an fp16 instruction: the other three slots are zero.
+__device__ __forceinline__ float4v mfma_step(float b, float a, float4v acc, bool half) {
+  if (half) return __builtin_amdgcn_mfma_f32_16x16x16f16(pack_half4(b, 0.f, 0.f, 0.f), pack_half4(a, 0.f, 0.f, 0.f), acc, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(b, a, acc, 0, 0, 0);
+}
 
 // reductions over 8 adjacent lanes, result in every lane of the group
 __device__ __forceinline__ float oct_sum(float v) {
@@ -103,16 +127,24 @@ struct RowOperands {
 #pragma unroll
     for (int r = 0; r < 4; ++r) load_b<NCT>(lds, b_at + r * ldb, m, b[r]);
   }
+  template <bool HALF>
   __device__ __forceinline__ void mma(float4v* acc) const {
-    const float av[4] = {a.x, a.y, a.z, a.w};
+    if constexpr (HALF) {
+      const half4v ha = pack_half4(a.x, a.y, a.z, a.w);
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+      for (int t = 0; t < NCT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack_half4(b[0][t], b[1][t], b[2][t], b[3][t]), ha, acc[t], 0, 0, 0);
+    } else {
+      const float av[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
-      for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[r][t], av[r], acc[t], 0, 0, 0);
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[r][t], av[r], acc[t], 0, 0, 0);
+    }
   }
 };
 
-template <int NCT>
+template <int NCT, bool HALF = false>
 __device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_at, int ldb, int kq, int m, int groups,
                                              int rest, float4v* acc) {
   a_at += 4 * kq;
@@ -123,17 +155,17 @@ __device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_a
   for (; gk + 2 <= groups; gk += 2) {
     y.load(lds, a_at + 16, b_at + 16 * ldb, ldb, m);
     __builtin_amdgcn_sched_barrier(0);
-    x.mma(acc);
+    x.template mma<HALF>(acc);
     __builtin_amdgcn_sched_barrier(0);
     a_at += 32;
     b_at += 32 * ldb;
     x.load(lds, a_at, b_at, ldb, m);
     __builtin_amdgcn_sched_barrier(0);
-    y.mma(acc);
+    y.template mma<HALF>(acc);
     __builtin_amdgcn_sched_barrier(0);
   }
   if (gk < groups) {
-    x.mma(acc);
+    x.template mma<HALF>(acc);
     a_at += 16;
     b_at += 16 * ldb;
   }
@@ -144,7 +176,7 @@ __device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_a
     float b1[NCT];
     load_b<NCT>(lds, b_at, m, b1);
 #pragma unroll
-    for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b1[t], a1, acc[t], 0, 0, 0);
+    for (int t = 0; t < NCT; ++t) acc[t] = mfma_step(b1[t], a1, acc[t], HALF);
     a_at += 4;
     b_at += 4 * ldb;
   }
@@ -154,11 +186,41 @@ __device__ __forceinline__ void sweep_a_rows(const float* lds, int a_at, int b_a
 // uniform negatives' gradient): the lane's A element of step ks is at a_at +
 // (4 ks + kq) * lda.  Returns the sum of the A elements the lane has fed (its
 // share of a column sum of the score block).  Reads up to two steps past the end.
-template <int NCT>
+template <int NCT, bool HALF = false>
 __device__ __forceinline__ float sweep_a_cols(const float* lds, int a_at, int lda, int b_at, int ldb, int kq, int m,
                                               int ksteps, float4v* acc) {
   a_at += kq * lda;
   b_at += kq * ldb;
+  if constexpr (HALF) {  // four steps' operands per instruction; nothing is read past the end
+    float asum = 0.f;
+    int ks = 0;
+    for (; ks + 4 <= ksteps; ks += 4) {
+      float a[4], b[4][NCT];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        a[r] = lds[a_at + 4 * r * lda];
+        load_b<NCT>(lds, b_at + 4 * r * ldb, m, b[r]);
+      }
+      const half4v ha = pack_half4(a[0], a[1], a[2], a[3]);
+#pragma unroll
+      for (int t = 0; t < NCT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack_half4(b[0][t], b[1][t], b[2][t], b[3][t]), ha, acc[t], 0, 0, 0);
+      asum += (a[0] + a[1]) + (a[2] + a[3]);
+      a_at += 16 * lda;
+      b_at += 16 * ldb;
+    }
+    for (; ks < ksteps; ++ks) {
+      const float a1 = lds[a_at];
+      float b1[NCT];
+      load_b<NCT>(lds, b_at, m, b1);
+#pragma unroll
+      for (int t = 0; t < NCT; ++t) acc[t] = mfma_step(b1[t], a1, acc[t], true);
+      asum += a1;
+      a_at += 4 * lda;
+      b_at += 4 * ldb;
+    }
+    return asum;
+  }
   float ax = lds[a_at], ay, asum = 0.f;
   float bx[NCT], by[NCT];
   load_b<NCT>(lds, b_at, m, bx);
@@ -205,19 +267,27 @@ struct K16Operands {
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) b[ct] = *reinterpret_cast<const float4*>(&lds[b_at + ct * b_tile]);
   }
+  template <bool HALF>
   __device__ __forceinline__ void mma(float4v* acc) const {
+    if constexpr (HALF) {
+      const half4v ha = pack_half4(a.x, a.y, a.z, a.w);
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].x, a.x, acc[ct], 0, 0, 0);
+      for (int ct = 0; ct < T; ++ct)
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack_half4(b[ct].x, b[ct].y, b[ct].z, b[ct].w), ha, acc[ct], 0, 0, 0);
+    } else {
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].y, a.y, acc[ct], 0, 0, 0);
+      for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].x, a.x, acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].z, a.z, acc[ct], 0, 0, 0);
+      for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].y, a.y, acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].w, a.w, acc[ct], 0, 0, 0);
+      for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].z, a.z, acc[ct], 0, 0, 0);
+#pragma unroll
+      for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[ct].w, a.w, acc[ct], 0, 0, 0);
+    }
   }
 };
 
-template <int T>
+template <int T, bool HALF = false>
 __device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b_at, int b_tile, int groups, int rest,
                                                int kq, float4v* acc) {
   a_at += 4 * kq;
@@ -232,17 +302,17 @@ __device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b
   for (; gk + 2 <= groups; gk += 2) {
     y.load(lds, a_at + 16, b_at + 16, b_tile);
     __builtin_amdgcn_sched_barrier(0);
-    x.mma(acc);
+    x.template mma<HALF>(acc);
     __builtin_amdgcn_sched_barrier(0);
     a_at += 32;
     b_at += 32;
     x.load(lds, a_at, b_at, b_tile);
     __builtin_amdgcn_sched_barrier(0);
-    y.mma(acc);
+    y.template mma<HALF>(acc);
     __builtin_amdgcn_sched_barrier(0);
   }
   if (gk < groups) {
-    x.mma(acc);
+    x.template mma<HALF>(acc);
     a_at += 16;
     b_at += 16;
   }
@@ -254,7 +324,7 @@ __device__ __forceinline__ void mfma_sweep_k16(const float* lds, int a_at, int b
 #pragma unroll
     for (int ct = 0; ct < T; ++ct) b1[ct] = lds[b_at + ct * b_tile];
 #pragma unroll
-    for (int ct = 0; ct < T; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(b1[ct], a1, acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < T; ++ct) acc[ct] = mfma_step(b1[ct], a1, acc[ct], HALF);
     a_at += 4;
     b_at += 4;
   }

@@ -1635,8 +1635,8 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   plan->sort_temp = take(sort_temp_bytes(npairs), 1);
   plan->nvh = (int)ceil_div((D + 1) / 2, kWave);
   // (the regularizer's terms live in the staged kernels only)
-  // (half_precision: the staged route only, whose products then run on the fp16 matrix instructions)
-  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && !c.half && getenv("PBG_DISABLE_FUSED") == nullptr;
+  // (half_precision: the fused and the staged route, whose products then run on the fp16 matrix instructions)
+  plan->fused = fused_layout(c, &plan->fl) && c.reg_coef == 0.f && !c.bias && getenv("PBG_DISABLE_FUSED") == nullptr;
   if (plan->fused) {  // the fused kernel writes every gradient row and every dz itself
     c.side[0].uni_direct = c.side[1].uni_direct = 0;
     c.side[0].uni_dz_direct = c.side[1].uni_dz_direct = 0;

@@ -82,6 +82,18 @@ HALF_CASES += [
     dict(operator="translation", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=4,
          num_uniform_negs=3, num_pos=9, dim=8, disable_lhs_negs=True),
 ]
+# the fused route's shapes (dims that are multiples of 4, batch + uniform negatives on both sides): full and partial
+# chunks, dims with and without a remainder of the 16-wide k groups, every tile count
+for op, cmp_, loss in itertools.product(("none", "diagonal", "translation"), ("dot", "cos"), ostep.LOSS_NAMES):
+    HALF_CASES.append(dict(operator=op, comparator=cmp_, loss=loss, dynamic=False, num_batch_negs=50, num_uniform_negs=50,
+                           num_pos=130, dim=100))
+HALF_CASES += [
+    dict(operator="none", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=64, num_uniform_negs=64, num_pos=200, dim=128),
+    dict(operator="none", comparator="cos", loss="softmax", dynamic=False, num_batch_negs=37, num_uniform_negs=20, num_pos=100, dim=64),
+    dict(operator="translation", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=16, num_uniform_negs=9, num_pos=40, dim=20),
+    dict(operator="diagonal", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=3, num_pos=75, dim=36),
+    dict(operator="none", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=13, num_uniform_negs=64, num_pos=30, dim=112),
+]
 
 
 def close16(got, want, what, units=2.0, floor=None):
@@ -110,17 +122,20 @@ def test_half_precision_step(pbg, case, workers):
     st, batches = make_inputs(cfg, num_pos, n_ent, workers, seed=num_pos + dim, shared=(dim % 2 == 0))
     before = [t.clone() for t in (st.w_lhs, st.w_rhs)]
     runner = to_runner(pbg, cfg, st, num_pos, workers)
-    assert runner.route == "staged"
+    assert runner.route in ("staged", "fused")  # (the streaming route does not take half_precision)
     fwd = runner.forward(*pack(cfg, batches))
     torch.cuda.synchronize()
     for k, b in enumerate(batches):
         sc = ostep.forward_backward(cfg, st, *b, keep_scores=True)[0].scores
         got = tuple(t[k].cpu() for t in fwd)
-        # positive scores are fp32 sums over float16 rows (model.py:177): not float16 numbers themselves, and far
-        # closer than float16's 2^-11 (what is left are the few coordinates that the two fp32 evaluations of
-        # prepare() put on different sides of a float16 rounding boundary)
-        pos_err = float((got[0] - sc.lhs_pos).abs().max())
-        assert pos_err <= 5e-5 * float(sc.lhs_pos.abs().max()) + 1e-7, ("positive scores", pos_err)
+        # Positive scores are fp32 sums over float16 rows (model.py:177), not float16 numbers: on average they agree
+        # far better than float16's 2^-12 (a score rounded to float16 would be off by a quarter unit on average).
+        # The largest difference may reach a unit: a coordinate that the two fp32 evaluations of prepare() put on
+        # different sides of a float16 rounding boundary moves its row's score.
+        pos_scale = float(sc.lhs_pos.abs().max())
+        pos_diff = (got[0] - sc.lhs_pos).abs()
+        assert float(pos_diff.mean()) <= 2e-5 * pos_scale + 1e-7, ("positive scores, mean", float(pos_diff.mean()))
+        assert float(pos_diff.max()) <= EPS16 * pos_scale + 1e-7, ("positive scores, max", float(pos_diff.max()))
         for g, w, name in ((got[2], sc.lhs_neg, "lhs_neg"), (got[3], sc.rhs_neg, "rhs_neg")):
             masked = w == -1e9
             assert torch.equal(g == -1e9, masked), name
@@ -138,7 +153,10 @@ def test_half_precision_step(pbg, case, workers):
     # bound is two units of the LARGEST step, for every entry.
     for got, want, was, name in ((runner.w_lhs, st.w_lhs, before[0], "w_lhs"), (runner.w_rhs, st.w_rhs, before[1], "w_rhs")):
         step = want - was
-        close16(got.cpu() - was, step, "step of " + name, units=2.0, floor=float(step.abs().max()))
+        # (cos: prepare's backward takes the row's own direction out of the float16 gradient; what is left is
+        # smaller than the gradient whose rounding noise it keeps)
+        close16(got.cpu() - was, step, "step of " + name, units=8.0 if cfg.comparator == "cos" else 2.0,
+                floor=float(step.abs().max()))
     close16(runner.g_lhs, st.g_lhs, "g_lhs", units=8.0)
     # Operator parameters: AsyncAdagrad's first steps are lr * g / |g|, so an entry whose gradient is float16
     # rounding noise around zero moves by a full step in either direction; a handful of such entries per matrix
