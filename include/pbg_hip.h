@@ -178,7 +178,7 @@ typedef struct pbg_step_desc {
                              * are float16 products and the prepared embeddings' gradients float16 tensors; positive
                              * scores, losses, operators and both optimizers stay fp32.  Tables, scores and gradients
                              * are still fp32 arrays here (holding float16 numbers where the reference holds Half
-                             * tensors); the products run on the fp16 matrix instructions.  dot and cos comparators,
+                             * tensors); the products run on the fp16 matrix instructions (fused and staged route).  dot and cos comparators,
                              * without bias and regularizer (anything else: PBG_ERR_UNSUPPORTED) */
 } pbg_step_desc;
 
