@@ -176,3 +176,42 @@ def test_half_precision_is_refused_where_it_is_not_built(pbg):
         st, _ = make_inputs(cfg, 10, 50, 1, seed=1)
         with pytest.raises(NotImplementedError, match="half_precision"):
             to_runner(pbg, cfg, st, 10, 1)
+
+
+@pytest.mark.parametrize("case", [
+    dict(operator="translation", comparator="cos", loss="softmax", dynamic=False, num_batch_negs=10, num_uniform_negs=10),
+    dict(operator="diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=8, num_uniform_negs=5),
+], ids=lambda c: "-".join(str(v) for v in c.values()))
+def test_half_precision_through_the_model_classes(pbg, case):
+    """MultiRelationEmbedder(half_precision=True) (model.py:409,444) hands the switch to forward and to the
+    Trainer's step."""
+    say("half model", case)
+    from tests.test_gpu_plugins import build_model
+
+    cfg = ostep.StepConfig(dim=16, num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01, margin=0.1,
+                           half_precision=True, **case)
+    st, batches = make_inputs(cfg, 33, 300, 1, seed=5, shared=True)
+    model, w_l, w_r = build_model(pbg, cfg, st, 1 if cfg.dynamic else 3)
+    assert model.half_precision
+    EL, ED, T = pbg.entitylist.EntityList, pbg.edgelist.EdgeList, pbg.train
+    lhs, rhs, rel, ul, ur = batches[0]
+    rel_t = rel.to(DEV) if cfg.dynamic else torch.tensor(rel)
+    edges = ED(EL.from_tensor(lhs.to(DEV)), EL.from_tensor(rhs.to(DEV)), rel_t)
+    scores, _ = model(edges, uniform_negs=(ul.to(DEV), ur.to(DEV)))
+    want, _ = ostep.forward_backward(cfg, st, lhs, rhs, rel, ul, ur, keep_scores=True)
+    got = scores.lhs_neg.cpu()
+    masked = want.scores.lhs_neg == -1e9
+    assert torch.equal(got == -1e9, masked)
+    assert torch.equal(got[~masked].half().float(), got[~masked]), "float16 numbers: the switch reached the kernels"
+    close16(got[~masked], want.scores.lhs_neg[~masked], "lhs_neg", units=3.0, floor=0.05 * float(want.scores.lhs_neg[~masked].abs().max()))
+    loss_fn = pbg.losses.LOSS_FUNCTIONS.get_class(cfg.loss)(margin=cfg.margin)
+    trainer = T.Trainer(T.make_optimizer(list(model.parameters()), False, cfg.lr, cfg.relation_lr), loss_fn, list(cfg.relation_weights))
+    trainer.partitioned_optimizers[("l", 0)] = T.make_optimizer([w_l], True, cfg.lr)
+    trainer.next_uniform_negs = (ul.to(DEV), ur.to(DEV))
+    before = st.w_lhs.clone()
+    stats = trainer.process_one_batch(model, edges)
+    out = ostep.train_step(cfg, st, lhs, rhs, rel, ul, ur)
+    assert float(stats.metrics["loss"]) == pytest.approx(out.loss, rel=4 * EPS16, abs=1e-5)
+    step = st.w_lhs - before
+    close16(w_l.detach().cpu() - before, step, "step of the table", units=8.0 if cfg.comparator == "cos" else 2.0,
+            floor=float(step.abs().max()))

@@ -211,7 +211,8 @@ def build_model(pbg, cfg, st, n_rel_schemas):
     model = M.MultiRelationEmbedder(
         cfg.dim, rels, ent, cfg.num_batch_negs, cfg.num_uniform_negs, cfg.disable_lhs_negs, cfg.disable_rhs_negs,
         lhs_ops, rhs_ops, comparator, regularizer=regularizer,
-        global_emb=cfg.global_emb, max_norm=cfg.max_norm, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0)
+        global_emb=cfg.global_emb, max_norm=cfg.max_norm, num_dynamic_rels=cfg.num_relations if cfg.dynamic else 0,
+        half_precision=cfg.half_precision)
     if cfg.global_emb:
         model.global_embs.to(DEV)
         with torch.no_grad():
