@@ -15,9 +15,11 @@ struct FusedLayout {
   int xch;                       // cos: [2 column groups][64 rows] partial <row, gradient row> of the product being written out
   int ids;                       // int32 row ids of the 2N operand rows (-1: padding), kFusedIds slots; last block
   int total;                     // floats
+  int sliced;                    // rows wider than 128 floats: they pass through LDS in slices of 128 columns (ldx is a slice's stride)
 };
 
-// Whether the route takes this configuration; fills the LDS layout.
+// Whether the route takes this configuration; fills the LDS layout.  (f->sliced: the chunk kernel then needs
+// fused_ids to have run.)
 bool fused_layout(const StepCtx& c, FusedLayout* f);
 
 // Row ids and sort keys of every chunk, ahead of the chunk kernel (c.fused_rowid set): the keys can

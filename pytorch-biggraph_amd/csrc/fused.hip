@@ -16,6 +16,8 @@
 // fit the instruction cache is paid for in fetch stalls by every workgroup.
 #include "fused.h"
 
+#include <cstdlib>
+
 #include "mfma_tiles.h"
 #include "row_ops.h"
 
@@ -732,6 +734,326 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same chain for rows too wide for LDS (dim 256 ... 4096 in multiples of 128,
+// at most 64 batch + 64 uniform negatives, no operator, dot / cos): the chunk's
+// 2 (P + U) rows pass through LDS in SLICES of 128 columns, twice.
+//
+//   sweep 1   per slice: rows -> LDS (raw; cos: the squared norms add up in
+//             registers), both score blocks accumulate S += A_slice N_slice^T in
+//             the matrix accumulators across all slices
+//   between   cos: scores times the two reciprocal norms; scores -> LDS; masks, loss,
+//             dLoss/dS in place, the fold G = dS_R + dS_L^T (+ dLoss/dpos on the
+//             diagonal), exactly as in the one-piece kernel; cos: <y, dLoss/dy> of every
+//             row from the scores and their gradients, t = sum_j dS_ij S_ij (the row is
+//             never in LDS as a whole, its gradient neither)
+//   sweep 2   per slice: rows -> LDS again (cos: normalised), the four gradient
+//             products of the one-piece kernel on the slice, results through
+//             (dy - t y) / ||x|| (cos) to the slice's columns of the gradient rows
+//
+// A row is read twice and its gradient written once; scores and their gradients never
+// leave LDS.  Eight waves, no split into roles: the next slice's rows are on their way
+// from HBM into registers while the products of the current one issue.
+// Row ids and sort keys come from fused_ids_kernel (c.fused_rowid).
+constexpr int kSliceCols = 128;
+constexpr int kSliceThreads = 512;
+
+template <int CMP, int LOSS>
+__global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr bool cosn = CMP == PBG_CMP_COS;
+  constexpr int T0 = 4;         // column tiles per wave: of the score columns, and of a slice's 128 columns
+  constexpr int kLossCols = 16; // score columns per lane of the 8 lanes that share a row (N <= 128)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  FusedGeom g;
+  g.D = kSliceCols; g.P = c.P; g.U = c.U; g.N = c.P + c.U; g.ldx = f.ldx; g.lds = f.lds;
+  g.xn0 = f.xn[0]; g.xn1 = f.xn[1]; g.sc0 = f.sc[0]; g.sc1 = f.sc[1];
+  g.sq0 = f.sq[0]; g.sq1 = f.sq[1]; g.rs0 = f.rs[0]; g.rs1 = f.rs[1]; g.cs0 = f.cs[0]; g.cs1 = f.cs[1];
+  const int D = c.D, P = g.P, U = g.U, N = g.N, ldx = g.ldx, lds_ = g.lds, CP = c.C * c.P;
+  const int xn0 = g.xn0, xn1 = g.xn1, sc0 = g.sc0, sc1 = g.sc1;
+  const int slices = D / kSliceCols, rounds = (N + 15) >> 4;
+  const int p4 = (P + 3) & ~3;
+  const int cp0 = xn0, cp1 = xn0 + p4 * lds_;  // cos: copies of the score blocks, in the operand rows' place between the sweeps
+  int* ids = reinterpret_cast<int*>(lds + f.ids);
+  const int rt = wave & 3, grp = wave >> 2, ct0 = grp * T0;
+
+  for (int t = (int)threadIdx.x * 4; t < f.ids; t += kSliceThreads * 4)
+    *reinterpret_cast<float4*>(&lds[t]) = make_float4(0.f, 0.f, 0.f, 0.f);
+  lds_barrier();
+
+  for (int kc = blockIdx.x; kc < num_chunks; kc += gridDim.x) {
+    // The thread-to-cell mapping is the same for every chunk; hidden from the optimiser once per chunk, so
+    // that it does not hoist every address of the loop body into registers that stay live (and spill).
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
+    const int m16 = lane & 15, kq = lane >> 4;
+    const int hw = lane >> 5, c4 = (lane & 31) << 2;  // half a wave per row, four columns per lane
+    const int k = kc / c.C, cc = kc - k * c.C;
+    const int valid = (cc == c.C - 1) ? c.last : P;
+    const int64_t rel = clamp_index(c.rel[k], c.num_relations);
+    float w_edge = c.rel_weights[rel];
+    if (c.edge_weight) w_edge *= c.edge_weight[(int64_t)k * c.B + min(cc * P + (tid >> 3), c.B - 1)];
+
+    if (tid < kFusedIds) ids[tid] = c.fused_rowid[(int64_t)kc * kFusedIds + tid];
+    lds_barrier();
+    // this thread's rows: row j = 16 u + 2 wave + hw of side s, u < rounds
+    int idv[2][8];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) idv[s][u] = ids[s * kFusedSide + 16 * u + 2 * wave + hw];
+    float4 v[2][8];
+    float sqp[2][8];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sqp[s][u] = 0.f;
+    const uint32_t row_bytes = (uint32_t)D * 4u;
+    auto load_slice = [&](int sl) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const char* w = reinterpret_cast<const char*>(c.side[s].w + sl * kSliceCols + c4);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u >= rounds) break;
+          v[s][u] = *reinterpret_cast<const float4*>(w + (uint64_t)(uint32_t)max(idv[s][u], 0) * row_bytes);
+        }
+      }
+    };
+    // the slice's rows into LDS; RAW: as they are (plus the type's global embedding), the squared norms
+    // adding up; else times the reciprocal norm (cos)
+    auto store_slice = [&](int sl, bool raw) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const float* glob = c.side[s].glob;
+        float4 gv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (glob) gv = *reinterpret_cast<const float4*>(glob + sl * kSliceCols + c4);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u >= rounds) break;
+          const int j = 16 * u + 2 * wave + hw;
+          float4 x = v[s][u];
+          x.x += gv.x; x.y += gv.y; x.z += gv.z; x.w += gv.w;
+          if (idv[s][u] < 0) x = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (cosn) {
+            if (raw) {
+              sqp[s][u] += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+            } else {
+              const float inv = lds[(s ? g.sq1 : g.sq0) + min(j, N - 1)];
+              x.x *= inv; x.y *= inv; x.z *= inv; x.w *= inv;
+            }
+          }
+          if (j < N) *reinterpret_cast<float4*>(&lds[(s ? xn1 : xn0) + j * ldx + c4]) = x;
+        }
+      }
+    };
+
+    // ---- sweep 1: the score blocks ----
+    float4v acc0[T0], acc1[T0];
+#pragma unroll
+    for (int ct = 0; ct < T0; ++ct) {
+      acc0[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+      acc1[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+    }
+    const bool score_live = rt * 16 < P && ct0 * 16 < N;
+    const int ar = min(rt * 16 + m16, P - 1);
+    load_slice(0);
+    for (int sl = 0; sl < slices; ++sl) {
+      lds_barrier();  // the products of the previous slice (or of the previous chunk) have let go of the rows
+      store_slice(sl, true);
+      lds_barrier();
+      if (sl + 1 < slices) load_slice(sl + 1);
+      if (score_live) {
+        // block b: rows = the positives of side 1 - b, columns = side b's negatives
+        mfma_sweep_k16<T0>(lds, xn1 + ar * ldx, xn0 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc0);
+        mfma_sweep_k16<T0>(lds, xn0 + ar * ldx, xn1 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc1);
+      }
+    }
+    if (cosn) {     // reciprocal norms (0 for a padded position: its row is zero)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u >= rounds) break;
+          const float tot = half_sum_at_31(sqp[s][u]);  // complete in lanes 31 and 63
+          const int j = 16 * u + 2 * wave + hw;
+          if ((lane & 31) == 31 && j < N) lds[(s ? g.sq1 : g.sq0) + j] = idv[s][u] < 0 ? 0.f : 1.0f / sqrtf(tot);
+        }
+    }
+    lds_barrier();  // every product has read its rows; the norms are there
+    {
+      const int row = rt * 16 + m16;
+      const int n8 = (N + 7) & ~7;
+      if (score_live && row < P) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const float4v* acc = b ? acc1 : acc0;
+          const float ia = cosn ? lds[(b ? g.sq0 : g.sq1) + row] : 1.0f;
+          const int at = (b ? sc1 : sc0) + row * lds_ + ct0 * 16 + 4 * kq;
+          const int cat = (b ? cp1 : cp0) + row * lds_ + ct0 * 16 + 4 * kq;
+#pragma unroll
+          for (int ct = 0; ct < T0; ++ct) {
+            const int col = (ct0 + ct) * 16 + 4 * kq;
+            float sv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float x = acc[ct][r];
+              if (cosn) x *= ia * lds[(b ? g.sq1 : g.sq0) + min(col + r, N - 1)];
+              sv[r] = col + r < N ? x : -INFINITY;
+            }
+            if (col < n8) {
+              *reinterpret_cast<float4*>(&lds[at + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
+              if (cosn) *reinterpret_cast<float4*>(&lds[cat + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
+            }
+            if (b == 0 && row >= col && row < col + 4) {
+              const int r = row - col;
+              lds[f.pos + row] = r == 0 ? sv[0] : (r == 1 ? sv[1] : (r == 2 ? sv[2] : sv[3]));
+            }
+          }
+        }
+      }
+    }
+    lds_barrier();
+
+    // ---- the loss: side 0, then side 1; eight lanes per edge, columns interleaved ----
+    for (int s = 0; s < 2; ++s) {
+      if (tid < 8 * P) {
+        const int i = tid >> 3, qd = tid & 7;
+        const int row_at = (s ? sc1 : sc0) + i * lds_;
+        float loss_w = 0.f, dpos_s = 0.f, rowsum = 0.f;
+        int viol = 0;
+        if (i >= valid) {
+          for (int j = qd; j < lds_; j += 8) lds[row_at + j] = 0.f;
+        } else {
+          if (qd == (i & 7)) lds[row_at + i] = -1e9f;  // model.py:566-580,836-839
+          if (valid < P)
+            for (int j = valid + ((qd - valid) & 7); j < P; j += 8) lds[row_at + j] = -1e9f;
+          fused_row_loss<CMP, LOSS, kLossCols, false>(lds, row_at, 0, 0.f, c.margin, 1.0f / (float)N, (N + 7) >> 3, lds[f.pos + i],
+                                                        w_edge, qd, &loss_w, &dpos_s, &viol, &rowsum);
+        }
+        if (qd == 0) {
+          lds[f.part + (s * 3 + 0) * P + i] = dpos_s;
+          lds[f.part + (s * 3 + 1) * P + i] = loss_w;
+          lds[f.part + (s * 3 + 2) * P + i] = __int_as_float(viol);
+        }
+      }
+    }
+    lds_barrier();
+    // statistics out
+    if (tid < P) {
+      const int64_t job = (int64_t)k * CP + cc * P + tid;
+      c.lossrow[job] = lds[f.part + 1 * P + tid] + lds[f.part + 4 * P + tid];
+      c.violrow[job * 2] = __float_as_int(lds[f.part + 2 * P + tid]);
+      c.violrow[job * 2 + 1] = __float_as_int(lds[f.part + 5 * P + tid]);
+    }
+    if (cosn) {
+      // <y, dLoss/dy> of a row = sum over the scores it takes part in of dLoss/dscore * score:
+      // per block the sums along its rows (the positives as left operands) and along its
+      // columns (the negatives); masked and padded entries have a zero gradient
+      if (tid < 2 * N) {
+        const int b = tid >= N, j = tid - b * N;
+        const int da = (b ? sc1 : sc0) + j, ca = (b ? cp1 : cp0) + j;
+        float acc = 0.f;
+        for (int i = 0; i < P; ++i) acc += lds[da + i * lds_] * lds[ca + i * lds_];
+        lds[(b ? g.cs1 : g.cs0) + j] = acc;
+      } else if (tid >= 256 && tid < 256 + 2 * P) {
+        const int b = tid - 256 >= P, i = tid - 256 - b * P;
+        const int da = (b ? sc1 : sc0) + i * lds_, ca = (b ? cp1 : cp0) + i * lds_;
+        float acc = 0.f;
+        for (int j = 0; j < N; ++j) acc += lds[da + j] * lds[ca + j];
+        lds[(b ? g.rs1 : g.rs0) + i] = acc;
+      }
+      lds_barrier();
+    }
+    // the fold (see fused_chunk_kernel): G = dS_R[:, :P] + dS_L[:, :P]^T, dLoss/dpos on its diagonal
+    {
+      int i = tid / P, j = tid - i * P;
+      const int di = kSliceThreads / P, dj = kSliceThreads - di * P;
+      for (int e = tid; e < P * P; e += kSliceThreads) {
+        float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
+        if (i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
+        lds[sc1 + i * lds_ + j] = sum;
+        lds[sc0 + j * lds_ + i] = sum;
+        i += di;
+        j += dj;
+        if (j >= P) {
+          j -= P;
+          ++i;
+        }
+      }
+    }
+    // (the barrier at the head of sweep 2 orders the fold before the products)
+
+    // ---- sweep 2: the gradient rows, slice by slice ----
+    load_slice(0);
+    for (int sl = 0; sl < slices; ++sl) {
+      lds_barrier();
+      store_slice(sl, false);
+      lds_barrier();
+      if (sl + 1 < slices) load_slice(sl + 1);
+      const int col0 = sl * kSliceCols + ct0 * 16;
+      // uniform negatives of side m: (dS_m[:, P:])^T (U x P) times the other side's positives
+      for (int m = 0; m < 2; ++m) {
+        const SideCtx& sd = c.side[m];
+        const int dsn = m ? sc1 : sc0, bx = m ? xn0 : xn1, xs = m ? xn1 : xn0;
+        if (rt * 16 >= U) continue;
+        float4v acc[T0];
+#pragma unroll
+        for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+        const int au = min(rt * 16 + m16, U - 1);
+        sweep_a_cols<T0>(lds, dsn + P + au, lds_, bx + ct0 * 16, ldx, kq, m16, (P + 3) >> 2, acc);
+        const int u = rt * 16 + m16;
+        if (u < U) {
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + cc * U + u) * D + col0;
+          const int self_at = xs + (P + u) * ldx + ct0 * 16;
+          const float inv = cosn ? lds[(m ? g.sq1 : g.sq0) + P + u] : 1.0f;
+          const float tt = cosn ? lds[(m ? g.cs1 : g.cs0) + P + u] : 0.f;
+          for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+            if (cosn) {
+              const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
+              r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
+              r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
+            }
+            *reinterpret_cast<float4*>(out + col) = r4;
+          });
+        }
+      }
+      // positives of side m: [G | dS_a[:, P:]] (P x N) times the other side's N rows
+      for (int m = 0; m < 2; ++m) {
+        const SideCtx& sd = c.side[m];
+        const int dsa = m ? sc0 : sc1, bx = m ? xn0 : xn1, xs = m ? xn1 : xn0;
+        if (rt * 16 >= P) continue;
+        float4v acc[T0];
+#pragma unroll
+        for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+        const int ksteps = (N + 3) >> 2;
+        sweep_a_rows<T0>(lds, dsa + ar * lds_, bx + ct0 * 16, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
+        const int i = rt * 16 + m16;
+        if (i < valid) {
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + cc * P + i) * D + col0;
+          const int self_at = xs + i * ldx + ct0 * 16;
+          const float inv = cosn ? lds[(m ? g.sq1 : g.sq0) + i] : 1.0f;
+          // the row was the left operand of block 1 - m, a batch negative (column i) of block m, and one of the positive pair
+          float tt = 0.f;
+          if (cosn)
+            tt = lds[(m ? g.rs0 : g.rs1) + i] + lds[(m ? g.cs1 : g.cs0) + i] +
+                 (lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i]) * lds[f.pos + i];
+          for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+            if (cosn) {
+              const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
+              r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
+              r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
+            }
+            *reinterpret_cast<float4*>(out + col) = r4;
+          });
+        }
+      }
+    }
+    lds_barrier();  // the last slice's products are done before the next chunk's ids and rows arrive
+  }
+}
+
 // One thread per operand-row slot of every chunk (kFusedIds per chunk, see fused_load_ids): the slot's
 // row id (-1: a slot past the operand rows or a padded position of the last chunk) and, for real
 // slots, the sort key and value of the slot's gradient row.  Nothing here depends on the
@@ -792,18 +1114,44 @@ int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, 
   }
 }
 
+template <int CMP, int LOSS>
+int launch_sliced_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
+  static LdsLimit limit;
+  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS>, &limit, lds_bytes);
+  if (rc != PBG_OK) return rc;
+  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c, fl,
+                     c.K * c.C);
+  return PBG_OK;
+}
+
+template <int CMP>
+int launch_sliced_loss(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
+  switch (c.loss) {
+    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC>(c, fl, lds_bytes, s, blocks);
+    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX>(c, fl, lds_bytes, s, blocks);
+  }
+}
+
 }  // namespace
 
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
+  f->sliced = 0;
   if (c.dynamic) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
-  if (c.D > 128 || c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
+  if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
+  // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): no operator, dot / cos, fp32
+  const bool sliced = c.D > 128;
+  if (sliced && (c.D % kSliceCols != 0 || c.op != PBG_OP_NONE || c.cmp == PBG_CMP_L2 || c.half ||
+                 getenv("PBG_DISABLE_SLICED") != nullptr))
+    return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;
   for (int s = 0; s < 2; ++s)
     if (c.side[s].nb != c.P || c.side[s].u != c.U) return false;
   const int N = c.P + c.U;
-  f->ldx = lds_stride(c.D);
+  f->sliced = sliced;
+  f->ldx = lds_stride(sliced ? kSliceCols : c.D);
   f->lds = lds_stride((N + 7) / 8 * 8);  // the loss reads whole groups of 8 columns
   int off = 0;
   auto take = [&](int count) { int o = off; off += (count + 3) / 4 * 4; return o; };
@@ -818,7 +1166,7 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   f->pos = take(c.P);
   f->dpos = take(c.P);
   f->part = take(6 * c.P);
-  f->xch = take(c.cmp == PBG_CMP_COS ? 128 : 0);
+  f->xch = take(c.cmp == PBG_CMP_COS && !sliced ? 128 : 0);
   f->ids = take(kFusedIds);
   f->total = off;
   return (size_t)off * sizeof(float) <= 160 * 1024 - 512;
@@ -832,6 +1180,11 @@ int fused_ids(const StepCtx& c, hipStream_t s) {
 
 int fused_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_t s) {
   const size_t lds_bytes = (size_t)fl.total * sizeof(float);
+  if (fl.sliced) {
+    if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
+    if (c.cmp == PBG_CMP_COS) return launch_sliced_loss<PBG_CMP_COS>(c, fl, lds_bytes, s, blocks);
+    return launch_sliced_loss<PBG_CMP_DOT>(c, fl, lds_bytes, s, blocks);
+  }
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
   // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 104 floats)
   if (small_tiles && fl.ldx == 104 && fl.lds == 104) return launch_fused_cmp<7, 104>(c, fl, lds_bytes, s, blocks);

@@ -2135,15 +2135,18 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     SideStream* ss = nullptr;
     if (chunks >= 128 && cus > 1 && getenv("PBG_DISABLE_SIDE_STREAM") == nullptr) {
       const int rounds_beside = (int)ceil_div(chunks, cus - 1);
-      if (rounds_beside == rounds || sort_bits - c.kbits > 17) {
+      // (the sliced chunk kernel's rounds are far longer than any sort: beside it only when that is free)
+      if (rounds_beside == rounds || (sort_bits - c.kbits > 17 && !plan.fl.sliced)) {
         ss = side_stream();
         if (ss) blocks = (int)ceil_div(chunks, rounds_beside);
       }
     }
     unsigned slot = 0;
-    if (ss) {
+    if (ss || plan.fl.sliced) {
       plan.c.fused_rowid = plan.fused_rowid;
       if ((rc = fused_ids(c, s)) != PBG_OK) return rc;
+    }
+    if (ss) {
       slot = ss->next.fetch_add(1) & 7u;
       if (hipEventRecord(ss->fork[slot], s) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
     }

@@ -923,6 +923,65 @@ def test_fused_kernel_shapes(pbg, case):
     compare_state(cfg, runner, st, rtol, "step", st64)
 
 
+def _sliced_cases():
+    """Rows wider than 128 floats with at most 64 + 64 negatives: the chunk kernel takes them in slices of
+    128 columns (no operator, dot / cos)."""
+    import random
+
+    rng = random.Random(5)
+    cases = [
+        dict(comparator="cos", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=1024),
+        dict(comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=50, num_pos=100, dim=256),
+        dict(comparator="cos", loss="logistic", num_batch_negs=64, num_uniform_negs=64, num_pos=200, dim=384),
+    ]
+    for _ in range(15):
+        p = rng.choice([1, 3, 16, 17, 33, 48, 50, 63, 64])
+        u = rng.choice([1, 5, 16, 17, 49, 50, 64])
+        chunks = rng.choice([1, 2, 3])
+        cases.append(dict(comparator=rng.choice(["dot", "cos"]), loss=rng.choice(["ranking", "logistic", "softmax"]),
+                          num_batch_negs=p, num_uniform_negs=u, num_pos=max(1, p * chunks - rng.choice([0, 0, 1, p // 2])),
+                          dim=rng.choice([256, 384, 512, 640, 2048])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sliced_cases(), ids=ids)
+@pytest.mark.parametrize("extras", ["plain", "global_emb+weights"])
+def test_sliced_chunk_kernel(pbg, case, extras):
+    say("sliced", case, extras)
+    case = dict(case)
+    num_pos, dim = case.pop("num_pos"), case.pop("dim")
+    cfg = ostep.StepConfig(dim=dim, operator="none", dynamic=False, num_relations=2, relation_weights=[1.0, 0.5], lr=0.1,
+                           relation_lr=0.01, margin=0.1, global_emb=(extras != "plain"), **case)
+    workers = 3
+    st, batches = make_inputs(cfg, num_pos, max(300, num_pos * 4), workers, seed=num_pos * 7 + dim, shared=(num_pos % 2 == 0))
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    if cfg.num_batch_negs + cfg.num_uniform_negs <= 100:  # (two score blocks and a slice of more rows do not fit LDS)
+        assert runner.route == "fused"
+    weight = None
+    if extras != "plain":
+        weight = torch.rand(workers, num_pos, generator=torch.Generator().manual_seed(3)) * 2
+    runner.train(*pack(cfg, batches), edge_weight=None if weight is None else weight.to(DEV))
+    torch.cuda.synchronize()
+    outs = ostep.train_lockstep(cfg, st, [b + (weight[k],) for k, b in enumerate(batches)] if weight is not None else batches,
+                                keep_scores=True)
+    for k, out in enumerate(outs):
+        assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
+        sc = out.scores
+        for side, pos, neg, want in ((0, sc.lhs_pos, sc.lhs_neg, out.violators_lhs),
+                                     (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
+            ties = violator_ties(pos, neg)
+            assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
+    assert_close(runner.w_lhs, st.w_lhs, 1e-5, "sliced w_lhs")
+    assert_close(runner.g_lhs, st.g_lhs, 1e-5, "sliced g_lhs")
+    if not st.shared:
+        assert_close(runner.w_rhs, st.w_rhs, 1e-5, "sliced w_rhs")
+        assert_close(runner.g_rhs, st.g_rhs, 1e-5, "sliced g_rhs")
+    if st.glob_lhs is not None:
+        # a type's vector takes the sum of ALL the call's gradient rows: thousands of terms that largely cancel
+        assert_close(runner.global_embs[0], st.glob_lhs, 1e-5, "sliced glob_lhs", atol_scale=1e-5)
+        assert_close(runner.global_embs[1], st.glob_rhs, 1e-5, "sliced glob_rhs", atol_scale=1e-5)
+
+
 def test_lockstep_training_learns_like_sequential(pbg):
     """End to end on a graph with planted structure (a ring with chords: i -> i+1,
     i -> i+7): ten passes with 1 batch per call and with 16 batches per call both
