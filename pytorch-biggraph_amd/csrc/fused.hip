@@ -797,12 +797,9 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 
     if (tid < kFusedIds) ids[tid] = c.fused_rowid[(int64_t)kc * kFusedIds + tid];
     lds_barrier();
-    // this thread's rows: row j = 16 u + 2 wave + hw of side s, u < rounds
-    int idv[2][8];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int u = 0; u < 8; ++u) idv[s][u] = ids[s * kFusedSide + 16 * u + 2 * wave + hw];
+    // this thread's rows: row j = 16 u + 2 wave + hw of side s, u < rounds (their ids are read from LDS where
+    // they are needed: sixteen registers less)
+    const int id_at = 2 * wave + hw;
     float4 v[2][8];
     float sqp[2][8];
 #pragma unroll
@@ -817,7 +814,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
-          v[s][u] = *reinterpret_cast<const float4*>(w + (uint64_t)(uint32_t)max(idv[s][u], 0) * row_bytes);
+          v[s][u] = *reinterpret_cast<const float4*>(w + (uint64_t)(uint32_t)max(ids[s * kFusedSide + 16 * u + id_at], 0) * row_bytes);
         }
       }
     };
@@ -835,7 +832,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           const int j = 16 * u + 2 * wave + hw;
           float4 x = v[s][u];
           x.x += gv.x; x.y += gv.y; x.z += gv.z; x.w += gv.w;
-          if (idv[s][u] < 0) x = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (ids[s * kFusedSide + 16 * u + id_at] < 0) x = make_float4(0.f, 0.f, 0.f, 0.f);
           if (cosn) {
             if (raw) {
               sqp[s][u] += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
@@ -878,7 +875,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           if (u >= rounds) break;
           const float tot = half_sum_at_31(sqp[s][u]);  // complete in lanes 31 and 63
           const int j = 16 * u + 2 * wave + hw;
-          if ((lane & 31) == 31 && j < N) lds[(s ? g.sq1 : g.sq0) + j] = idv[s][u] < 0 ? 0.f : 1.0f / sqrtf(tot);
+          if ((lane & 31) == 31 && j < N) lds[(s ? g.sq1 : g.sq0) + j] = ids[s * kFusedSide + j] < 0 ? 0.f : 1.0f / sqrtf(tot);
         }
     }
     lds_barrier();  // every product has read its rows; the norms are there
