@@ -735,7 +735,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 }
 
 // ---------------------------------------------------------------------------
-// The same chain for rows too wide for LDS (dim 256 ... 4096 in multiples of 128,
+// The same chain for rows too wide for LDS (dim 132 ... 4096 in multiples of 4,
 // at most 64 batch + 64 uniform negatives, no operator, dot / cos): the chunk's
 // 2 (P + U) rows pass through LDS in SLICES of 128 columns, twice.
 //
@@ -771,7 +771,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
   g.sq0 = f.sq[0]; g.sq1 = f.sq[1]; g.rs0 = f.rs[0]; g.rs1 = f.rs[1]; g.cs0 = f.cs[0]; g.cs1 = f.cs[1];
   const int D = c.D, P = g.P, U = g.U, N = g.N, ldx = g.ldx, lds_ = g.lds, CP = c.C * c.P;
   const int xn0 = g.xn0, xn1 = g.xn1, sc0 = g.sc0, sc1 = g.sc1;
-  const int slices = D / kSliceCols, rounds = (N + 15) >> 4;
+  const int slices = (D + kSliceCols - 1) / kSliceCols, rounds = (N + 15) >> 4;  // (the last slice may be a partial one)
   const int p4 = (P + 3) & ~3;
   const int cp0 = xn0, cp1 = xn0 + p4 * lds_;  // cos: copies of the score blocks, in the operand rows' place between the sweeps
   int* ids = reinterpret_cast<int*>(lds + f.ids);
@@ -810,7 +810,8 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
     auto load_slice = [&](int sl) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const char* w = reinterpret_cast<const char*>(c.side[s].w + sl * kSliceCols + c4);
+        // (columns past D: read from the row's last four instead and dropped when the slice is stored)
+        const char* w = reinterpret_cast<const char*>(c.side[s].w + min(sl * kSliceCols + c4, D - 4));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
@@ -824,15 +825,16 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const float* glob = c.side[s].glob;
+        const bool col_ok = sl * kSliceCols + c4 < D;
         float4 gv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (glob) gv = *reinterpret_cast<const float4*>(glob + sl * kSliceCols + c4);
+        if (glob) gv = *reinterpret_cast<const float4*>(glob + min(sl * kSliceCols + c4, D - 4));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
           const int j = 16 * u + 2 * wave + hw;
           float4 x = v[s][u];
           x.x += gv.x; x.y += gv.y; x.z += gv.z; x.w += gv.w;
-          if (ids[s * kFusedSide + 16 * u + id_at] < 0) x = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (ids[s * kFusedSide + 16 * u + id_at] < 0 || !col_ok) x = make_float4(0.f, 0.f, 0.f, 0.f);
           if (cosn) {
             if (raw) {
               sqp[s][u] += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
@@ -1012,7 +1014,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
             }
-            *reinterpret_cast<float4*>(out + col) = r4;
+            if (col0 + col < D) *reinterpret_cast<float4*>(out + col) = r4;
           });
         }
       }
@@ -1042,7 +1044,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
             }
-            *reinterpret_cast<float4*>(out + col) = r4;
+            if (col0 + col < D) *reinterpret_cast<float4*>(out + col) = r4;
           });
         }
       }
@@ -1140,7 +1142,7 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
   // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): no operator, dot / cos, fp32
   const bool sliced = c.D > 128;
-  if (sliced && (c.D % kSliceCols != 0 || c.op != PBG_OP_NONE || c.cmp == PBG_CMP_L2 || c.half ||
+  if (sliced && (c.op != PBG_OP_NONE || c.cmp == PBG_CMP_L2 || c.half ||
                  getenv("PBG_DISABLE_SLICED") != nullptr))
     return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;

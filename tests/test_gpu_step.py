@@ -941,6 +941,14 @@ def _sliced_cases():
         cases.append(dict(comparator=rng.choice(["dot", "cos"]), loss=rng.choice(["ranking", "logistic", "softmax"]),
                           num_batch_negs=p, num_uniform_negs=u, num_pos=max(1, p * chunks - rng.choice([0, 0, 1, p // 2])),
                           dim=rng.choice([256, 384, 512, 640, 2048])))
+    # dims that end in a partial slice
+    cases += [
+        dict(comparator="cos", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=400),
+        dict(comparator="dot", loss="logistic", num_batch_negs=50, num_uniform_negs=50, num_pos=75, dim=200),
+        dict(comparator="cos", loss="softmax", num_batch_negs=33, num_uniform_negs=17, num_pos=66, dim=132),
+        dict(comparator="cos", loss="softmax", num_batch_negs=16, num_uniform_negs=49, num_pos=40, dim=300),
+        dict(comparator="dot", loss="ranking", num_batch_negs=48, num_uniform_negs=5, num_pos=100, dim=1028),
+    ]
     return cases
 
 

@@ -89,6 +89,13 @@ def lockstep64(cfg, st, batches, keep_scores=False):
     return outs, st64
 
 
+@pytest.fixture(autouse=True)
+def _keep_to_the_streaming_kernels(monkeypatch):
+    """A shape without operator whose chunk has at most about 100 negatives is taken by the chunk kernel on
+    slices first; these tests are about the streaming kernels."""
+    monkeypatch.setenv("PBG_DISABLE_SLICED", "1")
+
+
 def build(pbg, case, workers, seed_shift=0):
     case = dict(case)
     num_pos, dim = case.pop("num_pos"), case.pop("dim")
