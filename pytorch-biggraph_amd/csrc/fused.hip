@@ -736,7 +736,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 
 // ---------------------------------------------------------------------------
 // The same chain for rows too wide for LDS (dim 132 ... 4096 in multiples of 4,
-// at most 64 batch + 64 uniform negatives, no operator, dot / cos): the chunk's
+// at most 64 batch + 64 uniform negatives, operator none / translation / diagonal, dot / cos): the chunk's
 // 2 (P + U) rows pass through LDS in SLICES of 128 columns, twice.
 //
 //   sweep 1   per slice: rows -> LDS (raw; cos: the squared norms add up in
@@ -828,12 +828,23 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
         const bool col_ok = sl * kSliceCols + c4 < D;
         float4 gv = make_float4(0.f, 0.f, 0.f, 0.f);
         if (glob) gv = *reinterpret_cast<const float4*>(glob + min(sl * kSliceCols + c4, D - 4));
+        // the relation's operator acts on side 1's rows (model.py:666-703); both kinds are local to a slice
+        const bool has_op = s == 1 && c.op != PBG_OP_NONE;
+        float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (has_op) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + min(sl * kSliceCols + c4, D - 4));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
           const int j = 16 * u + 2 * wave + hw;
           float4 x = v[s][u];
           x.x += gv.x; x.y += gv.y; x.z += gv.z; x.w += gv.w;
+          if (has_op) {
+            if (c.op == PBG_OP_DIAGONAL) {
+              x.x *= par.x; x.y *= par.y; x.z *= par.z; x.w *= par.w;
+            } else {
+              x.x += par.x; x.y += par.y; x.z += par.z; x.w += par.w;
+            }
+          }
           if (ids[s * kFusedSide + 16 * u + id_at] < 0 || !col_ok) x = make_float4(0.f, 0.f, 0.f, 0.f);
           if (cosn) {
             if (raw) {
@@ -1008,13 +1019,23 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           const int self_at = xs + (P + u) * ldx + ct0 * 16;
           const float inv = cosn ? lds[(m ? g.sq1 : g.sq0) + P + u] : 1.0f;
           const float tt = cosn ? lds[(m ? g.cs1 : g.cs0) + P + u] : 0.f;
+          const bool has_op = m == 1 && c.op != PBG_OP_NONE;
+          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + cc * U + u) * D + col0 : nullptr;
+          const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
           for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
             }
-            if (col0 + col < D) *reinterpret_cast<float4*>(out + col) = r4;
+            if (col0 + col < D) {
+              if (dz) *reinterpret_cast<float4*>(dz + col) = r4;  // the gradient at the operator's output: the parameter stage reads it
+              if (par) {
+                const float4 pv = *reinterpret_cast<const float4*>(par + col);
+                r4.x *= pv.x; r4.y *= pv.y; r4.z *= pv.z; r4.w *= pv.w;
+              }
+              *reinterpret_cast<float4*>(out + col) = r4;
+            }
           });
         }
       }
@@ -1038,13 +1059,23 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           if (cosn)
             tt = lds[(m ? g.rs0 : g.rs1) + i] + lds[(m ? g.cs1 : g.cs0) + i] +
                  (lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i]) * lds[f.pos + i];
+          const bool has_op = m == 1 && c.op != PBG_OP_NONE;
+          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + cc * P + i) * D + col0 : nullptr;
+          const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
           for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
             }
-            if (col0 + col < D) *reinterpret_cast<float4*>(out + col) = r4;
+            if (col0 + col < D) {
+              if (dz) *reinterpret_cast<float4*>(dz + col) = r4;
+              if (par) {
+                const float4 pv = *reinterpret_cast<const float4*>(par + col);
+                r4.x *= pv.x; r4.y *= pv.y; r4.z *= pv.z; r4.w *= pv.w;
+              }
+              *reinterpret_cast<float4*>(out + col) = r4;
+            }
           });
         }
       }
@@ -1140,9 +1171,9 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
-  // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): no operator, dot / cos, fp32
+  // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): dot / cos, fp32
   const bool sliced = c.D > 128;
-  if (sliced && (c.op != PBG_OP_NONE || c.cmp == PBG_CMP_L2 || c.half ||
+  if (sliced && (c.cmp == PBG_CMP_L2 || c.half ||
                  getenv("PBG_DISABLE_SLICED") != nullptr))
     return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;

@@ -949,6 +949,10 @@ def _sliced_cases():
         dict(comparator="cos", loss="softmax", num_batch_negs=16, num_uniform_negs=49, num_pos=40, dim=300),
         dict(comparator="dot", loss="ranking", num_batch_negs=48, num_uniform_negs=5, num_pos=100, dim=1028),
     ]
+    # the two operators that act on a slice's columns alone
+    for op, cmp_, loss, dim in itertools.product(("translation", "diagonal"), ("dot", "cos"), ("ranking", "softmax"), (256, 200)):
+        cases.append(dict(operator=op, comparator=cmp_, loss=loss, num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=dim))
+    cases.append(dict(operator="diagonal", comparator="cos", loss="logistic", num_batch_negs=17, num_uniform_negs=33, num_pos=40, dim=1024))
     return cases
 
 
@@ -958,7 +962,8 @@ def test_sliced_chunk_kernel(pbg, case, extras):
     say("sliced", case, extras)
     case = dict(case)
     num_pos, dim = case.pop("num_pos"), case.pop("dim")
-    cfg = ostep.StepConfig(dim=dim, operator="none", dynamic=False, num_relations=2, relation_weights=[1.0, 0.5], lr=0.1,
+    case.setdefault("operator", "none")
+    cfg = ostep.StepConfig(dim=dim, dynamic=False, num_relations=2, relation_weights=[1.0, 0.5], lr=0.1,
                            relation_lr=0.01, margin=0.1, global_emb=(extras != "plain"), **case)
     workers = 3
     st, batches = make_inputs(cfg, num_pos, max(300, num_pos * 4), workers, seed=num_pos * 7 + dim, shared=(num_pos % 2 == 0))
@@ -988,6 +993,9 @@ def test_sliced_chunk_kernel(pbg, case, extras):
         # a type's vector takes the sum of ALL the call's gradient rows: thousands of terms that largely cancel
         assert_close(runner.global_embs[0], st.glob_lhs, 1e-5, "sliced glob_lhs", atol_scale=1e-5)
         assert_close(runner.global_embs[1], st.glob_rhs, 1e-5, "sliced glob_rhs", atol_scale=1e-5)
+    for name, got, want in (("rhs_op", runner.rhs_op, st.rhs_op), ("rhs_op_sum", runner.rhs_op_sum, st.rhs_op_sum)):
+        for key in want:
+            assert_close(got[key], want[key], 1e-5, f"sliced {name}.{key}")
 
 
 def test_lockstep_training_learns_like_sequential(pbg):
