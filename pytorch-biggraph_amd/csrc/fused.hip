@@ -758,7 +758,9 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 constexpr int kSliceCols = 128;
 constexpr int kSliceThreads = 512;
 
-template <int CMP, int LOSS>
+// LDS != 0: the score rows' stride, known at compile time like the slice rows' (136 floats), so that the
+// products' LDS addresses are one register plus immediates.
+template <int CMP, int LOSS, int LDS>
 __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool cosn = CMP == PBG_CMP_COS;
@@ -766,10 +768,13 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
   constexpr int kLossCols = 16; // score columns per lane of the 8 lanes that share a row (N <= 128)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   FusedGeom g;
-  g.D = kSliceCols; g.P = c.P; g.U = c.U; g.N = c.P + c.U; g.ldx = f.ldx; g.lds = f.lds;
+  constexpr int kSliceLd = lds_stride(kSliceCols);
+  g.D = kSliceCols; g.P = c.P; g.U = c.U; g.N = c.P + c.U; g.ldx = kSliceLd; g.lds = LDS ? LDS : f.lds;
   g.xn0 = f.xn[0]; g.xn1 = f.xn[1]; g.sc0 = f.sc[0]; g.sc1 = f.sc[1];
   g.sq0 = f.sq[0]; g.sq1 = f.sq[1]; g.rs0 = f.rs[0]; g.rs1 = f.rs[1]; g.cs0 = f.cs[0]; g.cs1 = f.cs[1];
-  const int D = c.D, P = g.P, U = g.U, N = g.N, ldx = g.ldx, lds_ = g.lds, CP = c.C * c.P;
+  const int D = c.D, P = g.P, U = g.U, N = g.N, CP = c.C * c.P;
+  constexpr int ldx = kSliceLd;
+  const int lds_ = LDS ? LDS : f.lds;
   const int xn0 = g.xn0, xn1 = g.xn1, sc0 = g.sc0, sc1 = g.sc1;
   const int slices = (D + kSliceCols - 1) / kSliceCols, rounds = (N + 15) >> 4;  // (the last slice may be a partial one)
   const int p4 = (P + 3) & ~3;
@@ -1144,23 +1149,30 @@ int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, 
   }
 }
 
-template <int CMP, int LOSS>
+template <int CMP, int LOSS, int LDS>
 int launch_sliced_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   static LdsLimit limit;
-  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS>, &limit, lds_bytes);
+  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS, LDS>, &limit, lds_bytes);
   if (rc != PBG_OK) return rc;
-  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c, fl,
+  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS, LDS>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c, fl,
                      c.K * c.C);
   return PBG_OK;
 }
 
-template <int CMP>
+template <int CMP, int LDS>
 int launch_sliced_loss(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   switch (c.loss) {
-    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING>(c, fl, lds_bytes, s, blocks);
-    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC>(c, fl, lds_bytes, s, blocks);
-    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING, LDS>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC, LDS>(c, fl, lds_bytes, s, blocks);
+    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX, LDS>(c, fl, lds_bytes, s, blocks);
   }
+}
+
+template <int CMP>
+int launch_sliced_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
+  // 50 + 50 negatives (and everything else whose score rows come out at 104 floats)
+  if (fl.lds == 104) return launch_sliced_loss<CMP, 104>(c, fl, lds_bytes, s, blocks);
+  return launch_sliced_loss<CMP, 0>(c, fl, lds_bytes, s, blocks);
 }
 
 }  // namespace
@@ -1212,8 +1224,8 @@ int fused_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_
   const size_t lds_bytes = (size_t)fl.total * sizeof(float);
   if (fl.sliced) {
     if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
-    if (c.cmp == PBG_CMP_COS) return launch_sliced_loss<PBG_CMP_COS>(c, fl, lds_bytes, s, blocks);
-    return launch_sliced_loss<PBG_CMP_DOT>(c, fl, lds_bytes, s, blocks);
+    if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS>(c, fl, lds_bytes, s, blocks);
+    return launch_sliced_cmp<PBG_CMP_DOT>(c, fl, lds_bytes, s, blocks);
   }
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
   // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 104 floats)
