@@ -84,6 +84,10 @@ WORKLOADS = {
                     entities=100_000, edges=1_000_000, dim=400, batch=1000, batch_negs=50, uniform_negs=50,
                     operator="none", comparator="cos", loss="ranking", relations=1, dynamic=False,
                     init_scale=1e-3, zipf=None, two_tables=False),
+    "d200transe": dict(desc="TransE at dim 200: translation/l2/ranking(0.1), 100k entities, B=1000, 50 batch + 50 uniform negatives",
+                       entities=100_000, edges=1_000_000, dim=200, batch=1000, batch_negs=50, uniform_negs=50,
+                       operator="translation", comparator="l2", loss="ranking", relations=1, dynamic=False,
+                       init_scale=1e-3, zipf=None, two_tables=False),
     "d200": dict(desc="as d400 at dim 200 (13 column tiles, the last half padding)",
                  entities=14_951, edges=483_142, dim=200, batch=1000, batch_negs=50, uniform_negs=50,
                  operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=False,
@@ -499,7 +503,7 @@ def main():
         return spec, calls * per_call / dt, dt / calls * 1e3, dt, stages, loss
 
     workers = max(1, args.workers)
-    default_batches = {"cfg1": 64000, "cfg1cos": 64000, "cfg2": 400, "cfg2d": 400, "fb15k": 400, "d400": 6400, "d200": 6400, "d256dot": 6400, "d400cos": 6400, "livejournal": 3200, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
+    default_batches = {"cfg1": 64000, "cfg1cos": 64000, "cfg2": 400, "cfg2d": 400, "fb15k": 400, "d400": 6400, "d200": 6400, "d256dot": 6400, "d400cos": 6400, "d200transe": 6400, "livejournal": 3200, "cfg3": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}[args.workload]
     steps = args.steps if args.steps is not None else max(1, default_batches // workers)
     warmup = args.warmup if args.warmup is not None else max(1, steps // 10)
     spec, eps, ms_per_step, wall_s, stages, loss = run(workers, steps, warmup, profile_calls=10)

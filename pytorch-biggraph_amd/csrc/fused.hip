@@ -736,7 +736,7 @@ __global__ __launch_bounds__(2 * kFusedThreads) void fused_chunk_kernel(StepCtx 
 
 // ---------------------------------------------------------------------------
 // The same chain for rows too wide for LDS (dim 132 ... 4096 in multiples of 4,
-// at most 64 batch + 64 uniform negatives, operator none / translation / diagonal, dot / cos): the chunk's
+// at most 64 batch + 64 uniform negatives, operator none / translation / diagonal, dot / cos / l2): the chunk's
 // 2 (P + U) rows pass through LDS in SLICES of 128 columns, twice.
 //
 //   sweep 1   per slice: rows -> LDS (raw; cos: the squared norms add up in
@@ -764,6 +764,8 @@ template <int CMP, int LOSS, int LDS>
 __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool cosn = CMP == PBG_CMP_COS;
+  constexpr bool l2 = CMP == PBG_CMP_L2;  // as in fused_chunk_kernel: squared norms, positive scores in the direct form,
+                                          // dS stored as -2 dLoss/dq, the rows' own terms added as the gradients leave
   constexpr int T0 = 4;         // column tiles per wave: of the score columns, and of a slice's 128 columns
   constexpr int kLossCols = 16; // score columns per lane of the 8 lanes that share a row (N <= 128)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -851,10 +853,10 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
             }
           }
           if (ids[s * kFusedSide + 16 * u + id_at] < 0 || !col_ok) x = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (cosn) {
+          if (cosn || l2) {
             if (raw) {
               sqp[s][u] += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
-            } else {
+            } else if (cosn) {
               const float inv = lds[(s ? g.sq1 : g.sq0) + min(j, N - 1)];
               x.x *= inv; x.y *= inv; x.z *= inv; x.w *= inv;
             }
@@ -873,19 +875,33 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
     }
     const bool score_live = rt * 16 < P && ct0 * 16 < N;
     const int ar = min(rt * 16 + m16, P - 1);
+    float pos_part = 0.f;
     load_slice(0);
     for (int sl = 0; sl < slices; ++sl) {
       lds_barrier();  // the products of the previous slice (or of the previous chunk) have let go of the rows
       store_slice(sl, true);
       lds_barrier();
       if (sl + 1 < slices) load_slice(sl + 1);
+      if (l2 && tid < 4 * P) {  // positive scores in the direct form (model.py:267-274): this slice's share
+        const int i = tid >> 2, qd = tid & 3;
+        for (int d0 = qd; d0 < kSliceCols; d0 += 32) {
+          float a[8], bb[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            a[u] = lds[xn0 + i * ldx + d0 + 4 * u];
+            bb[u] = lds[xn1 + i * ldx + d0 + 4 * u];
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) pos_part += (a[u] - bb[u]) * (a[u] - bb[u]);
+        }
+      }
       if (score_live) {
         // block b: rows = the positives of side 1 - b, columns = side b's negatives
         mfma_sweep_k16<T0>(lds, xn1 + ar * ldx, xn0 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc0);
         mfma_sweep_k16<T0>(lds, xn0 + ar * ldx, xn1 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc1);
       }
     }
-    if (cosn) {     // reciprocal norms (0 for a padded position: its row is zero)
+    if (cosn || l2) {  // cos: reciprocal norms (0 for a padded position: its row is zero); l2: squared norms as norm().pow(2)
 #pragma unroll
       for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -893,8 +909,14 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           if (u >= rounds) break;
           const float tot = half_sum_at_31(sqp[s][u]);  // complete in lanes 31 and 63
           const int j = 16 * u + 2 * wave + hw;
-          if ((lane & 31) == 31 && j < N) lds[(s ? g.sq1 : g.sq0) + j] = ids[s * kFusedSide + j] < 0 ? 0.f : 1.0f / sqrtf(tot);
+          const float nrm = sqrtf(tot);
+          if ((lane & 31) == 31 && j < N)
+            lds[(s ? g.sq1 : g.sq0) + j] = l2 ? nrm * nrm : (ids[s * kFusedSide + j] < 0 ? 0.f : 1.0f / nrm);
         }
+    }
+    if (l2) {
+      pos_part = quad_sum(pos_part);
+      if (tid < 4 * P && (tid & 3) == 0) lds[f.pos + (tid >> 2)] = -sqrtf(fmaxf(pos_part, 1e-30f));
     }
     lds_barrier();  // every product has read its rows; the norms are there
     {
@@ -921,7 +943,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               *reinterpret_cast<float4*>(&lds[at + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
               if (cosn) *reinterpret_cast<float4*>(&lds[cat + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
             }
-            if (b == 0 && row >= col && row < col + 4) {
+            if (!l2 && b == 0 && row >= col && row < col + 4) {
               const int r = row - col;
               lds[f.pos + row] = r == 0 ? sv[0] : (r == 1 ? sv[1] : (r == 2 ? sv[2] : sv[3]));
             }
@@ -941,13 +963,16 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
         if (i >= valid) {
           for (int j = qd; j < lds_; j += 8) lds[row_at + j] = 0.f;
         } else {
-          if (qd == (i & 7)) lds[row_at + i] = -1e9f;  // model.py:566-580,836-839
+          const float masked = l2 ? -INFINITY : -1e9f;  // model.py:566-580,836-839
+          if (qd == (i & 7)) lds[row_at + i] = masked;
           if (valid < P)
-            for (int j = valid + ((qd - valid) & 7); j < P; j += 8) lds[row_at + j] = -1e9f;
-          fused_row_loss<CMP, LOSS, kLossCols, false>(lds, row_at, 0, 0.f, c.margin, 1.0f / (float)N, (N + 7) >> 3, lds[f.pos + i],
-                                                        w_edge, qd, &loss_w, &dpos_s, &viol, &rowsum);
+            for (int j = valid + ((qd - valid) & 7); j < P; j += 8) lds[row_at + j] = masked;
+          fused_row_loss<CMP, LOSS, kLossCols, false>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f,
+                                                        c.margin, 1.0f / (float)N, (N + 7) >> 3, lds[f.pos + i], w_edge, qd, &loss_w,
+                                                        &dpos_s, &viol, &rowsum);
         }
         if (qd == 0) {
+          if (l2) lds[(s ? g.rs1 : g.rs0) + i] = rowsum;
           lds[f.part + (s * 3 + 0) * P + i] = dpos_s;
           lds[f.part + (s * 3 + 1) * P + i] = loss_w;
           lds[f.part + (s * 3 + 2) * P + i] = __int_as_float(viol);
@@ -961,6 +986,20 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
       c.lossrow[job] = lds[f.part + 1 * P + tid] + lds[f.part + 4 * P + tid];
       c.violrow[job * 2] = __float_as_int(lds[f.part + 2 * P + tid]);
       c.violrow[job * 2 + 1] = __float_as_int(lds[f.part + 5 * P + tid]);
+    }
+    if (l2) {
+      // column sums of the stored -2 dLoss/dq over the batch-negative columns of both blocks (before the fold
+      // rewrites them), and dLoss/dpos of both sides together
+      if (tid < 2 * P) {
+        const int b = tid >= P, j = tid - b * P;
+        float acc = 0.f;
+        for (int i = 0; i < P; ++i) acc += lds[(b ? sc1 : sc0) + i * lds_ + j];
+        lds[(b ? g.cs1 : g.cs0) + j] = acc;
+      } else if (tid >= 256 && tid < 256 + P) {
+        const int i = tid - 256;
+        lds[f.dpos + i] = lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
+      }
+      lds_barrier();
     }
     if (cosn) {
       // <y, dLoss/dy> of a row = sum over the scores it takes part in of dLoss/dscore * score:
@@ -987,7 +1026,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
       const int di = kSliceThreads / P, dj = kSliceThreads - di * P;
       for (int e = tid; e < P * P; e += kSliceThreads) {
         float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
-        if (i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
+        if (!l2 && i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
         lds[sc1 + i * lds_ + j] = sum;
         lds[sc0 + j * lds_ + i] = sum;
         i += di;
@@ -1017,7 +1056,11 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
         for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int au = min(rt * 16 + m16, U - 1);
-        sweep_a_cols<T0>(lds, dsn + P + au, lds_, bx + ct0 * 16, ldx, kq, m16, (P + 3) >> 2, acc);
+        float asum = sweep_a_cols<T0>(lds, dsn + P + au, lds_, bx + ct0 * 16, ldx, kq, m16, (P + 3) >> 2, acc);
+        if (l2) {  // the column sum of the stored -2 dLoss/dq: the lane's share, then the other three k slots'
+          asum += __shfl_xor(asum, 16);
+          asum += __shfl_xor(asum, 32);
+        }
         const int u = rt * 16 + m16;
         if (u < U) {
           float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + cc * U + u) * D + col0;
@@ -1032,6 +1075,10 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
+            }
+            if (l2) {  // ||b||^2's share: minus the column sum times the row itself
+              const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
+              r4.x -= asum * y.x; r4.y -= asum * y.y; r4.z -= asum * y.z; r4.w -= asum * y.w;
             }
             if (col0 + col < D) {
               if (dz) *reinterpret_cast<float4*>(dz + col) = r4;  // the gradient at the operator's output: the parameter stage reads it
@@ -1064,6 +1111,13 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           if (cosn)
             tt = lds[(m ? g.rs0 : g.rs1) + i] + lds[(m ? g.cs1 : g.cs0) + i] +
                  (lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i]) * lds[f.pos + i];
+          float l2_coef = 0.f, l2_pcoef = 0.f;
+          const int other_at = bx + i * ldx + ct0 * 16;
+          if (l2) {
+            const float dpz = lds[f.dpos + i], pz = lds[f.pos + i];
+            l2_coef = 2.0f * lds[(m ? g.rs0 : g.rs1) + i] - lds[(m ? g.cs1 : g.cs0) + i];
+            l2_pcoef = pz * pz > 2e-30f ? dpz / pz : 0.f;
+          }
           const bool has_op = m == 1 && c.op != PBG_OP_NONE;
           float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + cc * P + i) * D + col0 : nullptr;
           const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
@@ -1072,6 +1126,12 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
               r4.z = inv * (r4.z - tt * y.z); r4.w = inv * (r4.w - tt * y.w);
+            }
+            if (l2) {  // the row's own terms of ||a||^2 - 2ab + ||b||^2, and the positive pair's (see fused_emit)
+              const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
+              const float4 o4 = *reinterpret_cast<const float4*>(&lds[other_at + col]);
+              r4.x += l2_coef * y.x + l2_pcoef * (y.x - o4.x); r4.y += l2_coef * y.y + l2_pcoef * (y.y - o4.y);
+              r4.z += l2_coef * y.z + l2_pcoef * (y.z - o4.z); r4.w += l2_coef * y.w + l2_pcoef * (y.w - o4.w);
             }
             if (col0 + col < D) {
               if (dz) *reinterpret_cast<float4*>(dz + col) = r4;
@@ -1183,9 +1243,9 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
-  // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): dot / cos, fp32
+  // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): fp32
   const bool sliced = c.D > 128;
-  if (sliced && (c.cmp == PBG_CMP_L2 || c.half ||
+  if (sliced && (c.half ||
                  getenv("PBG_DISABLE_SLICED") != nullptr))
     return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;
@@ -1225,6 +1285,7 @@ int fused_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_
   if (fl.sliced) {
     if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
     if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS>(c, fl, lds_bytes, s, blocks);
+    if (c.cmp == PBG_CMP_L2) return launch_sliced_cmp<PBG_CMP_L2>(c, fl, lds_bytes, s, blocks);
     return launch_sliced_cmp<PBG_CMP_DOT>(c, fl, lds_bytes, s, blocks);
   }
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
