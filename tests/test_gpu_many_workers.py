@@ -73,6 +73,11 @@ CASES = {
                            num_uniform_negs=5, entities=300, relations=3, scale=0.03, ks=(1, 3)),
     "affine-dim2048": dict(operator="affine", comparator="l2", loss="ranking", dim=2048, num_pos=24, num_batch_negs=8,
                            num_uniform_negs=5, entities=300, relations=2, scale=0.03, shared=False, ks=(2,)),
+    # rows wider than LDS (the chunk kernel on slices of 128 columns), power-law ids: the LiveJournal example's kind of step
+    "sliced-cos": dict(operator="none", comparator="cos", loss="ranking", dim=256, num_pos=200, num_batch_negs=50,
+                       num_uniform_negs=50, entities=3000, scale=0.1, zipf=1.5, ks=(20, 65)),
+    "sliced-transe": dict(operator="translation", comparator="l2", loss="ranking", dim=200, num_pos=200, num_batch_negs=50,
+                          num_uniform_negs=50, entities=20000, relations=4, scale=0.1, zipf=1.5, shared=False, ks=(64,)),
     # global embeddings: their update walks the batches in blocks of 64
     "global-fused": dict(operator="none", comparator="dot", loss="logistic", dim=100, num_pos=200, num_batch_negs=50,
                          num_uniform_negs=50, entities=3000, scale=0.1, global_emb=True, ks=(64, 65, 130)),
