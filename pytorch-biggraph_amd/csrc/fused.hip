@@ -760,7 +760,10 @@ constexpr int kSliceThreads = 512;
 
 // LDS != 0: the score rows' stride, known at compile time like the slice rows' (136 floats), so that the
 // products' LDS addresses are one register plus immediates.
-template <int CMP, int LOSS, int LDS>
+// HALF (config.half_precision, dot / cos): the rounding points of fused_chunk_kernel<..., HALF>.  The prepared row
+// is what gets rounded, so with cos the norms must be known before the first product: one more pass over the rows
+// ("sweep 0", nothing stored) adds up the squared norms, and both sweeps then store normalised, rounded rows.
+template <int CMP, int LOSS, int LDS, bool HALF>
 __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool cosn = CMP == PBG_CMP_COS;
@@ -826,9 +829,12 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
         }
       }
     };
-    // the slice's rows into LDS; RAW: as they are (plus the type's global embedding), the squared norms
-    // adding up; else times the reciprocal norm (cos)
-    auto store_slice = [&](int sl, bool raw) {
+    // The slice's rows (plus the type's global embedding, through the operator) into LDS.  kRaw: as they are, the
+    // squared norms adding up; kNorms: the squared norms only, nothing stored; kPrepared: times the reciprocal norm
+    // (cos), rounded to float16 numbers (HALF).
+    constexpr int kRaw = 0, kPrepared = 1, kNorms = 2;
+    auto store_slice = [&](int sl, int mode) {
+      const bool raw = mode != kPrepared;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const float* glob = c.side[s].glob;
@@ -861,10 +867,37 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               x.x *= inv; x.y *= inv; x.z *= inv; x.w *= inv;
             }
           }
-          if (j < N) *reinterpret_cast<float4*>(&lds[(s ? xn1 : xn0) + j * ldx + c4]) = x;
+          if (HALF && !raw) {  // embs.half() (model.py:504-505)
+            x.x = half_round(x.x); x.y = half_round(x.y); x.z = half_round(x.z); x.w = half_round(x.w);
+          }
+          if (j < N && mode != kNorms) *reinterpret_cast<float4*>(&lds[(s ? xn1 : xn0) + j * ldx + c4]) = x;
         }
       }
     };
+    // cos: reciprocal norms (0 for a padded position: its row is zero); l2: squared norms as norm().pow(2)
+    auto finish_norms = [&]() {
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u >= rounds) break;
+          const float tot = half_sum_at_31(sqp[s][u]);  // complete in lanes 31 and 63
+          const int j = 16 * u + 2 * wave + hw;
+          const float nrm = sqrtf(tot);
+          if ((lane & 31) == 31 && j < N)
+            lds[(s ? g.sq1 : g.sq0) + j] = l2 ? nrm * nrm : (ids[s * kFusedSide + j] < 0 ? 0.f : 1.0f / nrm);
+        }
+    };
+    constexpr bool pre_norms = HALF && cosn;  // the norms before the first product
+    if (pre_norms) {
+      load_slice(0);
+      for (int sl = 0; sl < slices; ++sl) {
+        store_slice(sl, kNorms);
+        if (sl + 1 < slices) load_slice(sl + 1);
+      }
+      finish_norms();
+      // (the first barrier of sweep 1 orders the norms before the stores that read them)
+    }
 
     // ---- sweep 1: the score blocks ----
     float4v acc0[T0], acc1[T0];
@@ -879,7 +912,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
     load_slice(0);
     for (int sl = 0; sl < slices; ++sl) {
       lds_barrier();  // the products of the previous slice (or of the previous chunk) have let go of the rows
-      store_slice(sl, true);
+      store_slice(sl, pre_norms || (HALF && !cosn) ? kPrepared : kRaw);
       lds_barrier();
       if (sl + 1 < slices) load_slice(sl + 1);
       if (l2 && tid < 4 * P) {  // positive scores in the direct form (model.py:267-274): this slice's share
@@ -897,23 +930,11 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
       }
       if (score_live) {
         // block b: rows = the positives of side 1 - b, columns = side b's negatives
-        mfma_sweep_k16<T0>(lds, xn1 + ar * ldx, xn0 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc0);
-        mfma_sweep_k16<T0>(lds, xn0 + ar * ldx, xn1 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc1);
+        mfma_sweep_k16<T0, HALF>(lds, xn1 + ar * ldx, xn0 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc0);
+        mfma_sweep_k16<T0, HALF>(lds, xn0 + ar * ldx, xn1 + (ct0 * 16 + m16) * ldx, 16 * ldx, kSliceCols / 16, 0, kq, acc1);
       }
     }
-    if (cosn || l2) {  // cos: reciprocal norms (0 for a padded position: its row is zero); l2: squared norms as norm().pow(2)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          if (u >= rounds) break;
-          const float tot = half_sum_at_31(sqp[s][u]);  // complete in lanes 31 and 63
-          const int j = 16 * u + 2 * wave + hw;
-          const float nrm = sqrtf(tot);
-          if ((lane & 31) == 31 && j < N)
-            lds[(s ? g.sq1 : g.sq0) + j] = l2 ? nrm * nrm : (ids[s * kFusedSide + j] < 0 ? 0.f : 1.0f / nrm);
-        }
-    }
+    if ((cosn || l2) && !pre_norms) finish_norms();
     if (l2) {
       pos_part = quad_sum(pos_part);
       if (tid < 4 * P && (tid & 3) == 0) lds[f.pos + (tid >> 2)] = -sqrtf(fmaxf(pos_part, 1e-30f));
@@ -926,7 +947,8 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
           const float4v* acc = b ? acc1 : acc0;
-          const float ia = cosn ? lds[(b ? g.sq0 : g.sq1) + row] : 1.0f;
+          constexpr bool scale = cosn && !pre_norms;  // (with the norms known beforehand the rows were normalised as they were stored)
+          const float ia = scale ? lds[(b ? g.sq0 : g.sq1) + row] : 1.0f;
           const int at = (b ? sc1 : sc0) + row * lds_ + ct0 * 16 + 4 * kq;
           const int cat = (b ? cp1 : cp0) + row * lds_ + ct0 * 16 + 4 * kq;
 #pragma unroll
@@ -936,16 +958,21 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float x = acc[ct][r];
-              if (cosn) x *= ia * lds[(b ? g.sq1 : g.sq0) + min(col + r, N - 1)];
+              if (scale) x *= ia * lds[(b ? g.sq1 : g.sq0) + min(col + r, N - 1)];
               sv[r] = col + r < N ? x : -INFINITY;
+            }
+            // (HALF: the positive score is the fp32 sum itself, model.py:177; the block holds float16 numbers)
+            if (!l2 && b == 0 && row >= col && row < col + 4) {
+              const int r = row - col;
+              lds[f.pos + row] = r == 0 ? sv[0] : (r == 1 ? sv[1] : (r == 2 ? sv[2] : sv[3]));
+            }
+            if (HALF) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) sv[r] = half_round(sv[r]);
             }
             if (col < n8) {
               *reinterpret_cast<float4*>(&lds[at + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
               if (cosn) *reinterpret_cast<float4*>(&lds[cat + ct * 16]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
-            }
-            if (!l2 && b == 0 && row >= col && row < col + 4) {
-              const int r = row - col;
-              lds[f.pos + row] = r == 0 ? sv[0] : (r == 1 ? sv[1] : (r == 2 ? sv[2] : sv[3]));
             }
           }
         }
@@ -967,7 +994,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           if (qd == (i & 7)) lds[row_at + i] = masked;
           if (valid < P)
             for (int j = valid + ((qd - valid) & 7); j < P; j += 8) lds[row_at + j] = masked;
-          fused_row_loss<CMP, LOSS, kLossCols, false>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f,
+          fused_row_loss<CMP, LOSS, kLossCols, HALF>(lds, row_at, s ? g.sq1 : g.sq0, l2 ? lds[(s ? g.sq0 : g.sq1) + i] : 0.f,
                                                         c.margin, 1.0f / (float)N, (N + 7) >> 3, lds[f.pos + i], w_edge, qd, &loss_w,
                                                         &dpos_s, &viol, &rowsum);
         }
@@ -1027,6 +1054,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
       for (int e = tid; e < P * P; e += kSliceThreads) {
         float sum = lds[sc1 + i * lds_ + j] + lds[sc0 + j * lds_ + i];
         if (!l2 && i == j) sum += lds[f.part + 0 * P + i] + lds[f.part + 3 * P + i];
+        if (HALF) sum = half_round(sum);
         lds[sc1 + i * lds_ + j] = sum;
         lds[sc0 + j * lds_ + i] = sum;
         i += di;
@@ -1043,7 +1071,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
     load_slice(0);
     for (int sl = 0; sl < slices; ++sl) {
       lds_barrier();
-      store_slice(sl, false);
+      store_slice(sl, kPrepared);
       lds_barrier();
       if (sl + 1 < slices) load_slice(sl + 1);
       const int col0 = sl * kSliceCols + ct0 * 16;
@@ -1056,7 +1084,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
         for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int au = min(rt * 16 + m16, U - 1);
-        float asum = sweep_a_cols<T0>(lds, dsn + P + au, lds_, bx + ct0 * 16, ldx, kq, m16, (P + 3) >> 2, acc);
+        float asum = sweep_a_cols<T0, HALF>(lds, dsn + P + au, lds_, bx + ct0 * 16, ldx, kq, m16, (P + 3) >> 2, acc);
         if (l2) {  // the column sum of the stored -2 dLoss/dq: the lane's share, then the other three k slots'
           asum += __shfl_xor(asum, 16);
           asum += __shfl_xor(asum, 32);
@@ -1071,6 +1099,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + cc * U + u) * D + col0 : nullptr;
           const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
           for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+            if (HALF) r4 = make_float4(half_round(r4.x), half_round(r4.y), half_round(r4.z), half_round(r4.w));
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
@@ -1100,7 +1129,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
         for (int ct = 0; ct < T0; ++ct) acc[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
         const int ksteps = (N + 3) >> 2;
-        sweep_a_rows<T0>(lds, dsa + ar * lds_, bx + ct0 * 16, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
+        sweep_a_rows<T0, HALF>(lds, dsa + ar * lds_, bx + ct0 * 16, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
         const int i = rt * 16 + m16;
         if (i < valid) {
           float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + cc * P + i) * D + col0;
@@ -1122,6 +1151,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + cc * P + i) * D + col0 : nullptr;
           const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
           for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+            if (HALF) r4 = make_float4(half_round(r4.x), half_round(r4.y), half_round(r4.z), half_round(r4.w));
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x = inv * (r4.x - tt * y.x); r4.y = inv * (r4.y - tt * y.y);
@@ -1209,30 +1239,30 @@ int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, 
   }
 }
 
-template <int CMP, int LOSS, int LDS>
+template <int CMP, int LOSS, int LDS, bool HALF>
 int launch_sliced_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   static LdsLimit limit;
-  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS, LDS>, &limit, lds_bytes);
+  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS, LDS, HALF>, &limit, lds_bytes);
   if (rc != PBG_OK) return rc;
-  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS, LDS>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c, fl,
-                     c.K * c.C);
+  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS, LDS, HALF>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c,
+                     fl, c.K * c.C);
   return PBG_OK;
 }
 
-template <int CMP, int LDS>
+template <int CMP, int LDS, bool HALF>
 int launch_sliced_loss(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   switch (c.loss) {
-    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING, LDS>(c, fl, lds_bytes, s, blocks);
-    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC, LDS>(c, fl, lds_bytes, s, blocks);
-    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX, LDS>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING, LDS, HALF>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC, LDS, HALF>(c, fl, lds_bytes, s, blocks);
+    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX, LDS, HALF>(c, fl, lds_bytes, s, blocks);
   }
 }
 
-template <int CMP>
+template <int CMP, bool HALF>
 int launch_sliced_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   // 50 + 50 negatives (and everything else whose score rows come out at 104 floats)
-  if (fl.lds == 104) return launch_sliced_loss<CMP, 104>(c, fl, lds_bytes, s, blocks);
-  return launch_sliced_loss<CMP, 0>(c, fl, lds_bytes, s, blocks);
+  if (fl.lds == 104) return launch_sliced_loss<CMP, 104, HALF>(c, fl, lds_bytes, s, blocks);
+  return launch_sliced_loss<CMP, 0, HALF>(c, fl, lds_bytes, s, blocks);
 }
 
 }  // namespace
@@ -1245,8 +1275,7 @@ bool fused_layout(const StepCtx& c, FusedLayout* f) {
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
   // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): fp32
   const bool sliced = c.D > 128;
-  if (sliced && (c.half ||
-                 getenv("PBG_DISABLE_SLICED") != nullptr))
+  if (sliced && getenv("PBG_DISABLE_SLICED") != nullptr)
     return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;
   for (int s = 0; s < 2; ++s)
@@ -1284,9 +1313,14 @@ int fused_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_
   const size_t lds_bytes = (size_t)fl.total * sizeof(float);
   if (fl.sliced) {
     if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
-    if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS>(c, fl, lds_bytes, s, blocks);
-    if (c.cmp == PBG_CMP_L2) return launch_sliced_cmp<PBG_CMP_L2>(c, fl, lds_bytes, s, blocks);
-    return launch_sliced_cmp<PBG_CMP_DOT>(c, fl, lds_bytes, s, blocks);
+    if (c.half) {  // (dot and cos only: the step's validation has refused the rest)
+      if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS, true>(c, fl, lds_bytes, s, blocks);
+      if (c.cmp == PBG_CMP_DOT) return launch_sliced_cmp<PBG_CMP_DOT, true>(c, fl, lds_bytes, s, blocks);
+      return fail(PBG_ERR_UNSUPPORTED, "step: half_precision on the fused route is built for dot and cos");
+    }
+    if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS, false>(c, fl, lds_bytes, s, blocks);
+    if (c.cmp == PBG_CMP_L2) return launch_sliced_cmp<PBG_CMP_L2, false>(c, fl, lds_bytes, s, blocks);
+    return launch_sliced_cmp<PBG_CMP_DOT, false>(c, fl, lds_bytes, s, blocks);
   }
   const bool small_tiles = c.P + c.U <= 112 && c.D <= 112;
   // dim 100 with 50 + 50 negatives (and everything else whose two row strides come out as 104 floats)

@@ -94,6 +94,14 @@ HALF_CASES += [
     dict(operator="diagonal", comparator="cos", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=3, num_pos=75, dim=36),
     dict(operator="none", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=13, num_uniform_negs=64, num_pos=30, dim=112),
 ]
+# rows wider than 128 floats: the chunk kernel on slices (cos: after a pass of its own for the norms)
+for op, cmp_, loss in itertools.product(("none", "translation", "diagonal"), ("dot", "cos"), ("ranking", "softmax")):
+    HALF_CASES.append(dict(operator=op, comparator=cmp_, loss=loss, dynamic=False, num_batch_negs=50, num_uniform_negs=50,
+                           num_pos=130, dim=256))
+HALF_CASES += [
+    dict(operator="none", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=33, num_uniform_negs=17, num_pos=70, dim=200),
+    dict(operator="none", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=16, num_uniform_negs=49, num_pos=40, dim=132),
+]
 
 
 def close16(got, want, what, units=2.0, floor=None):
