@@ -10,7 +10,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = pathlib.Path(__file__).resolve().parent
-SOURCES = ["common.hip", "sort.hip", "row_adagrad.hip", "perm.hip", "gemm.hip", "seg_linear.hip", "step.hip", "fused.hip", "stream.hip", "plugins.hip"]
+SOURCES = ["common.hip", "sort.hip", "row_adagrad.hip", "perm.hip", "gemm.hip", "seg_linear.hip", "step.hip", "fused.hip", "sliced.hip", "stream.hip", "plugins.hip"]
 LIB = HERE.parent / "libpbg_hip.so"
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

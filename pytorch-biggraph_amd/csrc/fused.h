@@ -27,6 +27,11 @@ bool fused_layout(const StepCtx& c, FusedLayout* f);
 // makes both itself.
 int fused_ids(const StepCtx& c, hipStream_t stream);
 
+// Width of a slice of the sliced chunk kernel (sliced.hip), in columns.
+constexpr int kSliceCols = 128;
+// (fused_chunks hands a layout with `sliced` set on to this one)
+int sliced_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_t stream);
+
 // The chunk kernel on `blocks` workgroups, each of which takes chunks blockIdx, blockIdx + blocks, ...
 int fused_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_t stream);
 
