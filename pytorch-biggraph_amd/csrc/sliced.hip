@@ -34,7 +34,7 @@ constexpr int kSliceThreads = 512;
 // HALF (config.half_precision, dot / cos): the rounding points of fused_chunk_kernel<..., HALF>.  The prepared row
 // is what gets rounded, so with cos the norms must be known before the first product: one more pass over the rows
 // ("sweep 0", nothing stored) adds up the squared norms, and both sweeps then store normalised, rounded rows.
-template <int CMP, int LOSS, int LDS, bool HALF>
+template <int CMP, int LOSS, int LDS, bool HALF, bool CPLX>
 __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, FusedLayout f, int num_chunks) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool cosn = CMP == PBG_CMP_COS;
@@ -52,7 +52,27 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
   constexpr int ldx = kSliceLd;
   const int lds_ = LDS ? LDS : f.lds;
   const int xn0 = g.xn0, xn1 = g.xn1, sc0 = g.sc0, sc1 = g.sc1;
-  const int slices = (D + kSliceCols - 1) / kSliceCols, rounds = (N + 15) >> 4;  // (the last slice may be a partial one)
+  // CPLX (complex_diagonal, operators.py:118-152): the operator pairs coordinate h with h + D/2, so a slice holds 64 such
+  // pairs instead of 128 consecutive coordinates -- LDS columns [0, 32) and [64, 96) are the real parts of the slice's
+  // pairs 0..31 and 32..63, [32, 64) and [96, 128) their imaginary parts -- and a product that sums over all
+  // coordinates does not care.  The partner of LDS column p is p ^ 32: in the stores, lane ^ 8; in the results of
+  // the gradient products, register r ^ 2 of the same lane (for_each_out's columns are 16 r + 4 q).
+  const int H = D >> 1;
+  const int slices = CPLX ? (H + 63) / 64 : (D + kSliceCols - 1) / kSliceCols;  // (the last slice may be a partial one)
+  const int rounds = (N + 15) >> 4;
+  // LDS column p (a multiple of 4) of slice sl: its first coordinate (the last whole quad of the row, or of the
+  // row's half, when the slice ends before p) and whether the column exists
+  auto coord = [&](int sl, int p, bool* ok) -> int {
+    if constexpr (CPLX) {
+      const int h = sl * 64 + ((p >> 6) << 5) + (p & 31);
+      *ok = h < H;
+      return ((p >> 5) & 1) * H + min(h, H - 4);
+    } else {
+      const int col = sl * kSliceCols + p;
+      *ok = col < D;
+      return min(col, D - 4);
+    }
+  };
   const int p4 = (P + 3) & ~3;
   const int cp0 = xn0, cp1 = xn0 + p4 * lds_;  // cos: copies of the score blocks, in the operand rows' place between the sweeps
   int* ids = reinterpret_cast<int*>(lds + f.ids);
@@ -92,7 +112,8 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         // (columns past D: read from the row's last four instead and dropped when the slice is stored)
-        const char* w = reinterpret_cast<const char*>(c.side[s].w + min(sl * kSliceCols + c4, D - 4));
+        bool ok;
+        const char* w = reinterpret_cast<const char*>(c.side[s].w + coord(sl, c4, &ok));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
@@ -109,13 +130,23 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const float* glob = c.side[s].glob;
-        const bool col_ok = sl * kSliceCols + c4 < D;
+        bool col_ok;
+        const int col = coord(sl, c4, &col_ok);
         float4 gv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (glob) gv = *reinterpret_cast<const float4*>(glob + min(sl * kSliceCols + c4, D - 4));
+        if (glob) gv = *reinterpret_cast<const float4*>(glob + col);
         // the relation's operator acts on side 1's rows (model.py:666-703); both kinds are local to a slice
         const bool has_op = s == 1 && c.op != PBG_OP_NONE;
         float4 par = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (has_op) par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + min(sl * kSliceCols + c4, D - 4));
+        const bool imag = CPLX && (c4 & 32) != 0;
+        float4 par_o = par;  // CPLX: the partner's share of the parameter (imaginary for a real lane and the reverse)
+        if (has_op) {
+          if constexpr (CPLX) {
+            par = *reinterpret_cast<const float4*>(imag ? c.side[1].p1 + (rel * H + col - H) : c.side[1].p0 + (rel * H + col));
+            par_o = make_float4(__shfl_xor(par.x, 8), __shfl_xor(par.y, 8), __shfl_xor(par.z, 8), __shfl_xor(par.w, 8));
+          } else {
+            par = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + col);
+          }
+        }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           if (u >= rounds) break;
@@ -123,7 +154,17 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
           float4 x = v[s][u];
           x.x += gv.x; x.y += gv.y; x.z += gv.z; x.w += gv.w;
           if (has_op) {
-            if (c.op == PBG_OP_DIAGONAL) {
+            if constexpr (CPLX) {
+              // real: x_re a_re - x_im a_im; imaginary: x_im a_re + x_re a_im (operators.py:143-148)
+              const float4 o = make_float4(__shfl_xor(x.x, 8), __shfl_xor(x.y, 8), __shfl_xor(x.z, 8), __shfl_xor(x.w, 8));
+              if (imag) {
+                x.x = x.x * par_o.x + o.x * par.x; x.y = x.y * par_o.y + o.y * par.y;
+                x.z = x.z * par_o.z + o.z * par.z; x.w = x.w * par_o.w + o.w * par.w;
+              } else {
+                x.x = x.x * par.x - o.x * par_o.x; x.y = x.y * par.y - o.y * par_o.y;
+                x.z = x.z * par.z - o.z * par_o.z; x.w = x.w * par.w - o.w * par_o.w;
+              }
+            } else if (c.op == PBG_OP_DIAGONAL) {
               x.x *= par.x; x.y *= par.y; x.z *= par.z; x.w *= par.w;
             } else {
               x.x += par.x; x.y += par.y; x.z += par.z; x.w += par.w;
@@ -345,7 +386,51 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
       store_slice(sl, kPrepared);
       lds_barrier();
       if (sl + 1 < slices) load_slice(sl + 1);
-      const int col0 = sl * kSliceCols + ct0 * 16;
+      // Where a finished quad of a gradient row goes: the row's place in the gradient array, at the operator's output
+      // (dz, for the parameter stage) and, through the operator's transpose, at the raw row.  `lc`: the quad's LDS column.
+      auto put = [&](float* out, float* dz, int lc, float4 r4, bool diag) {
+        bool ok;
+        const int col = coord(sl, ct0 * 16 + lc, &ok);
+        if (!ok) return;
+        if (dz) *reinterpret_cast<float4*>(dz + col) = r4;
+        if (diag) {
+          const float4 pv = *reinterpret_cast<const float4*>(c.side[1].p0 + rel * D + col);
+          r4.x *= pv.x; r4.y *= pv.y; r4.z *= pv.z; r4.w *= pv.w;
+        }
+        *reinterpret_cast<float4*>(out + col) = r4;
+      };
+      // CPLX, a row the operator acted on: the real quad at LDS column lc and the imaginary one at lc + 32;
+      // d/dx_re = a_re g_re + a_im g_im, d/dx_im = a_re g_im - a_im g_re
+      auto put_pair = [&](float* out, float* dz, int lc, float4 gre, float4 gim) {
+        bool ok;
+        const int col = coord(sl, ct0 * 16 + lc, &ok);
+        if (!ok) return;
+        if (dz) {
+          *reinterpret_cast<float4*>(dz + col) = gre;
+          *reinterpret_cast<float4*>(dz + col + H) = gim;
+        }
+        const float4 are = *reinterpret_cast<const float4*>(c.side[1].p0 + (rel * H + col));
+        const float4 aim = *reinterpret_cast<const float4*>(c.side[1].p1 + (rel * H + col));
+        *reinterpret_cast<float4*>(out + col) = make_float4(are.x * gre.x + aim.x * gim.x, are.y * gre.y + aim.y * gim.y,
+                                                            are.z * gre.z + aim.z * gim.z, are.w * gre.w + aim.w * gim.w);
+        *reinterpret_cast<float4*>(out + col + H) = make_float4(are.x * gim.x - aim.x * gre.x, are.y * gim.y - aim.y * gre.y,
+                                                                are.z * gim.z - aim.z * gre.z, are.w * gim.w - aim.w * gre.w);
+      };
+      // all quads of the lane's row: each through `adjust`, then to their places
+      auto emit = [&](const float4v* acc, float* out, float* dz, bool has_op, auto&& adjust) {
+        if constexpr (CPLX) {
+          if (has_op) {
+            float4 q4[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) q4[r] = adjust(16 * r + 4 * kq, make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]));
+            put_pair(out, dz, 4 * kq, q4[0], q4[2]);
+            put_pair(out, dz, 16 + 4 * kq, q4[1], q4[3]);
+            return;
+          }
+        }
+        const bool diag = has_op && c.op == PBG_OP_DIAGONAL;
+        for_each_out<T0>(acc, kq, [&](int lc, float4 r4) { put(out, dz, lc, adjust(lc, r4), diag); });
+      };
       // uniform negatives of side m: (dS_m[:, P:])^T (U x P) times the other side's positives
       for (int m = 0; m < 2; ++m) {
         const SideCtx& sd = c.side[m];
@@ -362,14 +447,13 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
         }
         const int u = rt * 16 + m16;
         if (u < U) {
-          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + cc * U + u) * D + col0;
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_uni + cc * U + u) * D;
           const int self_at = xs + (P + u) * ldx + ct0 * 16;
           const float inv = cosn ? lds[(m ? g.sq1 : g.sq0) + P + u] : 1.0f;
           const float tt = cosn ? lds[(m ? g.cs1 : g.cs0) + P + u] : 0.f;
           const bool has_op = m == 1 && c.op != PBG_OP_NONE;
-          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + cc * U + u) * D + col0 : nullptr;
-          const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
-          for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + c.B + cc * U + u) * D : nullptr;
+          emit(acc, out, dz, has_op, [&](int col, float4 r4) {
             if (HALF) r4 = make_float4(half_round(r4.x), half_round(r4.y), half_round(r4.z), half_round(r4.w));
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
@@ -380,14 +464,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
               r4.x -= asum * y.x; r4.y -= asum * y.y; r4.z -= asum * y.z; r4.w -= asum * y.w;
             }
-            if (col0 + col < D) {
-              if (dz) *reinterpret_cast<float4*>(dz + col) = r4;  // the gradient at the operator's output: the parameter stage reads it
-              if (par) {
-                const float4 pv = *reinterpret_cast<const float4*>(par + col);
-                r4.x *= pv.x; r4.y *= pv.y; r4.z *= pv.z; r4.w *= pv.w;
-              }
-              *reinterpret_cast<float4*>(out + col) = r4;
-            }
+            return r4;
           });
         }
       }
@@ -403,7 +480,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
         sweep_a_rows<T0, HALF>(lds, dsa + ar * lds_, bx + ct0 * 16, ldx, kq, m16, ksteps >> 2, ksteps & 3, acc);
         const int i = rt * 16 + m16;
         if (i < valid) {
-          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + cc * P + i) * D + col0;
+          float* out = c.gr + ((int64_t)k * c.rk + sd.slot_pos + cc * P + i) * D;
           const int self_at = xs + i * ldx + ct0 * 16;
           const float inv = cosn ? lds[(m ? g.sq1 : g.sq0) + i] : 1.0f;
           // the row was the left operand of block 1 - m, a batch negative (column i) of block m, and one of the positive pair
@@ -419,9 +496,8 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
             l2_pcoef = pz * pz > 2e-30f ? dpz / pz : 0.f;
           }
           const bool has_op = m == 1 && c.op != PBG_OP_NONE;
-          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + cc * P + i) * D + col0 : nullptr;
-          const float* par = (has_op && c.op == PBG_OP_DIAGONAL) ? sd.p0 + rel * D + col0 : nullptr;
-          for_each_out<T0>(acc, kq, [&](int col, float4 r4) {
+          float* dz = (has_op && sd.dz) ? sd.dz + ((int64_t)k * sd.op_rows + cc * P + i) * D : nullptr;
+          emit(acc, out, dz, has_op, [&](int col, float4 r4) {
             if (HALF) r4 = make_float4(half_round(r4.x), half_round(r4.y), half_round(r4.z), half_round(r4.w));
             if (cosn) {
               const float4 y = *reinterpret_cast<const float4*>(&lds[self_at + col]);
@@ -434,14 +510,7 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
               r4.x += l2_coef * y.x + l2_pcoef * (y.x - o4.x); r4.y += l2_coef * y.y + l2_pcoef * (y.y - o4.y);
               r4.z += l2_coef * y.z + l2_pcoef * (y.z - o4.z); r4.w += l2_coef * y.w + l2_pcoef * (y.w - o4.w);
             }
-            if (col0 + col < D) {
-              if (dz) *reinterpret_cast<float4*>(dz + col) = r4;
-              if (par) {
-                const float4 pv = *reinterpret_cast<const float4*>(par + col);
-                r4.x *= pv.x; r4.y *= pv.y; r4.z *= pv.z; r4.w *= pv.w;
-              }
-              *reinterpret_cast<float4*>(out + col) = r4;
-            }
+            return r4;
           });
         }
       }
@@ -450,30 +519,30 @@ __global__ __launch_bounds__(kSliceThreads) void sliced_chunk_kernel(StepCtx c, 
   }
 }
 
-template <int CMP, int LOSS, int LDS, bool HALF>
+template <int CMP, int LOSS, int LDS, bool HALF, bool CPLX>
 int launch_sliced_as(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   static LdsLimit limit;
-  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS, LDS, HALF>, &limit, lds_bytes);
+  const int rc = reserve_lds((const void*)sliced_chunk_kernel<CMP, LOSS, LDS, HALF, CPLX>, &limit, lds_bytes);
   if (rc != PBG_OK) return rc;
-  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS, LDS, HALF>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c,
+  hipLaunchKernelGGL((sliced_chunk_kernel<CMP, LOSS, LDS, HALF, CPLX>), dim3((unsigned)blocks), dim3(kSliceThreads), lds_bytes, s, c,
                      fl, c.K * c.C);
   return PBG_OK;
 }
 
-template <int CMP, int LDS, bool HALF>
+template <int CMP, int LDS, bool HALF, bool CPLX>
 int launch_sliced_loss(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   switch (c.loss) {
-    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING, LDS, HALF>(c, fl, lds_bytes, s, blocks);
-    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC, LDS, HALF>(c, fl, lds_bytes, s, blocks);
-    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX, LDS, HALF>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_RANKING: return launch_sliced_as<CMP, PBG_LOSS_RANKING, LDS, HALF, CPLX>(c, fl, lds_bytes, s, blocks);
+    case PBG_LOSS_LOGISTIC: return launch_sliced_as<CMP, PBG_LOSS_LOGISTIC, LDS, HALF, CPLX>(c, fl, lds_bytes, s, blocks);
+    default: return launch_sliced_as<CMP, PBG_LOSS_SOFTMAX, LDS, HALF, CPLX>(c, fl, lds_bytes, s, blocks);
   }
 }
 
-template <int CMP, bool HALF>
+template <int CMP, bool HALF, bool CPLX = false>
 int launch_sliced_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, hipStream_t s, int blocks) {
   // 50 + 50 negatives (and everything else whose score rows come out at 104 floats)
-  if (fl.lds == 104) return launch_sliced_loss<CMP, 104, HALF>(c, fl, lds_bytes, s, blocks);
-  return launch_sliced_loss<CMP, 0, HALF>(c, fl, lds_bytes, s, blocks);
+  if (fl.lds == 104) return launch_sliced_loss<CMP, 104, HALF, CPLX>(c, fl, lds_bytes, s, blocks);
+  return launch_sliced_loss<CMP, 0, HALF, CPLX>(c, fl, lds_bytes, s, blocks);
 }
 
 }  // namespace
@@ -481,6 +550,8 @@ int launch_sliced_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes,
 int sliced_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_t s) {
   const size_t lds_bytes = (size_t)fl.total * sizeof(float);
   if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
+  // (complex_diagonal: with dot, in fp32 -- what fused_layout lets through)
+  if (c.op == PBG_OP_COMPLEX_DIAGONAL) return launch_sliced_cmp<PBG_CMP_DOT, false, true>(c, fl, lds_bytes, s, blocks);
   if (c.half) {  // (dot and cos only: the step's validation has refused the rest)
     if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS, true>(c, fl, lds_bytes, s, blocks);
     if (c.cmp == PBG_CMP_DOT) return launch_sliced_cmp<PBG_CMP_DOT, true>(c, fl, lds_bytes, s, blocks);

@@ -209,10 +209,10 @@ TRAIN_CASES += [
 ]
 
 
-def lockstep(cfg, st, batches, keep_scores=False):
-    """oracle.step.train_lockstep on `st`; for the l2 comparator also on a float64
-    copy, the anchor of compare_state's criterion for that comparator."""
-    st64 = double_state(st) if cfg.comparator == "l2" else None
+def lockstep(cfg, st, batches, keep_scores=False, anchor=False):
+    """oracle.step.train_lockstep on `st`; for the l2 comparator (or with `anchor`) also on a
+    float64 copy, the anchor of compare_state's criterion for that comparator."""
+    st64 = double_state(st) if cfg.comparator == "l2" or anchor else None
     outs = ostep.train_lockstep(cfg, st, batches, keep_scores=keep_scores)
     if st64 is not None:
         for out, exact in zip(outs, ostep.train_lockstep(cfg, st64, batches)):
@@ -961,6 +961,17 @@ def _sliced_cases():
         dict(operator="diagonal", comparator="l2", loss="softmax", num_batch_negs=33, num_uniform_negs=17, num_pos=70, dim=132),
         dict(operator="translation", comparator="l2", loss="logistic", num_batch_negs=16, num_uniform_negs=49, num_pos=40, dim=1024),
     ]
+    # complex_diagonal pairs coordinate h with h + dim / 2: slices of 64 such pairs (dot; dims whose half is and is
+    # not a multiple of 64, a last slice of 8 and of 4 pairs, one partial chunk)
+    for loss, dim in itertools.product(ostep.LOSS_NAMES, (400, 256)):
+        cases.append(dict(operator="complex_diagonal", comparator="dot", loss=loss, num_batch_negs=50, num_uniform_negs=50,
+                          num_pos=130, dim=dim))
+    cases += [
+        dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=33, num_uniform_negs=17, num_pos=70, dim=136),
+        dict(operator="complex_diagonal", comparator="dot", loss="ranking", num_batch_negs=17, num_uniform_negs=64, num_pos=40, dim=1024),
+        dict(operator="complex_diagonal", comparator="dot", loss="logistic", num_batch_negs=64, num_uniform_negs=5, num_pos=100, dim=200),
+        dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=48, num_uniform_negs=16, num_pos=96, dim=648),
+    ]
     return cases
 
 
@@ -988,8 +999,11 @@ def test_sliced_chunk_kernel(pbg, case, extras):
         weight = torch.rand(workers, num_pos, generator=torch.Generator().manual_seed(3)) * 2
     runner.train(*pack(cfg, batches), edge_weight=None if weight is None else weight.to(DEV))
     torch.cuda.synchronize()
+    # (complex_diagonal: four products per coordinate pair, whose order of rounding is the compiler's on both sides;
+    # a gradient that nearly cancels then differs in its last bits, and Adagrad's division scales that up: the
+    # float64 result is the anchor there as it is for l2)
     outs, st64 = lockstep(cfg, st, [b + (weight[k],) for k, b in enumerate(batches)] if weight is not None else batches,
-                          keep_scores=True)
+                          keep_scores=True, anchor=cfg.operator == "complex_diagonal")
     for k, out in enumerate(outs):
         assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
         sc = out.scores
@@ -997,7 +1011,7 @@ def test_sliced_chunk_kernel(pbg, case, extras):
                                      (1, sc.rhs_pos, sc.rhs_neg, out.violators_rhs)):
             ties = violator_ties(pos, neg)
             assert abs(int(runner.violators_out[k, side]) - want) <= ties, ("violators", side, k, ties)
-    if st64 is not None:  # l2: the float64-anchored criterion
+    if st64 is not None:  # l2, complex_diagonal: the float64-anchored criterion
         compare_state(cfg, runner, st, 1e-5, "sliced", st64)
         return
     assert_close(runner.w_lhs, st.w_lhs, 1e-5, "sliced w_lhs")
