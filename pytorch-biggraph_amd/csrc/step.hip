@@ -987,6 +987,140 @@ __global__ __launch_bounds__(kParamGroups * 64) void param_grad_kernel(StepCtx c
   }
 }
 
+// The same sums for rows whose length is a multiple of 4 (of 8 with complex_diagonal): four columns per lane --
+// with complex_diagonal four (real, imaginary) pairs -- as 128-bit loads, four rows in flight.  The rows a group
+// takes, their order and the order of the groups are param_grad_kernel's, and so is every sum.  On the fused
+// route the rows' ids are the ones its id kernel has left behind (c.fused_rowid), not drawn again.
+template <int OP>
+__global__ __launch_bounds__(kParamGroups * 64) void param_grad_quad_kernel(StepCtx c, int s, float* __restrict__ dth,
+                                                                             int slices, int reg_op) {
+  constexpr bool cplx = OP == PBG_OP_COMPLEX_DIAGONAL;
+  constexpr int NA = cplx ? 2 : 1;
+  constexpr int kFusedSide = kFusedIds / 2;
+  __shared__ float4 sh[NA][kParamGroups][64];
+  const SideCtx& sd = c.side[s];
+  const int lane = threadIdx.x & 63, rg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int k = blockIdx.y, slice = blockIdx.z;
+  const int D = c.D, H = D / 2;
+  const int quads = (cplx ? H : D) >> 2;
+  const int q = blockIdx.x * 64 + lane;
+  const int e = 4 * min(q, quads - 1);  // (lanes past the last quad read the last one and store nothing)
+  const int step = slices * kParamGroups;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 acc[NA];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) acc[a] = zero;
+  float4 gl[NA];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) gl[a] = (OP != PBG_OP_TRANSLATION && sd.glob) ? *reinterpret_cast<const float4*>(sd.glob + e + a * H) : zero;
+  auto dz_of = [&](int r) -> const float* {
+    if (sd.uni_dz_direct && r >= c.B) {
+      const int cc = (r - c.B) / sd.u, uu = (r - c.B) - cc * sd.u;
+      return sd.dxn + (((int64_t)k * c.C + cc) * sd.nn + sd.nb + uu) * D;
+    }
+    return sd.dz + ((int64_t)k * sd.op_rows + r) * D;
+  };
+  auto x_of = [&](int r) -> const float* {  // the operator's input row (without the global embedding)
+    int64_t id;
+    if (c.fused_rowid) {
+      const bool uni = r >= c.B;
+      const int cc = uni ? (r - c.B) / c.U : r / c.P;
+      const int j = uni ? c.P + (r - c.B) - cc * c.U : r - cc * c.P;
+      id = c.fused_rowid[((int64_t)k * c.C + cc) * kFusedIds + s * kFusedSide + j];
+      if (id < 0) id = 0;
+    } else if (r < c.B) {
+      id = clamp_index(sd.idx[(int64_t)k * c.B + r], sd.num_rows);
+    } else {
+      id = clamp_index(uniform_negative(sd, s, (int64_t)k * c.C * sd.u + (r - c.B)), sd.num_rows);
+    }
+    return sd.w + id * D;
+  };
+  for (int r0 = slice * kParamGroups + rg; r0 < sd.op_rows; r0 += 4 * step) {
+    float4 g[4][NA], x[4][NA];
+    bool live[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = r0 + j * step;
+      live[j] = r < sd.op_rows;
+      const int rr = live[j] ? r : r0;
+      const float* dz = dz_of(rr);
+      const float* xr = OP == PBG_OP_TRANSLATION ? dz : x_of(rr);
+#pragma unroll
+      for (int a = 0; a < NA; ++a) {
+        g[j][a] = *reinterpret_cast<const float4*>(dz + e + a * H);
+        x[j][a] = OP == PBG_OP_TRANSLATION ? zero : *reinterpret_cast<const float4*>(xr + e + a * H);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (!live[j]) break;
+      if constexpr (OP == PBG_OP_TRANSLATION) {
+        acc[0].x += g[j][0].x; acc[0].y += g[j][0].y; acc[0].z += g[j][0].z; acc[0].w += g[j][0].w;
+      } else if constexpr (!cplx) {
+        acc[0].x += (x[j][0].x + gl[0].x) * g[j][0].x; acc[0].y += (x[j][0].y + gl[0].y) * g[j][0].y;
+        acc[0].z += (x[j][0].z + gl[0].z) * g[j][0].z; acc[0].w += (x[j][0].w + gl[0].w) * g[j][0].w;
+      } else {
+        const float4 xr = make_float4(x[j][0].x + gl[0].x, x[j][0].y + gl[0].y, x[j][0].z + gl[0].z, x[j][0].w + gl[0].w);
+        const float4 xi = make_float4(x[j][1].x + gl[1].x, x[j][1].y + gl[1].y, x[j][1].z + gl[1].z, x[j][1].w + gl[1].w);
+        const float4 gr = g[j][0], gi = g[j][1];
+        acc[0].x += xr.x * gr.x + xi.x * gi.x; acc[0].y += xr.y * gr.y + xi.y * gi.y;
+        acc[0].z += xr.z * gr.z + xi.z * gi.z; acc[0].w += xr.w * gr.w + xi.w * gi.w;
+        acc[1].x += xr.x * gi.x - xi.x * gr.x; acc[1].y += xr.y * gi.y - xi.y * gr.y;
+        acc[1].z += xr.z * gi.z - xi.z * gr.z; acc[1].w += xr.w * gi.w - xi.w * gr.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < NA; ++a) sh[a][rg][lane] = acc[a];
+  __syncthreads();
+  if (rg == 0 && q < quads) {
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < kParamGroups; ++g) {
+        const float4 v = sh[a][g][lane];
+        t[0] += v.x; t[1] += v.y; t[2] += v.z; t[3] += v.w;
+      }
+      if (slice == 0 && c.reg_coef != 0.f) {  // N3 on the operator's parameters, as in param_grad_kernel
+        const int64_t r = clamp_index(c.rel[k], c.num_relations);
+        const float c3 = 3.0f * c.reg_coef * (float)c.C;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (reg_op == PBG_OP_COMPLEX_DIAGONAL) {
+            const int col = e + a * H + i, h = col < H ? col : col - H;
+            const float re = sd.p0[r * H + h], im = sd.p1[r * H + h];
+            t[i] += c3 * sqrtf(re * re + im * im) * (col < H ? re : im);
+          } else {
+            const float pv = sd.p0[r * D + e + a * H + i];
+            t[i] += c3 * fabsf(pv) * pv;
+          }
+        }
+      }
+      *reinterpret_cast<float4*>(dth + ((int64_t)k * slices + slice) * D + e + a * H) = make_float4(t[0], t[1], t[2], t[3]);
+    }
+  }
+}
+
+// param_grad_kernel, or its 128-bit form where the rows' length allows it
+void launch_param_grad(const StepCtx& c, int s, float* dth, int slices, int reg_op, hipStream_t stream) {
+  const int D = c.D, K = c.K;
+  const dim3 block(kParamGroups * 64);
+  if (c.op == PBG_OP_COMPLEX_DIAGONAL && D % 8 == 0) {
+    hipLaunchKernelGGL((param_grad_quad_kernel<PBG_OP_COMPLEX_DIAGONAL>), dim3((unsigned)ceil_div(D / 8, 64), (unsigned)K, (unsigned)slices),
+                       block, 0, stream, c, s, dth, slices, reg_op);
+  } else if (c.op == PBG_OP_DIAGONAL && D % 4 == 0) {
+    hipLaunchKernelGGL((param_grad_quad_kernel<PBG_OP_DIAGONAL>), dim3((unsigned)ceil_div(D / 4, 64), (unsigned)K, (unsigned)slices),
+                       block, 0, stream, c, s, dth, slices, reg_op);
+  } else if (c.op == PBG_OP_TRANSLATION && D % 4 == 0) {
+    hipLaunchKernelGGL((param_grad_quad_kernel<PBG_OP_TRANSLATION>), dim3((unsigned)ceil_div(D / 4, 64), (unsigned)K, (unsigned)slices),
+                       block, 0, stream, c, s, dth, slices, reg_op);
+  } else {
+    hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)slices), block, 0, stream, c, s,
+                       dth, slices, reg_op);
+  }
+}
+
 // AsyncAdagrad (async_adagrad.py:75-85), the K batches' gradients applied in order.
 __global__ void param_update_kernel(StepCtx c, int s, const float* __restrict__ dth, int slices, int64_t psize,
                                     float* p0, float* p1, float* s0, float* s1, float lr) {
@@ -1958,15 +2092,13 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
     } else {
       StepCtx cg = c;
       if (edge_terms) cg.op = PBG_OP_TRANSLATION;  // (whose gradient is the column sum of dz)
-      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)plan.pslices[s]),
-                         dim3(kParamGroups * 64), 0, stream, cg, s, plan.dth[s], plan.pslices[s], c.op);
+      launch_param_grad(cg, s, plan.dth[s], plan.pslices[s], c.op, stream);
     }
     if (c.affine) {  // the translation: column sums of dz, then its own Adagrad steps (parameters in the second slot)
       StepCtx ct = c;
       ct.op = PBG_OP_TRANSLATION;
       const int sl = plan.pslices_t[s];
-      hipLaunchKernelGGL(param_grad_kernel, dim3((unsigned)ceil_div(D, 64), (unsigned)K, (unsigned)sl),
-                         dim3(kParamGroups * 64), 0, stream, ct, s, plan.dth_t[s], sl, PBG_OP_TRANSLATION);
+      launch_param_grad(ct, s, plan.dth_t[s], sl, PBG_OP_TRANSLATION, stream);
       if (K <= kWave) {
         hipLaunchKernelGGL(param_update_wave_kernel, dim3((unsigned)ceil_div(D, kWavesPerBlock)), dim3(kRowThreads), 0,
                            stream, ct, s, plan.dth_t[s], sl, (int64_t)D, p1, nullptr, s1, nullptr, d->relation_lr);
