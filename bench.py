@@ -88,7 +88,7 @@ WORKLOADS = {
                        entities=100_000, edges=1_000_000, dim=200, batch=1000, batch_negs=50, uniform_negs=50,
                        operator="translation", comparator="l2", loss="ranking", relations=1, dynamic=False,
                        init_scale=1e-3, zipf=None, two_tables=False),
-    "d200": dict(desc="as d400 at dim 200 (13 column tiles, the last half padding)",
+    "d200": dict(desc="as d400 at dim 200",
                  entities=14_951, edges=483_142, dim=200, batch=1000, batch_negs=50, uniform_negs=50,
                  operator="complex_diagonal", comparator="dot", loss="softmax", relations=1345, dynamic=False,
                  init_scale=1e-3, zipf=1.1, two_tables=False),

@@ -676,9 +676,9 @@ int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, 
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
   f->sliced = 0;
   if (c.dynamic) return false;
-  // complex_diagonal: on slices only (pairs of coordinates, see sliced_chunk_kernel), with dot, in fp32
+  // complex_diagonal: on slices only (pairs of coordinates, see sliced_chunk_kernel), with dot
   const bool cplx = c.op == PBG_OP_COMPLEX_DIAGONAL;
-  if (cplx && (c.D <= 128 || c.D % 8 != 0 || c.cmp != PBG_CMP_DOT || c.half)) return false;
+  if (cplx && (c.D <= 128 || c.D % 8 != 0 || c.cmp != PBG_CMP_DOT)) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL && !cplx) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;

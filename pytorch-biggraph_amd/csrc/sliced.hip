@@ -550,8 +550,11 @@ int launch_sliced_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes,
 int sliced_chunks(const StepCtx& c, const FusedLayout& fl, int blocks, hipStream_t s) {
   const size_t lds_bytes = (size_t)fl.total * sizeof(float);
   if (!c.fused_rowid) return fail(PBG_ERR_INVALID, "step: the sliced chunk kernel reads its row ids from fused_ids");
-  // (complex_diagonal: with dot, in fp32 -- what fused_layout lets through)
-  if (c.op == PBG_OP_COMPLEX_DIAGONAL) return launch_sliced_cmp<PBG_CMP_DOT, false, true>(c, fl, lds_bytes, s, blocks);
+  // (complex_diagonal: with dot -- what fused_layout lets through)
+  if (c.op == PBG_OP_COMPLEX_DIAGONAL) {
+    if (c.half) return launch_sliced_cmp<PBG_CMP_DOT, true, true>(c, fl, lds_bytes, s, blocks);
+    return launch_sliced_cmp<PBG_CMP_DOT, false, true>(c, fl, lds_bytes, s, blocks);
+  }
   if (c.half) {  // (dot and cos only: the step's validation has refused the rest)
     if (c.cmp == PBG_CMP_COS) return launch_sliced_cmp<PBG_CMP_COS, true>(c, fl, lds_bytes, s, blocks);
     if (c.cmp == PBG_CMP_DOT) return launch_sliced_cmp<PBG_CMP_DOT, true>(c, fl, lds_bytes, s, blocks);

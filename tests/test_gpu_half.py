@@ -101,6 +101,10 @@ for op, cmp_, loss in itertools.product(("none", "translation", "diagonal"), ("d
 HALF_CASES += [
     dict(operator="none", comparator="cos", loss="logistic", dynamic=False, num_batch_negs=33, num_uniform_negs=17, num_pos=70, dim=200),
     dict(operator="none", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=16, num_uniform_negs=49, num_pos=40, dim=132),
+    # complex_diagonal on slices of 64 coordinate pairs
+    dict(operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=400),
+    dict(operator="complex_diagonal", comparator="dot", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=50, num_pos=100, dim=256),
+    dict(operator="complex_diagonal", comparator="dot", loss="logistic", dynamic=False, num_batch_negs=33, num_uniform_negs=17, num_pos=70, dim=136),
 ]
 
 
