@@ -1337,6 +1337,152 @@ __global__ __launch_bounds__(64) void dyn_param_apply_kernel(StepCtx c, const ui
   }
 }
 
+// The same two kernels for rows whose length is a multiple of 4 (of 8 with complex_diagonal): four columns -- four
+// (real, imaginary) pairs -- per lane as 128-bit loads, so one workgroup per run instead of one per 64 elements,
+// every sum in dyn_param_grad_kernel's order.  The grad kernel also leaves at a run's first position where the
+// relation's next run starts (-1: none), so that the apply kernel's walk is one dependent load per run instead
+// of a scan of the run's keys.
+template <int OP>
+__global__ __launch_bounds__(256) void dyn_param_grad_quad_kernel(StepCtx c, int s, const uint64_t* __restrict__ keys,
+                                                                  const uint32_t* __restrict__ vals, float* __restrict__ grun,
+                                                                  int64_t* __restrict__ run_next) {
+  constexpr bool cplx = OP == PBG_OP_COMPLEX_DIAGONAL;
+  constexpr int NA = cplx ? 2 : 1;
+  __shared__ float4 sh[NA][4][64];
+  __shared__ int64_t sh_end;
+  const SideCtx& sd = c.side[s];
+  const int64_t n = (int64_t)c.K * c.B;
+  const int64_t i = blockIdx.x;
+  const uint64_t key = keys[i];
+  if (i > 0 && keys[i - 1] == key) return;  // not the first position of a run
+  const int lane = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int D = c.D, H = D / 2;
+  const int quads = (cplx ? H : D) >> 2;
+  const int q = blockIdx.y * 64 + lane;
+  const int e = 4 * min(q, quads - 1);  // (lanes past the last quad read the last one and store nothing)
+  const int64_t end = block_scan_end(keys, i, n, key, 0, &sh_end);
+  if (blockIdx.y == 0 && threadIdx.x == 0)
+    run_next[i] = (end < n && (keys[end] >> c.kbits) == (key >> c.kbits)) ? end : -1;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 acc[NA];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) acc[a] = zero;
+  auto add_term = [&](const float4 (&g)[NA], const float4 (&x)[NA]) {
+    if constexpr (OP == PBG_OP_TRANSLATION) {
+      acc[0].x += g[0].x; acc[0].y += g[0].y; acc[0].z += g[0].z; acc[0].w += g[0].w;
+    } else if constexpr (!cplx) {
+      acc[0].x += x[0].x * g[0].x; acc[0].y += x[0].y * g[0].y; acc[0].z += x[0].z * g[0].z; acc[0].w += x[0].w * g[0].w;
+    } else {
+      acc[0].x += x[0].x * g[0].x + x[1].x * g[1].x; acc[0].y += x[0].y * g[0].y + x[1].y * g[1].y;
+      acc[0].z += x[0].z * g[0].z + x[1].z * g[1].z; acc[0].w += x[0].w * g[0].w + x[1].w * g[1].w;
+      acc[1].x += x[0].x * g[1].x - x[1].x * g[0].x; acc[1].y += x[0].y * g[1].y - x[1].y * g[0].y;
+      acc[1].z += x[0].z * g[1].z - x[1].z * g[0].z; acc[1].w += x[0].w * g[1].w - x[1].w * g[0].w;
+    }
+  };
+  auto load_edge = [&](int64_t edge, float4 (&g)[NA], float4 (&x)[NA]) {
+    const float* dz = sd.dz + edge * D + e;
+    const float* xr = OP == PBG_OP_TRANSLATION ? dz : sd.w + clamp_index(sd.idx[edge], sd.num_rows) * D + e;
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      g[a] = *reinterpret_cast<const float4*>(dz + a * H);
+      x[a] = OP == PBG_OP_TRANSLATION ? zero : *reinterpret_cast<const float4*>(xr + a * H);
+    }
+  };
+  int64_t r = i + rg;
+  for (; r + 4 < end; r += 8) {  // two edges' chains of loads (value -> index -> rows) in flight
+    const int64_t e0 = vals[r], e1 = vals[r + 4];
+    float4 g0[NA], x0[NA], g1[NA], x1[NA];
+    load_edge(e0, g0, x0);
+    load_edge(e1, g1, x1);
+    add_term(g0, x0);
+    add_term(g1, x1);
+  }
+  if (r < end) {
+    float4 g0[NA], x0[NA];
+    load_edge(vals[r], g0, x0);
+    add_term(g0, x0);
+  }
+#pragma unroll
+  for (int a = 0; a < NA; ++a) sh[a][rg][lane] = acc[a];
+  __syncthreads();
+  if (rg == 0 && q < quads) {
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      const float4 v0 = sh[a][0][lane], v1 = sh[a][1][lane], v2 = sh[a][2][lane], v3 = sh[a][3][lane];
+      float4 g = make_float4((v0.x + v1.x) + (v2.x + v3.x), (v0.y + v1.y) + (v2.y + v3.y), (v0.z + v1.z) + (v2.z + v3.z),
+                             (v0.w + v1.w) + (v2.w + v3.w));
+      // N3 on the parameters of the run's edges (regularizers.py:73-76), from the values before this call
+      if (c.reg_coef != 0.f) {
+        const float4 rp = *reinterpret_cast<const float4*>(sd.reg_pgrad + (key >> c.kbits) * D + e + a * H);
+        const float cnt = (float)(end - i);
+        g.x += cnt * rp.x; g.y += cnt * rp.y; g.z += cnt * rp.z; g.w += cnt * rp.w;
+      }
+      *reinterpret_cast<float4*>(grun + i * D + e + a * H) = g;
+    }
+  }
+}
+
+__global__ __launch_bounds__(64) void dyn_param_apply_quad_kernel(StepCtx c, const uint64_t* __restrict__ keys,
+                                                                  const float* __restrict__ grun,
+                                                                  const int64_t* __restrict__ run_next, float* p0, float* p1,
+                                                                  float* s0, float* s1, float lr) {
+  const int64_t i = blockIdx.x;
+  const uint64_t rel = keys[i] >> c.kbits;
+  if (i > 0 && (keys[i - 1] >> c.kbits) == rel) return;  // not the first position of a relation
+  const int lane = threadIdx.x;
+  const int D = c.D, H = D / 2;
+  const int q = blockIdx.y * 64 + lane;
+  const bool on = q < (D >> 2);
+  const int e = 4 * min(q, (D >> 2) - 1);
+  float* p;
+  float* st;
+  if (c.op == PBG_OP_COMPLEX_DIAGONAL) {  // (H is a multiple of 4 here: a quad lies in one half)
+    p = (e < H) ? p0 + rel * H + e : p1 + rel * H + (e - H);
+    st = (e < H) ? s0 + rel * H + e : s1 + rel * H + (e - H);
+  } else {
+    p = p0 + rel * D + e;
+    st = s0 + rel * D + e;
+  }
+  float4 pv = *reinterpret_cast<const float4*>(p), sum = *reinterpret_cast<const float4*>(st);
+  int64_t j = i;
+  while (j >= 0) {
+    const float4 g = *reinterpret_cast<const float4*>(grun + j * D + e);
+    const int64_t next = run_next[j];
+    sum.x += g.x * g.x; sum.y += g.y * g.y; sum.z += g.z * g.z; sum.w += g.w * g.w;
+    pv.x += -lr * (g.x / (sqrtf(sum.x) + 1e-10f)); pv.y += -lr * (g.y / (sqrtf(sum.y) + 1e-10f));
+    pv.z += -lr * (g.z / (sqrtf(sum.z) + 1e-10f)); pv.w += -lr * (g.w / (sqrtf(sum.w) + 1e-10f));
+    j = next;
+  }
+  if (on) {
+    *reinterpret_cast<float4*>(st) = sum;
+    *reinterpret_cast<float4*>(p) = pv;
+  }
+}
+
+// The two kernels of an element-wise operator's parameters with one relation per edge, in their 128-bit form where
+// the rows' length allows it.
+void launch_dyn_params(const StepCtx& c, int s, int64_t ne, const uint64_t* rkeys, const uint32_t* rvals, float* grun,
+                       int64_t* run_next, float* p0, float* p1, float* s0, float* s1, float lr, hipStream_t stream) {
+  const int D = c.D;
+  const bool cplx = c.op == PBG_OP_COMPLEX_DIAGONAL;
+  if (D % (cplx ? 8 : 4) != 0 || (c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL && !cplx)) {
+    hipLaunchKernelGGL(dyn_param_grad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c, s,
+                       rkeys, rvals, grun);
+    hipLaunchKernelGGL(dyn_param_apply_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(64), 0, stream, c, rkeys,
+                       grun, p0, p1, s0, s1, lr);
+    return;
+  }
+  const dim3 grid((unsigned)ne, (unsigned)ceil_div((cplx ? D / 2 : D) / 4, 64));
+  if (cplx)
+    hipLaunchKernelGGL((dyn_param_grad_quad_kernel<PBG_OP_COMPLEX_DIAGONAL>), grid, dim3(256), 0, stream, c, s, rkeys, rvals, grun, run_next);
+  else if (c.op == PBG_OP_DIAGONAL)
+    hipLaunchKernelGGL((dyn_param_grad_quad_kernel<PBG_OP_DIAGONAL>), grid, dim3(256), 0, stream, c, s, rkeys, rvals, grun, run_next);
+  else
+    hipLaunchKernelGGL((dyn_param_grad_quad_kernel<PBG_OP_TRANSLATION>), grid, dim3(256), 0, stream, c, s, rkeys, rvals, grun, run_next);
+  hipLaunchKernelGGL(dyn_param_apply_quad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D / 4, 64)), dim3(64), 0, stream, c,
+                     rkeys, grun, run_next, p0, p1, s0, s1, lr);
+}
+
 // ---------------------------------------------------------------------------
 // N3 regularizer: parameter terms and the per-batch value
 // ---------------------------------------------------------------------------
@@ -1536,6 +1682,7 @@ struct Plan {
   uint32_t *rvals_a, *rvals_b;
   void* rsort_temp;
   void* rel_start;  // first sorted position of every relation (`linear` only)
+  int64_t* dyn_next;  // ... and at the same position where the relation's next run starts (-1: none) [K * B]
   float* dyn_grun;  // element-wise operators: the parameter gradient of every (relation, batch) run, at the run's first sorted position [K * B, D]
   int nvh;
   float* gth;   // partial sums of the global embeddings' gradients [2, K, gslices, D]
@@ -1743,7 +1890,10 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
     plan->rvals_b = (uint32_t*)take(ne, 4);
     plan->rsort_temp = take(sort_temp_bytes(ne), 1);
     if (c.op == PBG_OP_LINEAR) plan->rel_start = take(seg_linear_update_temp_bytes(c.num_relations, ne, D, K), 1);
-    if (c.op != PBG_OP_LINEAR || c.affine) plan->dyn_grun = takef((size_t)ne * D);
+    if (c.op != PBG_OP_LINEAR || c.affine) {
+      plan->dyn_grun = takef((size_t)ne * D);
+      plan->dyn_next = (int64_t*)take(ne, 8);
+    }
   }
   for (int s = 0; s < 2; ++s) {
     plan->pslices[s] = 1;
@@ -2054,16 +2204,10 @@ int run_params(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan& pl
         if (c.affine) {  // the translations: the element-wise kernel on dz, parameters in the second slot
           StepCtx ct = c;
           ct.op = PBG_OP_TRANSLATION;
-          hipLaunchKernelGGL(dyn_param_grad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream,
-                             ct, s, rkeys, rvals, plan.dyn_grun);
-          hipLaunchKernelGGL(dyn_param_apply_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(64), 0, stream,
-                             ct, rkeys, plan.dyn_grun, p1, nullptr, s1, nullptr, d->relation_lr);
+          launch_dyn_params(ct, s, ne, rkeys, rvals, plan.dyn_grun, plan.dyn_next, p1, nullptr, s1, nullptr, d->relation_lr, stream);
         }
       } else {
-        hipLaunchKernelGGL(dyn_param_grad_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(256), 0, stream, c,
-                           s, rkeys, rvals, plan.dyn_grun);
-        hipLaunchKernelGGL(dyn_param_apply_kernel, dim3((unsigned)ne, (unsigned)ceil_div(D, 64)), dim3(64), 0, stream, c,
-                           rkeys, plan.dyn_grun, p0, p1, s0, s1, d->relation_lr);
+        launch_dyn_params(c, s, ne, rkeys, rvals, plan.dyn_grun, plan.dyn_next, p0, p1, s0, s1, d->relation_lr, stream);
       }
     }
     return check_launch("step params (dynamic)");
