@@ -32,7 +32,7 @@ FP16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16, what --half-precision's products a
 # WRITE_SIZE runs summarised in profiles/train_step_pmc_traffic.md (not measured live);
 # any other combination reports null.
 TRAFFIC = {("cfg1", "fused_chunk", 64): 233.3e6, ("cfg4", "fused_chunk", 64): 225.5e6,
-           ("cfg2", "stream_chunk", 64): 13960.2e6}
+           ("cfg2", "stream_chunk", 64): 13957.7e6}
 
 # name -> the fields of BASELINE.json's configs
 WORKLOADS = {
