@@ -78,6 +78,12 @@ CASES = {
                        num_uniform_negs=50, entities=3000, scale=0.1, zipf=1.5, ks=(20, 65)),
     "sliced-transe": dict(operator="translation", comparator="l2", loss="ranking", dim=200, num_pos=200, num_batch_negs=50,
                           num_uniform_negs=50, entities=20000, relations=4, scale=0.1, zipf=1.5, shared=False, ks=(64,)),
+    # a table of 40 rows under a power law: the update takes a wave per table row, and the hot rows' runs are
+    # hundreds of sorted positions long (many windows of 64 positions per run)
+    "hot-row-walk": dict(operator="none", comparator="dot", loss="logistic", dim=100, num_pos=400, num_batch_negs=50,
+                         num_uniform_negs=50, entities=40, scale=0.1, zipf=1.5, ks=(8, 20)),
+    "hot-row-walk-wide": dict(operator="diagonal", comparator="cos", loss="softmax", dim=256, num_pos=300, num_batch_negs=50,
+                              num_uniform_negs=50, entities=25, relations=3, scale=0.1, zipf=1.3, shared=False, ks=(5,)),
     # global embeddings: their update walks the batches in blocks of 64
     "global-fused": dict(operator="none", comparator="dot", loss="logistic", dim=100, num_pos=200, num_batch_negs=50,
                          num_uniform_negs=50, entities=3000, scale=0.1, global_emb=True, ks=(64, 65, 130)),
