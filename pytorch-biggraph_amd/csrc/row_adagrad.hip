@@ -662,22 +662,40 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
   // round trips per 32 positions.)
   const int nb = 1 << kbits;
   const int64_t row_end = lower_bound_key(keys, long_i, n, (long_row + 1) << kbits);
-  uint32_t run = 0;  // start (relative to long_i) of the run whose gradient long_g holds
+  // (The starts do not decrease with the batch, and an absent batch has the start of the next one present: the runs
+  // still to apply are the starts that differ from the one before them -- from 0, the run in hand, for the first.)
+  uint32_t last_st = 0;  // the start of the last batch of the 32 before
+  constexpr int kAhead = 8;  // gradient rows in flight: a hot row's runs are otherwise one memory round trip each
 #pragma unroll 1
   for (int b0 = 0; b0 < nb; b0 += 32) {
     const int b = b0 + gl;
     const int64_t at = b < nb ? lower_bound_key(keys, long_i, row_end, (long_row << kbits) | (uint64_t)b) : row_end;
     const uint32_t st = (uint32_t)(at - long_i);    // first position of batch b (of the next batch present, if absent)
     const uint32_t sv = vals[at < n ? at : n - 1];  // and the gradient row there
+    uint32_t st_prev = (uint32_t)__shfl_up((int)st, 1, 32);
+    if (gl == 0) st_prev = last_st;
+    uint32_t todo = (uint32_t)(__ballot(b < nb && st != st_prev && (int64_t)st < row_end - long_i) >> gbase);
+    last_st = (uint32_t)__shfl((int)st, gbase + 31, 64);
 #pragma unroll 1
-    for (int j = 0; j < 32 && b0 + j < nb; ++j) {
-      const uint32_t s_b = (uint32_t)__shfl((int)st, gbase + j, 64);
-      if (s_b == run || (int64_t)s_b >= row_end - long_i) continue;  // batch absent, or it is the run in hand
-      const uint32_t v_b = (uint32_t)__shfl((int)sv, gbase + j, 64);
-      const float4 next = load_or_zero(grad_rows + (int64_t)v_b * dim + col, has);
-      long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
-      long_g = next;
-      run = s_b;
+    while (todo != 0u) {
+      int js[kAhead];
+      float4 nx[kAhead];
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t) {
+        js[t] = todo != 0u ? __ffs((int)todo) - 1 : -1;
+        todo &= todo - 1;  // (0 stays 0)
+      }
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t) {
+        const uint32_t v_b = (uint32_t)__shfl((int)sv, gbase + (js[t] >= 0 ? js[t] : 0), 64);
+        nx[t] = load_or_zero(grad_rows + (int64_t)v_b * dim + col, has && js[t] >= 0);
+      }
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t) {
+        if (js[t] < 0) break;
+        long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
+        long_g = nx[t];
+      }
     }
   }
   long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
