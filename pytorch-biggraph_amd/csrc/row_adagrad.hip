@@ -316,6 +316,17 @@ __device__ __forceinline__ float adagrad_apply(RowRegs<NV, VEC>& w, const RowReg
   return gsum;
 }
 
+// first position in [lo, hi) whose key is >= want (hi if none)
+__device__ __forceinline__ int64_t lower_bound_key(const uint64_t* __restrict__ keys, int64_t lo, int64_t hi,
+                                                   uint64_t want) {
+  while (lo < hi) {
+    const int64_t mid = lo + ((hi - lo) >> 1);
+    if (keys[mid] < want) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo;
+}
+
 // One wave looks at R consecutive sorted positions; a position that starts a row
 // gets the row's update.  All loads that do not depend on each other (the R key
 // windows, then the weight rows and first gradient rows of the positions that
@@ -373,6 +384,7 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
         g[r].add_if(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane, fold && t < run_len);
     }
   }
+  int long_r = -1;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (!head[r]) continue;
@@ -394,19 +406,75 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
         g[r] = next;
       }
       gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+    } else if (kbits == 0) {  // a single-worker call has one run per row
+      gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
     } else {
-      int64_t j = i;
-      while (true) {
-        // a single-worker call has one run per row: no need to look for its end
-        j = (kbits == 0) ? n : scan_end(keys, j, n, keys[j], 0, lane);
-        gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
-        if (j >= n || (keys[j] >> kbits) != row) break;
-        g[r].load(grad_rows + (int64_t)vals[j] * dim, nv, lane);
-      }
+      // A long row: handled after this loop.  There is at most one per wave (the positions after its head belong
+      // to it), so the code below exists once instead of once per position, in the registers that this loop's rows
+      // no longer need.
+      long_r = r;
+      continue;
     }
     w[r].store(wrow[r], nv, lane);
     if (lane == 0) *gptr[r] = gsum[r];
   }
+  if (long_r < 0) return;
+  // (only the position is carried out of the loop above: the row's weights, sum and first gradient are fetched again)
+  const int64_t i = first + long_r;
+  const uint64_t row = keys[i] >> kbits;
+  float* long_wrow = (int64_t)row < rows0 ? w0 + (int64_t)row * dim : w1 + ((int64_t)row - rows0) * dim;
+  float* long_gptr = (int64_t)row < rows0 ? g0 + row : g1 + ((int64_t)row - rows0);
+  RowRegs<NV, VEC> lw, lg;
+  lw.load(long_wrow, nv, lane);
+  float lsum = *long_gptr;
+  lg.load(grad_rows + (int64_t)vals[i] * dim, nv, lane);
+  // A long row (a hot entity of a power-law graph): one run per batch that names it, hundreds of positions
+  // each.  Lane l finds the first position of batch b0 + l by binary search in the sorted keys, 64 batches at
+  // once, and fetches the number of the gradient row there; the runs are then applied in batch order with the
+  // next kAhead runs' gradients in flight.  (Walking from run to run costs a chain of dependent loads per run:
+  // the keys of every 64 positions of the run, the row's number, the row.)
+  // The starts do not decrease with the batch, and an absent batch has the start of the next one present: the
+  // runs still to apply are the starts that differ from the one before them -- from 0, the run in hand, at first.
+  constexpr int kRowRegs = NV * RowRegs<NV, VEC>::W;
+  constexpr int kAhead = kRowRegs >= 32 ? 1 : (kRowRegs >= 16 ? 2 : (kRowRegs >= 8 ? 4 : 8));
+  const int nb = 1 << kbits;
+  const int64_t row_end = lower_bound_key(keys, i, n, (row + 1) << kbits);
+  uint32_t last_st = 0;
+#pragma unroll 1
+  for (int b0 = 0; b0 < nb; b0 += kWave) {
+    const int b = b0 + lane;
+    const int64_t at = b < nb ? lower_bound_key(keys, i, row_end, (row << kbits) | (uint64_t)b) : row_end;
+    const uint32_t st = (uint32_t)(at - i);
+    const uint32_t sv = vals[at < n ? at : n - 1];
+    uint32_t st_prev = (uint32_t)__shfl_up((int)st, 1, 64);
+    if (lane == 0) st_prev = last_st;
+    uint64_t todo = __ballot(b < nb && st != st_prev && (int64_t)st < row_end - i);
+    last_st = lane_u32(st, kWave - 1);
+#pragma unroll 1
+    while (todo != 0ull) {
+      int js[kAhead];
+      RowRegs<NV, VEC> nx[kAhead];
+      const int j0 = __ffsll((unsigned long long)todo) - 1;
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t) {
+        js[t] = todo != 0ull ? __ffsll((unsigned long long)todo) - 1 : -1;
+        todo &= todo - 1;  // (0 stays 0)
+      }
+      // all loads are issued before the first is used; slots past the last run read the first row again and are dropped
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t)
+        nx[t].load(grad_rows + (int64_t)lane_u32(sv, js[t] >= 0 ? js[t] : j0) * dim, nv, lane);
+#pragma unroll
+      for (int t = 0; t < kAhead; ++t) {
+        if (js[t] < 0) break;
+        lsum = adagrad_apply(lw, lg, lsum, fdim, lr);
+        lg = nx[t];
+      }
+    }
+  }
+  lsum = adagrad_apply(lw, lg, lsum, fdim, lr);
+  lw.store(long_wrow, nv, lane);
+  if (lane == 0) *long_gptr = lsum;
 }
 
 // One wave per TABLE row, for calls whose gradient rows outnumber the tables' rows many
@@ -525,16 +593,6 @@ __device__ __forceinline__ float half_sum(float v) {  // sum over the 32 lanes o
   return v + __shfl_xor(v, 16, 64);
 }
 constexpr int kMaxBatchSlots = 8;  // batches per lane of a half wave: 256 batches per call at most
-// first position in [lo, hi) whose key is >= want (hi if none)
-__device__ __forceinline__ int64_t lower_bound_key(const uint64_t* __restrict__ keys, int64_t lo, int64_t hi,
-                                                   uint64_t want) {
-  while (lo < hi) {
-    const int64_t mid = lo + ((hi - lo) >> 1);
-    if (keys[mid] < want) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo;
-}
 __device__ __forceinline__ float4 load_or_zero(const float* __restrict__ p, bool has) {
   return has ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
 }
