@@ -436,7 +436,7 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   // The starts do not decrease with the batch, and an absent batch has the start of the next one present: the
   // runs still to apply are the starts that differ from the one before them -- from 0, the run in hand, at first.
   constexpr int kRowRegs = NV * RowRegs<NV, VEC>::W;
-  constexpr int kAhead = kRowRegs >= 32 ? 1 : (kRowRegs >= 16 ? 2 : (kRowRegs >= 8 ? 4 : 8));
+  constexpr int kAhead = kRowRegs > 16 ? 1 : (kRowRegs * R > 16 ? 4 : (kRowRegs > 4 ? 2 : 8));  // (within the registers of the loop above)
   const int nb = 1 << kbits;
   const int64_t row_end = lower_bound_key(keys, i, n, (row + 1) << kbits);
   uint32_t last_st = 0;
