@@ -809,9 +809,9 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
   const int64_t borders = ceil_div(n, kTile) - 1;
   const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
-  // gradient rows outnumbering the tables' rows 16 times over: a wave per table row (row_walk_kernel)
+  // gradient rows outnumbering the tables' rows 32 times over: a wave per table row (row_walk_kernel)
   const int64_t table_rows = rows0 + rows1;
-  const bool walk = kbits > 0 && table_rows > 0 && n >= 16 * table_rows && getenv("PBG_DISABLE_ROW_WALK") == nullptr;
+  const bool walk = kbits > 0 && table_rows > 0 && n >= 32 * table_rows && getenv("PBG_DISABLE_ROW_WALK") == nullptr;
   const dim3 walk_grid((unsigned)ceil_div(table_rows > 0 ? table_rows : 1, wpb));
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
