@@ -676,14 +676,14 @@ int launch_fused_cmp(const StepCtx& c, const FusedLayout& fl, size_t lds_bytes, 
 bool fused_layout(const StepCtx& c, FusedLayout* f) {
   f->sliced = 0;
   if (c.dynamic) return false;
-  // complex_diagonal: on slices only (pairs of coordinates, see sliced_chunk_kernel), with dot
+  // complex_diagonal: on slices only (pairs of coordinates, see sliced_chunk_kernel; a single slice up to dim 128), with dot
   const bool cplx = c.op == PBG_OP_COMPLEX_DIAGONAL;
-  if (cplx && (c.D <= 128 || c.D % 8 != 0 || c.cmp != PBG_CMP_DOT)) return false;
+  if (cplx && (c.D % 8 != 0 || c.cmp != PBG_CMP_DOT)) return false;
   if (c.op != PBG_OP_NONE && c.op != PBG_OP_TRANSLATION && c.op != PBG_OP_DIAGONAL && !cplx) return false;
   if (c.cmp != PBG_CMP_DOT && c.cmp != PBG_CMP_L2 && c.cmp != PBG_CMP_COS) return false;
   if (c.D % 4 != 0 || c.P > 64 || c.U > 64) return false;
   // rows wider than 128 floats pass through LDS in slices (sliced_chunk_kernel): fp32
-  const bool sliced = c.D > 128;
+  const bool sliced = c.D > 128 || cplx;
   if (sliced && getenv("PBG_DISABLE_SLICED") != nullptr)
     return false;
   if (c.side[0].num_rows >= ((int64_t)1 << 31) || c.side[1].num_rows >= ((int64_t)1 << 31)) return false;

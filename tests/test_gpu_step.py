@@ -971,6 +971,11 @@ def _sliced_cases():
         dict(operator="complex_diagonal", comparator="dot", loss="ranking", num_batch_negs=17, num_uniform_negs=64, num_pos=40, dim=1024),
         dict(operator="complex_diagonal", comparator="dot", loss="logistic", num_batch_negs=64, num_uniform_negs=5, num_pos=100, dim=200),
         dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=48, num_uniform_negs=16, num_pos=96, dim=648),
+        # ... and a single slice up to dim 128
+        dict(operator="complex_diagonal", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=130, dim=128),
+        dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=50, num_uniform_negs=50, num_pos=100, dim=64),
+        dict(operator="complex_diagonal", comparator="dot", loss="logistic", num_batch_negs=17, num_uniform_negs=33, num_pos=40, dim=104),
+        dict(operator="complex_diagonal", comparator="dot", loss="softmax", num_batch_negs=5, num_uniform_negs=3, num_pos=12, dim=8),
     ]
     return cases
 
