@@ -161,6 +161,35 @@ def test_group_by_relation_type_and_batchers(pbg):
     assert seen == sorted(zip(lhs.tolist(), rhs.tolist(), rel.tolist()))
 
 
+def test_relation_batches_of_a_group_beyond_2_pow_24_edges(pbg, monkeypatch):
+    """A relation type with more than 2**24 edges (a single-relation bucket of the
+    LiveJournal example has 62 M): a float32 count of the edges left cannot step by
+    one there.  Groups are stand-ins that only know their length."""
+    import itertools
+    B = pbg.batching
+
+    class Span:
+        def __init__(self, n):
+            self.n = n
+
+        def __len__(self):
+            return self.n
+
+        def __getitem__(self, sl):
+            start, stop, _ = sl.indices(self.n)
+            return Span(max(stop - start, 0))
+
+    sizes = [2 ** 24 + 3, 5, 2 ** 24 + 1]
+    monkeypatch.setattr(B, "group_by_relation_type", lambda edges: [Span(n) for n in sizes])
+    torch.manual_seed(0)
+    batch_size = 4099
+    want = sum(-(-n // batch_size) for n in sizes)
+    got = list(itertools.islice(B.batch_edges_group_by_relation_type(None, batch_size=batch_size), want + 10))
+    assert len(got) == want
+    assert sum(len(g) for g in got) == sum(sizes)
+    assert all(0 < len(g) <= batch_size for g in got)
+
+
 def test_argument_validation_without_gpu(pbg):
     with pytest.raises(ValueError, match="even dimension"):
         pbg.operators.ComplexDiagonalOperator(3)
