@@ -434,7 +434,10 @@ class StepRunner:
     def route(self) -> str:
         """Which kernels the step runs: "staged", "fused" (one LDS-resident chunk
         kernel) or "stream" (positives in LDS, negatives streamed past them)."""
-        return ("staged", "fused", "stream")[_lib.lib().pbg_train_step_route(ctypes.byref(self.desc))]
+        code = _lib.lib().pbg_train_step_route(ctypes.byref(self.desc))
+        if code < 0:  # an invalid descriptor: -1 must not read as the last name
+            raise ValueError(_lib.lib().pbg_last_error().decode("utf-8", "replace") or "invalid step descriptor")
+        return ("staged", "fused", "stream")[code]
 
     def train_profiled(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None,
                        uniform_seed=None) -> List[float]:

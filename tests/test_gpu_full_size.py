@@ -71,8 +71,13 @@ FULL = {
     "cfg2-1000-batch-negs": dict(entities=14_951, relations=1345, dim=400, batch=1000, nb=1000, nu=0,
                                  operator="complex_diagonal", comparator="dot", loss="softmax", dynamic=False,
                                  zipf=1.1, two_tables=False),
+    # the graph as BASELINE states it: out-degree Zipf(2.0) capped at 20 000, targets by preferential attachment
+    # (bench.livejournal_like_edges, all 68 993 773 edges, the same generator the bench line runs on)
     "cfg3": dict(entities=4_847_571, relations=1, dim=1024, batch=10_000, nb=1000, nu=100, operator="none",
-                 comparator="dot", loss="softmax", dynamic=False, zipf=2.0, two_tables=False),
+                 comparator="dot", loss="softmax", dynamic=False, zipf=2.0, two_tables=False, graph="livejournal"),
+    # a harsher graph than stated: both endpoints i.i.d. Zipf(2.0) without a cap, one entity holds 60 % of a batch
+    "cfg3-hot": dict(entities=4_847_571, relations=1, dim=1024, batch=10_000, nb=1000, nu=100, operator="none",
+                     comparator="dot", loss="softmax", dynamic=False, zipf=2.0, two_tables=False),
     "cfg4": dict(entities=10_413_058, relations=1, dim=100, batch=1000, nb=50, nu=50, operator="translation",
                  comparator="l2", loss="ranking", dynamic=False, zipf=1.8, two_tables=True),
     "cfg5-standard": dict(entities=2_000_000, relations=500, dim=256, batch=2000, nb=100, nu=100, operator="linear",
@@ -109,9 +114,16 @@ def test_full_shape_step(pbg, name, workers):
     def draw(n):
         return zipf_ids(n, e, w["zipf"], gen) if w["zipf"] else torch.randint(0, e, (n,), generator=gen)
 
+    graph = None
+    if w.get("graph") == "livejournal":
+        import bench
+        graph = bench.livejournal_like_edges(e, 68_993_773, w["zipf"], 20_000, dgen, DEV)
+        graph = (graph[0][:workers * b].cpu(), graph[1][:workers * b].cpu())
+        torch.cuda.empty_cache()
+
     batches = []
-    for _ in range(workers):
-        lhs, rhs = draw(b), draw(b)
+    for k in range(workers):
+        lhs, rhs = (graph[0][k * b:(k + 1) * b], graph[1][k * b:(k + 1) * b]) if graph else (draw(b), draw(b))
         ul = torch.randint(0, e, (c, u), generator=gen)
         ur = torch.randint(0, e, (c, u), generator=gen)
         if w["dynamic"]:
