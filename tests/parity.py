@@ -160,6 +160,33 @@ def hinge_ties(cfg, scores, eps=2e-6):
     return n
 
 
+def tie_free_batches(cfg, st64, candidates, steps, eps):
+    """The first `steps` of `candidates` that, taken in order along a float64 run of
+    the oracle from `st64`, have no live hinge argument (neg - pos) + margin within
+    eps * max(1, largest |score|) of 0; a candidate that has one is skipped.  `st64`
+    is advanced through the kept batches.  Returns (kept, number of candidates looked at)."""
+    from oracle import step as ostep
+
+    kept, looked = [], 0
+    for b in candidates:
+        if len(kept) == steps:
+            break
+        looked += 1
+        sc = ostep.forward_backward(cfg, st64, *b, keep_scores=True)[0].scores
+        nearest, largest = float("inf"), 1.0
+        for pos, neg in ((sc.lhs_pos, sc.lhs_neg), (sc.rhs_pos, sc.rhs_neg)):
+            live = neg > -1e8  # masked entries hold -1e9 and never reach the hinge
+            x = ((neg - pos.unsqueeze(1)) + cfg.margin)[live]
+            if x.numel():
+                nearest = min(nearest, float(x.abs().min()))
+                largest = max(largest, float(neg[live].abs().max()), float(pos.abs().max()))
+        if nearest < eps * largest:
+            continue
+        ostep.train_step(cfg, st64, *b)
+        kept.append(b)
+    return kept, looked
+
+
 def hinge_tie_rows(cfg, scores, lhs, rhs, uniform_lhs, uniform_rhs, eps=2e-6):
     """(rows of the lhs table, rows of the rhs table) that a hinge tie of this batch
     reaches: the tied edge's two entities and the tied negative's entity (a batch

@@ -190,3 +190,6 @@ def test_many_workers_match_the_lockstep_oracle(pbg, name, workers):
     anchored_state(cfg, runner, st, st64, 1e-5, f"{name} K={workers}", census, loose_rows=loose_rows,
                    loose_steps=2 * tied_batches, param_slack=slack)
     say("  ", census)
+    # the float64 anchor is for the odd entry whose fp32 sum depends on the order of summation,
+    # not a second criterion that everything may pass on
+    assert census.anchored <= max(5, 1e-4 * census.entries), str(census)

@@ -19,7 +19,7 @@ def test_bench_line_has_the_contract_fields():
 
     root = pathlib.Path(__file__).resolve().parent.parent
     out = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "1", "--steps", "20", "--warmup", "5",
-                          "--cpu-seconds", "0", "--no-sequential"], capture_output=True, text=True, timeout=240, cwd=root)
+                          "--cpu-seconds", "0", "--no-sequential", "--configs", "cfg2b,cfg4"], capture_output=True, text=True, timeout=240, cwd=root)
     assert out.returncode == 0, out.stderr[-2000:]
     lines = [ln for ln in out.stdout.splitlines() if ln.startswith("{")]
     assert len(lines) == 1
@@ -38,3 +38,9 @@ def test_bench_line_has_the_contract_fields():
         assert key in roof, key
     assert roof["bound"] in ("hbm", "mfma") and 0 < roof["frac"] < 1
     assert roof["frac"] == pytest.approx(roof["achieved"] / roof["peak"], rel=1e-6)
+    # the other configurations ride along under "configs", each with its own roofline entry
+    assert set(line["configs"]) == {"cfg2b", "cfg4"}
+    for name, entry in line["configs"].items():
+        assert entry["value"] > 0 and entry["sequential_value"] > 0, name
+        assert entry["roofline"]["bound"] in ("hbm", "mfma") and 0 < entry["roofline"]["frac"] < 1, name
+        assert cfg[f"{name}_edges_per_s"] == entry["value"]

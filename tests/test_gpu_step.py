@@ -704,8 +704,18 @@ def test_regularizer_is_refused_for_linear(pbg):
 ], ids=ids)
 def test_hundred_steps(pbg, case):
     """Updated embeddings, Adagrad state and operator parameters after 100
-    sequential steps stay within 1e-4 relative of the CPU path."""
-    from tests.parity import zipf_ids
+    sequential steps stay within 1e-4 relative of the CPU path: ONE run of 100
+    steps on the GPU and one on the oracle, neither ever seeing the other's state.
+
+    max(0, x) has a gradient of 0 on one side of x = 0 and 1 on the other, so two
+    correct fp32 evaluations of a hinge argument within rounding distance of 0 may
+    take different sides, and the runs then part for good (every later hinge near
+    the changed rows may flip too): on such a batch no tolerance means anything.
+    The ranking cases therefore draw their batches along a float64 run of the
+    oracle and redraw a batch in which some live hinge argument lies within 4e-6
+    of 0, relative to the largest score (the GPU's and the CPU's scores agree to
+    about 1e-7); how many were redrawn is printed."""
+    from tests.parity import double_state, tie_free_batches, zipf_ids
 
     say("hundred", case)
     case = dict(case)
@@ -713,30 +723,26 @@ def test_hundred_steps(pbg, case):
     shared, zipf = case.pop("shared", True), case.pop("zipf", None)
     cfg = ostep.StepConfig(dim=dim, num_relations=2, relation_weights=[1.0, 1.0], lr=0.1,
                            dynamic=case.pop("dynamic", False), **case)
-    st, batches = make_inputs(cfg, num_pos, 2000, 100, seed=1, shared=shared,
+    steps = 100
+    st, batches = make_inputs(cfg, num_pos, 2000, steps * (5 if cfg.loss == "ranking" else 1), seed=1, shared=shared,
                               scale=1e-3 if case["operator"] == "none" else 0.1)
     if zipf:
         g = torch.Generator().manual_seed(2)
         batches = [(zipf_ids(num_pos, 2000, zipf, g), zipf_ids(num_pos, 2000, zipf, g)) + b[2:] for b in batches]
+    st64 = double_state(st)
+    if cfg.loss == "ranking":
+        batches, drawn = tie_free_batches(cfg, st64, batches, steps, 4e-6)  # (advances st64 through the kept batches)
+        say("  batches drawn for", steps, "steps without a hinge tie:", drawn)
+    else:
+        for b in batches:
+            ostep.train_step(cfg, st64, *b)
+    assert len(batches) == steps
     runner = to_runner(pbg, cfg, st, num_pos, 1)
-    resyncs = 0
-    for n, b in enumerate(batches):
+    for b in batches:
         runner.train(*pack(cfg, [b]))
-        out = ostep.train_step(cfg, st, *b, keep_scores=cfg.loss == "ranking")
-        if cfg.loss == "ranking" and hinge_ties(cfg, out.scores) > 0:
-            # A negative within rounding distance of the hinge: max(0, x) has a
-            # gradient of 0 on one side and 1 on the other, so two correct fp32
-            # evaluations may take different sides and then drift apart for good.
-            # Such a step is checked on its own at a tolerance that admits one
-            # flipped hinge per row, then the GPU state restarts from the oracle's.
-            torch.cuda.synchronize()
-            compare_state(cfg, runner, st, 5e-2, f"step {n} (hinge tie)")
-            copy_state(runner, st)
-            resyncs += 1
+        ostep.train_step(cfg, st, *b)
     torch.cuda.synchronize()
-    say("  steps restarted from the oracle's state after a hinge tie:", resyncs, "of", len(batches))
-    assert resyncs <= 10, resyncs
-    compare_state(cfg, runner, st, 1e-4, "100 steps")
+    compare_state(cfg, runner, st, 1e-4, "100 steps", st64 if cfg.comparator == "l2" else None)
 
 
 @pytest.mark.parametrize("workers", [1, 8])
