@@ -370,7 +370,8 @@ def standalone_kernels(pkg):
 def perm_kernels(pkg, small=False):
     """Achieved HBM bandwidth of the permutation helpers on cfg4's sizes (41.65M entities in 4 partitions of
     10.4M rows, one bucket of 91.8M edges split 8 x 8).  Algorithmic bytes: reverse_permutation 16 per entry
-    (id read, position written); shuffle_rows 2 * row + 8 per row; randperm 8 per entry (the output alone);
+    (id read, position written); shuffle_rows (in place: scatter into the scratch and copy back) and shuffle_rows_out
+    (into a second buffer) 2 * row + 8 per row; randperm 8 per entry (the output alone);
     sub_bucket 64 per edge (three ids read, two permutation entries looked up, three ids written)."""
     nat = pkg.native
     lib = pkg._lib.lib()
@@ -394,7 +395,11 @@ def perm_kernels(pkg, small=False):
         t = timed(lambda: nat.shuffle_rows(tab, p, scratch))
         out[f"shuffle_rows_{rows}x{d}"] = {"rows": rows, "row_bytes": 4 * d, "ms": t * 1e3,
                                            "GBs": rows * (8 * d + 8) / t / 1e9}
-        del tab, p, scratch
+        dst = scratch.view(torch.float32).view(tab.shape)
+        t = timed(lambda: nat.shuffle_rows_out(tab, p, dst))
+        out[f"shuffle_rows_out_{rows}x{d}"] = {"rows": rows, "row_bytes": 4 * d, "ms": t * 1e3,
+                                               "GBs": rows * (8 * d + 8) / t / 1e9}
+        del tab, p, scratch, dst
     parts = 8
     lhs = torch.randint(0, n_part, (n_edges,), device=dev)
     rhs = torch.randint(0, n_part, (n_edges,), device=dev)
@@ -406,8 +411,16 @@ def perm_kernels(pkg, small=False):
     out["sub_bucket"] = {"edges": n_edges, "parts": f"{parts}x{parts}", "ms": t * 1e3, "GBs": n_edges * 64 / t / 1e9}
     for v in out.values():
         v["frac_of_8TBs"] = v["GBs"] / HBM_PEAK_GBS
+    # The same launches priced in the 128-byte lines they move: an 8-byte access at a random place is a whole line.
+    # reverse_permutation: the id read in order + one line per position written; sub_bucket: 48 bytes per edge in
+    # order + two permutation look-ups of one line each.
+    for name, per_item, count in (("reverse_permutation", 8 + 128, n_ent), ("sub_bucket", 48 + 2 * 128, n_edges)):
+        v = out[name]
+        v["line_granular_GBs"] = count * per_item / (v["ms"] * 1e-3) / 1e9
+        v["line_granular_frac_of_8TBs"] = v["line_granular_GBs"] / HBM_PEAK_GBS
     return {"metric": "permutation helpers, achieved HBM GB/s on algorithmic bytes", "peak_GBs": HBM_PEAK_GBS,
-            "note": "shuffle_rows and sub_bucket include the host read of their error flag (one synchronisation per call)",
+            "note": "shuffle_rows and sub_bucket include the host read of their error flag (one synchronisation per call); "
+                    "randperm is arithmetic (a keyed bijection per entry), priced here on the 8 bytes it writes",
             "cases": out}
 
 

@@ -12,7 +12,11 @@
  *   - the caller owns every buffer, including workspaces (query the *_bytes
  *     function, allocate, pass in); the library never allocates device memory;
  *   - work is enqueued on `stream` (a hipStream_t) and the call returns without
- *     synchronising;
+ *     synchronising.  pbg_train_step may also run its key sort on one more
+ *     stream that the library creates per device on first use (default
+ *     priority): it is forked from `stream` and joined back into it with two
+ *     events inside the call, so the caller sees the step's work as if it were
+ *     all on `stream` (a HIP graph capture records the fork and the join);
  *   - return value: PBG_OK or a negative pbg_status; pbg_last_error() gives the
  *     message of the last failure on the calling thread.
  */
@@ -342,9 +346,20 @@ int pbg_reverse_permutation(const int64_t* perm, int64_t n, int64_t* out, pbg_st
 int pbg_shuffle_rows(void* rows, int64_t n, int64_t row_bytes, const int64_t* perm, void* scratch,
                      int32_t* oob_flag, pbg_stream_t stream);
 
-/* _C.randperm (util.cpp:14-102): a uniform random permutation of [0, n).  The
+/* The same move out of place: out[perm[i]] <- rows[i], `rows` untouched, `out`
+ * (n * row_bytes bytes) not overlapping it.  For a caller that holds two
+ * buffers and swaps them, so that the copy back of the in-place form (half of
+ * its traffic) is not paid.  The reference only has the in-place form
+ * (util.cpp:127-220, whose cycle-following needs no second buffer on a CPU). */
+int pbg_shuffle_rows_out(const void* rows, int64_t n, int64_t row_bytes, const int64_t* perm, void* out,
+                         int32_t* oob_flag, pbg_stream_t stream);
+
+/* _C.randperm (util.cpp:14-102): a random permutation of [0, n).  The
  * reference's bit pattern depends on its thread count; only the contract is
- * kept.  Deterministic in (n, seed). */
+ * kept.  Deterministic in (n, seed).  out[i] is a keyed bijection of i (a
+ * Feistel network on the bits of n - 1, cycle-walked into [0, n)): no sort and
+ * no workspace -- pbg_randperm_workspace_bytes returns 0 and the workspace
+ * arguments are ignored (kept so that existing callers link). */
 size_t pbg_randperm_workspace_bytes(int64_t n);
 int pbg_randperm(int64_t n, uint64_t seed, int64_t* out, void* workspace, size_t workspace_bytes,
                  pbg_stream_t stream);

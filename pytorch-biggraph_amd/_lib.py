@@ -114,6 +114,7 @@ SIGNATURES = {
                                     c_void_p, c_void_p, c_void_p]),
     "pbg_reverse_permutation": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p]),
     "pbg_shuffle_rows": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "pbg_shuffle_rows_out": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "pbg_randperm_workspace_bytes": (c_size_t, [c_int64]),
     "pbg_randperm": (c_int32, [c_int64, c_uint64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "pbg_sub_bucket_workspace_bytes": (c_size_t, [c_int64]),

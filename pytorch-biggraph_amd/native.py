@@ -157,11 +157,26 @@ def shuffle_rows(tensor: torch.Tensor, perm: torch.Tensor, scratch: Optional[tor
         raise ValueError("Permutation has out-of-bound values")
 
 
+def shuffle_rows_out(tensor: torch.Tensor, perm: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[perm[i]] = tensor[i] into a second buffer (returned): the in-place form without its copy back."""
+    if not tensor.is_contiguous():
+        raise ValueError("tensor must be contiguous")
+    if out is None:
+        out = torch.empty_like(tensor)
+    n = tensor.shape[0]
+    row_bytes = tensor[0].numel() * tensor.element_size() if n > 0 else 0
+    if n == 0 or row_bytes == 0:
+        return out
+    flag = torch.zeros(1, dtype=torch.int32, device=tensor.device)
+    check(_lib.lib().pbg_shuffle_rows_out(_ptr(tensor), n, row_bytes, _ptr(perm), _ptr(out), _ptr(flag), _stream()))
+    if int(flag.item()) != 0:
+        raise ValueError("Permutation has out-of-bound values")
+    return out
+
+
 def randperm(n: int, seed: int, device) -> torch.Tensor:
     out = torch.empty(n, dtype=torch.int64, device=device)
-    nbytes = _lib.lib().pbg_randperm_workspace_bytes(n)
-    ws = _workspace(nbytes, device)
-    check(_lib.lib().pbg_randperm(n, seed & (2**64 - 1), _ptr(out), _ptr(ws), ws.numel(), _stream()))
+    check(_lib.lib().pbg_randperm(n, seed & (2**64 - 1), _ptr(out), None, 0, _stream()))
     return out
 
 

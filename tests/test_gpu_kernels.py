@@ -113,11 +113,20 @@ def test_permutation_helpers_bit_exact(pbg, n):
     p = np.random.default_rng(n).permutation(n).astype(np.int64)
     tp = torch.from_numpy(p).to(DEV)
     assert np.array_equal(pbg.native.reverse_permutation(tp).cpu().numpy(), operm.reverse_permutation(p))
+    # row widths on either side of every kernel's border: 4 / 8 bytes, up to 128 / 256 / 512 / 1024 bytes in
+    # 16-byte words, wider than that, and widths that are no multiple of 16
     for shape, dtype in (((n, 100), torch.float32), ((n,), torch.float32), ((n,), torch.int64), ((n, 3), torch.float32),
-                         ((n, 2, 2), torch.float64)):
+                         ((n, 2, 2), torch.float64), ((n, 32), torch.float32), ((n, 36), torch.float32),
+                         ((n, 64), torch.float32), ((n, 128), torch.float32), ((n, 132), torch.float32),
+                         ((n, 256), torch.float32), ((n, 260), torch.float32), ((n, 1030), torch.float32)):
+        if n * int(np.prod(shape[1:])) > 40_000_000:
+            continue
         t = (torch.randn(shape) * 1000).to(dtype)
         want = operm.shuffle(t.numpy(), p)
         td = t.to(DEV)
+        out = pbg.native.shuffle_rows_out(td, tp)   # into a second buffer, the input untouched
+        assert np.array_equal(out.cpu().numpy(), want), (shape, dtype, "out of place")
+        assert torch.equal(td.cpu(), t)
         pbg.native.shuffle_rows(td, tp)
         assert np.array_equal(td.cpu().numpy(), want), (shape, dtype)
     # undo with the reverse permutation (train_gpu.py:627-632)
@@ -132,21 +141,46 @@ def test_shuffle_rejects_bad_permutation(pbg):
     t = torch.randn(4, 4, device=DEV)
     with pytest.raises(ValueError):
         pbg.native.shuffle_rows(t, torch.tensor([0, 1, 2, 4], device=DEV))
+    with pytest.raises(ValueError):
+        pbg.native.shuffle_rows_out(t, torch.tensor([0, -1, 2, 3], device=DEV))
+    both = torch.randn(8, 4, device=DEV)
+    with pytest.raises(ValueError, match="overlap"):  # the out-of-place form needs two buffers
+        pbg.native.shuffle_rows_out(both[:6], torch.arange(6, device=DEV), both[2:])
 
 
-@pytest.mark.parametrize("n", [1, 5000, 200003])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 65, 5000, 65536, 65537, 200003, 1 << 20, 4_000_001])
 def test_randperm_contract(pbg, n):
+    """_C.randperm's contract (util.cpp:14-102; its bits depend on the thread count, so only the contract
+    travels): a permutation, the same for the same seed, another for another seed, and uniform to first
+    and second order -- where the first tenth of the elements lands, the differences of neighbouring
+    outputs, and the joint position of neighbouring outputs on an 8 x 8 grid."""
     a = pbg.native.randperm(n, 7, DEV).cpu().numpy()
     assert operm.is_permutation(a)
     assert np.array_equal(a, pbg.native.randperm(n, 7, DEV).cpu().numpy())
     if n > 1000:
         b = pbg.native.randperm(n, 8, DEV).cpu().numpy()
         assert (a != b).mean() > 0.99
-        # first-order uniformity: where element 0..n/10 land, in 10 bins (chi-square, 9 dof)
-        inv = operm.reverse_permutation(a)
-        counts = np.bincount(inv[: n // 10] * 10 // n, minlength=10)
-        expected = (n // 10) / 10
-        assert ((counts - expected) ** 2 / expected).sum() < 40
+
+        def chi2(counts):
+            expected = counts.sum() / counts.size
+            return float(((counts - expected) ** 2 / expected).sum())
+
+        for perm in (a, b):
+            inv = np.empty(n, dtype=np.int64)
+            inv[perm] = np.arange(n)
+            assert chi2(np.bincount(inv[: n // 10] * 10 // n, minlength=10)) < 40                   # 9 dof
+            assert chi2(np.bincount(np.diff(perm) % 16, minlength=16)) < 55                          # 15 dof
+            assert chi2(np.bincount((perm[:-1] * 8 // n) * 8 + perm[1:] * 8 // n, minlength=64)) < 130  # 63 dof
+            assert int((perm == np.arange(n)).sum()) < 12  # fixed points: Poisson(1)
+
+
+def test_randperm_small_sizes_reach_every_permutation(pbg):
+    """n = 4 has 24 permutations; over 600 seeds each must appear (expected 25 times)."""
+    seen = {}
+    for seed in range(600):
+        key = tuple(pbg.native.randperm(4, seed, DEV).tolist())
+        seen[key] = seen.get(key, 0) + 1
+    assert len(seen) == 24 and min(seen.values()) >= 5, seen
 
 
 @pytest.mark.parametrize("dynamic", [False, True])
