@@ -46,17 +46,27 @@ inline int bits_for(uint64_t max_value) {  // number of bits needed to hold max_
 // out ordered by all bits below key_bits.  Both buffer pairs are clobbered; the
 // result is in whichever pair *keys_sorted / *vals_sorted name on return.
 // `temp` holds sort_temp_bytes(n) bytes.
+// With `indices` the input pairs are made by the sort's first kernel instead of being read: key i = indices[i]
+// (an index outside [0, park) becomes `park`), value i = i; keys_in / vals_in are then only written.
+// If `long_runs` is given it receives a device pointer (into `temp`) to a word that is zero after the
+// sort only if no value of the sorted bits occurs more than kFoldMax times -- what lets a single-worker
+// RowAdagrad step skip its duplicate-summation kernels.
+constexpr int kFoldMax = 16;
 size_t sort_temp_bytes(int64_t n);
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
-               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted);
+               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted,
+               const uint32_t** long_runs = nullptr, const int64_t* indices = nullptr, int64_t park = 0);
 
 // ---- segmented RowAdagrad over sorted (row << kbits | worker) keys ---------
 // keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim], which is
 // clobbered (duplicate sums are formed in place).  A key's row field addresses table 0 for row < rows0, table 1 (row - rows0) for
 // row < rows0 + rows1, and is ignored beyond.
+// `long_runs` (single-worker calls, kbits == 0): the word sort_pairs leaves behind; where it is zero the
+// duplicate-summation kernels return at once (no key occurs more than kFoldMax times, and the update
+// kernel sums such runs itself).  nullptr: not known.
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits,
                        float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
-                       float* g1, int64_t rows1, float lr, hipStream_t stream);
+                       float* g1, int64_t rows1, float lr, hipStream_t stream, const uint32_t* long_runs = nullptr);
 
 // ---- plain fp32 batched GEMM on MFMA ----------------------------------------
 // C[b] (M x N, row-major, ldc) = alpha * A[b] * B[b] + beta * C[b], for b in [0, batch).

@@ -106,22 +106,19 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_multi_kernel(const fl
 //   row_update    a wave per few sorted positions; at each position that starts
 //                 a row it walks the row's runs (one gradient row each), the
 //                 keys of the next 64 positions held in registers.
-// In a single-worker call (kbits == 0: a row has ONE run, all its duplicates) most
-// runs are two or three positions long.  Sending those through tile_reduce costs
-// a read of every row of the run, a write of the sum and another read of it;
-// instead a run of at most kShort positions that lies inside one tile is left
-// alone by tile_reduce (and never concerns run_combine) and summed, in position
-// order, by the update kernel as it reads it, with the loads of the same phase.
-// (With several workers a row has a run per worker and the update kernels' loop
-// over them is latency bound: the extra loads cost more there than they save.
-// row_walk_kernel, which streams a table row's whole stretch anyway, takes every
-// whole run that lies inside one tile, whatever its length.)
+// In a single-worker call (kbits == 0: a row has ONE run, all its duplicates) nearly all
+// runs are two or three positions long.  Sending those through tile_reduce costs a read of
+// every row of the run, a write of the sum and another read of it; instead a run of at most
+// kFoldMax positions -- wherever it lies -- is left alone by tile_reduce and run_combine and
+// summed, in position order, by the update kernel as it reads it.  Longer runs (a hot row of
+// a power-law graph) keep the three-kernel scheme.  Whether a run is short is decided from
+// its length alone, so the three kernels agree, and the sort says whether any long run
+// exists at all (`long_runs`): where none does, tile_reduce and run_combine return at once.
+// (With several workers a row has a run per worker and the update kernels' loop over them is
+// latency bound: the extra loads cost more there than they save.  row_walk_kernel, which
+// streams a table row's whole stretch anyway, takes every whole run that lies inside one
+// tile, whatever its length.)
 constexpr int kTile = 32;
-constexpr int kShort = 4;
-// [s, s + len) in sorted positions: summed by the update kernels themselves (single-worker calls)
-__device__ __forceinline__ bool folded_run(int64_t s, int64_t len) {
-  return len >= 2 && len <= kShort && (s / kTile) == ((s + len - 1) / kTile);
-}
 
 template <int NV, bool VEC>
 struct RowRegs {
@@ -213,11 +210,15 @@ __device__ __forceinline__ uint64_t lane_u64(uint64_t v, int l) {
   return ((uint64_t)hi << 32) | lo;
 }
 
+// leave_mode 0: every piece of two or more positions is summed; 1 (single-worker calls): pieces of runs
+// of at most kFoldMax positions are left to the update kernel; 2 (row_walk_kernel follows): whole runs
+// inside the tile are left alone.
 template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
                                                                   float* __restrict__ grad_rows, int dim,
-                                                                  int leave_short) {
+                                                                  int leave_mode, const uint32_t* __restrict__ long_runs) {
+  if (leave_mode == 1 && long_runs && *long_runs == 0u) return;  // the sort saw no run of more than kFoldMax positions
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
   const int64_t begin = tile * kTile;
@@ -231,20 +232,30 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
   const uint64_t prev = __shfl_up(key, 1, 64);
   const bool starts = (mine < end) && (lane == 0 || prev != key);
   uint64_t heads = __ballot(starts);  // bit l set: a piece starts at begin + l
-  // the keys next to the tile tell whether a piece at its edge is a whole run
-  const bool has_before = begin > 0, has_after = end < n;
-  const uint64_t key_before = (leave_short && has_before) ? keys[begin - 1] : 0ull;
-  const uint64_t key_after = (leave_short && has_after) ? keys[end] : 0ull;
+  // How far the runs at the tile's two edges go on outside it, up to kFoldMax positions each way:
+  // lanes 0 .. 15 look at the positions before the tile (nearest first), lanes 16 .. 31 at those after it.
+  int before = 0, after = 0;
+  if (leave_mode != 0) {
+    const uint64_t first_key = lane_u64(key, 0), last_key = lane_u64(key, (int)(end - begin) - 1);
+    const int64_t q = lane < kFoldMax ? begin - 1 - lane : end + (lane - kFoldMax);
+    const bool there = lane < 2 * kFoldMax && q >= 0 && q < n;
+    const uint64_t other = there ? keys[q] : 0ull;
+    const uint32_t same_before = (uint32_t)__ballot(there && lane < kFoldMax && other == first_key) & 0xffffu;
+    const uint32_t same_after = (uint32_t)(__ballot(there && lane >= kFoldMax && other == last_key) >> kFoldMax) & 0xffffu;
+    before = same_before == 0xffffu ? kFoldMax : __ffs((int)~same_before) - 1;  // leading ones
+    after = same_after == 0xffffu ? kFoldMax : __ffs((int)~same_after) - 1;
+  }
   while (heads != 0ull) {
     const int a = __ffsll((unsigned long long)heads) - 1;
     heads &= heads - 1;
     const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
-    if (b - a < 2) continue;
-    if (b - a <= leave_short) {  // a whole run of at most leave_short positions inside the tile is the update kernel's
-      const uint64_t kp = lane_u64(key, a);
-      const bool whole = (a > 0 || !has_before || key_before != kp) && (b < (int)(end - begin) || !has_after || key_after != kp);
-      if (whole) continue;
+    if (leave_mode != 0) {
+      const bool whole = (a > 0 || before == 0) && (b < (int)(end - begin) || after == 0);
+      if (leave_mode == 2 && whole) continue;  // (a single position needs no sum either way)
+      const int run_len = (b - a) + (a == 0 ? before : 0) + (b == (int)(end - begin) ? after : 0);
+      if (leave_mode == 1 && run_len <= kFoldMax) continue;
     }
+    if (b - a < 2) continue;
     RowRegs<NV, VEC> acc;
     float* head = grad_rows + (int64_t)lane_u32(val, a) * dim;
     acc.load(head, nv, lane);
@@ -266,7 +277,9 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
 template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
-                                                                  float* __restrict__ grad_rows, int dim) {
+                                                                  float* __restrict__ grad_rows, int dim,
+                                                                  int leave_mode, const uint32_t* __restrict__ long_runs) {
+  if (leave_mode == 1 && long_runs && *long_runs == 0u) return;  // as in tile_reduce_kernel
   const int lane = threadIdx.x & 63;
   const int64_t b = ((int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6) + 1) * kTile;
   if (b >= n) return;
@@ -280,6 +293,9 @@ __global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t
   const int head_lane = not_before ? 32 - __clz(not_before) : 0;
   if (head_lane == 0 && b - kTile > 0 && keys[b - kTile - 1] == key) return;  // an earlier border owns this run
   const uint32_t not_after = ~(uint32_t)(same >> 32);
+  // a run that begins and ends inside the window shows its whole length: a short one is the update kernel's
+  if (leave_mode == 1 && head_lane > 0 && not_after != 0u && (kTile - head_lane) + (__ffs((int)not_after) - 1) <= kFoldMax)
+    return;
   const int64_t end = not_after ? b + (__ffs(not_after) - 1) : scan_end(keys, b + kTile - 1, n, key, 0, lane);
   const int nv = VEC ? (dim >> 2) : dim;
   RowRegs<NV, VEC> acc;
@@ -375,13 +391,14 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     w[r].load(wrow[r], nv, lane);
     gsum[r] = *gptr[r];
     g[r].load(grad_rows + (int64_t)lane_u32(vv[r], 0) * dim, nv, lane);  // each run's sum sits in its first row ...
-    if (kbits == 0) {  // ... unless it is a short run left to this kernel (folded_run)
+    if (kbits == 0) {  // ... unless it is a short run, left to this kernel: summed here in position order
       const uint64_t same = __ballot(i + lane < n && kk[r] == lane_u64(kk[r], 0));
       const int run_len = ~same != 0ull ? __ffsll((unsigned long long)~same) - 1 : kWave;
-      const bool fold = folded_run(i, run_len);
+      const bool fold = run_len <= kFoldMax;
 #pragma unroll
-      for (int t = 1; t < kShort; ++t)
+      for (int t = 1; t < 4; ++t)  // the common lengths with their loads in flight together
         g[r].add_if(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane, fold && t < run_len);
+      for (int t = 4; fold && t < run_len; ++t) g[r].add(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane);
     }
   }
   int long_r = -1;
@@ -484,7 +501,7 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
 // of dependent loads along a row's runs.  Here the wave finds its row's first position
 // by a 64-ary search, then walks the row's stretch of sorted positions window by
 // window: the rows to read -- the head row of every run, or all rows of a short run that
-// tile_reduce left alone (folded_run) -- are known from the keys of the window alone, so
+// tile_reduce left alone -- are known from the keys of the window alone, so
 // R of them are in flight at a time whatever run they belong to, and the runs' Adagrad
 // steps follow in worker order on registers.
 template <int NV, bool VEC, int R>
@@ -652,13 +669,15 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     w[r] = load_or_zero(wrow[r], has);
     gsum[r] = *gptr[r];
     g[r] = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase, 64) * dim + col, has);
-    if (kbits == 0) {  // the row's one run, if it is a short one left to this kernel (folded_run)
+    if (kbits == 0) {  // the row's one run, if it is a short one left to this kernel: summed here in position order
       const uint32_t same = (uint32_t)(__ballot(i + gl < n && kk[r] == half_bcast_u64(kk[r], gbase)) >> gbase);
       const int run_len = same != 0xffffffffu ? __ffs((int)~same) - 1 : 32;
-      const bool fold = folded_run(i, run_len);
+      const bool fold = run_len <= kFoldMax;
 #pragma unroll
-      for (int t = 1; t < kShort; ++t)
+      for (int t = 1; t < 4; ++t)  // the common lengths with their loads in flight together
         add4(g[r], load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + t, 64) * dim + col, has && fold && t < run_len));
+      // (rare: the two halves of the wave differ in their counts here, so the row numbers come from memory, not from a shuffle)
+      for (int t = 4; fold && t < run_len; ++t) add4(g[r], load_or_zero(grad_rows + (int64_t)vals[i + t] * dim + col, has));
     }
   }
   int long_r = -1;
@@ -761,17 +780,6 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
   if (gl == 0) *long_gptr = long_gsum;
 }
 
-// keys for the stand-alone sparse step: key = row index, value = position
-__global__ void make_keys_kernel(const int64_t* __restrict__ idx, int64_t n, int64_t num_rows,
-                                 uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int64_t r = idx[i];
-  if (r < 0 || r >= num_rows) r = num_rows;  // parked past the table, skipped by the update
-  keys[i] = (uint64_t)r;
-  vals[i] = (uint32_t)i;
-}
-
 // ---- dense branches ------------------------------------------------------------
 __global__ __launch_bounds__(kRowThreads) void row_adagrad_dense_kernel(float* __restrict__ w, float* __restrict__ gs,
                                                                         int64_t num_rows, int dim,
@@ -803,7 +811,7 @@ __global__ void async_adagrad_dense_kernel(float* __restrict__ p, float* __restr
 template <bool VEC>
 int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                   int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                  hipStream_t stream) {
+                  const uint32_t* long_runs, hipStream_t stream) {
   const int wpb = kRowThreads / kWave;
   const dim3 block(kRowThreads);
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
@@ -813,12 +821,14 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
   const int64_t table_rows = rows0 + rows1;
   const bool walk = kbits > 0 && table_rows > 0 && n >= 32 * table_rows && getenv("PBG_DISABLE_ROW_WALK") == nullptr;
   const dim3 walk_grid((unsigned)ceil_div(table_rows > 0 ? table_rows : 1, wpb));
+  const int leave_mode = walk ? 2 : (kbits == 0 ? 1 : 0);
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim,       \
-                       walk ? kTile : (kbits == 0 ? kShort : 0));                                                              \
+                       leave_mode, long_runs);                                                                     \
     if (borders > 0)                                                                                              \
-      hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim); \
+      hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim,  \
+                         leave_mode, long_runs);                                                                   \
     if (walk) {                                                                                                    \
       constexpr int R = NV <= 2 ? 8 : (NV <= 4 ? 4 : 2);                                                           \
       hipLaunchKernelGGL((row_walk_kernel<NV, VEC, R>), walk_grid, block, 0, stream, keys, vals, n, kbits, grad_rows,  \
@@ -853,15 +863,15 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                        int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                       hipStream_t stream) {
+                       hipStream_t stream, const uint32_t* long_runs) {
   if (n <= 0) return PBG_OK;
   int rc;
   if (dim % 4 == 0) {
     rc = launch_sorted<true>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
-                             g1, rows1, lr, stream);
+                             g1, rows1, lr, long_runs, stream);
   } else {
     rc = launch_sorted<false>((int)ceil_div(dim, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1, g1,
-                              rows1, lr, stream);
+                              rows1, lr, long_runs, stream);
   }
   if (rc != PBG_OK) return rc;
   return check_launch("row_adagrad_sorted");
@@ -998,16 +1008,15 @@ extern "C" int pbg_row_adagrad_sparse(float* weight, float* state_sum, int64_t n
   if (!workspace || workspace_bytes < ws.total)
     return fail(PBG_ERR_WORKSPACE, "pbg_row_adagrad_sparse: workspace needs %zu bytes", ws.total);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(make_keys_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, idx, n, num_rows, ws.keys_a,
-                     ws.vals_a);
   uint64_t* skeys;
   uint32_t* svals;
+  const uint32_t* long_runs;
   int rc = sort_pairs(ws.keys_a, ws.vals_a, ws.keys_b, ws.vals_b, n, 0, bits_for((uint64_t)num_rows), ws.temp, s,
-                      &skeys, &svals);
+                      &skeys, &svals, &long_runs, idx, num_rows);
   if (rc != PBG_OK) return rc;
-  // out-of-range indices were parked at key == num_rows and are skipped by the update
+  // out-of-range indices are parked at key == num_rows and are skipped by the update
   return row_adagrad_sorted(skeys, svals, n, 0, grad_rows, dim, weight, state_sum, num_rows, nullptr,
-                            nullptr, 0, lr, s);
+                            nullptr, 0, lr, s, long_runs);
 }
 
 // ---------------------------------------------------------------------------

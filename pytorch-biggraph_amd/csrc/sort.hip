@@ -8,11 +8,17 @@
 // small), ranks its keys slice by slice (ballot matching inside a wave, LDS
 // counts across the 16 waves, a running per-digit cursor across slices) and
 // scatters them.  That leaves one bucket per digit value, contiguous in memory;
-// the remaining low bits are sorted inside each bucket, one block per bucket,
-// 8 bits per launch from the lowest up: no counts to exchange between blocks, no
-// atomics on global memory.  Every step is stable, so equal keys keep the order
-// of the input, which keeps segmented gradient sums deterministic and lets a
-// caller whose input is already ordered by the low bits leave those bits out.
+// the remaining low bits are sorted inside each bucket, one block per bucket, in
+// ONE launch: no counts to exchange between blocks, no atomics on global memory.
+// A bucket of up to `cap` keys (the common case: a few times the mean bucket) is
+// sorted inside LDS -- its remaining bits and its positions packed into 32-bit
+// words that go through all the digit passes there, then one gather of the
+// bucket's pairs in sorted order -- so its keys cross HBM once more instead of
+// once per digit; a larger bucket (swollen by a hot key) walks its digit passes
+// through global memory, 8 bits per pass from the lowest up, with block barriers
+// between them.  Every step is stable, so equal keys keep the order of the
+// input, which keeps segmented gradient sums deterministic and lets a caller
+// whose input is already ordered by the low bits leave those bits out.
 #include "pbg_internal.h"
 
 namespace pbg {
@@ -38,19 +44,36 @@ SortPlan plan_sort(int64_t n) {
   return p;
 }
 
-// counts[block][kMaxDigits] of the global pass
-__global__ __launch_bounds__(kGlobalWaves * 64) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n,
+// counts[block][kMaxDigits] of the global pass.  With `idx` the pairs are made on the way: key = idx[i]
+// (an index outside [0, park) is parked at `park`), value = i -- the stand-alone RowAdagrad step's keys
+// need no pass of their own then.
+__global__ __launch_bounds__(kGlobalWaves * 64) void sort_hist_kernel(uint64_t* __restrict__ keys, int64_t n,
                                                                       int tile_shift, int shift, int digit_bits,
-                                                                      uint32_t* __restrict__ counts) {
+                                                                      uint32_t* __restrict__ counts,
+                                                                      uint32_t* __restrict__ long_flag,
+                                                                      uint32_t long_init,
+                                                                      const int64_t* __restrict__ idx, int64_t park,
+                                                                      uint32_t* __restrict__ vals) {
   __shared__ uint32_t hist[kMaxDigits];
+  if (blockIdx.x == 0 && threadIdx.x == 0) *long_flag = long_init;
   const uint32_t mask = (1u << digit_bits) - 1u;
   if (threadIdx.x < kMaxDigits) hist[threadIdx.x] = 0;
   __syncthreads();
   const int64_t begin = (int64_t)blockIdx.x << tile_shift;
   int64_t end = begin + ((int64_t)1 << tile_shift);
   if (end > n) end = n;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kGlobalWaves * 64)
-    atomicAdd(&hist[(uint32_t)(keys[i] >> shift) & mask], 1u);
+  if (idx) {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kGlobalWaves * 64) {
+      int64_t r = idx[i];
+      if (r < 0 || r >= park) r = park;
+      keys[i] = (uint64_t)r;
+      vals[i] = (uint32_t)i;
+      atomicAdd(&hist[(uint32_t)((uint64_t)r >> shift) & mask], 1u);
+    }
+  } else {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kGlobalWaves * 64)
+      atomicAdd(&hist[(uint32_t)(keys[i] >> shift) & mask], 1u);
+  }
   __syncthreads();
   if (threadIdx.x < kMaxDigits) counts[(int64_t)blockIdx.x * kMaxDigits + threadIdx.x] = hist[threadIdx.x];
 }
@@ -323,34 +346,18 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
                                                               shift, (1u << digit_bits) - 1u, first_keys, first_vals);
 }
 
-// A local pass: block b sorts bucket b (positions [bucket_off[b], bucket_off[b + 1]))
-// by one digit of up to 8 bits, reading from the "in" pair and writing the same
-// positions of the "out" pair.
-__global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
-    const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
-    uint32_t* __restrict__ vals_out, const uint32_t* __restrict__ bucket_off, int shift, int digit_bits) {
-  __shared__ SliceState<kBucketWaves, 8> st;
+// One digit pass of a bucket through global memory (a bucket too large for LDS).
+__device__ __forceinline__ void bucket_pass_global(SliceState<kBucketWaves, 8>& st, const uint64_t* keys_in,
+                                                   const uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out,
+                                                   int64_t begin, int64_t end, int shift, int digit_bits) {
   const int t = threadIdx.x;
-  const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
-  if (begin >= end) return;
   const uint32_t mask = (1u << digit_bits) - 1u;
-  const bool wide = end - begin > 2 * kBucketWaves * 64;  // a swollen bucket
-  uint64_t key_next = 0;
-  uint32_t val_next = 0;
-  if (begin + t < end) {
-    key_next = keys_in[begin + t];
-    val_next = vals_in[begin + t];
-  }
   if (t < 256) {
     st.cursor[t] = 0;
     for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
   }
   __syncthreads();
-  if (!wide) {
-    if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
-    for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
-      atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
-  } else {
+  {
     // equal keys would queue up on one counter: one addition per wave and digit value present.
     // Eight loads per thread in flight (the ballots would otherwise wait for each load in turn).
     const int lane = t & 63;
@@ -377,24 +384,168 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(
   const uint32_t excl = block_exclusive_scan(t < 256 ? st.cursor[t] : 0u, 4, st.wave_total, &grand);
   if (t < 256) st.cursor[t] = (uint32_t)begin + excl;
   __syncthreads();
-  if (wide)
-    scatter_range_wide<kBucketWaves, 8, 4>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask);
-  else
-    scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
-                                   val_next);
+  scatter_range_wide<kBucketWaves, 8, 4>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask);
+}
+
+// One digit pass of a bucket's packed words inside LDS: `from` -> `to`, m words, digit = bits
+// [shift, shift + digit_bits) of a word.  Same ranking as the global passes (a wave owns 4 x 64
+// consecutive words of a slice of 4096, so (wave, round, lane) is the order of the positions).
+__device__ __forceinline__ void bucket_pass_lds(SliceState<kBucketWaves, 8>& st, const uint32_t* from, uint32_t* to,
+                                                int m, int shift, int digit_bits) {
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+  const uint32_t mask = (1u << digit_bits) - 1u;
+  constexpr int kKpt = 4, kSlice = kBucketWaves * 64 * kKpt;
+  if (t < 256) {
+    st.cursor[t] = 0;
+    for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
+  }
+  __syncthreads();
+  for (int i = t; i < m; i += kBucketWaves * 64) atomicAdd(&st.cursor[(from[i] >> shift) & mask], 1u);
+  __syncthreads();
+  uint32_t grand;
+  const uint32_t excl = block_exclusive_scan(t < 256 ? st.cursor[t] : 0u, 4, st.wave_total, &grand);
+  if (t < 256) st.cursor[t] = excl;
+  __syncthreads();
+  const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  int parity = 0;
+  for (int base = 0; base < m; base += kSlice) {
+    uint32_t word[kKpt], digit[kKpt], rank[kKpt];
+    bool valid[kKpt];
+#pragma unroll
+    for (int q = 0; q < kKpt; ++q) {
+      const int i = base + wave * (64 * kKpt) + q * 64 + lane;
+      valid[q] = i < m;
+      word[q] = valid[q] ? from[i] : 0u;
+      digit[q] = (word[q] >> shift) & mask;
+      const uint64_t peers = digit_peers<8>(digit[q], valid[q]);
+      const int rank_in_round = __popcll(peers & below);
+      const uint32_t prior = valid[q] ? st.wave_count[parity][wave][digit[q]] : 0u;  // this wave's earlier rounds
+      rank[q] = prior + (uint32_t)rank_in_round;
+      if (valid[q] && rank_in_round == 0) st.wave_count[parity][wave][digit[q]] = (uint16_t)(prior + __popcll(peers));
+    }
+    __syncthreads();
+    if (t < 256) {
+      uint32_t at = 0;
+#pragma unroll
+      for (int w = 0; w < kBucketWaves; ++w) {
+        const uint32_t c = st.wave_count[parity][w][t];
+        st.wave_count[parity][w][t] = (uint16_t)at;
+        at += c;
+        st.wave_count[parity ^ 1][w][t] = 0;
+      }
+      const uint32_t first = st.cursor[t];
+      st.slot[t] = first;
+      st.cursor[t] = first + at;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kKpt; ++q)
+      if (valid[q]) to[st.slot[digit[q]] + st.wave_count[parity][wave][digit[q]] + rank[q]] = word[q];
+    parity ^= 1;
+  }
+  __syncthreads();
+}
+
+constexpr int kLdsIndexBits = 14;              // a bucket sorted inside LDS holds at most 2^14 keys ...
+constexpr int kLdsMaxRestBits = 32 - kLdsIndexBits;  // ... and its remaining bits share a 32-bit word with the position
+
+// All the bucket passes of one sort.  Block b sorts bucket b (positions [bucket_off[b],
+// bucket_off[b + 1]) of the pair (ka, va), where the global pass left it) by bits
+// [low_bit, low_bit + rest) of the key; the result goes to the same positions of (kfin, vfin), which
+// is (ka, va) or (kb, vb) depending on the parity of `passes` (the number of digit passes a bucket too
+// large for LDS takes through global memory).  `long_flag`, if given, is raised when some value of the
+// sorted bits occurs more than kFoldMax times in a bucket sorted here (or the bucket was not looked at).
+__global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t* ka, uint32_t* va, uint64_t* kb,
+                                                                        uint32_t* vb, uint64_t* kfin, uint32_t* vfin,
+                                                                        const uint32_t* __restrict__ bucket_off,
+                                                                        int low_bit, int rest, int passes, int cap,
+                                                                        uint32_t* __restrict__ long_flag) {
+  __shared__ SliceState<kBucketWaves, 8> st;
+  extern __shared__ uint32_t lds_words[];  // 2 * cap packed words
+  const int t = threadIdx.x;
+  const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
+  if (begin >= end) return;
+  const int64_t m64 = end - begin;
+  if (m64 <= cap && rest <= kLdsMaxRestBits) {
+    const int m = (int)m64;
+    uint32_t* from = lds_words;
+    uint32_t* to = lds_words + cap;
+    const uint32_t rest_mask = rest >= 32 ? 0xffffffffu : ((1u << rest) - 1u);
+    for (int i = t; i < m; i += kBucketWaves * 64)
+      from[i] = (((uint32_t)(ka[begin + i] >> low_bit) & rest_mask) << kLdsIndexBits) | (uint32_t)i;
+    // (bucket_pass_lds starts with a barrier)
+    const int lds_passes = (rest + 7) / 8;
+    int shift = kLdsIndexBits;
+    for (int pass = 0; pass < lds_passes; ++pass) {  // lowest digit first; digits of (almost) equal width
+      const int width = (rest - (shift - kLdsIndexBits) + (lds_passes - pass) - 1) / (lds_passes - pass);
+      bucket_pass_lds(st, from, to, m, shift, width);
+      shift += width;
+      uint32_t* tmp = from; from = to; to = tmp;
+    }
+    if (long_flag) {
+      bool found = false;
+      for (int i = t; i + kFoldMax < m; i += kBucketWaves * 64)
+        found |= (from[i] >> kLdsIndexBits) == (from[i + kFoldMax] >> kLdsIndexBits);
+      if (found) *long_flag = 1u;
+    }
+    // The pairs in sorted order.  All of a thread's reads come before its first write, and a barrier
+    // in between: the result may go where the bucket was read from.
+    constexpr int kMaxPerThread = (1 << kLdsIndexBits) / (kBucketWaves * 64);
+    uint64_t k[kMaxPerThread];
+    uint32_t v[kMaxPerThread];
+#pragma unroll
+    for (int r = 0; r < kMaxPerThread; ++r) {
+      const int j = r * kBucketWaves * 64 + t;
+      if (j < m) {
+        const int64_t src = begin + (from[j] & ((1u << kLdsIndexBits) - 1u));
+        k[r] = ka[src];
+        v[r] = va[src];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kMaxPerThread; ++r) {
+      const int j = r * kBucketWaves * 64 + t;
+      if (j < m) {
+        kfin[begin + j] = k[r];
+        vfin[begin + j] = v[r];
+      }
+    }
+    return;
+  }
+  if (long_flag && t == 0) *long_flag = 1u;
+  uint64_t* ksrc = ka;
+  uint32_t* vsrc = va;
+  uint64_t* kdst = kb;
+  uint32_t* vdst = vb;
+  int shift = low_bit;
+  for (int pass = 0; pass < passes; ++pass) {
+    const int width = (rest - (shift - low_bit) + (passes - pass) - 1) / (passes - pass);
+    bucket_pass_global(st, ksrc, vsrc, kdst, vdst, begin, end, shift, width);
+    shift += width;
+    uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
+    uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
+    __syncthreads();  // the next pass reads what this one wrote (same block, workgroup scope)
+  }
 }
 
 }  // namespace
 
 size_t sort_temp_bytes(int64_t n) {
   SortPlan p = plan_sort(n);
-  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 1) * sizeof(uint32_t), 256);
+  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 2) * sizeof(uint32_t), 256);
+}
+
+namespace {
+LdsLimit g_bucket_lds;
 }
 
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
-               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted) {
+               int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted,
+               const uint32_t** long_runs, const int64_t* indices, int64_t park) {
   *keys_sorted = keys_in;
   *vals_sorted = vals_in;
+  if (long_runs) *long_runs = nullptr;
   if (n <= 0) return PBG_OK;
   if (n >= (int64_t)1 << 32)
     return fail(PBG_ERR_UNSUPPORTED, "sort_pairs: n=%lld does not fit 32-bit offsets", (long long)n);
@@ -402,31 +553,37 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   SortPlan p = plan_sort(n);
   uint32_t* counts = (uint32_t*)temp;
   uint32_t* bucket_off = counts + (size_t)kMaxDigits * p.blocks;
+  uint32_t* long_flag = bucket_off + kMaxDigits + 1;
   int bits = key_bits - low_bit;
   if (bits < 1) bits = 1;
   const int top = bits < kMaxDigitBits ? bits : kMaxDigitBits;  // width of the global pass
   const int rest = bits - top;                                  // bits left for the bucket passes
   const int local = (rest + 7) / 8;
   const int top_shift = low_bit + rest;
+  // without bucket passes nobody looks at the lengths of the runs: the flag then says "there may be long ones"
   hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, n, p.tile_shift,
-                     top_shift, top, counts);
+                     top_shift, top, counts, long_flag, local == 0 ? 1u : 0u, indices, park, vals_in);
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, vals_in,
                      keys_out, vals_out, n, p.tile_shift, top_shift, top, counts, bucket_off);
-  uint64_t* ksrc = keys_out;
-  uint32_t* vsrc = vals_out;
-  uint64_t* kdst = keys_in;
-  uint32_t* vdst = vals_in;
-  int shift = low_bit;
-  for (int pass = 0; pass < local; ++pass) {  // lowest digit first; digits of (almost) equal width
-    const int width = (rest - (shift - low_bit) + (local - pass) - 1) / (local - pass);
-    hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kBucketWaves * 64), 0, stream, ksrc, vsrc, kdst, vdst,
-                       bucket_off, shift, width);
-    shift += width;
-    uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
-    uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
+  if (long_runs) *long_runs = long_flag;
+  if (local == 0) {
+    *keys_sorted = keys_out;
+    *vals_sorted = vals_out;
+    return check_launch("sort_pairs");
   }
-  *keys_sorted = ksrc;
-  *vals_sorted = vsrc;
+  // buckets of up to `cap` keys are sorted inside LDS: four times the mean bucket, between 2048 and 2^14 keys
+  int64_t cap = 4 * ceil_div(n, (int64_t)1 << top);
+  cap = cap < 2048 ? 2048 : (cap > (1 << kLdsIndexBits) ? (1 << kLdsIndexBits) : cap);
+  cap = (cap + 1023) / 1024 * 1024;
+  const size_t lds_bytes = (size_t)cap * 2 * sizeof(uint32_t);
+  const int rc = reserve_lds((const void*)sort_bucket_kernel, &g_bucket_lds, lds_bytes);
+  if (rc != PBG_OK) return rc;
+  uint64_t* kfin = (local & 1) ? keys_in : keys_out;
+  uint32_t* vfin = (local & 1) ? vals_in : vals_out;
+  hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kBucketWaves * 64), lds_bytes, stream, keys_out, vals_out,
+                     keys_in, vals_in, kfin, vfin, bucket_off, low_bit, rest, local, (int)cap, long_flag);
+  *keys_sorted = kfin;
+  *vals_sorted = vfin;
   return check_launch("sort_pairs");
 }
 

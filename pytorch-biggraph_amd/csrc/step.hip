@@ -2379,7 +2379,17 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   const int sort_bits = bits_for(rows - 1) + c.kbits;
   uint64_t* skeys = nullptr;
   uint32_t* svals = nullptr;
+  const uint32_t* long_runs = nullptr;  // the sort's word on runs of equal keys (read by a single-worker update)
   hipEvent_t sort_done = nullptr;  // set: the sort was queued on the side stream and ends with this event
+  // Once the side stream has been forked from `s` it must be joined back on EVERY way out of this function:
+  // under a HIP graph capture an unjoined fork leaves the library's stream inside the caller's capture.
+  struct JoinOnExit {
+    hipStream_t into;
+    hipEvent_t ev = nullptr;
+    ~JoinOnExit() {
+      if (ev) (void)hipStreamWaitEvent(into, ev, 0);
+    }
+  } join_guard{s};
   mark(0);
   if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
   if (stream) {
@@ -2430,12 +2440,12 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if (ss) {
       if (hipStreamWaitEvent(ss->stream, ss->fork[slot], 0) != hipSuccess)
         return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
-      if ((rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, ss->stream,
-                           &skeys, &svals)) != PBG_OK)
-        return rc;
+      const int sort_rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp,
+                                     ss->stream, &skeys, &svals, &long_runs);
       if (hipEventRecord(ss->join[slot], ss->stream) != hipSuccess)
         return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
-      sort_done = ss->join[slot];
+      join_guard.ev = sort_done = ss->join[slot];
+      if (sort_rc != PBG_OK) return sort_rc;
     }
     mark(1);
     mark(2);
@@ -2474,18 +2484,21 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   }
   mark(8);
   if (sort_done) {
+    join_guard.ev = nullptr;
     if (hipStreamWaitEvent(s, sort_done, 0) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot join the side stream");
   } else {
-    rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, s, &skeys, &svals);
+    rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, s, &skeys, &svals,
+                    &long_runs);
     if (rc != PBG_OK) return rc;
   }
   mark(9);
+  if (c.kbits != 0) long_runs = nullptr;  // the word counts positions per ROW; only with one batch per call is that a run
   if (desc->shared_table) {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
-                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s);
+                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s, long_runs);
   } else {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
-                            desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s);
+                            desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s, long_runs);
   }
   mark(10);
   return rc;
