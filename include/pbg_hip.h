@@ -283,6 +283,23 @@ int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_buffers* bu
 int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos,
                       float* rhs_pos, float* lhs_neg, float* rhs_neg, pbg_stream_t stream);
 
+/* RankingEvaluator._process_one_batch (eval.py:43-81) without the [B, N] score
+ * matrices: the same forward as pbg_model_forward, then per edge e of the call
+ * (K * batch_size of them) lhs_pos[e], rhs_pos[e], the ranks lhs_rank[e] /
+ * rhs_rank[e] = 1 + the number of that side's negatives scoring at least as
+ * high as the positive (entries the model masks to -1e9 take part with that
+ * value, as they do in the reference's matrices; 0 for a side without
+ * negatives, which the evaluator skips), and loss_edge[e] = relation weight x
+ * edge weight x (lhs loss + rhs loss) of the edge under desc->loss / margin
+ * (batching.py:139-150; sum over the edges = the batch's loss).  With
+ * auc_samples > 0 also compute_randomized_auc's count (util.py:420-428):
+ * auc_hits[side] (device, two int64) = how many of auc_samples random
+ * (positive, negative-entry) pairs of the call have positive > negative, drawn
+ * with Philox4x32-10 from auc_seed. */
+int pbg_model_ranks(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos, float* rhs_pos,
+                    int64_t* lhs_rank, int64_t* rhs_rank, float* loss_edge, int64_t auc_samples, uint64_t auc_seed,
+                    int64_t* auc_hits, pbg_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Plugin-level entry points: one operator / comparator / loss at a time, forward
  * and backward, for code that calls the plugin classes directly (the reference's

@@ -96,6 +96,8 @@ SIGNATURES = {
     "pbg_train_step_is_fused": (c_int32, [POINTER(StepDesc)]),
     "pbg_train_step_route": (c_int32, [POINTER(StepDesc)]),
     "pbg_train_step_profile": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, POINTER(c_float)]),
+    "pbg_model_ranks": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_int64, c_uint64, c_void_p, c_void_p]),
     "pbg_model_forward": (c_int32, [POINTER(StepDesc), POINTER(StepBuffers), c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),
     "pbg_operator_forward": (c_int32, [c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,

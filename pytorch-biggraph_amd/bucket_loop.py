@@ -32,7 +32,7 @@ from typing import Callable, Dict, List, Optional, Sequence, Tuple
 import torch
 
 from . import native
-from .eval import ranking_stats
+from .eval import ranking_stats_from_ranks
 from .losses import LOSS_FUNCTIONS
 from .stats import Stats
 from .util import round_up_to_nearest_multiple
@@ -346,6 +346,7 @@ class BucketLoop:
         # call (`self.calls_log`), for a caller that wants to replay the epoch elsewhere
         self.calls_log: Optional[List[dict]] = [] if record_calls else None
         self.calls = 0
+        self.eval_calls = 0  # seeds of the evaluation's AUC samples
         self.epoch = 0
 
     def _keys(self, b: Bucket) -> List[PartitionKey]:
@@ -449,13 +450,15 @@ class BucketLoop:
             c = runner.spec.num_chunks
             ul = self._uniform(k, c, nu, rows_l, 0) if nu else None
             ur = self._uniform(k, c, nu, rows_r, 1) if nu else None
-            lhs_pos, rhs_pos, lhs_neg, rhs_neg = runner.forward(l, r, t, ul, ur)
             count = k * b_now
-            sides = [(lhs_pos.reshape(count), lhs_neg.reshape(count, -1)),
-                     (rhs_pos.reshape(count), rhs_neg.reshape(count, -1))]
-            # AbstractBatchProcessor.calc_loss (batching.py:139-150) with relation weights of 1
-            loss = sum(float(self.loss_fn(pos, neg, None)) for pos, neg in sides)
-            stats.append(ranking_stats(sides, loss, count))
+            # ranks, loss (AbstractBatchProcessor.calc_loss, batching.py:139-150, with relation weights of 1) and the
+            # AUC count per edge from one call; the [K, B, N] score tensors are never formed
+            self.eval_calls += 1
+            _, _, lhs_rank, rhs_rank, loss_edge, hits = runner.ranks(l, r, t, ul, ur, auc_samples=count,
+                                                                     auc_seed=(self.seed << 20) + self.eval_calls)
+            sides = [s for s, off in ((0, runner.spec.disable_lhs_negs), (1, runner.spec.disable_rhs_negs)) if not off]
+            stats.append(ranking_stats_from_ranks([(lhs_rank, rhs_rank)[s] for s in sides], float(loss_edge.sum()), count,
+                                                  [hits[s] for s in sides], count))
         return Stats.sum(stats)
 
     def _train_bucket(self, b: Bucket, tables) -> BucketStats:

@@ -713,6 +713,109 @@ __global__ __launch_bounds__(kRowThreads) void scores_out_kernel(StepCtx c, floa
   }
 }
 
+// Ranking evaluation without the [B, N] score matrices (eval.py:57-81, batching.py:139-150): per edge
+// the two positive scores, per side the rank of the positive among its negatives -- one more than the
+// number of negatives scoring at least as high, masked entries (-1e9) included as they are in the
+// reference's matrices -- and the edge's loss.  One wave per edge reads the chunk's score rows where the
+// score GEMMs left them.
+__device__ __forceinline__ void row_rank_and_loss(int loss, float margin, const ScoreRow& sr, int nn, float pos, int lane,
+                                                  float* loss_acc, int* at_least) {
+  bool live;
+  int ge = 0;
+  float mx = pos;
+  for (int j = lane; j < nn; j += kWave) {
+    const float t = sr.at(j, &live);
+    if (t >= pos) ++ge;
+    if (loss == PBG_LOSS_RANKING) {
+      const float x = (t - pos) + margin;
+      if (x > 0.f) *loss_acc += x;
+    } else if (loss == PBG_LOSS_LOGISTIC) {
+      float sg;
+      *loss_acc += softplus_sigmoid(t, &sg) / (float)nn;
+    } else {
+      mx = fmaxf(mx, t);
+    }
+  }
+  if (loss == PBG_LOSS_SOFTMAX) {
+    mx = wave_max(mx);
+    float z = 0.f;
+    for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
+    z = wave_sum(z) + expf(pos - mx);
+    if (lane == 0) *loss_acc += (mx + logf(z)) - pos;
+  } else if (loss == PBG_LOSS_LOGISTIC) {
+    if (lane == 0) *loss_acc += softplusf(-pos);
+  }
+  *at_least = wave_sum_int(ge);
+}
+
+__global__ __launch_bounds__(kRowThreads) void ranks_out_kernel(StepCtx c, float* __restrict__ lhs_pos,
+                                                                float* __restrict__ rhs_pos,
+                                                                int64_t* __restrict__ lhs_rank,
+                                                                int64_t* __restrict__ rhs_rank,
+                                                                float* __restrict__ loss_edge) {
+  const int lane = threadIdx.x & 63;
+  const int64_t job = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (job >= (int64_t)c.K * c.B) return;
+  const int k = (int)(job / c.B), q = (int)(job % c.B);
+  const int cc = q / c.P, i = q % c.P;
+  const int64_t kc = (int64_t)k * c.C + cc;
+  float posv[2];
+  positive_scores(c, kc, i, lane, posv);
+  float w = c.rel_weights[c.dynamic ? 0 : clamp_index(c.rel[k], c.num_relations)];
+  if (c.edge_weight) w *= c.edge_weight[job];
+  float loss_acc = 0.f;
+  int64_t rank[2] = {0, 0};  // 0: the side has no negatives (the evaluator skips it, eval.py:61-62)
+  for (int s = 0; s < 2; ++s) {
+    const int nn = c.side[s].nn;
+    if (nn == 0) {
+      if (c.loss == PBG_LOSS_LOGISTIC && lane == 0) loss_acc += softplusf(-posv[s]);  // losses.py:63
+      continue;
+    }
+    ScoreRow sr = score_row(c, s, kc, cc, i);
+    int ge;
+    row_rank_and_loss(c.loss, c.margin, sr, nn, posv[s], lane, &loss_acc, &ge);
+    rank[s] = (int64_t)ge + 1;
+  }
+  const float loss_row = wave_sum(loss_acc) * w;
+  if (lane == 0) {
+    lhs_pos[job] = posv[0];
+    rhs_pos[job] = posv[1];
+    lhs_rank[job] = rank[0];
+    rhs_rank[job] = rank[1];
+    loss_edge[job] = loss_row;
+  }
+}
+
+// util.py:420-428 over the call's edges: sample (a positive, an entry of the side's negatives), count
+// "positive > negative".  One thread per sample and side; pos = the scores ranks_out_kernel wrote.
+__global__ __launch_bounds__(256) void auc_sample_kernel(StepCtx c, const float* __restrict__ lhs_pos,
+                                                         const float* __restrict__ rhs_pos, int64_t samples,
+                                                         uint64_t seed, unsigned long long* __restrict__ hits) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int s = blockIdx.y;
+  const int nn = c.side[s].nn;
+  bool hit = false;
+  if (n < samples && nn > 0) {
+    const int64_t edges = (int64_t)c.K * c.B;
+    const uint64_t r0 = philox_u64(seed, (uint64_t)n, (uint32_t)(2 * s)), r1 = philox_u64(seed, (uint64_t)n, (uint32_t)(2 * s + 1));
+    const int64_t ep = (int64_t)(r0 % (uint64_t)edges);
+    const uint64_t flat = r1 % ((uint64_t)edges * (uint64_t)nn);
+    const int64_t en = (int64_t)(flat / (uint64_t)nn);
+    const int j = (int)(flat % (uint64_t)nn);
+    const int k = (int)(en / c.B), q = (int)(en % c.B);
+    const int cc = q / c.P, i = q % c.P;
+    ScoreRow sr = score_row(c, s, (int64_t)k * c.C + cc, cc, i);
+    bool live;
+    hit = (s == 0 ? lhs_pos : rhs_pos)[ep] > sr.at(j, &live);
+  }
+  const uint64_t m = __ballot(hit);
+  if ((threadIdx.x & 63) == 0 && m != 0ull) atomicAdd(&hits[s], (unsigned long long)__popcll(m));
+}
+
+__global__ void zero_u64_kernel(unsigned long long* p, int n) {
+  if ((int)threadIdx.x < n) p[threadIdx.x] = 0ull;
+}
+
 // ---------------------------------------------------------------------------
 // rowback
 // ---------------------------------------------------------------------------
@@ -2542,6 +2645,34 @@ extern "C" int pbg_train_step_profile(const pbg_step_desc* desc, const pbg_step_
   }
   for (int i = 0; i <= kStages; ++i) hipEventDestroy(ev[i]);
   return rc;
+}
+
+extern "C" int pbg_model_ranks(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos, float* rhs_pos,
+                               int64_t* lhs_rank, int64_t* rhs_rank, float* loss_edge, int64_t auc_samples,
+                               uint64_t auc_seed, int64_t* auc_hits, pbg_stream_t stream) {
+  int rc = validate(desc, false);
+  if (rc != PBG_OK) return rc;
+  Plan plan;
+  make_plan(desc, bufs, &plan);
+  if ((rc = check_buffers(desc, bufs, plan, false)) != PBG_OK) return rc;
+  const StepCtx& c = plan.c;
+  if (!lhs_pos || !rhs_pos || !lhs_rank || !rhs_rank || !loss_edge || (auc_samples > 0 && !auc_hits) || auc_samples < 0)
+    return fail(PBG_ERR_INVALID, "pbg_model_ranks: null output");
+  hipStream_t s = (hipStream_t)stream;
+  RelOrder rel_order;
+  if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
+  if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
+  if ((rc = run_operator_forward(plan, s, &rel_order)) != PBG_OK) return rc;
+  if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
+  hipLaunchKernelGGL(ranks_out_kernel, wave_grid((int64_t)c.K * c.B), dim3(kRowThreads), 0, s, c, lhs_pos, rhs_pos, lhs_rank,
+                     rhs_rank, loss_edge);
+  if (auc_samples > 0) {
+    static_assert(sizeof(unsigned long long) == sizeof(int64_t), "auc_hits is written as two 64-bit counters");
+    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(64), 0, s, (unsigned long long*)auc_hits, 2);
+    hipLaunchKernelGGL(auc_sample_kernel, dim3((unsigned)ceil_div(auc_samples, 256), 2), dim3(256), 0, s, c, lhs_pos, rhs_pos,
+                       auc_samples, auc_seed, (unsigned long long*)auc_hits);
+  }
+  return check_launch("pbg_model_ranks");
 }
 
 extern "C" int pbg_model_forward(const pbg_step_desc* desc, const pbg_step_buffers* bufs, float* lhs_pos,

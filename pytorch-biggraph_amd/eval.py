@@ -48,12 +48,44 @@ def ranking_stats(sides, loss: float, count: int) -> Stats:
     )
 
 
+def ranking_stats_from_ranks(ranks, loss: float, count: int, auc_hits=None, auc_samples: int = 0) -> Stats:
+    """The same sums from per-edge ranks (StepRunner.ranks / pbg_model_ranks), one
+    int64 tensor per side that has negatives.  auc_hits[side] of auc_samples random
+    (positive, negative) pairs had positive > negative (util.py:420-428)."""
+    ranks = [r.reshape(-1) for r in ranks]
+    if auc_hits is not None and auc_samples > 0:
+        auc = count * sum(float(h) / auc_samples for h in auc_hits) / len(auc_hits)
+    else:
+        auc = 0.0
+    return Stats(
+        loss=float(loss),
+        pos_rank=average_of_sums(*ranks),
+        mrr=average_of_sums(*(rank.float().reciprocal() for rank in ranks)),
+        r1=average_of_sums(*(rank.le(1) for rank in ranks)),
+        r10=average_of_sums(*(rank.le(10) for rank in ranks)),
+        r50=average_of_sums(*(rank.le(50) for rank in ranks)),
+        auc=auc,
+        count=count,
+    )
+
+
 class RankingEvaluator(AbstractBatchProcessor):
     """eval.py:43-86: rank of each positive among its negatives (ties count
     against the positive), MRR, hits@1/10/50 and a randomized AUC, averaged over
     the sides that have negatives; sums over the batch, to be divided by count."""
 
     def _process_one_batch(self, model: MultiRelationEmbedder, batch_edges: EdgeList) -> Stats:
+        # Without a score filter (the _adjust_scores hook) nothing needs the [B, N] score matrices: ranks,
+        # loss and the AUC count come from one call, per edge.
+        if type(self)._adjust_scores is RankingEvaluator._adjust_scores and len(batch_edges) > 0:
+            count = len(batch_edges)
+            kind = batch_edges.get_relation_type_as_scalar() if batch_edges.has_scalar_relation_type() else 0
+            out = model.forward_ranks(batch_edges, loss=self.loss_fn.loss_name, margin=self.loss_fn.fused_margin,
+                                      relation_weight=float(self.relation_weights[kind]), auc_samples=count,
+                                      auc_seed=int(torch.randint(0, 2**62, (1,))))
+            sides = [s for s in range(2) if out.has_negs[s]]
+            return ranking_stats_from_ranks([out.ranks[s] for s in sides], float(out.loss_edge.sum()), count,
+                                            [out.auc_hits[s] for s in sides], count)
         with torch.no_grad():
             scores, _ = model(batch_edges)
         self._adjust_scores(scores, batch_edges)

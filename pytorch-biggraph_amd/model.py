@@ -261,6 +261,16 @@ class Scores(NamedTuple):
     rhs_neg: FloatTensorType
 
 
+class RankOutput(NamedTuple):
+    """forward_ranks: per edge, without the [B, N] score matrices."""
+    lhs_pos: FloatTensorType
+    rhs_pos: FloatTensorType
+    ranks: Tuple[torch.Tensor, torch.Tensor]  # (lhs, rhs): 1 + negatives scoring at least as high as the positive
+    loss_edge: FloatTensorType                # relation weight x edge weight x (lhs loss + rhs loss)
+    auc_hits: Optional[torch.Tensor]          # [2]: random (positive, negative) pairs with positive > negative
+    has_negs: Tuple[bool, bool]               # a side without negatives has no rank
+
+
 class MultiRelationEmbedder(nn.Module):
     """A multi-relation embedding model scored against batch and uniform
     negatives (model.py:368-856)."""
@@ -424,6 +434,46 @@ class MultiRelationEmbedder(nn.Module):
             rhs_op, lhs_op = self.rhs_operators[relation_idx], self.lhs_operators[relation_idx]
             return (self.regularizer.forward_dynamic(chunked(lhs_pos, None), chunked(rhs_pos, rhs_op), rhs_op, rel)
                     + self.regularizer.forward_dynamic(chunked(rhs_pos, None), chunked(lhs_pos, lhs_op), lhs_op, rel))
+
+    def forward_ranks(self, edges: EdgeList, uniform_negs=None, *, loss: str = "ranking", margin: float = 0.1,
+                      relation_weight: float = 1.0, auc_samples: int = 0, auc_seed: int = 0) -> "RankOutput":
+        """What ranking evaluation takes from forward() -- the positive scores, the rank
+        of every positive among its negatives on either side, the loss -- computed per
+        edge on the device without the [B, N] score matrices (pbg_model_ranks;
+        reference: eval.py:43-81 over model.py:624-762).  The batch must not be empty."""
+        num_pos = len(edges)
+        relation_idx, lhs_module, rhs_module = self.resolve(edges)
+        if self.num_batch_negs == 0 and self.num_uniform_negs == 0 and not self.relations[relation_idx].all_negs:
+            raise ValueError("num_batch_negs and num_uniform_negs cannot both be 0")
+        if num_pos == 0:
+            raise ValueError("forward_ranks needs at least one edge")
+        w_l, w_r = lhs_module.weight, rhs_module.weight
+        dev = w_l.device
+        spec = self.step_spec(relation_idx, num_pos, w_l.shape[1], loss=loss, margin=float(margin))
+        key = ("ranks", relation_idx, num_pos, w_l.data_ptr(), w_r.data_ptr(), loss, float(margin))
+        runner = self._runners.get(key)
+        if runner is None:
+            rhs_op, lhs_op = self.operator_tensors(relation_idx)
+            glob = self.global_vectors(relation_idx)
+            runner = native.StepRunner(spec, w_l.data, torch.empty(0, device=dev), w_r.data, torch.empty(0, device=dev),
+                                       rhs_op, None, lhs_op, None,
+                                       global_embs=None if glob is None else (glob[0].data, glob[1].data))
+            self._runners[key] = runner
+        runner.relation_weights.fill_(float(relation_weight))
+        if uniform_negs is None:
+            uniform_negs = self.sample_uniform(lhs_module, rhs_module, spec.num_chunks)
+        ul, ur = uniform_negs
+        lhs = edges.lhs.to_tensor().to(dev).contiguous()
+        rhs = edges.rhs.to_tensor().to(dev).contiguous()
+        if self.num_dynamic_rels > 0:
+            rel = edges.get_relation_type_as_vector().to(dev).contiguous()
+        else:
+            rel = torch.zeros(1, dtype=torch.int64, device=dev)  # the runner holds this relation's operator only
+        weight = edges.weight.to(dev).float().contiguous() if edges.has_weight() else None
+        lp, rp, lr, rr, le, hits = runner.ranks(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
+                                                ur.contiguous() if ur is not None else None, weight, auc_samples, auc_seed)
+        has = (spec.num_negs(self.disable_lhs_negs, w_l.shape[0]) > 0, spec.num_negs(self.disable_rhs_negs, w_r.shape[0]) > 0)
+        return RankOutput(lp[0], rp[0], (lr[0], rr[0]), le[0], hits, has)
 
     def forward(self, edges: EdgeList, uniform_negs=None) -> Tuple[Scores, Optional[FloatTensorType]]:
         """Scores of a batch and the regularizer's value, None without a

@@ -464,6 +464,27 @@ class StepRunner:
         check(_lib.lib().pbg_train_step_profile(ctypes.byref(self.desc), ctypes.byref(bufs), _stream(), out))
         return [float(x) for x in out]
 
+    def ranks(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None, auc_samples: int = 0,
+              auc_seed: int = 0):
+        """What ranking evaluation needs of a forward pass, without the [K, B, N]
+        score tensors (pbg_model_ranks): (lhs_pos[K,B], rhs_pos[K,B], lhs_rank[K,B],
+        rhs_rank[K,B] -- 1 + negatives scoring at least as high, 0 for a side without
+        negatives --, loss_edge[K,B] under spec.loss, auc_hits[2] or None)."""
+        s = self.spec
+        k, b = s.num_workers, s.batch_size
+        bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight)
+        dev = self.device
+        lhs_pos = torch.empty((k, b), dtype=torch.float32, device=dev)
+        rhs_pos = torch.empty((k, b), dtype=torch.float32, device=dev)
+        lhs_rank = torch.empty((k, b), dtype=torch.int64, device=dev)
+        rhs_rank = torch.empty((k, b), dtype=torch.int64, device=dev)
+        loss_edge = torch.empty((k, b), dtype=torch.float32, device=dev)
+        hits = torch.empty(2, dtype=torch.int64, device=dev) if auc_samples > 0 else None
+        check(_lib.lib().pbg_model_ranks(ctypes.byref(self.desc), ctypes.byref(bufs), _ptr(lhs_pos), _ptr(rhs_pos),
+                                         _ptr(lhs_rank), _ptr(rhs_rank), _ptr(loss_edge), int(auc_samples),
+                                         auc_seed & (2**64 - 1), _ptr(hits), _stream()))
+        return lhs_pos, rhs_pos, lhs_rank, rhs_rank, loss_edge, hits
+
     def forward(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None):
         """Scores only: (lhs_pos[K,B], rhs_pos[K,B], lhs_neg[K,B,Nl], rhs_neg[K,B,Nr])."""
         s = self.spec

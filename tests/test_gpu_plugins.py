@@ -436,3 +436,20 @@ def test_ranking_evaluator(pbg):
     assert 0.0 <= m["auc"] <= num_pos
     avg = pbg.stats.Stats.sum([stats]).average()
     assert 0.0 <= avg.metrics["auc"] <= 1.0 and 1.0 <= avg.metrics["pos_rank"] <= 21.0
+
+    # An evaluator that overrides the score hook (a filtered evaluator, eval.py:82-86) needs the score
+    # matrices and takes the other way through the same numbers: everything but the sampled AUC is equal.
+    class Hooked(pbg.eval.RankingEvaluator):
+        seen = 0
+
+        def _adjust_scores(self, scores, batch_edges):
+            Hooked.seen += 1
+            assert scores.lhs_neg.shape == (num_pos, 20)
+
+    hooked = Hooked(loss_fn, list(cfg.relation_weights)).process_one_batch(
+        model, ED(EL.from_tensor(lhs.to(DEV)), EL.from_tensor(rhs.to(DEV)), torch.tensor(rel)))
+    assert Hooked.seen == 1
+    for key in ("pos_rank", "mrr", "r1", "r10", "r50"):
+        assert hooked.metrics[key] == m[key], key
+    assert hooked.metrics["loss"] == pytest.approx(m["loss"], rel=1e-5)
+    assert abs(hooked.metrics["auc"] - m["auc"]) < 0.35 * num_pos  # two random samples of num_pos pairs each

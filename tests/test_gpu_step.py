@@ -648,6 +648,59 @@ REG_CASES = [
 ]
 
 
+RANK_CASES = [
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=50, num_uniform_negs=50, num_pos=230, dim=100),
+    dict(operator="none", comparator="cos", loss="softmax", num_batch_negs=20, num_uniform_negs=300, num_pos=90, dim=32),
+    dict(operator="translation", comparator="l2", loss="ranking", num_batch_negs=16, num_uniform_negs=40, num_pos=70, dim=24,
+         shared=False),
+    dict(operator="complex_diagonal", comparator="dot", loss="logistic", dynamic=True, num_batch_negs=10, num_uniform_negs=25,
+         num_pos=45, dim=16),
+    dict(operator="diagonal", comparator="squared_l2", loss="softmax", num_batch_negs=0, num_uniform_negs=64, num_pos=40, dim=20),
+    dict(operator="linear", comparator="cos", loss="logistic", num_batch_negs=12, num_uniform_negs=0, num_pos=30, dim=16,
+         disable_lhs_negs=True),
+    dict(operator="none", comparator="dot", loss="softmax", num_batch_negs=8, num_uniform_negs=8, num_pos=20, dim=12, bias=True),
+    dict(operator="none", comparator="dot", loss="ranking", num_batch_negs=7, num_uniform_negs=0, num_pos=25, dim=12,
+         all_negs=True),
+]
+
+
+@pytest.mark.parametrize("case", RANK_CASES, ids=ids)
+@pytest.mark.parametrize("workers", [1, 3])
+def test_model_ranks(pbg, case, workers):
+    """pbg_model_ranks (the evaluator's ranks, loss and AUC count without the [B, N]
+    score matrices, eval.py:57-81) against the matrices of pbg_model_forward -- the
+    ranks count `negative >= positive` over the very same floats, so they are equal
+    bit for bit -- and against the oracle's loss; the AUC count against the exact
+    fraction of (positive, negative) pairs with positive > negative."""
+    say("ranks", case, workers)
+    case = dict(case)
+    num_pos, dim, shared = case.pop("num_pos"), case.pop("dim"), case.pop("shared", True)
+    cfg = ostep.StepConfig(dim=dim, num_relations=3, relation_weights=[1.0, 0.5, 2.0], margin=0.1, **case)
+    st, batches = make_inputs(cfg, num_pos, 300, workers, seed=3 * num_pos + dim, shared=shared)
+    runner = to_runner(pbg, cfg, st, num_pos, workers)
+    args = pack(cfg, batches)
+    g = torch.Generator().manual_seed(5)
+    weight = (torch.rand(workers, num_pos, generator=g) + 0.5).to(DEV)
+    lp, rp, ln, rn = runner.forward(*args)
+    samples = 200_000
+    for ew in (None, weight):
+        glp, grp, lrank, rrank, loss_edge, hits = runner.ranks(*args, edge_weight=ew, auc_samples=samples, auc_seed=11)
+        torch.cuda.synchronize()
+        assert torch.equal(glp, lp) and torch.equal(grp, rp)
+        for side, (pos, neg, rank) in enumerate(((lp, ln, lrank), (rp, rn, rrank))):
+            if neg.shape[-1] == 0:
+                assert int(rank.abs().sum()) == 0
+                continue
+            assert torch.equal(rank, (neg >= pos.unsqueeze(-1)).sum(-1) + 1), side
+            exact = float((pos.reshape(-1, 1) > neg.reshape(1, -1)).double().mean())
+            sigma = (max(exact * (1 - exact), 1e-4) / samples) ** 0.5
+            assert abs(int(hits[side]) / samples - exact) < 6 * sigma + 1e-4, (side, int(hits[side]) / samples, exact)
+        for k, b in enumerate(batches):
+            w = None if ew is None else ew[k].cpu()
+            out = ostep.forward_backward(cfg, copy_of(st), *b, weight=w)[0]
+            assert float(loss_edge[k].double().sum()) == pytest.approx(out.loss, rel=2e-5, abs=1e-6), (k, ew is not None)
+
+
 @pytest.mark.parametrize("case", REG_CASES, ids=ids)
 @pytest.mark.parametrize("workers", [1, 3])
 def test_train_step_with_n3_regularizer(pbg, case, workers):
