@@ -16,8 +16,9 @@ JSON line.
 Without `--workload` the line is cfg1's (the configuration the metric is quoted
 on) and carries, under "configs", the same measurement for every other BASELINE
 configuration (cfg2 standard and with one relation per edge, cfg2b = cfg2 with
-1000 batch negatives, cfg3 on the graph BASELINE states and on the harsher
-cfg3-hot, cfg4, cfg5), each with its own roofline entry, strictly sequential
+1000 batch negatives, cfg2cos = cfg2's shape under the reference's default
+comparator, cfg3 on the graph BASELINE states and on the harsher cfg3-hot, cfg4,
+cfg5), each with its own roofline entry, strictly sequential
 value and CPU baseline; under "k_sweep" cfg1 at 1 ... 64 batches per call; under
 "standalone" the gather / RowAdagrad kernels alone; under "perm_kernels" the
 permutation helpers; under "cfg4_epoch" one pass over cfg4's 16 buckets with
@@ -131,7 +132,7 @@ DEFAULT_BATCHES = {"cfg1": 64000, "cfg1cos": 64000, "cfg2": 400, "cfg2b": 1600, 
                    "d400": 6400, "d200": 6400, "d256dot": 6400, "d400cos": 6400, "d200transe": 6400, "livejournal": 3200,
                    "cfg3": 40, "cfg3-hot": 40, "cfg4": 32000, "cfg5": 400, "cfg5s": 800}
 # the configurations reported under "configs" beside the cfg1 line, with (timed calls, warm-up calls, CPU seconds)
-EXTRA_CONFIGS = {"cfg2": (10, 2, 4.0), "cfg2d": (10, 2, 4.0), "cfg2b": (10, 2, 4.0), "cfg3": (3, 1, 5.0),
+EXTRA_CONFIGS = {"cfg2": (10, 2, 4.0), "cfg2d": (10, 2, 4.0), "cfg2b": (10, 2, 4.0), "cfg2cos": (10, 2, 4.0), "cfg3": (3, 1, 5.0),
                  "cfg3-hot": (3, 1, 0.0), "cfg4": (100, 10, 4.0), "cfg5": (10, 2, 4.0)}
 
 

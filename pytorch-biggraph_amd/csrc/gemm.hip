@@ -237,7 +237,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g, int a
           if (row < g.m && col < g.n) {
             float* dst = c + (int64_t)row * g.ldc + col;
             float v = g.alpha * (tot[i][j][r] + acc[i][j][r]);
-            if (g.beta != 0.f) v += g.beta * *dst;
+            // HALF: the product is a Half tensor of its own before autograd adds it to what is there
+            // (two roundings: of the product, then of the sum)
+            if (g.beta != 0.f) v = (HALF ? (float)(_Float16)v : v) + g.beta * *dst;
             *dst = HALF ? (float)(_Float16)v : v;
           }
         }
@@ -435,7 +437,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dma_kernel(GemmArgs g) {
           if (row < g.m && col < g.n) {
             float* dst = c + (int64_t)row * g.ldc + col;
             float v = g.alpha * (tot[i][j][r] + acc[i][j][r]);
-            if (g.beta != 0.f) v += g.beta * *dst;
+            // HALF: the product is a Half tensor of its own before autograd adds it to what is there
+            // (two roundings: of the product, then of the sum)
+            if (g.beta != 0.f) v = (HALF ? (float)(_Float16)v : v) + g.beta * *dst;
             *dst = HALF ? (float)(_Float16)v : v;
           }
         }

@@ -51,7 +51,7 @@ inline int bits_for(uint64_t max_value) {  // number of bits needed to hold max_
 // If `long_runs` is given it receives a device pointer (into `temp`) to a word that is zero after the
 // sort only if no value of the sorted bits occurs more than kFoldMax times -- what lets a single-worker
 // RowAdagrad step skip its duplicate-summation kernels.
-constexpr int kFoldMax = 16;
+constexpr int kFoldMax = 8;
 size_t sort_temp_bytes(int64_t n);
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
                int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted,
@@ -64,9 +64,17 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
 // `long_runs` (single-worker calls, kbits == 0): the word sort_pairs leaves behind; where it is zero the
 // duplicate-summation kernels return at once (no key occurs more than kFoldMax times, and the update
 // kernel sums such runs itself).  nullptr: not known.
+// `cos_back`: the gradient rows are gradients at the NORMALISED rows y = x / |x| of the tables (a step with the
+// cos comparator that scored on a normalised copy of the tables): y0 / y1 are that copy of table 0 / 1 and
+// inv0 / inv1 the rows' 1 / |x|, all as they were when the call began.  Every run's summed gradient then goes back
+// through the normalisation, g <- (g - y <y, g>) / |x| (model.py:187-192 under autograd), before its Adagrad step.
+struct CosBack {
+  const float* y0; const float* inv0; const float* y1; const float* inv1;
+};
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits,
                        float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
-                       float* g1, int64_t rows1, float lr, hipStream_t stream, const uint32_t* long_runs = nullptr);
+                       float* g1, int64_t rows1, float lr, hipStream_t stream, const uint32_t* long_runs = nullptr,
+                       const CosBack* cos_back = nullptr);
 
 // ---- plain fp32 batched GEMM on MFMA ----------------------------------------
 // C[b] (M x N, row-major, ldc) = alpha * A[b] * B[b] + beta * C[b], for b in [0, batch).

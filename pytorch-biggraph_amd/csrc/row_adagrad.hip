@@ -233,17 +233,18 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
   const bool starts = (mine < end) && (lane == 0 || prev != key);
   uint64_t heads = __ballot(starts);  // bit l set: a piece starts at begin + l
   // How far the runs at the tile's two edges go on outside it, up to kFoldMax positions each way:
-  // lanes 0 .. 15 look at the positions before the tile (nearest first), lanes 16 .. 31 at those after it.
+  // lanes 0 .. kFoldMax - 1 look at the positions before the tile (nearest first), the next kFoldMax at those after it.
   int before = 0, after = 0;
   if (leave_mode != 0) {
     const uint64_t first_key = lane_u64(key, 0), last_key = lane_u64(key, (int)(end - begin) - 1);
     const int64_t q = lane < kFoldMax ? begin - 1 - lane : end + (lane - kFoldMax);
     const bool there = lane < 2 * kFoldMax && q >= 0 && q < n;
     const uint64_t other = there ? keys[q] : 0ull;
-    const uint32_t same_before = (uint32_t)__ballot(there && lane < kFoldMax && other == first_key) & 0xffffu;
-    const uint32_t same_after = (uint32_t)(__ballot(there && lane >= kFoldMax && other == last_key) >> kFoldMax) & 0xffffu;
-    before = same_before == 0xffffu ? kFoldMax : __ffs((int)~same_before) - 1;  // leading ones
-    after = same_after == 0xffffu ? kFoldMax : __ffs((int)~same_after) - 1;
+    constexpr uint32_t kAll = (1u << kFoldMax) - 1u;
+    const uint32_t same_before = (uint32_t)__ballot(there && lane < kFoldMax && other == first_key) & kAll;
+    const uint32_t same_after = (uint32_t)(__ballot(there && lane >= kFoldMax && other == last_key) >> kFoldMax) & kAll;
+    before = same_before == kAll ? kFoldMax : __ffs((int)~same_before) - 1;  // leading ones
+    after = same_after == kAll ? kFoldMax : __ffs((int)~same_after) - 1;
   }
   while (heads != 0ull) {
     const int a = __ffsll((unsigned long long)heads) - 1;
@@ -319,9 +320,21 @@ __global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t
   acc.store(head, nv, lane);
 }
 
-template <int NV, bool VEC>
-__device__ __forceinline__ float adagrad_apply(RowRegs<NV, VEC>& w, const RowRegs<NV, VEC>& g, float gsum, float fdim,
-                                               float lr) {
+// With COSB the gradient rows are gradients at the NORMALISED row y = x / |x| (the step scored on a normalised
+// copy of the table, see CosBack): a run's summed gradient first goes back through the normalisation,
+// g <- (g - y <y, g>) / |x|, which is linear in g and so may follow the sum over the run's duplicates.
+template <int NV, bool VEC, bool COSB = false>
+__device__ __forceinline__ float adagrad_apply(RowRegs<NV, VEC>& w, const RowRegs<NV, VEC>& g_in, float gsum, float fdim,
+                                               float lr, const RowRegs<NV, VEC>* y = nullptr, float inv = 0.f) {
+  RowRegs<NV, VEC> g = g_in;
+  if (COSB) {
+    float dot = 0.f;
+#pragma unroll
+    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) dot += y->v[q] * g.v[q];
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) g.v[q] = (g.v[q] - dot * y->v[q]) * inv;
+  }
   float sq = 0.f;
 #pragma unroll
   for (int q = 0; q < NV * RowRegs<NV, VEC>::W; ++q) sq += g.v[q] * g.v[q];
@@ -348,11 +361,11 @@ __device__ __forceinline__ int64_t lower_bound_key(const uint64_t* __restrict__ 
 // windows, then the weight rows and first gradient rows of the positions that
 // turned out to be row heads) are issued together: the kernel lives on memory
 // latency, and the rows in flight per wave are what hides it.
-template <int NV, bool VEC, int R>
+template <int NV, bool VEC, int R, bool COSB = false>
 __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
     const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
-    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
+    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr, CosBack cb) {
   const int lane = threadIdx.x & 63;
   const int64_t first = ((int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6)) * R;
   if (first >= n) return;
@@ -374,12 +387,15 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   float* gptr[R];
   float gsum[R];
   RowRegs<NV, VEC> w[R], g[R];
+  RowRegs<NV, VEC> y[COSB ? R : 1];
+  float inv[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int64_t i = first + r;
     const uint64_t row = lane_u64(kk[r], 0) >> kbits;
     // out-of-range indices are parked past both tables
     head[r] = i < n && !(i > 0 && (before[r] >> kbits) == row) && (int64_t)row < rows0 + rows1;
+    inv[r] = 0.f;
     if (!head[r]) continue;
     if ((int64_t)row < rows0) {
       wrow[r] = w0 + (int64_t)row * dim;
@@ -387,6 +403,11 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
     } else {
       wrow[r] = w1 + ((int64_t)row - rows0) * dim;
       gptr[r] = g1 + ((int64_t)row - rows0);
+    }
+    if (COSB) {
+      const bool t0 = (int64_t)row < rows0;
+      y[COSB ? r : 0].load(t0 ? cb.y0 + (int64_t)row * dim : cb.y1 + ((int64_t)row - rows0) * dim, nv, lane);
+      inv[r] = t0 ? cb.inv0[row] : cb.inv1[(int64_t)row - rows0];
     }
     w[r].load(wrow[r], nv, lane);
     gsum[r] = *gptr[r];
@@ -398,7 +419,14 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
 #pragma unroll
       for (int t = 1; t < 4; ++t)  // the common lengths with their loads in flight together
         g[r].add_if(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane, fold && t < run_len);
-      for (int t = 4; fold && t < run_len; ++t) g[r].add(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane);
+      for (int t = 4; fold && t < run_len; t += 2) {  // two rows in flight
+        RowRegs<NV, VEC> x, y;
+        x.load(grad_rows + (int64_t)lane_u32(vv[r], t) * dim, nv, lane);
+        y.zero();
+        if (t + 1 < run_len) y.load(grad_rows + (int64_t)lane_u32(vv[r], t + 1) * dim, nv, lane);
+        g[r].add(x);
+        g[r].add(y);
+      }
     }
   }
   int long_r = -1;
@@ -419,12 +447,12 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
         heads &= heads - 1;
         RowRegs<NV, VEC> next;
         next.load(grad_rows + (int64_t)lane_u32(vv[r], a) * dim, nv, lane);
-        gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+        gsum[r] = adagrad_apply<NV, VEC, COSB>(w[r], g[r], gsum[r], fdim, lr, &y[COSB ? r : 0], inv[r]);
         g[r] = next;
       }
-      gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+      gsum[r] = adagrad_apply<NV, VEC, COSB>(w[r], g[r], gsum[r], fdim, lr, &y[COSB ? r : 0], inv[r]);
     } else if (kbits == 0) {  // a single-worker call has one run per row
-      gsum[r] = adagrad_apply(w[r], g[r], gsum[r], fdim, lr);
+      gsum[r] = adagrad_apply<NV, VEC, COSB>(w[r], g[r], gsum[r], fdim, lr, &y[COSB ? r : 0], inv[r]);
     } else {
       // A long row: handled after this loop.  There is at most one per wave (the positions after its head belong
       // to it), so the code below exists once instead of once per position, in the registers that this loop's rows
@@ -441,7 +469,13 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
   const uint64_t row = keys[i] >> kbits;
   float* long_wrow = (int64_t)row < rows0 ? w0 + (int64_t)row * dim : w1 + ((int64_t)row - rows0) * dim;
   float* long_gptr = (int64_t)row < rows0 ? g0 + row : g1 + ((int64_t)row - rows0);
-  RowRegs<NV, VEC> lw, lg;
+  RowRegs<NV, VEC> lw, lg, ly;
+  float linv = 0.f;
+  if (COSB) {
+    const bool t0 = (int64_t)row < rows0;
+    ly.load(t0 ? cb.y0 + (int64_t)row * dim : cb.y1 + ((int64_t)row - rows0) * dim, nv, lane);
+    linv = t0 ? cb.inv0[row] : cb.inv1[(int64_t)row - rows0];
+  }
   lw.load(long_wrow, nv, lane);
   float lsum = *long_gptr;
   lg.load(grad_rows + (int64_t)vals[i] * dim, nv, lane);
@@ -484,12 +518,12 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
 #pragma unroll
       for (int t = 0; t < kAhead; ++t) {
         if (js[t] < 0) break;
-        lsum = adagrad_apply(lw, lg, lsum, fdim, lr);
+        lsum = adagrad_apply<NV, VEC, COSB>(lw, lg, lsum, fdim, lr, &ly, linv);
         lg = nx[t];
       }
     }
   }
-  lsum = adagrad_apply(lw, lg, lsum, fdim, lr);
+  lsum = adagrad_apply<NV, VEC, COSB>(lw, lg, lsum, fdim, lr, &ly, linv);
   lw.store(long_wrow, nv, lane);
   if (lane == 0) *long_gptr = lsum;
 }
@@ -504,11 +538,11 @@ __global__ __launch_bounds__(kRowThreads) void row_update_kernel(
 // tile_reduce left alone -- are known from the keys of the window alone, so
 // R of them are in flight at a time whatever run they belong to, and the runs' Adagrad
 // steps follow in worker order on registers.
-template <int NV, bool VEC, int R>
+template <int NV, bool VEC, int R, bool COSB = false>
 __global__ __launch_bounds__(kRowThreads) void row_walk_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
     const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
-    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
+    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr, CosBack cb) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
   if (row >= rows0 + rows1) return;
@@ -530,7 +564,12 @@ __global__ __launch_bounds__(kRowThreads) void row_walk_kernel(
   const float fdim = (float)dim;
   float* wrow = row < rows0 ? w0 + row * dim : w1 + (row - rows0) * dim;
   float* gptr = row < rows0 ? g0 + row : g1 + (row - rows0);
-  RowRegs<NV, VEC> w, acc;
+  RowRegs<NV, VEC> w, acc, y;
+  float inv = 0.f;
+  if (COSB) {
+    y.load(row < rows0 ? cb.y0 + row * dim : cb.y1 + (row - rows0) * dim, nv, lane);
+    inv = row < rows0 ? cb.inv0[row] : cb.inv1[row - rows0];
+  }
   w.load(wrow, nv, lane);
   float gsum = *gptr;
   acc.zero();
@@ -583,7 +622,7 @@ __global__ __launch_bounds__(kRowThreads) void row_walk_kernel(
         if (pos[r] < 0) break;
         acc.add(x[r]);
         if ((done >> pos[r]) & 1ull) {
-          gsum = adagrad_apply(w, acc, gsum, fdim, lr);
+          gsum = adagrad_apply<NV, VEC, COSB>(w, acc, gsum, fdim, lr, &y, inv);
           acc.zero();
         }
       }
@@ -616,7 +655,17 @@ __device__ __forceinline__ float4 load_or_zero(const float* __restrict__ p, bool
 __device__ __forceinline__ void add4(float4& a, const float4& b) {
   a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
 }
-__device__ __forceinline__ float adagrad_apply_half(float4& w, const float4& g, float gsum, float fdim, float lr) {
+template <bool COSB = false>
+__device__ __forceinline__ float adagrad_apply_half(float4& w, const float4& g_in, float gsum, float fdim, float lr,
+                                                    const float4& y = float4(), float inv = 0.f) {
+  float4 g = g_in;
+  if (COSB) {  // (see adagrad_apply)
+    const float dot = half_sum((y.x * g.x + y.y * g.y) + (y.z * g.z + y.w * g.w));
+    g.x = (g.x - dot * y.x) * inv;
+    g.y = (g.y - dot * y.y) * inv;
+    g.z = (g.z - dot * y.z) * inv;
+    g.w = (g.w - dot * y.w) * inv;
+  }
   gsum += half_sum(g.x * g.x + g.y * g.y + g.z * g.z + g.w * g.w) / fdim;
   const float stdv = sqrtf(gsum) + 1e-10f;
   w.x += (-lr * g.x) / stdv;
@@ -626,11 +675,11 @@ __device__ __forceinline__ float adagrad_apply_half(float4& w, const float4& g, 
   return gsum;
 }
 
-template <int R>
+template <int R, bool COSB = false>
 __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits,
     const float* __restrict__ grad_rows, int dim, float* __restrict__ w0, float* __restrict__ g0, int64_t rows0,
-    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr) {
+    float* __restrict__ w1, float* __restrict__ g1, int64_t rows1, float lr, CosBack cb) {
   const int lane = threadIdx.x & 63, gl = lane & 31, gbase = lane & 32;
   const int64_t first = ((((int64_t)blockIdx.x * kRowThreads) + threadIdx.x) >> 5) * R;
   const bool has = gl < (dim >> 2);
@@ -651,13 +700,16 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
   float* wrow[R];
   float* gptr[R];
   float gsum[R];
-  float4 w[R], g[R];
+  float4 w[R], g[R], y[R];
+  float inv[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int64_t i = first + r;
     const uint64_t row = half_bcast_u64(kk[r], gbase) >> kbits;
     // out-of-range indices are parked past both tables
     head[r] = i < n && !(i > 0 && (before[r] >> kbits) == row) && (int64_t)row < rows0 + rows1;
+    y[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+    inv[r] = 0.f;
     if (!head[r]) continue;
     if ((int64_t)row < rows0) {
       wrow[r] = w0 + (int64_t)row * dim + col;
@@ -665,6 +717,11 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
     } else {
       wrow[r] = w1 + ((int64_t)row - rows0) * dim + col;
       gptr[r] = g1 + ((int64_t)row - rows0);
+    }
+    if (COSB) {
+      const bool t0 = (int64_t)row < rows0;
+      y[r] = load_or_zero((t0 ? cb.y0 + (int64_t)row * dim : cb.y1 + ((int64_t)row - rows0) * dim) + col, has);
+      inv[r] = t0 ? cb.inv0[row] : cb.inv1[(int64_t)row - rows0];
     }
     w[r] = load_or_zero(wrow[r], has);
     gsum[r] = *gptr[r];
@@ -676,8 +733,15 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
 #pragma unroll
       for (int t = 1; t < 4; ++t)  // the common lengths with their loads in flight together
         add4(g[r], load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + t, 64) * dim + col, has && fold && t < run_len));
-      // (rare: the two halves of the wave differ in their counts here, so the row numbers come from memory, not from a shuffle)
-      for (int t = 4; fold && t < run_len; ++t) add4(g[r], load_or_zero(grad_rows + (int64_t)vals[i + t] * dim + col, has));
+      for (int t0 = 4; fold && t0 < run_len; t0 += 4) {  // (the halves of a wave may differ in their counts; a half reads its own lanes)
+        float4 x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          x[u] = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + min(t0 + u, 31), 64) * dim + col,
+                              has && t0 + u < run_len);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) add4(g[r], x[u]);
+      }
     }
   }
   int long_r = -1;
@@ -697,12 +761,12 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
         const int a = __ffs((int)heads) - 1;
         heads &= heads - 1;
         const float4 next = load_or_zero(grad_rows + (int64_t)__shfl((int)vv[r], gbase + a, 64) * dim + col, has);
-        gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+        gsum[r] = adagrad_apply_half<COSB>(w[r], g[r], gsum[r], fdim, lr, y[r], inv[r]);
         g[r] = next;
       }
-      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+      gsum[r] = adagrad_apply_half<COSB>(w[r], g[r], gsum[r], fdim, lr, y[r], inv[r]);
     } else if (kbits == 0) {  // a single-worker call has one run per row
-      gsum[r] = adagrad_apply_half(w[r], g[r], gsum[r], fdim, lr);
+      gsum[r] = adagrad_apply_half<COSB>(w[r], g[r], gsum[r], fdim, lr, y[r], inv[r]);
     } else {
       // A long row: handled after this loop.  There is at most one per half wave (the
       // positions after its head belong to it), so the code below exists once
@@ -727,6 +791,13 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
   } else {
     long_wrow = w1 + ((int64_t)long_row - rows0) * dim + col;
     long_gptr = g1 + ((int64_t)long_row - rows0);
+  }
+  float4 long_y = make_float4(0.f, 0.f, 0.f, 0.f);
+  float long_inv = 0.f;
+  if (COSB) {
+    const bool t0 = (int64_t)long_row < rows0;
+    long_y = load_or_zero((t0 ? cb.y0 + (int64_t)long_row * dim : cb.y1 + ((int64_t)long_row - rows0) * dim) + col, has);
+    long_inv = t0 ? cb.inv0[long_row] : cb.inv1[(int64_t)long_row - rows0];
   }
   float4 long_w = load_or_zero(long_wrow, has);
   float long_gsum = *long_gptr;
@@ -770,12 +841,12 @@ __global__ __launch_bounds__(kRowThreads) void row_update_half_kernel(
 #pragma unroll
       for (int t = 0; t < kAhead; ++t) {
         if (js[t] < 0) break;
-        long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
+        long_gsum = adagrad_apply_half<COSB>(long_w, long_g, long_gsum, fdim, lr, long_y, long_inv);
         long_g = nx[t];
       }
     }
   }
-  long_gsum = adagrad_apply_half(long_w, long_g, long_gsum, fdim, lr);
+  long_gsum = adagrad_apply_half<COSB>(long_w, long_g, long_gsum, fdim, lr, long_y, long_inv);
   if (has) *reinterpret_cast<float4*>(long_wrow) = long_w;
   if (gl == 0) *long_gptr = long_gsum;
 }
@@ -808,10 +879,10 @@ __global__ void async_adagrad_dense_kernel(float* __restrict__ p, float* __restr
   p[i] += -lr * (gi / (sqrtf(sum) + eps));
 }
 
-template <bool VEC>
+template <bool VEC, bool COSB>
 int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                   int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                  const uint32_t* long_runs, hipStream_t stream) {
+                  const uint32_t* long_runs, CosBack cb, hipStream_t stream) {
   const int wpb = kRowThreads / kWave;
   const dim3 block(kRowThreads);
   const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
@@ -831,18 +902,18 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
                          leave_mode, long_runs);                                                                   \
     if (walk) {                                                                                                    \
       constexpr int R = NV <= 2 ? 8 : (NV <= 4 ? 4 : 2);                                                           \
-      hipLaunchKernelGGL((row_walk_kernel<NV, VEC, R>), walk_grid, block, 0, stream, keys, vals, n, kbits, grad_rows,  \
-                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+      hipLaunchKernelGGL((row_walk_kernel<NV, VEC, R, COSB>), walk_grid, block, 0, stream, keys, vals, n, kbits,      \
+                         grad_rows, dim, w0, g0, rows0, w1, g1, rows1, lr, cb);                                    \
     } else if (VEC && dim <= 128) {                                                                                \
       constexpr int R = 4;                                                                                         \
       const dim3 hgrid((unsigned)ceil_div(ceil_div(n, R) * 32, kRowThreads));                                      \
-      hipLaunchKernelGGL((row_update_half_kernel<R>), hgrid, block, 0, stream, keys, vals, n, kbits, grad_rows,    \
-                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+      hipLaunchKernelGGL((row_update_half_kernel<R, COSB>), hgrid, block, 0, stream, keys, vals, n, kbits,        \
+                         grad_rows, dim, w0, g0, rows0, w1, g1, rows1, lr, cb);                                    \
     } else {                                                                                                       \
       constexpr int R = NV <= 2 ? 4 : (NV <= 4 ? 2 : 1);                                                           \
       const dim3 ugrid((unsigned)ceil_div(ceil_div(n, R), wpb));                                                   \
-      hipLaunchKernelGGL((row_update_kernel<NV, VEC, R>), ugrid, block, 0, stream, keys, vals, n, kbits, grad_rows, \
-                         dim, w0, g0, rows0, w1, g1, rows1, lr);                                                   \
+      hipLaunchKernelGGL((row_update_kernel<NV, VEC, R, COSB>), ugrid, block, 0, stream, keys, vals, n, kbits,    \
+                         grad_rows, dim, w0, g0, rows0, w1, g1, rows1, lr, cb);                                    \
     }                                                                                                              \
   } while (0)
   if (nvec <= 1) PBG_LAUNCH(1);
@@ -863,15 +934,20 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                        int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                       hipStream_t stream, const uint32_t* long_runs) {
+                       hipStream_t stream, const uint32_t* long_runs, const CosBack* cos_back) {
   if (n <= 0) return PBG_OK;
   int rc;
-  if (dim % 4 == 0) {
-    rc = launch_sorted<true>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
-                             g1, rows1, lr, long_runs, stream);
+  const CosBack none{nullptr, nullptr, nullptr, nullptr};
+  if (cos_back) {
+    if (dim % 4 != 0) return fail(PBG_ERR_UNSUPPORTED, "row_adagrad: the normalisation backward needs dim %% 4 == 0");
+    rc = launch_sorted<true, true>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
+                                   g1, rows1, lr, long_runs, *cos_back, stream);
+  } else if (dim % 4 == 0) {
+    rc = launch_sorted<true, false>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
+                                    g1, rows1, lr, long_runs, none, stream);
   } else {
-    rc = launch_sorted<false>((int)ceil_div(dim, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1, g1,
-                              rows1, lr, long_runs, stream);
+    rc = launch_sorted<false, false>((int)ceil_div(dim, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1, g1,
+                                     rows1, lr, long_runs, none, stream);
   }
   if (rc != PBG_OK) return rc;
   return check_launch("row_adagrad_sorted");

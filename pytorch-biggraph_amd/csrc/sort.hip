@@ -346,18 +346,29 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
                                                               shift, (1u << digit_bits) - 1u, first_keys, first_vals);
 }
 
-// One digit pass of a bucket through global memory (a bucket too large for LDS).
+// One digit pass of a bucket through global memory.
 __device__ __forceinline__ void bucket_pass_global(SliceState<kBucketWaves, 8>& st, const uint64_t* keys_in,
                                                    const uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out,
                                                    int64_t begin, int64_t end, int shift, int digit_bits) {
   const int t = threadIdx.x;
   const uint32_t mask = (1u << digit_bits) - 1u;
+  const bool wide = end - begin > 2 * kBucketWaves * 64;  // a swollen bucket
+  uint64_t key_next = 0;
+  uint32_t val_next = 0;
+  if (begin + t < end) {
+    key_next = keys_in[begin + t];
+    val_next = vals_in[begin + t];
+  }
   if (t < 256) {
     st.cursor[t] = 0;
     for (int w = 0; w < kBucketWaves; ++w) st.wave_count[0][w][t] = st.wave_count[1][w][t] = 0;
   }
   __syncthreads();
-  {
+  if (!wide) {
+    if (begin + t < end) atomicAdd(&st.cursor[(uint32_t)(key_next >> shift) & mask], 1u);
+    for (int64_t i = begin + kBucketWaves * 64 + t; i < end; i += kBucketWaves * 64)
+      atomicAdd(&st.cursor[(uint32_t)(keys_in[i] >> shift) & mask], 1u);
+  } else {
     // equal keys would queue up on one counter: one addition per wave and digit value present.
     // Eight loads per thread in flight (the ballots would otherwise wait for each load in turn).
     const int lane = t & 63;
@@ -384,7 +395,11 @@ __device__ __forceinline__ void bucket_pass_global(SliceState<kBucketWaves, 8>& 
   const uint32_t excl = block_exclusive_scan(t < 256 ? st.cursor[t] : 0u, 4, st.wave_total, &grand);
   if (t < 256) st.cursor[t] = (uint32_t)begin + excl;
   __syncthreads();
-  scatter_range_wide<kBucketWaves, 8, 4>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask);
+  if (wide)
+    scatter_range_wide<kBucketWaves, 8, 4>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask);
+  else
+    scatter_range<kBucketWaves, 8>(st, keys_in, vals_in, keys_out, vals_out, begin, end, shift, mask, key_next,
+                                   val_next);
 }
 
 // One digit pass of a bucket's packed words inside LDS: `from` -> `to`, m words, digit = bits
@@ -466,7 +481,8 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t
   const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
   if (begin >= end) return;
   const int64_t m64 = end - begin;
-  if (m64 <= cap && rest <= kLdsMaxRestBits) {
+  // (a single digit pass gains nothing from the detour through LDS: one read and one write either way)
+  if (passes >= 2 && m64 <= cap && rest <= kLdsMaxRestBits) {
     const int m = (int)m64;
     uint32_t* from = lds_words;
     uint32_t* to = lds_words + cap;
@@ -513,7 +529,6 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t
     }
     return;
   }
-  if (long_flag && t == 0) *long_flag = 1u;
   uint64_t* ksrc = ka;
   uint32_t* vsrc = va;
   uint64_t* kdst = kb;
@@ -526,6 +541,12 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t
     uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
     uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
     __syncthreads();  // the next pass reads what this one wrote (same block, workgroup scope)
+  }
+  if (long_flag) {  // the bucket as it lies now: is some value of the sorted bits there more than kFoldMax times?
+    bool found = false;
+    for (int64_t i = begin + t; i + kFoldMax < end; i += kBucketWaves * 64)
+      found |= (ksrc[i] >> low_bit) == (ksrc[i + kFoldMax] >> low_bit);
+    if (found) *long_flag = 1u;
   }
 }
 
@@ -581,7 +602,8 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   uint64_t* kfin = (local & 1) ? keys_in : keys_out;
   uint32_t* vfin = (local & 1) ? vals_in : vals_out;
   hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kBucketWaves * 64), lds_bytes, stream, keys_out, vals_out,
-                     keys_in, vals_in, kfin, vfin, bucket_off, low_bit, rest, local, (int)cap, long_flag);
+                     keys_in, vals_in, kfin, vfin, bucket_off, low_bit, rest, local, (int)cap,
+                     long_runs ? long_flag : nullptr);
   *keys_sorted = kfin;
   *vals_sorted = vfin;
   return check_launch("sort_pairs");

@@ -1780,6 +1780,12 @@ struct Plan {
   FusedLayout fl;
   bool stream;         // the chunk's positives fit LDS and its negatives are streamed past them
   StreamPlan sp;
+  // cos on the streaming route: the route's dot kernels score on a normalised copy of the tables (cos(a, b) is the
+  // dot product of the normalised rows, model.py:185-212), and the update takes every summed gradient back
+  // through the normalisation (CosBack)
+  bool stream_cos;
+  float* ynorm[2];  // the copy of the lhs / rhs table (one copy when the sides share a table)
+  float* yinv[2];   // 1 / |row|
   // dynamic relations: (relation, batch) keys of the positives and their sort buffers
   uint64_t *rkeys_a, *rkeys_b;
   uint32_t *rvals_a, *rvals_b;
@@ -2031,7 +2037,30 @@ int make_plan(const pbg_step_desc* d, const pbg_step_buffers* b, Plan* plan) {
   }
   // The streaming route's own buffers lie behind the staged ones: a call with global
   // embeddings (known only from its buffers) takes the staged route on the same workspace.
-  plan->stream = !plan->fused && !c.half && stream_geometry(c, &plan->sp) && getenv("PBG_DISABLE_STREAM") == nullptr;
+  // cos takes it as dot on a normalised copy of the tables: without an operator (prepare follows the operator,
+  // model.py:478-506, and a normalised copy per relation is not kept), when the copy is modest (2 GiB) and has no more
+  // rows than the call gathers anyway
+  StepCtx as_dot = c;
+  bool cos_copy = false;
+  {
+    const int64_t table_rows = d->num_lhs_rows + (d->shared_table ? 0 : d->num_rhs_rows);
+    if (c.cmp == PBG_CMP_COS && c.op == PBG_OP_NONE && c.reg_coef == 0.f && !c.bias && D % 4 == 0 &&
+        table_rows <= (int64_t)npairs && (size_t)table_rows * D * sizeof(float) <= ((size_t)2 << 30)) {
+      as_dot.cmp = PBG_CMP_DOT;
+      cos_copy = true;
+    }
+  }
+  plan->stream = !plan->fused && !c.half && stream_geometry(as_dot, &plan->sp) && getenv("PBG_DISABLE_STREAM") == nullptr;
+  plan->stream_cos = plan->stream && cos_copy;
+  plan->ynorm[0] = plan->ynorm[1] = plan->yinv[0] = plan->yinv[1] = nullptr;
+  if (plan->stream_cos) {
+    plan->ynorm[0] = takef((size_t)d->num_lhs_rows * D);
+    plan->yinv[0] = takef((size_t)d->num_lhs_rows);
+    if (!d->shared_table) {
+      plan->ynorm[1] = takef((size_t)d->num_rhs_rows * D);
+      plan->yinv[1] = takef((size_t)d->num_rhs_rows);
+    }
+  }
   if (plan->stream) {
     StreamPlan& sp = plan->sp;
     const size_t ne = (size_t)K * c.B;
@@ -2135,6 +2164,21 @@ int check_buffers(const pbg_step_desc* d, const pbg_step_buffers* b, const Plan&
   } while (0)
 
 dim3 wave_grid(int64_t jobs) { return dim3((unsigned)ceil_div(jobs > 0 ? jobs : 1, kWavesPerBlock)); }
+
+// comparator.prepare of the cos comparator on every row of a table (model.py:187-192): out[r] = table[r] * (1 / |table[r]|),
+// inv[r] = 1 / |table[r]|.  One wave per row.  (A zero row gives NaN, as it does in the reference.)
+template <int NVH>
+__global__ __launch_bounds__(kRowThreads) void normalize_rows_kernel(const float* __restrict__ table, int64_t num_rows, int D,
+                                                                     float* __restrict__ out, float* __restrict__ inv) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (r >= num_rows) return;
+  const int H = (D + 1) / 2;
+  RowV<NVH> x = row_load<NVH>(table + r * D, D, H, lane);
+  const float rn = prepare_row<NVH>(PBG_CMP_COS, x);
+  row_store<NVH>(out + r * D, x, D, H, lane);
+  if (lane == 0) inv[r] = rn;
+}
 
 int run_renorm(const Plan& plan, const pbg_step_buffers* b, hipStream_t stream) {
   if (plan.max_norm <= 0.f) return PBG_OK;
@@ -2495,16 +2539,34 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   } join_guard{s};
   mark(0);
   if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
+  CosBack cos_back{nullptr, nullptr, nullptr, nullptr};
+  const CosBack* cos_back_p = nullptr;
   if (stream) {
-    if ((rc = stream_prep(c, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
+    StepCtx cs = c;  // what the streaming kernels see
+    if (plan.stream_cos) {
+      // cos as dot on normalised rows: the tables' normalised copy (as they are now, after max_norm), the route's
+      // dot kernels on it, and the normalisation's backward where the update has summed a row's gradients
+      const int tables = desc->shared_table ? 1 : 2;
+      for (int t = 0; t < tables; ++t) {
+        const int64_t nrows = t ? desc->num_rhs_rows : desc->num_lhs_rows;
+        PBG_DISPATCH_NVH(plan.nvh, normalize_rows_kernel, wave_grid(nrows), s, t ? bufs->w_rhs : bufs->w_lhs, nrows, c.D,
+                         plan.ynorm[t], plan.yinv[t]);
+      }
+      cs.cmp = PBG_CMP_DOT;
+      cs.side[0].w = plan.ynorm[0];
+      cs.side[1].w = plan.ynorm[tables - 1];
+      cos_back = CosBack{plan.ynorm[0], plan.yinv[0], plan.ynorm[1], plan.yinv[1]};
+      cos_back_p = &cos_back;
+    }
+    if ((rc = stream_prep(cs, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
     mark(1);
     mark(2);
-    if ((rc = stream_chunks(c, plan.sp, s)) != PBG_OK) return rc;
+    if ((rc = stream_chunks(cs, plan.sp, s)) != PBG_OK) return rc;
     mark(3);
     mark(4);
     mark(5);
     mark(6);
-    if ((rc = stream_finish(c, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
+    if ((rc = stream_finish(cs, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
     hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
     launch_reg(c, s);
     mark(7);
@@ -2544,7 +2606,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
       if (hipStreamWaitEvent(ss->stream, ss->fork[slot], 0) != hipSuccess)
         return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
       const int sort_rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp,
-                                     ss->stream, &skeys, &svals, &long_runs);
+                                     ss->stream, &skeys, &svals, c.kbits == 0 ? &long_runs : nullptr);
       if (hipEventRecord(ss->join[slot], ss->stream) != hipSuccess)
         return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
       join_guard.ev = sort_done = ss->join[slot];
@@ -2591,17 +2653,18 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if (hipStreamWaitEvent(s, sort_done, 0) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot join the side stream");
   } else {
     rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp, s, &skeys, &svals,
-                    &long_runs);
+                    c.kbits == 0 ? &long_runs : nullptr);
     if (rc != PBG_OK) return rc;
   }
   mark(9);
   if (c.kbits != 0) long_runs = nullptr;  // the word counts positions per ROW; only with one batch per call is that a run
   if (desc->shared_table) {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
-                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s, long_runs);
+                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s, long_runs, cos_back_p);
   } else {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
-                            desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s, long_runs);
+                            desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s, long_runs,
+                            cos_back_p);
   }
   mark(10);
   return rc;

@@ -1,7 +1,9 @@
 // The streaming route of the training step, for chunks whose negatives do not fit
 // LDS next to their positives (hundreds or thousands of uniform negatives per
 // chunk, model.py:508-622 with num_uniform_negs large): dot comparator, operator
-// none / diagonal / complex_diagonal, every loss.
+// none / diagonal / complex_diagonal, every loss.  (The cos comparator without an
+// operator takes these kernels too: the caller hands them a normalised copy of the
+// tables and undoes the normalisation where it applies the gradients.)
 //
 // A work item is (chunk, side s): the chunk's P positives against side s's
 // P + U negatives (the chunk's own side-s rows, then its uniform draws).  The
@@ -821,13 +823,7 @@ bool stream_geometry(const StepCtx& c, StreamPlan* sp) {
   sp->g_at = sp->a_at + sp->pr * sp->lda;
   sp->total = sp->g_at + 2 * kTileFloats + kSlack;
   if ((size_t)sp->total * sizeof(float) > 160 * 1024 - 512) return false;
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-  }
+  const int cus = compute_units();  // (of the current device)
   const int items = 2 * c.K * c.C;
   sp->grid = items < cus ? items : cus;
   return true;

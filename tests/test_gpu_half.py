@@ -55,9 +55,14 @@ def test_half_product_matches_torch_half_bmm(pbg, batch, m, n, k, akm, bkm):
     base = c2.cpu().clone()
     pbg.native.gemm(ad, bd, c2, batch, m, n, k, m if akm else k, n if bkm else k, n, a[0].numel(), b[0].numel(), m * n,
                     akm, bkm, beta=1.0, half=True)
+    # Two roundings, as autograd adds two Half gradients: the product is a Half tensor of its own, then the sum is
+    # rounded -- within a unit of the product plus a unit of the sum of the exact value, and mostly equal to the
+    # same two steps on torch's Half tensors.
     want2 = (exact + base.double())
     ulp2 = torch.pow(2.0, torch.floor(torch.log2(want2.abs().clamp_min(2.0 ** -14))) - 10)
-    assert bool(((c2.cpu().double() - want2).abs() <= ulp2 + noise).all())
+    assert bool(((c2.cpu().double() - want2).abs() <= ulp + ulp2 + noise).all())
+    twice = (want.half() + base.half()).float()
+    assert float((c2.cpu() != twice).float().mean()) < 0.02
 
 
 HALF_CASES = []

@@ -71,6 +71,34 @@ CASES += [
 ]
 
 
+# The cos comparator (the reference's default, config.py:185-190) without an operator: the same kernels on a
+# normalised copy of the tables, the normalisation's backward in the update.  The three update kernels each
+# have that path: rows of up to 128 floats, wider rows, and a wave per table row where gradient rows
+# outnumber table rows 32 to 1; with 3 batches per call and 600 negatives per chunk on 300 entities a row
+# has more positions than one look at the sorted keys shows.
+COS_CASES = []
+for loss, dyn in itertools.product(ostep.LOSS_NAMES, (False, True)):
+    COS_CASES.append(dict(comparator="cos", operator="none", loss=loss, dynamic=dyn, num_batch_negs=50, num_uniform_negs=300,
+                          num_pos=130, dim=128))
+COS_CASES += [
+    dict(comparator="cos", operator="none", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=1000,
+         num_pos=173, dim=400),
+    dict(comparator="cos", operator="none", loss="ranking", dynamic=False, num_batch_negs=37, num_uniform_negs=291,
+         num_pos=100, dim=256, shared=False),
+    dict(comparator="cos", operator="none", loss="logistic", dynamic=True, num_batch_negs=50, num_uniform_negs=300,
+         num_pos=120, dim=200),
+    dict(comparator="cos", operator="none", loss="softmax", dynamic=False, num_batch_negs=0, num_uniform_negs=64,
+         num_pos=150, dim=128),
+    dict(comparator="cos", operator="none", loss="ranking", dynamic=False, num_batch_negs=50, num_uniform_negs=600,
+         num_pos=60, dim=128),
+    dict(comparator="cos", operator="none", loss="softmax", dynamic=False, num_batch_negs=50, num_uniform_negs=1000,
+         num_pos=60, dim=256),
+    dict(comparator="cos", operator="none", loss="logistic", dynamic=False, num_batch_negs=50, num_uniform_negs=1000,
+         num_pos=60, dim=128, shared=False),
+]
+CASES += COS_CASES
+
+
 def ids(case):
     return "-".join(f"{v}" for v in case.values())
 
@@ -100,8 +128,8 @@ def build(pbg, case, workers, seed_shift=0):
     case = dict(case)
     num_pos, dim = case.pop("num_pos"), case.pop("dim")
     shared = case.pop("shared", True)
-    cfg = ostep.StepConfig(dim=dim, comparator="dot", num_relations=3, relation_weights=[1.0, 0.5, 2.0], lr=0.1,
-                           relation_lr=0.01, margin=0.1, **case)
+    cfg = ostep.StepConfig(dim=dim, comparator=case.pop("comparator", "dot"), num_relations=3,
+                           relation_weights=[1.0, 0.5, 2.0], lr=0.1, relation_lr=0.01, margin=0.1, **case)
     st, batches = make_inputs(cfg, num_pos, max(300, num_pos * 4), workers, seed=num_pos + dim + seed_shift, shared=shared)
     return cfg, st, batches, num_pos
 
@@ -128,7 +156,7 @@ def test_stream_route_matches_the_oracle(pbg, case, workers):
     compare_state(cfg, runner, st, 1e-5, "stream", st64)
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[5], CASES[18], CASES[23]], ids=ids)
+@pytest.mark.parametrize("case", [CASES[0], CASES[5], CASES[18], CASES[23], COS_CASES[0], COS_CASES[7]], ids=ids)
 def test_stream_route_with_edge_weights(pbg, case):
     say("stream+weights", case)
     cfg, st, batches, num_pos = build(pbg, case, 2)
@@ -148,7 +176,7 @@ def test_stream_route_with_edge_weights(pbg, case):
     assert (st.w_lhs - unweighted.w_lhs).abs().max() > 1e-3 * st.w_lhs.abs().max()
 
 
-@pytest.mark.parametrize("case", [CASES[3], CASES[19]], ids=ids)
+@pytest.mark.parametrize("case", [CASES[3], CASES[19], COS_CASES[6]], ids=ids)
 def test_stream_route_draws_its_negatives(pbg, case):
     """A call that draws its uniform negatives from a seed equals, bit for bit, the call
     that is handed the same draw."""
