@@ -470,6 +470,7 @@ class MultiRelationEmbedder(nn.Module):
         else:
             rel = torch.zeros(1, dtype=torch.int64, device=dev)  # the runner holds this relation's operator only
         weight = edges.weight.to(dev).float().contiguous() if edges.has_weight() else None
+        runner._check_ids(lhs, rhs, rel, ul, ur)
         lp, rp, lr, rr, le, hits = runner.ranks(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
                                                 ur.contiguous() if ur is not None else None, weight, auc_samples, auc_seed)
         has = (spec.num_negs(self.disable_lhs_negs, w_l.shape[0]) > 0, spec.num_negs(self.disable_rhs_negs, w_r.shape[0]) > 0)
@@ -511,6 +512,7 @@ class MultiRelationEmbedder(nn.Module):
             rel = edges.get_relation_type_as_vector().to(dev).contiguous()
         else:
             rel = torch.zeros(1, dtype=torch.int64, device=dev)  # the runner holds this relation's operator only
+        runner._check_ids(lhs, rhs, rel, ul, ur)  # IndexError, as F.embedding raises it (model.py:60-61)
         lp, rp, ln, rn = runner.forward(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
                                         ur.contiguous() if ur is not None else None)
         reg = None

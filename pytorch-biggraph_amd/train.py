@@ -39,6 +39,8 @@ class Trainer(AbstractBatchProcessor):
         self._runners: Dict[tuple, native.StepRunner] = {}
         # set to (uniform_lhs [C,U], uniform_rhs [C,U]) to feed the next batch's negatives from outside
         self.next_uniform_negs = None
+        # False: ids outside their table are clamped by the kernels instead of raising IndexError
+        self.check_ids = True
 
     def _embedding_optimizer(self, weight: torch.nn.Parameter) -> RowAdagrad:
         for opt in list(self.unpartitioned_optimizers.values()) + list(self.partitioned_optimizers.values()):
@@ -112,8 +114,10 @@ class Trainer(AbstractBatchProcessor):
         weight = batch_edges.weight
         if weight is not None:
             weight = weight.to(device=dev, dtype=torch.float32).expand(num_pos).contiguous()
+        # An id outside its table raises IndexError here, as F.embedding does in the reference (model.py:60-61);
+        # the kernels themselves would clamp it.  The check's synchronisation is one this method has anyway.
         runner.train(lhs, rhs, rel, ul.contiguous() if ul is not None else None,
-                     ur.contiguous() if ur is not None else None, weight)
+                     ur.contiguous() if ur is not None else None, weight, check_ids=self.check_ids)
         # the reference reads loss and both violator counts on the host for every batch (train_cpu.py:95-101)
         viol = runner.violators_out[0].tolist()
         return Stats(loss=float(runner.loss_out[0]), reg=float(runner.reg_out[0]), violators_lhs=int(viol[0]), violators_rhs=int(viol[1]),

@@ -328,6 +328,39 @@ def test_model_forward_and_trainer_step(pbg, case):
                 assert_close(trainer.model_optimizer.state[getattr(op, k)]["sum"], st.rhs_op_sum[k][rel], rtol, k + ".sum")
 
 
+def test_model_and_trainer_raise_on_ids_outside_the_table(pbg):
+    """An entity id outside its table raises IndexError from MultiRelationEmbedder.forward and from
+    Trainer.process_one_batch, as F.embedding does in the reference (model.py:57-61), and leaves the
+    table as it was; with Trainer.check_ids switched off the kernels clamp the id instead."""
+    say("ids outside the table")
+    from tests.test_gpu_step import make_inputs
+
+    cfg = ostep.StepConfig(dim=12, operator="none", comparator="dot", loss="ranking", num_batch_negs=5, num_uniform_negs=4,
+                           num_relations=1, relation_weights=[1.0], margin=0.1)
+    st, batches = make_inputs(cfg, 20, 50, 1, seed=2)
+    model, w_l, _ = build_model(pbg, cfg, st, 1)
+    EL, ED, T = pbg.entitylist.EntityList, pbg.edgelist.EdgeList, pbg.train
+    loss_fn = pbg.losses.LOSS_FUNCTIONS.get_class(cfg.loss)(margin=cfg.margin)
+    trainer = T.Trainer(T.make_optimizer(list(model.parameters()), False, 0.1, 0.1), loss_fn, [1.0])
+    trainer.partitioned_optimizers[("l", 0)] = T.make_optimizer([w_l], True, 0.1)
+    lhs, rhs, rel, ul, ur = batches[0]
+    before = w_l.detach().clone()
+    for bad in (50, -1):
+        wrong = lhs.clone()
+        wrong[3] = bad
+        edges = ED(EL.from_tensor(wrong.to(DEV)), EL.from_tensor(rhs.to(DEV)), torch.tensor(rel))
+        with pytest.raises(IndexError):
+            model(edges, uniform_negs=(ul.to(DEV), ur.to(DEV)))
+        trainer.next_uniform_negs = (ul.to(DEV), ur.to(DEV))
+        with pytest.raises(IndexError):
+            trainer.process_one_batch(model, edges)
+        assert torch.equal(before, w_l.detach())
+    trainer.check_ids = False
+    trainer.next_uniform_negs = (ul.to(DEV), ur.to(DEV))
+    trainer.process_one_batch(model, edges)  # the id is clamped to the table's first row
+    assert not torch.equal(before, w_l.detach())
+
+
 def test_row_adagrad_and_async_adagrad_optimizers(pbg):
     torch.manual_seed(0)
     w0 = torch.randn(50, 12)
