@@ -375,6 +375,8 @@ MAX_NORM_CASES = [
          dim=9, disable_lhs_negs=True, shared=False),
     dict(operator="none", comparator="cos", loss="logistic", num_batch_negs=10, num_uniform_negs=5, num_pos=33, dim=16,
          global_emb=True),
+    # cos with a wide negative set: the streaming kernels on the normalised copy of the (renormalised) tables
+    dict(operator="none", comparator="cos", loss="softmax", num_batch_negs=50, num_uniform_negs=300, num_pos=130, dim=128),
 ]
 
 
@@ -408,7 +410,9 @@ def test_train_step_with_max_norm(pbg, case, workers):
     assert_close(runner.w_lhs, st.w_lhs, 1e-6, "renormalised table")
     runner.train(*pack(cfg, batches))
     torch.cuda.synchronize()
-    outs, st64 = lockstep(cfg, st, batches)
+    # (hundreds of exponentials per score row: the CPU path's own fp32 result is then further from the exact one
+    # than the tolerance, and the float64 run anchors the comparison, as in tests/test_gpu_stream.py)
+    outs, st64 = lockstep(cfg, st, batches, anchor=runner.route == "stream")
     rtol = 1e-5
     for k, out in enumerate(outs):
         assert loss_close(float(runner.loss_out[k]), out), ("loss", k, float(runner.loss_out[k]), out.loss)
