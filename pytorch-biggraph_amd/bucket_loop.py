@@ -178,6 +178,7 @@ class _Slot:
         self.ready: Optional[torch.cuda.Event] = None     # upload finished (copy stream)
         self.last_use: Optional[torch.cuda.Event] = None  # last training call finished (compute stream)
         self.stamp = 0
+        self.dirty = False  # trained on since it was last written back
 
 
 class PartitionCache:
@@ -212,6 +213,7 @@ class PartitionCache:
                 self.copy_stream.wait_event(slot.last_use)
             self.store.tables[key].copy_(slot.w[:n], non_blocking=True)
             self.store.sums[key].copy_(slot.g[:n], non_blocking=True)
+        slot.dirty = False
         self.bytes_written_back += n * (slot.w.shape[1] + 1) * 4
 
     def _load(self, key: PartitionKey, protected: Sequence[PartitionKey]) -> _Slot:
@@ -223,7 +225,8 @@ class PartitionCache:
             if not candidates:
                 raise RuntimeError("no device buffer left for partition %s" % (key,))
             slot = min(candidates, key=lambda s: s.stamp)  # least recently used
-            self._write_back(slot)
+            if slot.dirty:
+                self._write_back(slot)
             del self.by_key[slot.key]
         n = self.store.rows(key)
         with torch.cuda.stream(self.copy_stream):
@@ -232,7 +235,7 @@ class PartitionCache:
             slot.g[:n].copy_(self.store.sums[key], non_blocking=True)
             slot.ready = torch.cuda.Event()
             slot.ready.record(self.copy_stream)
-        slot.key, slot.last_use = key, None
+        slot.key, slot.last_use, slot.dirty = key, None, False
         self.by_key[key] = slot
         self.bytes_uploaded += n * (slot.w.shape[1] + 1) * 4
         return slot
@@ -265,13 +268,21 @@ class PartitionCache:
         """Marks the end of the current stream's work on `keys`."""
         for key in keys:
             slot = self.by_key[key]
+            slot.dirty = True
             slot.last_use = torch.cuda.Event()
             slot.last_use.record(torch.cuda.current_stream(self.device))
+
+    def write_back_idle(self, in_use: Sequence[PartitionKey]) -> None:
+        """Starts writing back every trained-on partition that the current bucket does not name (the last
+        bucket of a pass has no successor to upload for: its idle neighbours go home while it trains)."""
+        for slot in self.slots:
+            if slot.key is not None and slot.dirty and slot.key not in in_use:
+                self._write_back(slot)
 
     def flush(self) -> None:
         """Writes every resident partition back to the store and waits for it."""
         for slot in self.slots:
-            if slot.key is not None:
+            if slot.key is not None and slot.dirty:
                 self._write_back(slot)
         self.copy_stream.synchronize()
 
@@ -483,27 +494,29 @@ class BucketLoop:
         starts_dev = torch.tensor(starts, dtype=torch.int64, device=dev) if rels is not None else None
         rows_l, rows_r = tables[0][0].shape[0], tables[-1][0].shape[0]
         u = self.spec_args["num_uniform_negs"]
-        loss = torch.zeros((), dtype=torch.float64, device=dev)
-        viol = torch.zeros(2, dtype=torch.int64, device=dev)
+        # every call leaves its batches' statistics in its own row; one reduction per bucket
+        k_max = max((k for _, k, _ in calls), default=1)
+        loss_all = torch.zeros((len(calls), k_max), dtype=torch.float32, device=dev)
+        viol_all = torch.zeros((len(calls), k_max, 2), dtype=torch.int64, device=dev)
         runners: Dict[Tuple[int, int], native.StepRunner] = {}
-        for first, k, b_now in calls:
+        for i, (first, k, b_now) in enumerate(calls):
             runner = self._runner(runners, tables, k, b_now)
+            stats_out = (loss_all[i, :k], viol_all[i, :k])
             l, r, t = self._call_edges(lhs_t, rhs_t, rel_t, starts, rels, first, k, b_now, starts_dev)
             if self.calls_log is not None:
                 self.calls_log.append(dict(bucket=b, epoch=self.epoch, workers=k, batch_size=b_now, lhs=l.cpu(),
                                            rhs=r.cpu(), rel=t.cpu()))
             c = runner.spec.num_chunks
             if u and self.negatives is not None:
-                runner.train(l, r, t, self._uniform(k, c, u, rows_l, 0), self._uniform(k, c, u, rows_r, 1))
+                runner.train(l, r, t, self._uniform(k, c, u, rows_l, 0), self._uniform(k, c, u, rows_r, 1), stats_out=stats_out)
             else:
                 self.calls += 1
                 call_seed = (self.seed * 0x9E3779B97F4A7C15 + self.calls) & (2**64 - 1) if u else None
-                runner.train(l, r, t, uniform_seed=call_seed)
-            loss += runner.loss_out.double().sum()
-            viol += runner.violators_out.sum(dim=0)
+                runner.train(l, r, t, uniform_seed=call_seed, stats_out=stats_out)
         eval_after = self._evaluate(tables, lhs, rhs, rel, eval_idx) if eval_idx is not None else None
-        v = viol.tolist()
-        return BucketStats(b, num_train, float(loss), int(v[0]), int(v[1]), eval_before, eval_after)
+        loss = float(loss_all.double().sum())
+        v = viol_all.sum(dim=(0, 1)).tolist()
+        return BucketStats(b, num_train, loss, int(v[0]), int(v[1]), eval_before, eval_after)
 
     def train_epoch(self) -> List[BucketStats]:
         buckets = [b for b in create_ordered_buckets(self.nparts_lhs, self.nparts_rhs, self.bucket_order,
@@ -514,6 +527,8 @@ class BucketLoop:
             tables = self.cache.acquire(keys)
             if i + 1 < len(buckets):  # the next bucket's partitions travel while this one trains
                 self.cache.prefetch(self._keys(buckets[i + 1]), keys)
+            else:
+                self.cache.write_back_idle(keys)
             stats.append(self._train_bucket(b, tables))
             self.cache.release(keys)
         self.cache.flush()

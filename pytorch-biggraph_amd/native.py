@@ -394,9 +394,12 @@ class StepRunner:
         return bufs
 
     def train(self, lhs, rhs, rel, uniform_lhs=None, uniform_rhs=None, edge_weight=None, uniform_seed=None,
-              check_ids: bool = False) -> None:
+              check_ids: bool = False, stats_out=None) -> None:
         """One lock-step training step over num_workers batches; statistics land
-        in self.loss_out / self.violators_out (device, no sync).  The uniform
+        in self.loss_out / self.violators_out (device, no sync) or, with
+        `stats_out = (loss[K] float32, violators[K, 2] int64)`, in the caller's
+        tensors (a loop over many calls hands in rows of one buffer and reduces
+        them once).  The uniform
         negatives are either given ([K, C, U] per side) or drawn inside the step
         from `uniform_seed` (sample_uniform_negatives shows which).
 
@@ -407,6 +410,12 @@ class StepRunner:
         if check_ids:
             self._check_ids(lhs, rhs, rel, uniform_lhs, uniform_rhs)
         bufs = self._buffers(lhs, rhs, rel, uniform_lhs, uniform_rhs, edge_weight, uniform_seed)
+        if stats_out is not None:
+            loss, viol = stats_out
+            k = self.spec.num_workers
+            if _need(loss, torch.float32, "stats_out[0]").numel() != k or _need(viol, torch.int64, "stats_out[1]").numel() != 2 * k:
+                raise ValueError(f"stats_out must be (loss[{k}], violators[{k}, 2])")
+            bufs.loss_out, bufs.violators_out = _ptr(loss), _ptr(viol)
         check(_lib.lib().pbg_train_step(ctypes.byref(self.desc), ctypes.byref(bufs), _stream()))
 
     def _check_ids(self, lhs, rhs, rel, uniform_lhs, uniform_rhs) -> None:
