@@ -286,13 +286,14 @@ struct HotRuns {
 constexpr int kStage = 32;  // edges per step
 
 template <bool VEC, bool RUNS>
-__global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
+__global__ __launch_bounds__(kThreads, 4) void seg_linear_update_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, const uint32_t* __restrict__ rel_start,
     int kbits, const float* __restrict__ dz, const float* __restrict__ x, int dim, float* __restrict__ w,
     float* __restrict__ wsum, float lr, HotRuns hot) {
   __shared__ __attribute__((aligned(16))) float lds_a[2][kStage * LD];
   __shared__ __attribute__((aligned(16))) float lds_b[2][kStage * LD];
-  __shared__ uint32_t lds_batch[2][kStage];
+  // (the batch of a staged edge sits in the padding of its row of lds_a, column BM: with an array of its own
+  // the kernel's LDS would be 256 bytes above a quarter of the compute unit's)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
   const int tiles = (dim + BN - 1) / BN;
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
   for (int h = 0; h < 2; ++h) {
     *reinterpret_cast<float4*>(&lds_a[0][(kk + 16 * h) * LD + q4]) = make_float4(ra[h].v[0], ra[h].v[1], ra[h].v[2], ra[h].v[3]);
     *reinterpret_cast<float4*>(&lds_b[0][(kk + 16 * h) * LD + q4]) = make_float4(rb[h].v[0], rb[h].v[1], rb[h].v[2], rb[h].v[3]);
-    if ((tid & 15) == 0) lds_batch[0][kk + 16 * h] = sbt[h];
+    if ((tid & 15) == 0) lds_a[0][(kk + 16 * h) * LD + BM] = __uint_as_float(sbt[h]);
   }
   __syncthreads();
 
@@ -475,7 +476,7 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
       }
     }
     // batch of each staged edge in lanes 0..31; run heads as a bit mask
-    const uint32_t mine = lds_batch[buf][lane & (kStage - 1)];
+    const uint32_t mine = __float_as_uint(lds_a[buf][(lane & (kStage - 1)) * LD + BM]);
     const uint32_t prev = (uint32_t)__shfl_up((int)mine, 1, 64);
     const uint32_t valid = (uint32_t)__ballot(lane < kStage && mine != kNone);
     uint32_t heads = (uint32_t)__ballot(lane < kStage && mine != kNone && (lane == 0 || prev != mine));
@@ -521,7 +522,7 @@ __global__ __launch_bounds__(kThreads) void seg_linear_update_kernel(
       for (int h = 0; h < 2; ++h) {
         *reinterpret_cast<float4*>(&lds_a[buf ^ 1][(kk + 16 * h) * LD + q4]) = make_float4(ra[h].v[0], ra[h].v[1], ra[h].v[2], ra[h].v[3]);
         *reinterpret_cast<float4*>(&lds_b[buf ^ 1][(kk + 16 * h) * LD + q4]) = make_float4(rb[h].v[0], rb[h].v[1], rb[h].v[2], rb[h].v[3]);
-        if ((tid & 15) == 0) lds_batch[buf ^ 1][kk + 16 * h] = sbt[h];
+        if ((tid & 15) == 0) lds_a[buf ^ 1][(kk + 16 * h) * LD + BM] = __uint_as_float(sbt[h]);
       }
     }
     __syncthreads();
