@@ -90,11 +90,15 @@ __device__ __forceinline__ int64_t edge_row(uint32_t e, int edges_per_batch, int
   return (int64_t)(e / (uint32_t)edges_per_batch) * batch_stride + (e % (uint32_t)edges_per_batch);
 }
 
-template <bool TRANS>
+// VEC: dim is a multiple of 4 and both operands are 16-byte aligned, so a quad is whole or absent: it is loaded
+// without a branch from an address clamped into the operand and dropped afterwards (a load inside a branch makes
+// everything behind the branch wait for ALL loads in flight, which would undo the prefetch below).
+template <bool TRANS, bool VEC>
 __global__ __launch_bounds__(kThreads) void seg_linear_apply_kernel(
     const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, int64_t n, int kbits, int edges_per_batch,
     const float* __restrict__ in, int64_t in_batch_stride, const float* __restrict__ w, int dim,
-    float* __restrict__ out, int64_t out_batch_stride, int accumulate, int vec_ok) {
+    float* __restrict__ out, int64_t out_batch_stride, int accumulate) {
+  constexpr int vec_ok = VEC;
   __shared__ __attribute__((aligned(16))) float lds_a[2][BK * LD];
   __shared__ __attribute__((aligned(16))) float lds_b[2][BK * LD];
   __shared__ int64_t rel_s[BM];
@@ -134,11 +138,23 @@ __global__ __launch_bounds__(kThreads) void seg_linear_apply_kernel(
     const bool row_on = ar >= a && ar < b;
     const bool wave_on = a < wm0 + 32 && b > wm0;  // the wave's 32 rows meet [a, b)
 
+    auto quad_or_zero = [&](const float* p, bool keep) {
+      const float4 x = *reinterpret_cast<const float4*>(p);
+      Quad q;
+      q.v[0] = keep ? x.x : 0.f; q.v[1] = keep ? x.y : 0.f; q.v[2] = keep ? x.z : 0.f; q.v[3] = keep ? x.w : 0.f;
+      return q;
+    };
     auto fetch_a = [&](int k0) {
+      if constexpr (VEC) return quad_or_zero(arow + min(k0 + akq, dim - 4), row_on && k0 + akq < dim);
       const int count = row_on ? clamp_count(dim - (k0 + akq)) : 0;
       return load_quad(arow + k0 + akq, count, vec_ok);
     };
     auto fetch_b = [&](int k0) {
+      if constexpr (VEC) {
+        const bool keep = k0 + bk < dim && n0 + bj < dim;
+        if (TRANS) return quad_or_zero(wr + (int64_t)min(k0 + bk, dim - 1) * dim + min(n0 + bj, dim - 4), keep);
+        return quad_or_zero(wr + (int64_t)min(n0 + bj, dim - 1) * dim + min(k0 + bk, dim - 4), keep);
+      }
       if (TRANS) {
         const int count = (k0 + bk < dim) ? clamp_count(dim - (n0 + bj)) : 0;
         return load_quad(wr + (int64_t)(k0 + bk) * dim + n0 + bj, count, vec_ok);
@@ -157,15 +173,19 @@ __global__ __launch_bounds__(kThreads) void seg_linear_apply_kernel(
       }
     };
 
+    // operands travel two tiles ahead of the products (registers), one tile ahead sits in LDS
     Quad qa = fetch_a(0), qb = fetch_b(0);
+    Quad ra = fetch_a(BK), rb = fetch_b(BK);  // (past the last tile: counts of zero, clamped addresses)
     __syncthreads();  // the previous sweep may still be reading LDS
     stash(0, qa, qb);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
       const int cur = kt & 1;
-      if (kt + 1 < nk) {
-        qa = fetch_a((kt + 1) * BK);
-        qb = fetch_b((kt + 1) * BK);
+      qa = ra;
+      qb = rb;
+      if (VEC || kt + 2 < nk) {
+        ra = fetch_a((kt + 2) * BK);
+        rb = fetch_b((kt + 2) * BK);
       }
       if (wave_on) mfma_tile(lds_a[cur], lds_b[cur], wm0, wn0, lane, acc);
       if (kt + 1 < nk) stash(cur ^ 1, qa, qb);
@@ -546,15 +566,19 @@ int seg_linear_apply(const uint64_t* keys, const uint32_t* vals, int64_t n, int 
                      const float* in, int64_t in_batch_stride, const float* w, int dim, bool transpose_w, float* out,
                      int64_t out_batch_stride, bool accumulate, hipStream_t stream) {
   if (n <= 0) return PBG_OK;
-  const int vec_ok = dim % 4 == 0 && aligned16(in) && aligned16(w);
+  const bool vec_ok = dim % 4 == 0 && aligned16(in) && aligned16(w);
   const dim3 grid((unsigned)ceil_div(n, BM), (unsigned)ceil_div(dim, BN)), block(kThreads);
+#define PBG_SEG_APPLY(TRANS, VEC)                                                                                        \
+  hipLaunchKernelGGL((seg_linear_apply_kernel<TRANS, VEC>), grid, block, 0, stream, keys, vals, n, kbits, edges_per_batch, \
+                     in, in_batch_stride, w, dim, out, out_batch_stride, (int)accumulate)
   if (transpose_w) {
-    hipLaunchKernelGGL(seg_linear_apply_kernel<true>, grid, block, 0, stream, keys, vals, n, kbits, edges_per_batch, in,
-                       in_batch_stride, w, dim, out, out_batch_stride, (int)accumulate, vec_ok);
+    if (vec_ok) PBG_SEG_APPLY(true, true);
+    else PBG_SEG_APPLY(true, false);
   } else {
-    hipLaunchKernelGGL(seg_linear_apply_kernel<false>, grid, block, 0, stream, keys, vals, n, kbits, edges_per_batch, in,
-                       in_batch_stride, w, dim, out, out_batch_stride, (int)accumulate, vec_ok);
+    if (vec_ok) PBG_SEG_APPLY(false, true);
+    else PBG_SEG_APPLY(false, false);
   }
+#undef PBG_SEG_APPLY
   return check_launch("seg_linear_apply");
 }
 
