@@ -48,10 +48,12 @@ inline int bits_for(uint64_t max_value) {  // number of bits needed to hold max_
 // `temp` holds sort_temp_bytes(n) bytes.
 // With `indices` the input pairs are made by the sort's first kernel instead of being read: key i = indices[i]
 // (an index outside [0, park) becomes `park`), value i = i; keys_in / vals_in are then only written.
-// If `long_runs` is given it receives a device pointer (into `temp`) to a word that is zero after the
-// sort only if no value of the sorted bits occurs more than kFoldMax times -- what lets a single-worker
-// RowAdagrad step skip its duplicate-summation kernels.
+// If `long_runs` is given it receives a device pointer (into `temp`) to kLongWords words that are all zero after
+// the sort only if no value of the sorted bits occurs more than kFoldMax times -- what lets a single-worker
+// RowAdagrad step skip its duplicate-summation kernels.  (Several words: the kernel that sorts a small input
+// in one launch has every workgroup leave its own finding, and nobody has to clear a shared word first.)
 constexpr int kFoldMax = 8;
+constexpr int kLongWords = 512;
 size_t sort_temp_bytes(int64_t n);
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
                int key_bits, void* temp, hipStream_t stream, uint64_t** keys_sorted, uint32_t** vals_sorted,
@@ -61,7 +63,7 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
 // keys are sorted ascending; vals[i] indexes a row of grad_rows[*, dim], which is
 // clobbered (duplicate sums are formed in place).  A key's row field addresses table 0 for row < rows0, table 1 (row - rows0) for
 // row < rows0 + rows1, and is ignored beyond.
-// `long_runs` (single-worker calls, kbits == 0): the word sort_pairs leaves behind; where it is zero the
+// `long_runs` (single-worker calls, kbits == 0): the kLongWords words sort_pairs leaves behind; where all are zero the
 // duplicate-summation kernels return at once (no key occurs more than kFoldMax times, and the update
 // kernel sums such runs itself).  nullptr: not known.
 // `cos_back`: the gradient rows are gradients at the NORMALISED rows y = x / |x| of the tables (a step with the

@@ -210,6 +210,14 @@ __device__ __forceinline__ uint64_t lane_u64(uint64_t v, int l) {
   return ((uint64_t)hi << 32) | lo;
 }
 
+// The sort's word on runs of more than kFoldMax equal keys (kLongWords words, any of them raised); wave-uniform.
+__device__ __forceinline__ bool any_long_run(const uint32_t* __restrict__ long_runs) {
+  uint32_t any = 0u;
+#pragma unroll
+  for (int w = 0; w < kLongWords / kWave; ++w) any |= long_runs[w * kWave + (threadIdx.x & 63)];
+  return __ballot(any != 0u) != 0ull;
+}
+
 // leave_mode 0: every piece of two or more positions is summed; 1 (single-worker calls): pieces of runs
 // of at most kFoldMax positions are left to the update kernel; 2 (row_walk_kernel follows): whole runs
 // inside the tile are left alone.
@@ -218,7 +226,7 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
                                                                   const uint32_t* __restrict__ vals, int64_t n,
                                                                   float* __restrict__ grad_rows, int dim,
                                                                   int leave_mode, const uint32_t* __restrict__ long_runs) {
-  if (leave_mode == 1 && long_runs && *long_runs == 0u) return;  // the sort saw no run of more than kFoldMax positions
+  if (leave_mode == 1 && long_runs && !any_long_run(long_runs)) return;  // the sort saw no run of more than kFoldMax positions
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
   const int64_t begin = tile * kTile;
@@ -280,7 +288,7 @@ __global__ __launch_bounds__(kRowThreads) void run_combine_kernel(const uint64_t
                                                                   const uint32_t* __restrict__ vals, int64_t n,
                                                                   float* __restrict__ grad_rows, int dim,
                                                                   int leave_mode, const uint32_t* __restrict__ long_runs) {
-  if (leave_mode == 1 && long_runs && *long_runs == 0u) return;  // as in tile_reduce_kernel
+  if (leave_mode == 1 && long_runs && !any_long_run(long_runs)) return;  // as in tile_reduce_kernel
   const int lane = threadIdx.x & 63;
   const int64_t b = ((int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6) + 1) * kTile;
   if (b >= n) return;

@@ -19,6 +19,8 @@
 // between them.  Every step is stable, so equal keys keep the order of the
 // input, which keeps segmented gradient sums deterministic and lets a caller
 // whose input is already ordered by the low bits leave those bits out.
+#include <cstdlib>
+
 #include "pbg_internal.h"
 
 namespace pbg {
@@ -55,7 +57,7 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_hist_kernel(uint64_t* 
                                                                       const int64_t* __restrict__ idx, int64_t park,
                                                                       uint32_t* __restrict__ vals) {
   __shared__ uint32_t hist[kMaxDigits];
-  if (blockIdx.x == 0 && threadIdx.x == 0) *long_flag = long_init;
+  if (blockIdx.x == 0 && threadIdx.x < kLongWords) long_flag[threadIdx.x] = threadIdx.x == 0 ? long_init : 0u;
   const uint32_t mask = (1u << digit_bits) - 1u;
   if (threadIdx.x < kMaxDigits) hist[threadIdx.x] = 0;
   __syncthreads();
@@ -550,15 +552,98 @@ __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t
   }
 }
 
+// ---- a small input in ONE launch ------------------------------------------------------------------
+// Up to kRankMax pairs: three dependent launches of the radix sort cost more than their work there (a
+// single-batch training step has a few thousand keys).  The place of pair i in the stable order is the
+// number of pairs j whose field is smaller, plus the number of j < i whose field is equal.  A workgroup
+// owns kRankKeys consecutive pairs and copies ALL fields into LDS; the fields are cut into 64 shares, and
+// lane (share % 4) * 16 + p of wave share / 4 counts pair p against that share (the 16 lanes of a group read
+// the same words).  The 64 counts of a pair meet in LDS and the pair goes to its place.  n^2 comparisons in
+// all, spread over n / 16 workgroups: 16 M for the 4000 keys of a single batch.
+constexpr int kRankMax = 1 << 13;
+constexpr int kRankWaves = 16;
+constexpr int kRankKeys = 16;
+constexpr int kRankShares = kRankWaves * 4;
+
+template <bool FLAG>
+__global__ __launch_bounds__(kRankWaves * 64) void sort_rank_kernel(
+    const uint64_t* __restrict__ keys, const uint32_t* __restrict__ vals, uint64_t* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out, int n, int low_bit, uint32_t mask, uint32_t* __restrict__ long_flag,
+    const int64_t* __restrict__ idx, int64_t park) {
+  extern __shared__ uint32_t rank_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n4 = (n + 3) & ~3;
+  uint32_t* field = rank_lds;      // [n4]
+  uint32_t* part = rank_lds + n4;  // [3][kRankShares][kRankKeys]: smaller; equal and earlier; equal
+  auto key_of = [&](int j) -> uint64_t {
+    if (!idx) return keys[j];
+    const int64_t r = idx[j];
+    return (uint64_t)((r < 0 || r >= park) ? park : r);
+  };
+  for (int j = tid; j < n; j += kRankWaves * 64) field[j] = (uint32_t)(key_of(j) >> low_bit) & mask;
+  __syncthreads();
+
+  const int p = lane & (kRankKeys - 1), share = wave * 4 + (lane >> 4);
+  const int i = blockIdx.x * kRankKeys + p;
+  const uint32_t mine = field[i < n ? i : n - 1];
+  const int len = ((n4 / 4 + kRankShares - 1) / kRankShares) * 4;  // whole quads, except at the end of the input
+  const int s0 = min(share * len, n), s1 = min(s0 + len, n);
+  uint32_t lt = 0, eq = 0, eqb = 0;
+  int j = s0;
+  for (; j + 4 <= s1; j += 4) {
+    const uint4 f = *reinterpret_cast<const uint4*>(&field[j]);
+    lt += (uint32_t)(f.x < mine) + (uint32_t)(f.y < mine) + (uint32_t)(f.z < mine) + (uint32_t)(f.w < mine);
+    const uint32_t e0 = f.x == mine, e1 = f.y == mine, e2 = f.z == mine, e3 = f.w == mine;
+    if (FLAG) eq += e0 + e1 + e2 + e3;
+    eqb += (e0 & (uint32_t)(j < i)) + (e1 & (uint32_t)(j + 1 < i)) + (e2 & (uint32_t)(j + 2 < i)) + (e3 & (uint32_t)(j + 3 < i));
+  }
+  for (; j < s1; ++j) {
+    const uint32_t f = field[j];
+    lt += (uint32_t)(f < mine);
+    if (FLAG) eq += (uint32_t)(f == mine);
+    eqb += (uint32_t)(f == mine) & (uint32_t)(j < i);
+  }
+  part[(0 * kRankShares + share) * kRankKeys + p] = lt + eqb;
+  if (FLAG) part[(1 * kRankShares + share) * kRankKeys + p] = eq;
+  __syncthreads();
+  if (wave != 0) return;
+  // lane (q, p) adds the shares q, q + 4, ... of pair p; the four q meet through the lanes' exchange
+  uint32_t place = 0, same = 0;
+  const int q = lane >> 4;
+#pragma unroll
+  for (int w = 0; w < kRankWaves; ++w) {
+    place += part[(0 * kRankShares + w * 4 + q) * kRankKeys + p];
+    if (FLAG) same += part[(1 * kRankShares + w * 4 + q) * kRankKeys + p];
+  }
+  place += __shfl_xor(place, 16, 64);
+  place += __shfl_xor(place, 32, 64);
+  if (FLAG) {
+    same += __shfl_xor(same, 16, 64);
+    same += __shfl_xor(same, 32, 64);
+  }
+  const bool owner = lane < kRankKeys && i < n;
+  if (owner) {
+    keys_out[place] = key_of(i);
+    vals_out[place] = idx ? (uint32_t)i : vals[i];
+  }
+  if (FLAG) {
+    // every workgroup leaves its own word, and the first one clears the words no workgroup owns
+    const bool found = __ballot(owner && same > (uint32_t)kFoldMax) != 0ull;
+    if (lane == 0) long_flag[blockIdx.x] = found ? 1u : 0u;
+    if (blockIdx.x == 0)
+      for (int w = (int)gridDim.x + lane; w < kLongWords; w += 64) long_flag[w] = 0u;
+  }
+}
+
 }  // namespace
 
 size_t sort_temp_bytes(int64_t n) {
   SortPlan p = plan_sort(n);
-  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 2) * sizeof(uint32_t), 256);
+  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 1 + kLongWords) * sizeof(uint32_t), 256);
 }
 
 namespace {
-LdsLimit g_bucket_lds;
+LdsLimit g_bucket_lds, g_rank_lds[2];
 }
 
 int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, int64_t n, int low_bit,
@@ -577,6 +662,26 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   uint32_t* long_flag = bucket_off + kMaxDigits + 1;
   int bits = key_bits - low_bit;
   if (bits < 1) bits = 1;
+  if (n <= kRankMax && bits <= 32 && getenv("PBG_DISABLE_RANK_SORT") == nullptr) {  // one launch, see sort_rank_kernel
+    static_assert(kRankMax / kRankKeys <= kLongWords, "one word per workgroup");
+    const size_t lds_bytes = ((size_t)((n + 3) & ~(int64_t)3) + 2 * kRankShares * kRankKeys) * sizeof(uint32_t);
+    const uint32_t mask = bits == 32 ? 0xffffffffu : ((1u << bits) - 1u);
+    const dim3 grid((unsigned)ceil_div(n, kRankKeys)), block(kRankWaves * 64);
+    int rc;
+    if (long_runs) {
+      if ((rc = reserve_lds((const void*)sort_rank_kernel<true>, &g_rank_lds[1], lds_bytes)) != PBG_OK) return rc;
+      hipLaunchKernelGGL(sort_rank_kernel<true>, grid, block, lds_bytes, stream, keys_in, vals_in, keys_out, vals_out, (int)n,
+                         low_bit, mask, long_flag, indices, park);
+      *long_runs = long_flag;
+    } else {
+      if ((rc = reserve_lds((const void*)sort_rank_kernel<false>, &g_rank_lds[0], lds_bytes)) != PBG_OK) return rc;
+      hipLaunchKernelGGL(sort_rank_kernel<false>, grid, block, lds_bytes, stream, keys_in, vals_in, keys_out, vals_out, (int)n,
+                         low_bit, mask, long_flag, indices, park);
+    }
+    *keys_sorted = keys_out;
+    *vals_sorted = vals_out;
+    return check_launch("sort_pairs");
+  }
   const int top = bits < kMaxDigitBits ? bits : kMaxDigitBits;  // width of the global pass
   const int rest = bits - top;                                  // bits left for the bucket passes
   const int local = (rest + 7) / 8;
