@@ -89,6 +89,35 @@ def test_row_adagrad_sparse(pbg, dim, n_rows, n):
     assert torch.allclose(wd.cpu(), w, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("n, n_rows", [(1, 5), (15, 4), (16, 1000), (17, 3), (4000, 100000), (4001, 700), (8191, 50),
+                                       (8192, 1 << 20), (8192, 9), (8193, 1000)])
+def test_small_inputs_sort_in_one_launch_like_the_radix_sort(pbg, n, n_rows, monkeypatch):
+    """Up to 8192 indices are sorted by one rank-counting launch; the result (order of equal indices
+    included: the duplicates' sums are formed in that order) is that of the radix kernels bit for bit -- few
+    rows so that runs are long, many so that there is none, sizes on both sides of the workgroup's 16 pairs
+    and of the limit, and indices outside the table (parked behind it, ignored)."""
+    say("rank sort", n, n_rows)
+    g = torch.Generator().manual_seed(n + n_rows)
+    w = torch.randn(n_rows, 12, generator=g)
+    gs = torch.rand(n_rows, generator=g)
+    idx = torch.randint(0, n_rows, (n,), generator=g)
+    if n > 100:
+        idx[::97] = n_rows + 5  # out of range
+        idx[5::89] = -3
+    vals = torch.randn(n, 12, generator=g)
+    got = []
+    for off in ("", "1"):
+        if off:
+            monkeypatch.setenv("PBG_DISABLE_RANK_SORT", off)
+        wd, gd = w.clone().to(DEV), gs.clone().to(DEV)
+        pbg.native.row_adagrad_sparse(wd, gd, idx.to(DEV), vals.to(DEV), 0.1)
+        got.append((wd.cpu(), gd.cpu()))
+    assert torch.equal(got[0][0], got[1][0]) and torch.equal(got[0][1], got[1][1])
+    keep = (idx >= 0) & (idx < n_rows)
+    ostep.row_adagrad_sparse(w, gs, torch.sparse_coo_tensor(idx[keep].unsqueeze(0), vals[keep], (n_rows, 12)), 0.1)
+    assert torch.allclose(got[0][0], w, rtol=1e-5, atol=1e-6) and torch.allclose(got[0][1], gs, rtol=1e-5, atol=1e-7)
+
+
 def test_row_adagrad_empty_and_dense(pbg):
     w = torch.randn(6, 5)
     gs = torch.rand(6)
