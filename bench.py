@@ -303,8 +303,14 @@ def event_timer(reps):
     """median seconds of `reps` calls of fn, each bracketed by events on torch's current stream
     (the stand-alone entry points enqueue on the stream they are handed, which is that one)"""
     def timed(fn, n=reps):
-        fn()
-        torch.cuda.synchronize()
+        # warm-up: at least one call, and the device kept busy for 0.1 s (a handful of millisecond launches
+        # are over before the clocks have settled)
+        t0 = time.perf_counter()
+        while True:
+            fn()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t0 > 0.1:
+                break
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
         ev[0].record()
         for i in range(n):
