@@ -875,6 +875,12 @@ def main():
             config[f"{n}_cpu_edges_per_s"] = r["cpu_baseline"]["value"] if r.get("cpu_baseline") else None
     if epoch:
         config["cfg4_epoch_edges_per_s"] = epoch["value"]
+        # the epoch's calls are cfg4's calls: its kernels' roofline and the CPU's rate on the same step ride along
+        c4 = configs.get("cfg4") or {}
+        if "roofline" in c4:
+            epoch["roofline_of_the_calls"] = {k: c4["roofline"].get(k) for k in ("kernel", "bound", "achieved", "peak", "unit", "frac")}
+            epoch["cpu_baseline_of_the_calls"] = c4.get("cpu_baseline")
+            epoch["fraction_of_the_resident_rate"] = epoch["value"] / c4["value"]
     line = {
         "metric": "train edges/sec (100 negs/edge) on 1 MI355X",
         "value": eps, "unit": "edges/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
