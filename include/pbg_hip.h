@@ -251,7 +251,8 @@ int pbg_train_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, pbg_
  * durations in milliseconds to stage_ms (HOST memory).  Stages: 0 gather +
  * element-wise operator + prepare, 1 linear operator, 2 score GEMMs, 3 loss,
  * 4 dN GEMMs, 5 dA GEMMs, 6 chain rule to raw rows, 7 operator parameters,
- * 8 key sort, 9 RowAdagrad update.  When the step runs its key sort on the
+ * 8 key sort, 9 RowAdagrad update (whose first launch also sums the batches'
+ * losses and violator counts into loss_out / violators_out).  When the step runs its key sort on the
  * library's own stream beside the chunk kernel (see Conventions), that time
  * is hidden inside stage 0 and stage 8 reads as about zero.  No counterpart in
  * the reference (it logs wall-clock per bucket, train_cpu.py:696-703). */

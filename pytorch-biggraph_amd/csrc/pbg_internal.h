@@ -73,10 +73,16 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
 struct CosBack {
   const float* y0; const float* inv0; const float* y1; const float* inv1;
 };
+// `sums`: per-batch totals that ride along with the first of the update's launches (a launch of their own costs more
+// than their work: five microseconds per training step): loss_out[b] = sum of lossrow[b * per_batch ... + per_batch) and
+// violators[b][0 / 1] = sums of violrow[..][0 / 1], each in a fixed order.
+struct BatchSums {
+  const float* lossrow; const int* violrow; int per_batch; int batches; float* loss_out; unsigned long long* violators;
+};
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits,
                        float* grad_rows, int dim, float* w0, float* g0, int64_t rows0, float* w1,
                        float* g1, int64_t rows1, float lr, hipStream_t stream, const uint32_t* long_runs = nullptr,
-                       const CosBack* cos_back = nullptr);
+                       const CosBack* cos_back = nullptr, const BatchSums* sums = nullptr);
 
 // ---- plain fp32 batched GEMM on MFMA ----------------------------------------
 // C[b] (M x N, row-major, ldc) = alpha * A[b] * B[b] + beta * C[b], for b in [0, batch).

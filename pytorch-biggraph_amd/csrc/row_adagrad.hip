@@ -218,6 +218,38 @@ __device__ __forceinline__ bool any_long_run(const uint32_t* __restrict__ long_r
   return __ballot(any != 0u) != 0ull;
 }
 
+// One workgroup (kRowThreads = 256 threads): the totals of batch b, summed in a fixed order.
+__device__ __forceinline__ void batch_sums_block(const BatchSums& bs, int b) {
+  __shared__ float sh[kRowThreads];
+  __shared__ long long shv[2][kRowThreads];
+  const float* rows = bs.lossrow + (int64_t)b * bs.per_batch;
+  const int* viol = bs.violrow + (int64_t)b * bs.per_batch * 2;
+  float acc = 0.f;
+  long long v0 = 0, v1 = 0;
+  for (int q = threadIdx.x; q < bs.per_batch; q += kRowThreads) {
+    acc += rows[q];
+    v0 += viol[q * 2];
+    v1 += viol[q * 2 + 1];
+  }
+  sh[threadIdx.x] = acc;
+  shv[0][threadIdx.x] = v0;
+  shv[1][threadIdx.x] = v1;
+  __syncthreads();
+  for (int off = kRowThreads / 2; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) {
+      sh[threadIdx.x] += sh[threadIdx.x + off];
+      shv[0][threadIdx.x] += shv[0][threadIdx.x + off];
+      shv[1][threadIdx.x] += shv[1][threadIdx.x + off];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    bs.loss_out[b] = sh[0];
+    bs.violators[b * 2] = (unsigned long long)shv[0][0];
+    bs.violators[b * 2 + 1] = (unsigned long long)shv[1][0];
+  }
+}
+
 // leave_mode 0: every piece of two or more positions is summed; 1 (single-worker calls): pieces of runs
 // of at most kFoldMax positions are left to the update kernel; 2 (row_walk_kernel follows): whole runs
 // inside the tile are left alone.
@@ -225,7 +257,12 @@ template <int NV, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t* __restrict__ keys,
                                                                   const uint32_t* __restrict__ vals, int64_t n,
                                                                   float* __restrict__ grad_rows, int dim,
-                                                                  int leave_mode, const uint32_t* __restrict__ long_runs) {
+                                                                  int leave_mode, const uint32_t* __restrict__ long_runs,
+                                                                  BatchSums sums, unsigned tile_blocks) {
+  if (blockIdx.x >= tile_blocks) {  // the workgroups behind the tiles': one per batch of `sums`
+    batch_sums_block(sums, (int)(blockIdx.x - tile_blocks));
+    return;
+  }
   if (leave_mode == 1 && long_runs && !any_long_run(long_runs)) return;  // the sort saw no run of more than kFoldMax positions
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * (kRowThreads / kWave) + (threadIdx.x >> 6);
@@ -890,10 +927,11 @@ __global__ void async_adagrad_dense_kernel(float* __restrict__ p, float* __restr
 template <bool VEC, bool COSB>
 int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                   int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                  const uint32_t* long_runs, CosBack cb, hipStream_t stream) {
+                  const uint32_t* long_runs, CosBack cb, BatchSums sums, hipStream_t stream) {
   const int wpb = kRowThreads / kWave;
   const dim3 block(kRowThreads);
-  const dim3 tile_grid((unsigned)ceil_div(ceil_div(n, kTile), wpb));
+  const unsigned tile_blocks = (unsigned)ceil_div(ceil_div(n, kTile), wpb);
+  const dim3 tile_grid(tile_blocks + (unsigned)sums.batches);
   const int64_t borders = ceil_div(n, kTile) - 1;
   const dim3 border_grid((unsigned)ceil_div(borders > 0 ? borders : 1, wpb));
   // gradient rows outnumbering the tables' rows 32 times over: a wave per table row (row_walk_kernel)
@@ -904,7 +942,7 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 #define PBG_LAUNCH(NV)                                                                                             \
   do {                                                                                                             \
     hipLaunchKernelGGL((tile_reduce_kernel<NV, VEC>), tile_grid, block, 0, stream, keys, vals, n, grad_rows, dim,       \
-                       leave_mode, long_runs);                                                                     \
+                       leave_mode, long_runs, sums, tile_blocks);                                                  \
     if (borders > 0)                                                                                              \
       hipLaunchKernelGGL((run_combine_kernel<NV, VEC>), border_grid, block, 0, stream, keys, vals, n, grad_rows, dim,  \
                          leave_mode, long_runs);                                                                   \
@@ -942,20 +980,28 @@ int launch_sorted(int nvec, const uint64_t* keys, const uint32_t* vals, int64_t 
 
 int row_adagrad_sorted(const uint64_t* keys, const uint32_t* vals, int64_t n, int kbits, float* grad_rows,
                        int dim, float* w0, float* g0, int64_t rows0, float* w1, float* g1, int64_t rows1, float lr,
-                       hipStream_t stream, const uint32_t* long_runs, const CosBack* cos_back) {
-  if (n <= 0) return PBG_OK;
+                       hipStream_t stream, const uint32_t* long_runs, const CosBack* cos_back, const BatchSums* sums_in) {
+  const BatchSums sums = sums_in ? *sums_in : BatchSums{nullptr, nullptr, 0, 0, nullptr, nullptr};
+  if (n <= 0) {  // no gradient rows: a launch that only carries the sums, if any
+    if (sums.batches > 0) {
+      hipLaunchKernelGGL((tile_reduce_kernel<1, true>), dim3((unsigned)sums.batches), dim3(kRowThreads), 0, stream, keys, vals,
+                         (int64_t)0, grad_rows, dim, 0, (const uint32_t*)nullptr, sums, 0u);
+      return check_launch("row_adagrad_sorted");
+    }
+    return PBG_OK;
+  }
   int rc;
   const CosBack none{nullptr, nullptr, nullptr, nullptr};
   if (cos_back) {
     if (dim % 4 != 0) return fail(PBG_ERR_UNSUPPORTED, "row_adagrad: the normalisation backward needs dim %% 4 == 0");
     rc = launch_sorted<true, true>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
-                                   g1, rows1, lr, long_runs, *cos_back, stream);
+                                   g1, rows1, lr, long_runs, *cos_back, sums, stream);
   } else if (dim % 4 == 0) {
     rc = launch_sorted<true, false>((int)ceil_div(dim / 4, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1,
-                                    g1, rows1, lr, long_runs, none, stream);
+                                    g1, rows1, lr, long_runs, none, sums, stream);
   } else {
     rc = launch_sorted<false, false>((int)ceil_div(dim, kWave), keys, vals, n, kbits, grad_rows, dim, w0, g0, rows0, w1, g1,
-                                     rows1, lr, long_runs, none, stream);
+                                     rows1, lr, long_runs, none, sums, stream);
   }
   if (rc != PBG_OK) return rc;
   return check_launch("row_adagrad_sorted");

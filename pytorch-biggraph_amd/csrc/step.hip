@@ -653,39 +653,6 @@ __global__ __launch_bounds__(kRowThreads) void loss_kernel(StepCtx c) {
   }
 }
 
-// loss_out[k] = sum of the batch's per-edge losses, in a fixed order; violators likewise
-__global__ __launch_bounds__(256) void loss_reduce_kernel(StepCtx c) {
-  __shared__ float sh[256];
-  __shared__ long long shv[2][256];
-  const int CP = c.C * c.P;
-  const float* rows = c.lossrow + (int64_t)blockIdx.x * CP;
-  const int* viol = c.violrow + (int64_t)blockIdx.x * CP * 2;
-  float acc = 0.f;
-  long long v0 = 0, v1 = 0;
-  for (int q = threadIdx.x; q < CP; q += 256) {
-    acc += rows[q];
-    v0 += viol[q * 2];
-    v1 += viol[q * 2 + 1];
-  }
-  sh[threadIdx.x] = acc;
-  shv[0][threadIdx.x] = v0;
-  shv[1][threadIdx.x] = v1;
-  __syncthreads();
-  for (int off = 128; off > 0; off >>= 1) {
-    if ((int)threadIdx.x < off) {
-      sh[threadIdx.x] += sh[threadIdx.x + off];
-      shv[0][threadIdx.x] += shv[0][threadIdx.x + off];
-      shv[1][threadIdx.x] += shv[1][threadIdx.x + off];
-    }
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    c.loss_out[blockIdx.x] = sh[0];
-    c.violators[blockIdx.x * 2] = (unsigned long long)shv[0][0];
-    c.violators[blockIdx.x * 2 + 1] = (unsigned long long)shv[1][0];
-  }
-}
-
 // forward-only output: de-chunked, masked scores (model.py:842-844)
 __global__ __launch_bounds__(kRowThreads) void scores_out_kernel(StepCtx c, float* __restrict__ lhs_pos,
                                                                  float* __restrict__ rhs_pos,
@@ -2567,7 +2534,6 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(5);
     mark(6);
     if ((rc = stream_finish(cs, plan.sp, plan.nvh, s)) != PBG_OK) return rc;
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
     launch_reg(c, s);
     mark(7);
   } else if (plan.fused) {
@@ -2615,7 +2581,6 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(1);
     mark(2);
     mark(3);
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
     mark(4);
     mark(5);
     mark(6);
@@ -2628,7 +2593,6 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     if ((rc = run_scores(plan, s)) != PBG_OK) return rc;
     mark(3);
     launch_loss(c, s);
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3((unsigned)c.K), dim3(256), 0, s, c);
     mark(4);
     if ((rc = run_backward_dn(plan, s)) != PBG_OK) return rc;
     mark(5);
@@ -2658,13 +2622,15 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   }
   mark(9);
   if (c.kbits != 0) long_runs = nullptr;  // the word counts positions per ROW; only with one batch per call is that a run
+  // loss_out[k] and violators[k]: the batches' sums of the per-edge values, with the update's first launch
+  const BatchSums sums{c.lossrow, c.violrow, c.C * c.P, c.K, c.loss_out, c.violators};
   if (desc->shared_table) {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
-                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s, long_runs, cos_back_p);
+                            desc->num_lhs_rows, nullptr, nullptr, 0, desc->lr, s, long_runs, cos_back_p, &sums);
   } else {
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s, long_runs,
-                            cos_back_p);
+                            cos_back_p, &sums);
   }
   mark(10);
   return rc;
