@@ -291,10 +291,15 @@ __global__ __launch_bounds__(kRowThreads) void tile_reduce_kernel(const uint64_t
     before = same_before == kAll ? kFoldMax : __ffs((int)~same_before) - 1;  // leading ones
     after = same_after == kAll ? kFoldMax : __ffs((int)~same_after) - 1;
   }
-  while (heads != 0ull) {
-    const int a = __ffsll((unsigned long long)heads) - 1;
-    heads &= heads - 1;
-    const int b = heads != 0ull ? (__ffsll((unsigned long long)heads) - 1) : (int)(end - begin);
+  // Only a piece of two or more positions has anything to sum: a start whose next position exists and is no start.
+  // (Without duplicates -- most tiles of most calls -- the loop below does not run at all.)
+  const int len = (int)(end - begin);
+  uint64_t multi = heads & ~(heads >> 1) & (((1ull << len) - 1ull) >> 1);
+  while (multi != 0ull) {
+    const int a = __ffsll((unsigned long long)multi) - 1;
+    multi &= multi - 1;
+    const uint64_t later = heads & ~((2ull << a) - 1ull);
+    const int b = later != 0ull ? (__ffsll((unsigned long long)later) - 1) : len;
     if (leave_mode != 0) {
       const bool whole = (a > 0 || before == 0) && (b < (int)(end - begin) || after == 0);
       if (leave_mode == 2 && whole) continue;  // (a single position needs no sum either way)
