@@ -663,11 +663,11 @@ class Workload:
                 acc = ms if acc is None else [a + m for a, m in zip(acc, ms)]
             stages = dict(zip(runner.STAGES, [a / profile_calls for a in acc]))
             if runner.route == "fused":
-                # one kernel covers stages "prep" .. "rowback"; "loss" holds the per-batch reduction of the statistics
-                stages = {"fused_chunk": stages["prep"], "loss_reduce": stages["loss"], "params": stages["params"],
+                # one kernel covers stages "prep" .. "rowback" (the batches' sums of the statistics ride with the update)
+                stages = {"fused_chunk": stages["prep"], "params": stages["params"],
                           "sort": stages["sort"], "update": stages["update"]}
             elif runner.route == "stream":
-                # per-edge preparation + column ids | the chunk kernel | per-edge finish + the statistics' reduction
+                # per-edge preparation + column ids | the chunk kernel | per-edge finish
                 stages = {"stream_prep": stages["prep"], "stream_chunk": stages["scores"], "stream_finish": stages["rowback"],
                           "params": stages["params"], "sort": stages["sort"], "update": stages["update"]}
         loss = float(runner.loss_out.mean().item()) / b
