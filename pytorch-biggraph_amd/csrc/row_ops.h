@@ -319,6 +319,12 @@ __device__ __forceinline__ float sigmoidf(float z) {
   const float e = expf(z);
   return e / (1.0f + e);
 }
+// e^(x - m) for the softmax's terms (x <= m): the hardware's 2^y (1 ulp) on (x - m) log2 e, the subtraction first --
+// the correctly rounded expf costs a dozen instructions, twice per score of a row of a thousand, which made the
+// loss kernel arithmetic-bound; the same form as the streaming route's, and every term of a row (the positive's
+// included) goes through it, so that terms that must cancel still do.
+__device__ __forceinline__ float exp_below(float x, float m) { return __builtin_amdgcn_exp2f((x - m) * 1.4426950408889634f); }
+
 // softplus(z) and sigmoid(z) from one exponential (the same values as the two functions above)
 __device__ __forceinline__ float softplus_sigmoid(float z, float* sigmoid) {
   const float e = expf(-fabsf(z));

@@ -449,12 +449,12 @@ __device__ __forceinline__ void side_loss_held(int loss, float margin, int cmp, 
     mx = wave_max(mx);
     float z = 0.f;
 #pragma unroll
-    for (int u = 0; u < DEPTH; ++u) z += expf(t[u] - mx);
-    z = wave_sum(z) + expf(pos - mx);
+    for (int u = 0; u < DEPTH; ++u) z += exp_below(t[u], mx);
+    z = wave_sum(z) + exp_below(pos, mx);
     inv_z = 1.0f / z;
     if (first == 0) {
       *loss_acc += (mx + logf(z)) - pos;
-      dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+      dpos_part += (exp_below(pos, mx) * inv_z - 1.0f) * w;
     }
   } else if (loss == PBG_LOSS_LOGISTIC) {
     if (first == 0) {
@@ -480,7 +480,7 @@ __device__ __forceinline__ void side_loss_held(int loss, float margin, int cmp, 
       *loss_acc += softplus_sigmoid(tu, &sg) * inv_nn;
       g = sg * inv_nn * w;
     } else {
-      g = expf(tu - mx) * inv_z * w;
+      g = exp_below(tu, mx) * inv_z * w;
     }
     if (tu > pos) ++viol;
     if (!live) g = 0.f;
@@ -517,12 +517,12 @@ __device__ __forceinline__ void side_loss_long(int loss, float margin, int cmp, 
     for (int j = first; j < nn; j += kWave) mx = fmaxf(mx, sr.at(j, &live));
     mx = wave_max(mx);
     float z = 0.f;
-    for (int j = first; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
-    z = wave_sum(z) + expf(pos - mx);
+    for (int j = first; j < nn; j += kWave) z += exp_below(sr.at(j, &live), mx);
+    z = wave_sum(z) + exp_below(pos, mx);
     inv_z = 1.0f / z;
     if (first == 0) {
       *loss_acc += (mx + logf(z)) - pos;
-      dpos_part += (expf(pos - mx) * inv_z - 1.0f) * w;
+      dpos_part += (exp_below(pos, mx) * inv_z - 1.0f) * w;
     }
   } else if (loss == PBG_LOSS_LOGISTIC) {
     if (first == 0) {
@@ -543,7 +543,7 @@ __device__ __forceinline__ void side_loss_long(int loss, float margin, int cmp, 
       *loss_acc += softplus_sigmoid(t, &sg) * inv_nn;
       g = sg * inv_nn * w;
     } else {
-      g = expf(t - mx) * inv_z * w;
+      g = exp_below(t, mx) * inv_z * w;
     }
     if (t > pos) ++viol;
     if (!live) g = 0.f;
@@ -706,8 +706,8 @@ __device__ __forceinline__ void row_rank_and_loss(int loss, float margin, const 
   if (loss == PBG_LOSS_SOFTMAX) {
     mx = wave_max(mx);
     float z = 0.f;
-    for (int j = lane; j < nn; j += kWave) z += expf(sr.at(j, &live) - mx);
-    z = wave_sum(z) + expf(pos - mx);
+    for (int j = lane; j < nn; j += kWave) z += exp_below(sr.at(j, &live), mx);
+    z = wave_sum(z) + exp_below(pos, mx);
     if (lane == 0) *loss_acc += (mx + logf(z)) - pos;
   } else if (loss == PBG_LOSS_LOGISTIC) {
     if (lane == 0) *loss_acc += softplusf(-pos);
