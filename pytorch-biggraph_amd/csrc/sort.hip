@@ -298,7 +298,7 @@ __device__ __forceinline__ void wide_fetch(const uint64_t* __restrict__ keys_in,
 __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out, int64_t n, int tile_shift, int shift, int digit_bits,
-    const uint32_t* __restrict__ counts, uint32_t* __restrict__ bucket_off) {
+    const uint32_t* __restrict__ counts, uint32_t* __restrict__ bucket_off, uint32_t* __restrict__ bucket_order) {
   __shared__ SliceState<kGlobalWaves, kMaxDigitBits> st;
   __shared__ uint32_t part[2][2][kMaxDigits];  // [half][total, before][digit]
   const int t = threadIdx.x;
@@ -343,6 +343,17 @@ __global__ __launch_bounds__(kGlobalWaves * 64) void sort_scatter_kernel(
     if (me == 0) bucket_off[t] = excl;  // digits past the pass's width hold no keys: their offset is n
   }
   if (me == 0 && t == 0) bucket_off[kMaxDigits] = grand;
+  // The order in which the bucket passes' launch takes the buckets: those swollen by a hot key first (more than four
+  // times the mean), the others behind them, each group by digit.  A swollen bucket is one workgroup's long chain of
+  // slices, and it should be the first to start, not wait behind hundreds of ordinary ones.  The last block writes
+  // the order (its tile is the one that may be short).
+  if (bucket_order && me == blocks - 1) {
+    const uint32_t limit = 4u * (grand >> digit_bits) + 1024u;
+    const uint32_t big = (t < kMaxDigits && total > limit) ? 1u : 0u;
+    uint32_t num_big;
+    const uint32_t big_before = block_exclusive_scan(big, kMaxDigits / 64, st.wave_total, &num_big);
+    if (t < kMaxDigits) bucket_order[big ? big_before : num_big + ((uint32_t)t - big_before)] = (uint32_t)t;
+  }
   __syncthreads();
   scatter_range_wide<kGlobalWaves, kMaxDigitBits, kGlobalKpt>(st, keys_in, vals_in, keys_out, vals_out, begin, end,
                                                               shift, (1u << digit_bits) - 1u, first_keys, first_vals);
@@ -475,12 +486,14 @@ constexpr int kLdsMaxRestBits = 32 - kLdsIndexBits;  // ... and its remaining bi
 __global__ __launch_bounds__(kBucketWaves * 64) void sort_bucket_kernel(uint64_t* ka, uint32_t* va, uint64_t* kb,
                                                                         uint32_t* vb, uint64_t* kfin, uint32_t* vfin,
                                                                         const uint32_t* __restrict__ bucket_off,
+                                                                        const uint32_t* __restrict__ bucket_order,
                                                                         int low_bit, int rest, int passes, int cap,
                                                                         uint32_t* __restrict__ long_flag) {
   __shared__ SliceState<kBucketWaves, 8> st;
   extern __shared__ uint32_t lds_words[];  // 2 * cap packed words
   const int t = threadIdx.x;
-  const int64_t begin = bucket_off[blockIdx.x], end = bucket_off[blockIdx.x + 1];
+  const uint32_t bucket = bucket_order[blockIdx.x];  // largest first
+  const int64_t begin = bucket_off[bucket], end = bucket_off[bucket + 1];
   if (begin >= end) return;
   const int64_t m64 = end - begin;
   // (a single digit pass gains nothing from the detour through LDS: one read and one write either way)
@@ -639,7 +652,7 @@ __global__ __launch_bounds__(kRankWaves * 64) void sort_rank_kernel(
 
 size_t sort_temp_bytes(int64_t n) {
   SortPlan p = plan_sort(n);
-  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 1 + kLongWords) * sizeof(uint32_t), 256);
+  return align_up(((size_t)kMaxDigits * p.blocks + kMaxDigits + 1 + kLongWords + kMaxDigits) * sizeof(uint32_t), 256);
 }
 
 namespace {
@@ -660,6 +673,7 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   uint32_t* counts = (uint32_t*)temp;
   uint32_t* bucket_off = counts + (size_t)kMaxDigits * p.blocks;
   uint32_t* long_flag = bucket_off + kMaxDigits + 1;
+  uint32_t* bucket_order = long_flag + kLongWords;  // [kMaxDigits]
   int bits = key_bits - low_bit;
   if (bits < 1) bits = 1;
   if (n <= kRankMax && bits <= 32 && getenv("PBG_DISABLE_RANK_SORT") == nullptr) {  // one launch, see sort_rank_kernel
@@ -690,7 +704,7 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   hipLaunchKernelGGL(sort_hist_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, n, p.tile_shift,
                      top_shift, top, counts, long_flag, local == 0 ? 1u : 0u, indices, park, vals_in);
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(p.blocks), dim3(kGlobalWaves * 64), 0, stream, keys_in, vals_in,
-                     keys_out, vals_out, n, p.tile_shift, top_shift, top, counts, bucket_off);
+                     keys_out, vals_out, n, p.tile_shift, top_shift, top, counts, bucket_off, local > 0 ? bucket_order : nullptr);
   if (long_runs) *long_runs = long_flag;
   if (local == 0) {
     *keys_sorted = keys_out;
@@ -707,7 +721,7 @@ int sort_pairs(uint64_t* keys_in, uint32_t* vals_in, uint64_t* keys_out, uint32_
   uint64_t* kfin = (local & 1) ? keys_in : keys_out;
   uint32_t* vfin = (local & 1) ? vals_in : vals_out;
   hipLaunchKernelGGL(sort_bucket_kernel, dim3(1u << top), dim3(kBucketWaves * 64), lds_bytes, stream, keys_out, vals_out,
-                     keys_in, vals_in, kfin, vfin, bucket_off, low_bit, rest, local, (int)cap,
+                     keys_in, vals_in, kfin, vfin, bucket_off, bucket_order, low_bit, rest, local, (int)cap,
                      long_runs ? long_flag : nullptr);
   *keys_sorted = kfin;
   *vals_sorted = vfin;

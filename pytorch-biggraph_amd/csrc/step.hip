@@ -2420,7 +2420,7 @@ constexpr int kStages = 10;
 // event pairs, so that consecutive calls do not share one.  Default priority, like every stream here.
 struct SideStream {
   hipStream_t stream = nullptr;
-  hipEvent_t fork[8], join[8];
+  hipEvent_t fork[8], join[8], mid[8], tail[8];
   std::atomic<unsigned> next{0};
   bool ok = false;
 };
@@ -2437,7 +2437,9 @@ SideStream* side_stream() {
     bool ok = hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking) == hipSuccess;
     for (int i = 0; ok && i < 8; ++i)
       ok = hipEventCreateWithFlags(&ss.fork[i], hipEventDisableTiming) == hipSuccess &&
-           hipEventCreateWithFlags(&ss.join[i], hipEventDisableTiming) == hipSuccess;
+           hipEventCreateWithFlags(&ss.join[i], hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&ss.mid[i], hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&ss.tail[i], hipEventDisableTiming) == hipSuccess;
     ss.ok = ok;
     if (!ok) (void)hipGetLastError();
   }
@@ -2499,11 +2501,13 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
   // under a HIP graph capture an unjoined fork leaves the library's stream inside the caller's capture.
   struct JoinOnExit {
     hipStream_t into;
-    hipEvent_t ev = nullptr;
+    hipEvent_t ev = nullptr, ev2 = nullptr;
     ~JoinOnExit() {
       if (ev) (void)hipStreamWaitEvent(into, ev, 0);
+      if (ev2) (void)hipStreamWaitEvent(into, ev2, 0);
     }
   } join_guard{s};
+  hipEvent_t params_done = nullptr;  // set: the operator parameters' kernels were queued on the side stream
   mark(0);
   if ((rc = run_renorm(plan, bufs, s)) != PBG_OK) return rc;
   CosBack cos_back{nullptr, nullptr, nullptr, nullptr};
@@ -2577,6 +2581,19 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
         return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
       join_guard.ev = sort_done = ss->join[slot];
       if (sort_rc != PBG_OK) return sort_rc;
+      // A translation's gradient and Adagrad steps read the operator-output gradients the chunk kernel left and
+      // write the operator's parameters: nothing the table update touches (a diagonal's gradient reads table rows).
+      // Two short launches with a handful of waves each: behind the sort on the side stream they run beside the
+      // update instead of in front of it.
+      if (c.op == PBG_OP_TRANSLATION && !bufs->lhs_global && getenv("PBG_DISABLE_SIDE_PARAMS") == nullptr) {
+        if (hipEventRecord(ss->mid[slot], s) != hipSuccess || hipStreamWaitEvent(ss->stream, ss->mid[slot], 0) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot order the side stream behind the chunk kernel");
+        const int params_rc = run_params(desc, bufs, plan, ss->stream, &rel_order, false);
+        if (hipEventRecord(ss->tail[slot], ss->stream) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's second join");
+        join_guard.ev2 = params_done = ss->tail[slot];
+        if (params_rc != PBG_OK) return params_rc;
+      }
     }
     mark(1);
     mark(2);
@@ -2602,7 +2619,7 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     launch_reg(c, s);
     mark(7);
   }
-  if ((rc = run_params(desc, bufs, plan, s, &rel_order, stream)) != PBG_OK) return rc;
+  if (!params_done && (rc = run_params(desc, bufs, plan, s, &rel_order, stream)) != PBG_OK) return rc;
   if (bufs->lhs_global) {  // the raw-row gradients are complete and still one per gathered row
     hipLaunchKernelGGL(global_grad_kernel, dim3((unsigned)c.K, (unsigned)(2 * plan.gslices)), dim3(kGlobalHalves * 32), 0,
                        s, c, plan.gth, plan.gslices, plan.fused ? 1 : 0);
@@ -2631,6 +2648,10 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     rc = row_adagrad_sorted(skeys, svals, npairs, c.kbits, c.gr, c.D, bufs->w_lhs, bufs->g_lhs,
                             desc->num_lhs_rows, bufs->w_rhs, bufs->g_rhs, desc->num_rhs_rows, desc->lr, s, long_runs,
                             cos_back_p, &sums);
+  }
+  if (params_done) {
+    join_guard.ev2 = nullptr;
+    if (hipStreamWaitEvent(s, params_done, 0) != hipSuccess) return fail(PBG_ERR_LAUNCH, "step: cannot join the side stream");
   }
   mark(10);
   return rc;
