@@ -12,11 +12,12 @@
  *   - the caller owns every buffer, including workspaces (query the *_bytes
  *     function, allocate, pass in); the library never allocates device memory;
  *   - work is enqueued on `stream` (a hipStream_t) and the call returns without
- *     synchronising.  pbg_train_step may also run its key sort on one more
- *     stream that the library creates per device on first use (default
- *     priority): it is forked from `stream` and joined back into it with two
- *     events inside the call, so the caller sees the step's work as if it were
- *     all on `stream` (a HIP graph capture records the fork and the join);
+ *     synchronising.  pbg_train_step may also run its key sort (and behind it
+ *     the parameter kernels of a translation operator) on one more stream that
+ *     the library creates per device on first use (default priority): it is
+ *     forked from `stream` and joined back into it with events inside the
+ *     call, so the caller sees the step's work as if it were all on `stream`
+ *     (a HIP graph capture records the forks and the joins);
  *   - return value: PBG_OK or a negative pbg_status; pbg_last_error() gives the
  *     message of the last failure on the calling thread.
  */
