@@ -2533,6 +2533,22 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(1);
     mark(2);
     if ((rc = stream_chunks(cs, plan.sp, s)) != PBG_OK) return rc;
+    // The sort needs the keys alone (made before the chunk kernel): on the side stream it runs beside the per-edge
+    // finish and the parameter kernels instead of behind them.  (Beside the chunk kernel itself there is no room:
+    // its workgroups hold every compute unit's LDS.)
+    if (2 * c.K * c.C >= 128 && getenv("PBG_DISABLE_SIDE_STREAM") == nullptr) {
+      if (SideStream* ss = side_stream()) {
+        const unsigned slot = ss->next.fetch_add(1) & 7u;
+        if (hipEventRecord(ss->fork[slot], s) != hipSuccess || hipStreamWaitEvent(ss->stream, ss->fork[slot], 0) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
+        const int sort_rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp,
+                                       ss->stream, &skeys, &svals, c.kbits == 0 ? &long_runs : nullptr);
+        if (hipEventRecord(ss->join[slot], ss->stream) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
+        join_guard.ev = sort_done = ss->join[slot];
+        if (sort_rc != PBG_OK) return sort_rc;
+      }
+    }
     mark(3);
     mark(4);
     mark(5);
