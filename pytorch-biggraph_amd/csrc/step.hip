@@ -2620,6 +2620,21 @@ int run_step(const pbg_step_desc* desc, const pbg_step_buffers* bufs, hipStream_
     mark(7);
   } else {
     if ((rc = run_prep(plan, s)) != PBG_OK) return rc;
+    // The keys exist from here on and nothing before the update looks at them again (the global embeddings'
+    // gradient kernel does: not with those): a large call sorts them on the side stream beside the products.
+    if ((int64_t)c.K * c.C * c.P >= 16384 && !bufs->lhs_global && getenv("PBG_DISABLE_SIDE_STREAM") == nullptr) {
+      if (SideStream* ss = side_stream()) {
+        const unsigned slot = ss->next.fetch_add(1) & 7u;
+        if (hipEventRecord(ss->fork[slot], s) != hipSuccess || hipStreamWaitEvent(ss->stream, ss->fork[slot], 0) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot fork the side stream");
+        const int sort_rc = sort_pairs(c.keys, c.vals, plan.keys_b, plan.vals_b, npairs, c.kbits, sort_bits, plan.sort_temp,
+                                       ss->stream, &skeys, &svals, c.kbits == 0 ? &long_runs : nullptr);
+        if (hipEventRecord(ss->join[slot], ss->stream) != hipSuccess)
+          return fail(PBG_ERR_LAUNCH, "step: cannot record the side stream's join");
+        join_guard.ev = sort_done = ss->join[slot];
+        if (sort_rc != PBG_OK) return sort_rc;
+      }
+    }
     mark(1);
     if ((rc = run_operator_forward(plan, s, &rel_order)) != PBG_OK) return rc;
     mark(2);
